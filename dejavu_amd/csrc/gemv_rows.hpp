@@ -1,0 +1,155 @@
+// Row-wise GEMV kernels: every output element is the dot product of one weight
+// row (contiguous in memory) with an activation vector.  Lanes of a wavefront
+// stride along the row with 128-bit loads and reduce with a butterfly.
+//
+//  * canonical_gemv_kernel : dense rows, fully specified summation order
+//                            (predictor fc0 / fc1, bit-exact contract)
+//  * gather_rows_kernel    : rows picked by an index vector, bias + activation
+//                            fused (sparse-MLP fc1)
+#pragma once
+#include "common.hpp"
+
+namespace dv {
+
+// ---------------------------------------------------------------------------
+// Y[b, row] = fp16( sum_i W[row, i] * X[b, i] ) with the canonical order:
+// lane `sub` of the LANES lanes that share a row folds elements
+// c*8*LANES + 8*sub + e (c ascending, e = 0..7) into one fp32 accumulator, then
+// the LANES partials are combined with an xor butterfly (LANES/2 .. 1).
+// Requires n % 8 == 0 and ldw % 8 == 0.
+// ---------------------------------------------------------------------------
+template <int LANES, int B, int U>
+__global__ __launch_bounds__(256) void canonical_gemv_kernel(
+    const half_t* __restrict__ X, const half_t* __restrict__ W, int64_t ldw, int rows, int n,
+    half_t* __restrict__ Y) {
+  constexpr int RW = kWave / LANES;  // rows per wavefront pass
+  constexpr int CH = 8 * LANES;      // elements per chunk
+  const int lane = threadIdx.x & 63;
+  const int sub = lane % LANES;
+  const int grp = lane / LANES;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int waves_per_block = blockDim.x >> 6;
+  const int ntasks = (rows + RW - 1) / RW;
+  for (int t = blockIdx.x * waves_per_block + wave; t < ntasks; t += gridDim.x * waves_per_block) {
+    const int row = t * RW + grp;
+    const bool valid = row < rows;
+    const half_t* wr = W + (int64_t)(valid ? row : 0) * ldw + sub * 8;
+    const half_t* xr = X + sub * 8;
+    float acc[B];
+#pragma unroll
+    for (int b = 0; b < B; ++b) acc[b] = 0.f;
+    int base = 0;
+    for (; base + U * CH <= n; base += U * CH) {
+      half8_t w[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) w[u] = load8_stream(wr + base + u * CH);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+#pragma unroll
+        for (int b = 0; b < B; ++b)
+          acc[b] = fma8_ordered(w[u], load8(xr + (int64_t)b * n + base + u * CH), acc[b]);
+      }
+    }
+    for (; base < n; base += CH) {
+      if (base + sub * 8 < n) {
+        half8_t w = load8_stream(wr + base);
+#pragma unroll
+        for (int b = 0; b < B; ++b)
+          acc[b] = fma8_ordered(w, load8(xr + (int64_t)b * n + base), acc[b]);
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < B; ++b) acc[b] = butterfly_sum<LANES>(acc[b]);
+    if (valid && sub == 0) {
+#pragma unroll
+      for (int b = 0; b < B; ++b) Y[(int64_t)b * rows + row] = (half_t)acc[b];
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Y[b, m] = act( sum_i W[idx[m], i] * X[b, i] + bias[idx[m]] ), fp16 out.
+// One wavefront owns R gathered rows at a time (R independent load streams);
+// X is staged once per workgroup in LDS.  An index outside [0, Z) yields 0
+// instead of a wild read.  Requires n % 8 == 0 and ldw % 8 == 0.
+// ---------------------------------------------------------------------------
+template <int B, int R, int U, bool RELU>
+__global__ __launch_bounds__(256) void gather_rows_kernel(
+    const half_t* __restrict__ X, const half_t* __restrict__ W, const half_t* __restrict__ bias,
+    const void* __restrict__ idx, int idx_bytes, int n, int64_t ldw, int Z, int M,
+    half_t* __restrict__ Y) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  half_t* xs = reinterpret_cast<half_t*>(smem_raw);
+  for (int i = threadIdx.x * 8; i < B * n; i += blockDim.x * 8) store8(xs + i, load8(X + i));
+  __syncthreads();
+
+  constexpr int CH = 8 * kWave;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int waves_per_block = blockDim.x >> 6;
+  const int ntasks = (M + R - 1) / R;
+  for (int t = blockIdx.x * waves_per_block + wave; t < ntasks; t += gridDim.x * waves_per_block) {
+    const half_t* wr[R];
+    bool valid[R];
+    int64_t rid[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int m = t * R + r;
+      int64_t id = m < M ? load_index(idx, idx_bytes, m) : -1;
+      valid[r] = id >= 0 && id < Z;
+      rid[r] = valid[r] ? id : 0;
+      wr[r] = W + rid[r] * ldw + lane * 8;
+    }
+    float acc[R][B];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int b = 0; b < B; ++b) acc[r][b] = 0.f;
+
+    int base = 0;
+    for (; base + U * CH <= n; base += U * CH) {
+      half8_t w[U][R];
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int r = 0; r < R; ++r) w[u][r] = load8_stream(wr[r] + base + u * CH);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+#pragma unroll
+        for (int b = 0; b < B; ++b) {
+          const half8_t xv = load8(xs + b * n + base + u * CH + lane * 8);
+#pragma unroll
+          for (int r = 0; r < R; ++r) acc[r][b] = dot8_fast(w[u][r], xv, acc[r][b]);
+        }
+      }
+    }
+    for (; base < n; base += CH) {
+      if (base + lane * 8 < n) {
+        half8_t w[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) w[r] = load8_stream(wr[r] + base);
+#pragma unroll
+        for (int b = 0; b < B; ++b) {
+          const half8_t xv = load8(xs + b * n + base + lane * 8);
+#pragma unroll
+          for (int r = 0; r < R; ++r) acc[r][b] = dot8_fast(w[r], xv, acc[r][b]);
+        }
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int m = t * R + r;
+      float bv = 0.f;
+      if (bias != nullptr && valid[r]) bv = (float)bias[rid[r]];
+#pragma unroll
+      for (int b = 0; b < B; ++b) {
+        float v = butterfly_sum<kWave>(acc[r][b]) + bv;
+        if (RELU) v = relu_f(v);
+        if (!valid[r]) v = 0.f;
+        if (lane == 0 && m < M) Y[(int64_t)b * M + m] = (half_t)v;
+      }
+    }
+  }
+}
+
+}  // namespace dv

@@ -1,0 +1,491 @@
+"""CPU restatement (numpy) of DejaVu's contextual-sparsity decode path.
+
+TEST INFRASTRUCTURE ONLY -- never imported by the product package.
+
+Every function cites the reference file:line whose arithmetic it restates
+(paths relative to the reference checkout).  Storage dtype is fp16
+(``np.float16``), accumulation is fp32 unless a function says otherwise, and
+index outputs are integer arrays.
+
+How each function is pinned (see tests/test_oracle.py):
+
+* ``gather_gemv`` / ``gather_transposed_gemv`` / ``mlp_sparse``: against the
+  dense-then-masked form the accuracy simulator uses, against a pure-Python
+  brute force on tiny shapes, and against the dense library routine when
+  idx = arange(Z).
+* ``topk_lower_index``: against an O(n*k) brute-force selection, including
+  all-equal inputs, +-0 and ties straddling the boundary.
+* ``canonical_dot`` (the fixed summation order the predictor kernel uses):
+  against float64 dot products (error bound) and against a scalar pure-Python
+  walk of the same order (bit-exact).
+* ``qkv_proj_sparse`` / ``out_proj_sparse``: against the einsum expressions the
+  reference's own self-check prints (attention_proj_sparse.py:625-627, 646).
+* ``single_query_attention``: against
+  ``torch.nn.functional.scaled_dot_product_attention`` in fp32.
+  The reference calls an external FasterTransformer kernel here
+  (flash-attention v0.2.8 ``csrc/ft_attention``, not vendored) and holds no
+  vectors for it: parity unpinned against that binary, pinned against the
+  textbook definition the reference restates in CrossAttention.forward.
+* cache copies / window tracker: index arithmetic checked against a dense
+  always-recompute KV cache.
+* top-k tie order: the reference (``torch.topk(sorted=False)`` on CUDA) leaves
+  it unspecified and holds no vectors; the rule "ties go to the lower index" is
+  this build's definition: parity unpinned against the reference's CUDA tie
+  order, pinned against brute force for the stated rule.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+F16 = np.float16
+F32 = np.float32
+
+
+# --------------------------------------------------------------------------
+# helpers
+# --------------------------------------------------------------------------
+def f16_round(a) -> np.ndarray:
+    """Round an fp32/fp64 array to fp16 storage (round-to-nearest-even)."""
+    return np.asarray(a, dtype=F32).astype(F16)
+
+
+def relu(a: np.ndarray) -> np.ndarray:
+    """Dejavu/src/ops/triton/k_activations.py:73-80: ``where(x >= 0, x, 0)``."""
+    return np.where(a >= 0, a, np.zeros((), dtype=a.dtype))
+
+
+def _act(a: np.ndarray, activation: str) -> np.ndarray:
+    if activation == "id":
+        return a
+    if activation == "relu":
+        return relu(a)
+    raise ValueError(f"oracle implements 'id' and 'relu' only, got {activation!r}")
+
+
+# --------------------------------------------------------------------------
+# canonical fixed-order dot product (predictor numerics)
+# --------------------------------------------------------------------------
+def canonical_lanes(n: int) -> int:
+    """Lanes that cooperate on one row of length ``n`` in the predictor kernel.
+
+    Short rows (n <= 1024) are reduced by 16 lanes, longer ones by a whole
+    64-lane wavefront.  This is a definition of this build; the reference
+    leaves the summation order to cuBLAS (fused_dense_sparse_dejavu.py:124).
+    """
+    return 16 if n <= 1024 else 64
+
+
+def canonical_dot(W: np.ndarray, X: np.ndarray, lanes: int | None = None) -> np.ndarray:
+    """fp32 ``X @ W.T`` with a fully specified summation order.
+
+    W: (rows, n) fp16, X: (B, n) fp16 -> (B, rows) fp32.
+
+    Order: lane l of ``lanes`` owns elements ``c*8*lanes + 8*l + e`` for chunk
+    c = 0,1,.. and e = 0..7 and folds them into one fp32 accumulator in
+    (c, e) order, starting from +0; out-of-range elements contribute w = x = 0.
+    The ``lanes`` partial sums are then combined by an xor butterfly with
+    offsets lanes/2, .., 1 (``p[l] += p[l ^ off]``); lane 0 holds the result.
+    Products of two fp16 values are exact in fp32, so a fused multiply-add and
+    a separate multiply and add give the same bits.
+    """
+    W = np.asarray(W, dtype=F16)
+    X = np.asarray(X, dtype=F16)
+    rows, n = W.shape
+    B = X.shape[0]
+    assert X.shape == (B, n)
+    L = canonical_lanes(n) if lanes is None else lanes
+    chunk = 8 * L
+    C = -(-n // chunk)
+    pad = C * chunk - n
+    Wf = np.pad(W.astype(F32), ((0, 0), (0, pad))).reshape(rows, C, L, 8)
+    Xf = np.pad(X.astype(F32), ((0, 0), (0, pad))).reshape(B, C, L, 8)
+    out = np.empty((B, rows), dtype=F32)
+    lane = np.arange(L)
+    for b in range(B):
+        acc = np.zeros((rows, L), dtype=F32)
+        for c in range(C):
+            for e in range(8):
+                acc = acc + Wf[:, c, :, e] * Xf[b, c, :, e][None, :]
+        off = L // 2
+        while off >= 1:
+            acc = acc + acc[:, lane ^ off]
+            off //= 2
+        out[b] = acc[:, 0]
+    return out
+
+
+def canonical_dot_scalar(w_row, x_row, lanes: int) -> np.float32:
+    """Pure-Python walk of ``canonical_dot`` for one row (pins the vector form)."""
+    n = len(w_row)
+    part = [np.float32(0.0)] * lanes
+    chunk = 8 * lanes
+    C = -(-n // chunk)
+    for l in range(lanes):
+        acc = np.float32(0.0)
+        for c in range(C):
+            for e in range(8):
+                i = c * chunk + 8 * l + e
+                if i < n:
+                    acc = np.float32(acc + np.float32(w_row[i]) * np.float32(x_row[i]))
+        part[l] = acc
+    off = lanes // 2
+    while off >= 1:
+        part = [np.float32(part[l] + part[l ^ off]) for l in range(lanes)]
+        off //= 2
+    return part[0]
+
+
+# --------------------------------------------------------------------------
+# predictor + top-k
+# --------------------------------------------------------------------------
+def predictor_logits(x, Wa, Wb):
+    """Low-rank sparsity predictor, fp16 in / fp16 out.
+
+    Dejavu/src/ops/fused_dense_sparse_dejavu.py:73-76 (``fc1(fc0(x))``, both
+    bias-free; architecture fixed by sparse_predictor/main_mlp.py:150-153).
+    Both linears round their fp32-accumulated result to fp16, as nn.Linear in
+    fp16 does.  x: (B, d); Wa: (r, d); Wb: (out, r) -> (hidden (B, r) fp16,
+    logits (B, out) fp16).  The reference runs B = 1 only
+    (``x.view(self.embed_dim)``).
+    """
+    x = np.atleast_2d(np.asarray(x, dtype=F16))
+    hidden = canonical_dot(Wa, x).astype(F16)
+    logits = canonical_dot(Wb, hidden).astype(F16)
+    return hidden, logits
+
+
+def predictor_logits_f64(x, Wa, Wb):
+    """Same predictor in float64 with the fp16 rounding of the hidden vector
+    kept; used only to bound the error of the canonical order."""
+    x = np.atleast_2d(np.asarray(x, dtype=F16)).astype(np.float64)
+    hidden = (x @ np.asarray(Wa, dtype=np.float64).T).astype(F16)
+    return hidden, hidden.astype(np.float64) @ np.asarray(Wb, dtype=np.float64).T
+
+
+def topk_key(logits: np.ndarray) -> np.ndarray:
+    """Monotone map fp16 -> uint16 used for selection.
+
+    Larger logit <=> larger key; -0 and +0 share one key; every NaN maps to the
+    top key 0xFFFF (torch.topk also ranks NaN above everything).
+    """
+    h = np.asarray(logits, dtype=F16)
+    bits = h.view(np.uint16).astype(np.uint32)
+    bits = np.where(bits == 0x8000, 0, bits)
+    key = np.where(bits & 0x8000, (~bits) & 0xFFFF, bits | 0x8000)
+    key = np.where(np.isnan(h), 0xFFFF, key)
+    return key.astype(np.uint16)
+
+
+def batch_scores(logits: np.ndarray) -> np.ndarray:
+    """Per-neuron score for a batch: the maximum key over the batch rows.
+
+    The reference predictor is single-token; for B > 1 the active set is the
+    union of the per-token top-K sets capped at K, the cap keeping the K
+    neurons whose best (over tokens) logit is largest.  Every neuron kept this
+    way lies in the top-K of the token that gives it its best logit, so the
+    result is a subset of the union; for B = 1 it is the plain top-K.
+    """
+    key = topk_key(np.atleast_2d(logits))
+    return key.max(axis=0)
+
+
+def topk_lower_index(logits: np.ndarray, k: int) -> np.ndarray:
+    """Index SET of the k largest entries, ties to the lower index, returned in
+    ascending index order.
+
+    Dejavu/src/models/modules/mha_dejavu.py:1069, 1369, 1506
+    (``logits.topk(k, sorted=False)``: a set, order unspecified).  logits is
+    (n,) or (B, n); for B > 1 see ``batch_scores``.
+    """
+    score = batch_scores(logits).astype(np.int64)
+    n = score.shape[0]
+    assert 0 <= k <= n
+    order = np.argsort(-score, kind="stable")  # stable => lower index first among ties
+    return np.sort(order[:k]).astype(np.int64)
+
+
+def topk_bruteforce(logits, k: int) -> np.ndarray:
+    """O(n*k) selection by repeated scan; pins ``topk_lower_index``."""
+    vals = [float(v) for v in np.asarray(logits, dtype=F16).astype(np.float64).ravel()]
+    taken = [False] * len(vals)
+    out = []
+    for _ in range(k):
+        best = -1
+        for i, v in enumerate(vals):
+            if taken[i]:
+                continue
+            if best < 0:
+                best = i
+                continue
+            vb = vals[best]
+            # NaN ranks highest; otherwise strict > keeps the lower index on ties
+            if (v != v and vb == vb) or (vb == vb and v > vb):
+                best = i
+        taken[best] = True
+        out.append(best)
+    return np.array(sorted(out), dtype=np.int64)
+
+
+# --------------------------------------------------------------------------
+# sparse MLP
+# --------------------------------------------------------------------------
+def gather_gemv(x, weight, idx, bias=None, activation="id"):
+    """``y = act(x @ weight[idx].T + bias[idx])``, fp32 accumulate, fp16 out.
+
+    Dejavu/src/ops/triton/gather_gemv.py:198-254 (kernel 43-195: bias added in
+    fp32 before the activation, result stored in x.dtype at line 233).
+    x: (B, N); weight: (Z, N); idx: (M,); bias: (Z,) -> (B, M).
+    """
+    idx = np.asarray(idx).astype(np.int64)
+    acc = np.asarray(x, F16).astype(F32) @ np.asarray(weight, F16)[idx].astype(F32).T
+    if bias is not None:
+        acc = acc + np.asarray(bias, F16)[idx].astype(F32)[None, :]
+    return _act(acc, activation).astype(F16)
+
+
+def gather_transposed_gemv(x, weight, idx, bias=None):
+    """``y = x @ weight[idx] + bias``, fp32 accumulate, fp16 out.
+
+    Dejavu/src/ops/triton/gather_gemv.py:572-644 (atomic-add kernel 467-569
+    accumulates fp32, bias added once, cast to x.dtype at line 644).
+    x: (B, M); weight: (Z, N); idx: (M,); bias: (N,) -> (B, N).
+    """
+    idx = np.asarray(idx).astype(np.int64)
+    acc = np.asarray(x, F16).astype(F32) @ np.asarray(weight, F16)[idx].astype(F32)
+    if bias is not None:
+        acc = acc + np.asarray(bias, F16).astype(F32)[None, :]
+    return acc.astype(F16)
+
+
+def mlp_sparse(x, W1, W2t, idx, bias1=None, bias2=None):
+    """fc1 gather + bias + ReLU (rounded to fp16), then fc2 transposed gather.
+
+    Dejavu/src/ops/triton/gather_gemv.py:647-657.
+    """
+    h = gather_gemv(x, W1, idx, bias1, activation="relu")
+    return gather_transposed_gemv(h, W2t, idx, bias2)
+
+
+def mlp_dense_then_masked(x, W1, W2, idx, bias1=None, bias2=None, dtype=np.float64):
+    """Accuracy-simulator form: ``fc2(relu(fc1(x) * mask)) + b2``.
+
+    Decentralized_FM_alpha/modules/hf_opt_sparse_mlp_attention.py:493-501
+    (mask = scatter of top-k indices) and 552-558.  W2 is (d, ffn), i.e. NOT
+    transposed.  Computed in ``dtype`` without intermediate fp16 rounding.
+    """
+    x = np.asarray(x, F16).astype(dtype)
+    W1 = np.asarray(W1, F16).astype(dtype)
+    W2 = np.asarray(W2, F16).astype(dtype)
+    pre = x @ W1.T
+    if bias1 is not None:
+        pre = pre + np.asarray(bias1, F16).astype(dtype)[None, :]
+    mask = np.zeros(W1.shape[0], dtype=dtype)
+    mask[np.asarray(idx).astype(np.int64)] = 1
+    h = relu(pre * mask[None, :])
+    y = h @ W2.T
+    if bias2 is not None:
+        y = y + np.asarray(bias2, F16).astype(dtype)[None, :]
+    return y
+
+
+# --------------------------------------------------------------------------
+# head-sparse attention
+# --------------------------------------------------------------------------
+def qkv_proj_sparse(x, weight, head_idx, batch_idx, bias=None, out=None):
+    """QKV projection for the active heads and the live window tokens only.
+
+    Dejavu/src/ops/triton/attention_proj_sparse.py:110-194:
+    ``y[b, t, h, :] = x[b] @ weight[t, h].T + bias[t, h]`` for h in head_idx
+    and for the b listed (>= 0) in that head's row of batch_idx.
+    x: (nb, d); weight: (3, H, hd, d); head_idx: (nnz,) int32; batch_idx:
+    (nnz, nb) int32 -> (nb, 3, H, hd) fp16.  The reference returns
+    uninitialised memory elsewhere; the oracle leaves ``out`` (zeros by
+    default) untouched there.
+    """
+    x = np.asarray(x, F16)
+    weight = np.asarray(weight, F16)
+    three, H, hd, d = weight.shape
+    nb = x.shape[0]
+    if out is None:
+        out = np.zeros((nb, 3, H, hd), dtype=F16)
+    xf = x.astype(F32)
+    for i, h in enumerate(np.asarray(head_idx).astype(np.int64)):
+        for b in np.asarray(batch_idx)[i].astype(np.int64):
+            if b < 0:
+                continue
+            for t in range(3):
+                acc = weight[t, h].astype(F32) @ xf[b]
+                if bias is not None:
+                    acc = acc + np.asarray(bias, F16)[t, h].astype(F32)
+                out[b, t, h] = acc.astype(F16)
+    return out
+
+
+def out_proj_sparse(x, weight, head_idx, bias=None):
+    """``y[b, n] = sum_{h in head_idx} x[b, h, :] . weight[n, h, :] + bias[n]``.
+
+    Dejavu/src/ops/triton/attention_proj_sparse.py:274-338 (its self-check
+    expression is ``einsum("nhd,bhd->bn", W[:, idx], x[:, idx]) + bias``,
+    line 646).  x: (B, H, hd); weight: (d, H, hd) -> (B, d) fp16.
+    """
+    hi = np.asarray(head_idx).astype(np.int64)
+    xs = np.asarray(x, F16)[:, hi].astype(F32)
+    ws = np.asarray(weight, F16)[:, hi].astype(F32)
+    acc = np.einsum("nhd,bhd->bn", ws, xs).astype(F32)
+    if bias is not None:
+        acc = acc + np.asarray(bias, F16).astype(F32)[None, :]
+    return acc.astype(F16)
+
+
+def out_proj_head_masked(ctx, weight, head_idx, bias=None, dtype=np.float64):
+    """Accuracy-simulator form: zero the unselected heads, then dense out_proj.
+
+    Decentralized_FM_alpha/modules/hf_opt_sparse_mlp_attention.py:365-373.
+    """
+    ctx = np.asarray(ctx, F16).astype(dtype)
+    B, H, hd = ctx.shape
+    mask = np.zeros(H, dtype=dtype)
+    mask[np.asarray(head_idx).astype(np.int64)] = 1
+    flat = (ctx * mask[None, :, None]).reshape(B, H * hd)
+    y = flat @ np.asarray(weight, F16).astype(dtype).reshape(-1, H * hd).T
+    if bias is not None:
+        y = y + np.asarray(bias, F16).astype(dtype)[None, :]
+    return y
+
+
+def k_cache_copy_sparse(k, k_cache, head_idx, seqlen_idx, padding=0):
+    """Scatter recomputed keys into the packed key cache, in place.
+
+    Dejavu/src/ops/triton/attention_proj_sparse.py:460-590:
+    ``k_cache[0, h, dp, s + pad, p] = k[s, h, dp*8 + p]`` for h = head_idx[i],
+    s in seqlen_idx[i] with s >= 0.  k: (nb, H, hd); k_cache:
+    (1, H, hd/8, S, 8).
+    """
+    packs = k_cache.shape[-1]
+    for i, h in enumerate(np.asarray(head_idx).astype(np.int64)):
+        for s in np.asarray(seqlen_idx)[i].astype(np.int64):
+            if s < 0:
+                continue
+            k_cache[0, h, :, s + int(padding), :] = np.asarray(k)[s, h].reshape(-1, packs)
+    return k_cache
+
+
+def v_cache_copy_sparse(v, v_cache, head_idx, seqlen_idx, padding=0):
+    """``v_cache[0, h, s + pad, :] = v[s, h, :]``.
+
+    Dejavu/src/ops/triton/attention_proj_sparse.py:342-456.
+    """
+    for i, h in enumerate(np.asarray(head_idx).astype(np.int64)):
+        for s in np.asarray(seqlen_idx)[i].astype(np.int64):
+            if s < 0:
+                continue
+            v_cache[0, h, s + int(padding), :] = np.asarray(v)[s, h]
+    return v_cache
+
+
+def pack_k_cache(k_bshd: np.ndarray) -> np.ndarray:
+    """(B, S, H, hd) -> (B, H, hd/8, S, 8): the key-cache layout of
+    Dejavu/src/models/modules/mha_dejavu.py:430-435."""
+    B, S, H, hd = k_bshd.shape
+    return np.ascontiguousarray(k_bshd.reshape(B, S, H, hd // 8, 8).transpose(0, 2, 3, 1, 4))
+
+
+def unpack_k_cache(k_cache: np.ndarray) -> np.ndarray:
+    """(B, H, hd/8, S, 8) -> (B, H, S, hd)."""
+    B, H, dp, S, p = k_cache.shape
+    return np.ascontiguousarray(k_cache.transpose(0, 1, 3, 2, 4).reshape(B, H, S, dp * p))
+
+
+def single_query_attention(q, k, v, k_cache, v_cache, timestep, softmax_scale=None,
+                           head_idx=None, lengths_per_sample=None):
+    """One-query attention over the cache, appending the new k, v first.
+
+    Call sites Dejavu/src/models/modules/mha_dejavu.py:1045-1053, 1439-1456
+    (external FasterTransformer kernel); arithmetic as the reference's own
+    torch restatement CrossAttention.forward, mha_dejavu.py:333-375:
+    ``softmax(q . K^T * scale) . V`` with scale = hd**-0.5
+    (Dejavu/src/models/gpt_dejavu.py:175), no causal mask at decode (:1037).
+    q, k, v: (B, H, hd); k_cache: (B, H, hd/8, S, 8); v_cache: (B, H, S, hd).
+    k, v are written at position ``timestep`` and positions [0, timestep] are
+    attended (``lengths_per_sample[b]`` replaces timestep per sample if given).
+    Only heads in ``head_idx`` (all if None) are computed; the others are left
+    zero in the (B, H, hd) fp16 result.  Caches are updated in place for the
+    computed heads.
+    """
+    q = np.asarray(q, F16)
+    B, H, hd = q.shape
+    scale = F32(hd ** -0.5 if softmax_scale is None else softmax_scale)
+    heads = range(H) if head_idx is None else [int(h) for h in np.asarray(head_idx)]
+    out = np.zeros((B, H, hd), dtype=F16)
+    for b in range(B):
+        t = int(timestep if lengths_per_sample is None else lengths_per_sample[b])
+        for h in heads:
+            k_cache[b, h, :, t, :] = np.asarray(k, F16)[b, h].reshape(-1, k_cache.shape[-1])
+            v_cache[b, h, t, :] = np.asarray(v, F16)[b, h]
+            K = k_cache[b, h, :, : t + 1, :].transpose(1, 0, 2).reshape(t + 1, hd).astype(F32)
+            V = v_cache[b, h, : t + 1, :].astype(F32)
+            s = (K @ q[b, h].astype(F32)) * scale
+            s = s - s.max()
+            p = np.exp(s)
+            p = p / p.sum(dtype=F32)
+            out[b, h] = (p @ V).astype(F16)
+    return out
+
+
+# --------------------------------------------------------------------------
+# skipped-head KV back-fill window
+# --------------------------------------------------------------------------
+class WindowTracker:
+    """Which (head, window-token) K/V entries are still missing.
+
+    Dejavu/src/models/modules/mha_dejavu.py:1124-1149 (ParallelTracker) and the
+    counter / flush logic of ParallelMHASparseAttMlp.forward, :1318-1359 and
+    :1485-1492.  ``tracker[h, s]`` is s while token s of the current 16-token
+    window has no K/V for head h, and -1 once it has.
+    """
+
+    WINDOW = 16
+
+    def __init__(self, num_heads: int):
+        self.num_heads = num_heads
+        self.counter = 0
+        self.reset()
+
+    def reset(self):
+        self.tracker = np.tile(np.arange(self.WINDOW, dtype=np.int32), (self.num_heads, 1))
+
+    def begin_step(self, head_idx):
+        """Returns (head_idx used this step, batch_idx (nnz, counter+1))."""
+        head_idx = np.asarray(head_idx, dtype=np.int32)
+        if self.counter == self.WINDOW - 1:  # :1320-1325 flush: every head, every token
+            self.reset()
+            head_idx = np.arange(self.num_heads, dtype=np.int32)
+        batch_idx = self.tracker[head_idx][:, : self.counter + 1].copy()  # :1133-1135
+        return head_idx, batch_idx
+
+    def end_step(self, head_idx, batch_idx):
+        """Marks what was computed (:1355-1359, 1137-1142); returns True when the
+        window wrapped (:1485-1492: counter reset, cache_offset += 16)."""
+        if self.counter != self.WINDOW - 1:
+            sub = self.tracker[head_idx][:, : self.counter + 1]
+            sub[batch_idx != -1] = -1
+            self.tracker[head_idx, : self.counter + 1] = sub
+        self.counter += 1
+        if self.counter == self.WINDOW:
+            self.counter = 0
+            self.reset()
+            return True
+        return False
+
+
+# --------------------------------------------------------------------------
+# block-level algebra (the callers either side of the sparse modules)
+# --------------------------------------------------------------------------
+def layer_norm(x, weight, bias, eps=1e-5):
+    """nn.LayerNorm in fp32 on fp16 input, fp16 out
+    (Dejavu/src/models/modules/block_dejavu.py:575-584, 626-634)."""
+    xf = np.asarray(x, F16).astype(F32)
+    mu = xf.mean(axis=-1, keepdims=True)
+    var = ((xf - mu) ** 2).mean(axis=-1, keepdims=True)
+    y = (xf - mu) / np.sqrt(var + F32(eps))
+    return (y * np.asarray(weight, F16).astype(F32) + np.asarray(bias, F16).astype(F32)).astype(F16)

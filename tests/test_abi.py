@@ -1,0 +1,67 @@
+"""The C-ABI library loads without a GPU and exports every symbol that
+include/dejavu_hip.h declares; host-side argument checks return error codes."""
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "dejavu_hip.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\bDV_API\s+[\w\s\*]+?\b(dv_\w+)\s*\(", text)))
+
+
+def test_header_declares_symbols():
+    syms = declared_symbols()
+    assert "dv_version" in syms and "dv_gather_gemv_f16" in syms and len(syms) >= 8
+
+
+def test_library_exports_every_declared_symbol():
+    from dejavu_amd import _lib
+
+    for name in declared_symbols():
+        assert hasattr(_lib.lib, name), f"{name} declared in the header but not exported"
+        assert name in _lib.SIGNATURES, f"{name} has no ctypes signature"
+    assert set(_lib.SIGNATURES) == set(declared_symbols())
+    assert _lib.lib.dv_version() >= 100
+    assert _lib.lib.dv_error_string(0) == b"ok"
+
+
+def test_canonical_lanes_agrees_with_oracle():
+    from dejavu_amd import _lib
+    from oracle import dejavu_oracle as O
+
+    for n in [8, 128, 512, 1000, 1024, 1032, 4096, 12288]:
+        assert _lib.lib.dv_canonical_lanes(n) == O.canonical_lanes(n)
+
+
+def test_host_side_argument_checks_return_codes():
+    """Null pointers / bad sizes are rejected before anything is launched."""
+    from dejavu_amd import _lib
+
+    L = _lib.lib
+    assert L.dv_gather_gemv_f16(None, None, 8, None, None, 8, 1, 8, 8, 1, 0, None, None) == -1
+    assert L.dv_topk_f16(None, 1, 8, 1, None, 8, None) == -1
+    assert L.dv_topk_f16(0x1000, 1, 8, 9, 0x1000, 8, None) == -1  # k > n
+    assert L.dv_topk_f16(0x1000, 1, 8, 1, 0x1000, 3, None) == -1  # bad idx width
+    assert L.dv_topk_f16(0x1000, 1, 1 << 20, 1, 0x1000, 8, None) == -2  # n too large
+    assert L.dv_gather_gemv_f16(0x1000, 0x1000, 8, None, 0x1000, 8, 5, 8, 8, 1, 0, 0x1000, None) == -2  # B > 4
+    assert L.dv_gather_gemv_f16(0x1000, 0x1000, 12, None, 0x1000, 8, 1, 12, 8, 1, 0, 0x1000, None) == -3  # N % 8
+    assert L.dv_gather_transposed_gemv_f16(0x1000, 0x1000, 8, None, 0x1000, 8, 1, 8, 8, 4, 0x1000, None, 0, None) == -4
+    assert L.dv_predictor_logits_f16(0x1000, 0x1000, 8, 0x1000, 8, 9, 8, 8, 8, 0x1000, 0x1000, None) == -2
+
+
+def test_ops_refuse_cpu_tensors():
+    import torch
+
+    from dejavu_amd import ops
+
+    x = torch.zeros(1, 8, dtype=torch.float16)
+    W = torch.zeros(8, 8, dtype=torch.float16)
+    idx = torch.arange(4)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ops.gather_gemv(x, W, idx)

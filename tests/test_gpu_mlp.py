@@ -1,0 +1,168 @@
+"""GPU parity: predictor + top-k (bit-exact) and the gathered sparse MLP
+(max-abs 2e-2, relative L2 1e-3 against the fp32-accumulated oracle)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import dejavu_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS = 2e-2
+REL_L2 = 1e-3
+
+
+def assert_close(got, want, what=""):
+    got = np.asarray(got, dtype=np.float64)
+    want = np.asarray(want, dtype=np.float64)
+    max_abs = np.max(np.abs(got - want)) if got.size else 0.0
+    rel = np.linalg.norm(got - want) / max(np.linalg.norm(want), 1e-30)
+    assert max_abs <= MAX_ABS and rel <= REL_L2, f"{what}: max_abs={max_abs:.3e} rel_l2={rel:.3e}"
+
+
+def dev(t):
+    return t.cuda() if isinstance(t, torch.Tensor) else t
+
+
+def np16(t):
+    return t.detach().cpu().numpy()
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from dejavu_amd import ops as _ops
+
+    return _ops
+
+
+def make(cfg_name, batch, seed=0):
+    from dejavu_amd.workloads import CONFIGS, make_mlp
+
+    return make_mlp(CONFIGS[cfg_name], batch=batch, device="cpu", seed=seed)
+
+
+# ------------------------------------------------------------------ predictor
+@pytest.mark.parametrize("cfg,batch", [("opt-125m", 1), ("opt-125m", 3), ("opt-6.7b", 1), ("opt-6.7b", 8)])
+def test_predictor_logits_bit_exact(ops, cfg, batch):
+    t = make(cfg, batch)
+    print(f"case predictor {cfg} B={batch}", flush=True)
+    hidden = torch.empty(batch, t["mlp_Wa"].shape[0], dtype=torch.float16, device="cuda")
+    got = ops.predictor_logits(dev(t["residual"]), dev(t["mlp_Wa"]), dev(t["mlp_Wb"]), hidden=hidden)
+    torch.cuda.synchronize()
+    h_ref, l_ref = O.predictor_logits(np16(t["residual"]), np16(t["mlp_Wa"]), np16(t["mlp_Wb"]))
+    assert np.array_equal(np16(hidden).view(np.uint16), h_ref.view(np.uint16)), "hidden vector differs"
+    assert np.array_equal(np16(got).view(np.uint16), l_ref.view(np.uint16)), "logits differ"
+
+
+@pytest.mark.parametrize("cfg,batch,k", [("opt-125m", 1, 1024), ("opt-6.7b", 1, 4096), ("opt-6.7b", 4, 2048),
+                                         ("opt-6.7b", 1, 16384)])
+def test_predictor_topk_indices_bit_exact(ops, cfg, batch, k):
+    t = make(cfg, batch)
+    print(f"case predictor+topk {cfg} B={batch} k={k}", flush=True)
+    logits = ops.predictor_logits(dev(t["residual"]), dev(t["mlp_Wa"]), dev(t["mlp_Wb"]))
+    idx = ops.topk_indices(logits, k)
+    torch.cuda.synchronize()
+    _, l_ref = O.predictor_logits(np16(t["residual"]), np16(t["mlp_Wa"]), np16(t["mlp_Wb"]))
+    want = O.topk_lower_index(l_ref, k)
+    assert idx.dtype == torch.int64
+    assert np.array_equal(np16(idx), want)
+
+
+# ---------------------------------------------------------------------- top-k
+@pytest.mark.parametrize("n", [12, 96, 97, 512, 3072, 16384, 20480, 36864, 49152, 65536])
+def test_topk_random_and_ties(ops, n):
+    g = np.random.default_rng(n)
+    cases = {
+        "normal": (g.standard_normal(n) * 8).astype(np.float16),
+        "few_values": np.round(g.standard_normal(n) * 2).astype(np.float16),
+        "all_equal": np.full(n, -1.5, dtype=np.float16),
+        "signed_zeros": np.where(g.random(n) < 0.5, 0.0, -0.0).astype(np.float16),
+    }
+    cases["with_nan_inf"] = cases["normal"].copy()
+    cases["with_nan_inf"][[0, n // 2]] = np.nan
+    cases["with_nan_inf"][[1, n - 1]] = [np.inf, -np.inf]
+    for name, x in cases.items():
+        for k in sorted({0, 1, n // 3, n - 1, n}):
+            print(f"case topk n={n} {name} k={k}", flush=True)
+            for dt in (torch.int64, torch.int32):
+                got = ops.topk_indices(torch.from_numpy(x).cuda(), k, dtype=dt)
+                torch.cuda.synchronize()
+                assert np.array_equal(np16(got).astype(np.int64), O.topk_lower_index(x, k)), (name, k)
+
+
+def test_topk_batched_scores(ops):
+    g = np.random.default_rng(3)
+    L = (g.standard_normal((8, 16384)) * 4).astype(np.float16)
+    got = ops.topk_indices(torch.from_numpy(L).cuda(), 4096)
+    torch.cuda.synchronize()
+    assert np.array_equal(np16(got), O.topk_lower_index(L, 4096))
+
+
+# ----------------------------------------------------------------- sparse MLP
+@pytest.mark.parametrize("cfg,batch,K", [("opt-125m", 1, 1024), ("opt-125m", 4, 1024), ("opt-6.7b", 1, 1024),
+                                         ("opt-6.7b", 1, 4096), ("opt-6.7b", 4, 2048), ("opt-6.7b", 2, 16384)])
+@pytest.mark.parametrize("idx_dtype", [torch.int64, torch.int32])
+def test_mlp_sparse_matches_oracle(ops, cfg, batch, K, idx_dtype):
+    t = make(cfg, batch)
+    print(f"case mlp_sparse {cfg} B={batch} K={K} {idx_dtype}", flush=True)
+    _, l_ref = O.predictor_logits(np16(t["residual"]), np16(t["mlp_Wa"]), np16(t["mlp_Wb"]))
+    idx = O.topk_lower_index(l_ref, K)
+    idx_t = torch.from_numpy(idx).to(idx_dtype).cuda()
+    x, W1, W2t, b1, b2 = (dev(t[n]) for n in ("x2", "W1", "W2t", "b1", "b2"))
+    h = ops.gather_gemv(x, W1, idx_t, b1, activation="relu")
+    y = ops.gather_transposed_gemv(h, W2t, idx_t, b2)
+    y2 = ops.mlp_sparse(x, W1, W2t, idx_t, b1, b2)
+    torch.cuda.synchronize()
+    h_ref = O.gather_gemv(np16(t["x2"]), np16(t["W1"]), idx, np16(t["b1"]), "relu")
+    assert_close(np16(h), h_ref, "fc1")
+    # fc2 checked on the kernel's own fp16 intermediate, and end to end
+    assert_close(np16(y), O.gather_transposed_gemv(np16(h), np16(t["W2t"]), idx, np16(t["b2"])), "fc2")
+    assert_close(np16(y2), O.mlp_sparse(np16(t["x2"]), np16(t["W1"]), np16(t["W2t"]), idx, np16(t["b1"]), np16(t["b2"])),
+                 "mlp_sparse")
+    assert torch.equal(y, y2), "two runs of the same MLP differ (reduction must be deterministic)"
+    if K == 1024 and cfg == "opt-125m":
+        W2 = np.ascontiguousarray(np16(t["W2t"]).T)
+        dm = O.mlp_dense_then_masked(np16(t["x2"]), np16(t["W1"]), W2, idx, np16(t["b1"]), np16(t["b2"]))
+        assert_close(np16(y2), dm, "dense-then-masked")
+
+
+def test_gather_gemv_edge_cases(ops):
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(2, 776, generator=g).half()  # N not a multiple of the 512-element chunk
+    W = (torch.randn(300, 776, generator=g) * 0.05).half()
+    bias = torch.randn(300, generator=g).half()
+    # ragged M, duplicates, unsorted, and out-of-range entries (contribute zero)
+    idx = torch.tensor([299, 0, 0, 17, 5, 299, 123, 1000, -3], dtype=torch.int64)
+    print("case gather edge", flush=True)
+    got = ops.gather_gemv(x.cuda(), W.cuda(), idx.cuda(), bias.cuda(), activation="id")
+    torch.cuda.synchronize()
+    valid = (idx >= 0) & (idx < 300)
+    want = O.gather_gemv(x.numpy(), W.numpy(), idx[valid].numpy(), bias.numpy(), "id")
+    assert_close(np16(got)[:, valid.numpy()], want, "gather edge")
+    assert np.all(np16(got)[:, ~valid.numpy()] == 0)
+    # empty index vector
+    e = ops.gather_gemv(x.cuda(), W.cuda(), idx[:0].cuda(), bias.cuda())
+    assert e.shape == (2, 0)
+    # fc2 with ragged sizes, strided weight rows, invalid entries skipped
+    Wbig = (torch.randn(300, 1000, generator=g) * 0.05).half().cuda()
+    Wv = Wbig[:, :776]  # row stride 1000, contiguous last dim
+    h = torch.randn(2, idx.numel(), generator=g).half()
+    b2 = torch.randn(776, generator=g).half()
+    got2 = ops.gather_transposed_gemv(h.cuda(), Wv, idx.cuda(), b2.cuda())
+    torch.cuda.synchronize()
+    want2 = O.gather_transposed_gemv(h[:, valid].numpy(), Wv.cpu().numpy(), idx[valid].numpy(), b2.numpy())
+    assert_close(np16(got2), want2, "fc2 edge")
+    # M == 0: bias only
+    got3 = ops.gather_transposed_gemv(h[:, :0].cuda(), Wv, idx[:0].cuda(), b2.cuda())
+    torch.cuda.synchronize()
+    assert np.array_equal(np16(got3), np.tile(b2.numpy(), (2, 1)))
+
+
+def test_reference_style_assertions(ops):
+    x = torch.zeros(5, 64, dtype=torch.float16, device="cuda")
+    W = torch.zeros(128, 64, dtype=torch.float16, device="cuda")
+    idx = torch.arange(8, device="cuda")
+    with pytest.raises(AssertionError):
+        ops.gather_gemv(x, W, idx)  # batch 5 not in 1..4
+    with pytest.raises(AssertionError):
+        ops.gather_gemv(x[:1].float(), W, idx)  # dtype mismatch
