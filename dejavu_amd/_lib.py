@@ -43,6 +43,28 @@ SIGNATURES = {
         [_c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_size,
          _c_ptr],
     ),
+    "dv_qkv_proj_sparse_f16": (
+        _c_int, [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr]),
+    "dv_kv_cache_copy_sparse_f16": (
+        _c_int,
+        [_c_ptr, _c_ptr, _c_i64, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_int,
+         _c_int, _c_ptr]),
+    "dv_kv_append_f16": (
+        _c_int,
+        [_c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int,
+         _c_ptr]),
+    "dv_decode_attention_workspace_bytes": (_c_size, [_c_int, _c_int, _c_int, _c_int]),
+    "dv_decode_attention_f16": (
+        _c_int,
+        [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int,
+         ctypes.c_float, _c_ptr, _c_i64, _c_ptr, _c_size, _c_ptr]),
+    "dv_out_proj_sparse_f16": (
+        _c_int, [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr]),
+    "dv_out_proj_sparse_t_workspace_bytes": (_c_size, [_c_int, _c_int, _c_int, _c_int]),
+    "dv_out_proj_sparse_t_f16": (
+        _c_int,
+        [_c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_size,
+         _c_ptr]),
 }
 
 

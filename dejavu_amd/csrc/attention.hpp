@@ -1,0 +1,322 @@
+// Head-sparse attention kernels for the decode step:
+//   qkv_sparse_kernel     QKV projection of the active heads for the live window tokens
+//   kv_cache_copy_kernel  scatter of (re)computed K / V rows into the caches
+//   decode_attn_kernel    one-query attention over the fp16 KV cache, split along the sequence
+//   decode_attn_combine_kernel  log-sum-exp merge of the sequence splits
+//   out_proj_rows_kernel  out_proj over the active heads with the weight in (d, H, hd) layout
+//
+// Cache layouts (kept from the reference so the caches are interchangeable):
+//   k_cache (B, H, hd/8, S, 8): for a fixed head and 8-wide slice of head_dim the S
+//   positions are contiguous 16-byte packets, so a wavefront that maps lanes to
+//   positions reads 1 KiB contiguous per load;  v_cache (B, H, S, hd).
+#pragma once
+#include "common.hpp"
+
+namespace dv {
+
+// ---------------------------------------------------------------------------
+// Y[b, t, h, j] = X[b, :] . W[t, h, j, :] + bias[t, h, j]
+//   for i < nnz, h = head_idx[i], every slot s < nb with b = batch_idx[i, s] >= 0.
+// X (nb, d); W (3, H, hd, d) contiguous; Y (nb, 3, H, hd).  Rows of one (t, h)
+// are hd consecutive weight rows; a wavefront owns R of them at a time and
+// keeps one accumulator per live slot.  Nothing is written for dead slots or
+// unselected heads.
+// ---------------------------------------------------------------------------
+template <int NBMAX, int R, int U>
+__global__ __launch_bounds__(256) void qkv_sparse_kernel(
+    const half_t* __restrict__ X, const half_t* __restrict__ W, const half_t* __restrict__ bias,
+    const int* __restrict__ head_idx, const int* __restrict__ batch_idx, int nb, int d, int H,
+    int hd, int nnz, half_t* __restrict__ Y) {
+  constexpr int CH = 8 * kWave;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int waves_per_block = blockDim.x >> 6;
+  const int groups_per_head = hd / R;  // hd % R == 0 (checked on the host)
+  const int ntasks = nnz * 3 * groups_per_head;
+  for (int task = blockIdx.x * waves_per_block + wave; task < ntasks;
+       task += gridDim.x * waves_per_block) {
+    const int i = task / (3 * groups_per_head);
+    const int rem = task - i * 3 * groups_per_head;
+    const int t = rem / groups_per_head;
+    const int j0 = (rem - t * groups_per_head) * R;
+    const int h = head_idx[i];
+    if (h < 0 || h >= H) continue;
+    int slot[NBMAX];
+    bool any = false;
+#pragma unroll
+    for (int s = 0; s < NBMAX; ++s) {
+      int b = s < nb ? batch_idx[i * nb + s] : -1;
+      if (b >= nb) b = -1;
+      slot[s] = b;
+      any |= b >= 0;
+    }
+    if (!any) continue;
+    const int64_t row0 = ((int64_t)t * H + h) * hd + j0;
+    const half_t* wr = W + row0 * d + lane * 8;
+
+    float acc[R][NBMAX];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int s = 0; s < NBMAX; ++s) acc[r][s] = 0.f;
+
+    int base = 0;
+    for (; base + U * CH <= d; base += U * CH) {
+      half8_t w[U][R];
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int r = 0; r < R; ++r) w[u][r] = load8_stream(wr + (int64_t)r * d + base + u * CH);
+#pragma unroll
+      for (int s = 0; s < NBMAX; ++s) {
+        if (slot[s] >= 0) {
+          const half_t* xr = X + (int64_t)slot[s] * d + base + lane * 8;
+#pragma unroll
+          for (int u = 0; u < U; ++u) {
+            const half8_t xv = load8(xr + u * CH);
+#pragma unroll
+            for (int r = 0; r < R; ++r) acc[r][s] = dot8_fast(w[u][r], xv, acc[r][s]);
+          }
+        }
+      }
+    }
+    for (; base < d; base += CH) {
+      if (base + lane * 8 < d) {
+        half8_t w[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) w[r] = load8_stream(wr + (int64_t)r * d + base);
+#pragma unroll
+        for (int s = 0; s < NBMAX; ++s) {
+          if (slot[s] >= 0) {
+            const half8_t xv = load8(X + (int64_t)slot[s] * d + base + lane * 8);
+#pragma unroll
+            for (int r = 0; r < R; ++r) acc[r][s] = dot8_fast(w[r], xv, acc[r][s]);
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int s = 0; s < NBMAX; ++s) {
+      if (slot[s] >= 0) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          float v = butterfly_sum<kWave>(acc[r][s]);
+          if (bias != nullptr) v += (float)bias[row0 + r];
+          if (lane == 0) Y[(int64_t)slot[s] * 3 * H * hd + row0 + r] = (half_t)v;
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// For i < nnz, h = head_idx[i], every slot with s = seq_idx[i, slot] >= 0:
+//   k_cache[0, h, dp, s + pad, p] = K[s, h, dp*8 + p]      (if k_cache != null)
+//   v_cache[0, h, s + pad, :]     = V[s, h, :]             (if v_cache != null)
+// K / V are (nsrc, H, hd) views with row stride `ld_src` elements (rows of the
+// (nb, 3, H, hd) projection output).  `padding` is a device int32 (or null = 0).
+// One workgroup of hd threads per (slot, head).
+// ---------------------------------------------------------------------------
+__global__ void kv_cache_copy_kernel(const half_t* __restrict__ K, const half_t* __restrict__ V,
+                                     int64_t ld_src, int nsrc, half_t* __restrict__ k_cache,
+                                     half_t* __restrict__ v_cache, const int* __restrict__ head_idx,
+                                     const int* __restrict__ seq_idx, int nslots,
+                                     const int* __restrict__ padding, int H, int hd, int S) {
+  const int i = blockIdx.x;
+  const int slot = blockIdx.y;
+  const int j = threadIdx.x;
+  const int h = head_idx[i];
+  const int s = seq_idx[i * nslots + slot];
+  if (h < 0 || h >= H || s < 0 || s >= nsrc || j >= hd) return;
+  const int dst = s + (padding ? padding[0] : 0);
+  if (dst < 0 || dst >= S) return;
+  const int64_t src = (int64_t)s * ld_src + (int64_t)h * hd + j;
+  if (k_cache) k_cache[(((int64_t)h * (hd / 8) + j / 8) * S + dst) * 8 + (j & 7)] = K[src];
+  if (v_cache) v_cache[((int64_t)h * S + dst) * hd + j] = V[src];
+}
+
+// Appends the newest token: for every batch row b and head (all, or head_idx):
+//   k_cache[b, h, :, pos_b, :] = K[b, h, :],  v_cache[b, h, pos_b, :] = V[b, h, :]
+// with pos_b = lengths[b] if lengths else pos.  K / V: (B, H, hd) with batch
+// stride ld_src.  Grid (heads, B), hd threads.
+__global__ void kv_append_kernel(const half_t* __restrict__ K, const half_t* __restrict__ V,
+                                 int64_t ld_src, half_t* __restrict__ k_cache,
+                                 half_t* __restrict__ v_cache, const int* __restrict__ head_idx,
+                                 const int* __restrict__ lengths, int pos, int H, int hd, int S) {
+  const int h = head_idx ? head_idx[blockIdx.x] : (int)blockIdx.x;
+  const int b = blockIdx.y;
+  const int j = threadIdx.x;
+  const int p = lengths ? lengths[b] : pos;
+  if (h < 0 || h >= H || p < 0 || p >= S || j >= hd) return;
+  const int64_t src = (int64_t)b * ld_src + (int64_t)h * hd + j;
+  const int64_t bh = (int64_t)b * H + h;
+  k_cache[((bh * (hd / 8) + j / 8) * S + p) * 8 + (j & 7)] = K[src];
+  v_cache[(bh * S + p) * hd + j] = V[src];
+}
+
+// ---------------------------------------------------------------------------
+// One-query attention, one wavefront per (64-position split, head, batch row).
+// Lanes map to positions for q.K (each lane reads its position's hd/8 packets)
+// and to (row, 8-wide slice) for p.V.  All K and V loads of the split are
+// issued before any arithmetic.  Writes un-normalised partials
+//   part[(b, i, split)] = { max, sum, o[hd] }  (fp32)
+// n_len = number of cached positions to attend (lengths[b] + 1 if lengths).
+// ---------------------------------------------------------------------------
+template <int HD>
+__global__ __launch_bounds__(64) void decode_attn_kernel(
+    const half_t* __restrict__ Q, int64_t ldq, const half_t* __restrict__ k_cache,
+    const half_t* __restrict__ v_cache, const int* __restrict__ head_idx,
+    const int* __restrict__ lengths, int n_len, int H, int S, float scale, int nsplit,
+    float* __restrict__ part) {
+  constexpr int PK = HD / 8;     // 16-byte packets per position / lanes per V row
+  constexpr int RPI = kWave / PK;  // V rows per load instruction
+  constexpr int VIT = kWave / RPI;  // V load instructions per split (= PK)
+  const int lane = threadIdx.x;
+  const int split = blockIdx.x;
+  const int i = blockIdx.y;
+  const int b = blockIdx.z;
+  const int h = head_idx ? head_idx[i] : i;
+  const int len = lengths ? lengths[b] + 1 : n_len;
+  float* out = part + (((int64_t)b * gridDim.y + i) * nsplit + split) * (HD + 2);
+  const int p0 = split * kWave;
+  if (h < 0 || h >= H || p0 >= len) {  // empty split: neutral element of the merge
+    if (lane == 0) {
+      out[0] = -INFINITY;
+      out[1] = 0.f;
+    }
+#pragma unroll
+    for (int e = lane; e < HD; e += kWave) out[2 + e] = 0.f;
+    return;
+  }
+  const int64_t bh = (int64_t)b * H + h;
+  const int pos = p0 + lane;
+  const bool pos_ok = pos < len;
+  const int pos_c = pos_ok ? pos : len - 1;  // clamp: always a valid address
+
+  // K packets of this lane's position
+  half8_t kp[PK];
+  const half_t* kbase = k_cache + (bh * PK * S + pos_c) * 8;
+#pragma unroll
+  for (int dp = 0; dp < PK; ++dp) kp[dp] = load8_stream(kbase + (int64_t)dp * S * 8);
+  // V rows: instruction it covers rows it*RPI + grp
+  const int grp = lane / PK, sub = lane % PK;
+  half8_t vv[VIT];
+#pragma unroll
+  for (int it = 0; it < VIT; ++it) {
+    int row = p0 + it * RPI + grp;
+    if (row >= len) row = len - 1;
+    vv[it] = load8_stream(v_cache + (bh * S + row) * HD + sub * 8);
+  }
+  // q (uniform across lanes)
+  const half_t* q = Q + (int64_t)b * ldq + (int64_t)h * HD;
+  float s = 0.f;
+#pragma unroll
+  for (int dp = 0; dp < PK; ++dp) s = dot8_fast(kp[dp], load8(q + dp * 8), s);
+  s = pos_ok ? s * scale : -INFINITY;
+  const float m = butterfly_max<kWave>(s);
+  const float p = pos_ok ? __expf(s - m) : 0.f;
+  const float l = butterfly_sum<kWave>(p);
+
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+#pragma unroll
+  for (int it = 0; it < VIT; ++it) {
+    const float pr = __shfl(p, it * RPI + grp, kWave);  // 0 for positions >= len
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(pr, (float)vv[it][e], acc[e]);
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+#pragma unroll
+    for (int off = PK; off < kWave; off <<= 1) acc[e] += __shfl_xor(acc[e], off, kWave);
+  }
+  if (lane == 0) {
+    out[0] = m;
+    out[1] = l;
+  }
+  if (grp == 0) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) out[2 + sub * 8 + e] = acc[e];
+  }
+}
+
+// out[b, h, :] = sum_s o_s * exp(m_s - m) / sum_s l_s * exp(m_s - m).  Grid (heads, B), HD threads.
+template <int HD>
+__global__ __launch_bounds__(HD) void decode_attn_combine_kernel(
+    const float* __restrict__ part, const int* __restrict__ head_idx, int H, int nsplit,
+    half_t* __restrict__ out, int64_t ldo) {
+  const int i = blockIdx.x;
+  const int b = blockIdx.y;
+  const int j = threadIdx.x;
+  const int h = head_idx ? head_idx[i] : i;
+  if (h < 0 || h >= H) return;
+  const float* p = part + ((int64_t)b * gridDim.x + i) * nsplit * (HD + 2);
+  float m = -INFINITY;
+  for (int s = 0; s < nsplit; ++s) m = fmaxf(m, p[s * (HD + 2)]);
+  float num = 0.f, den = 0.f;
+  for (int s = 0; s < nsplit; ++s) {
+    const float ms = p[s * (HD + 2)];
+    const float w = ms == -INFINITY ? 0.f : __expf(ms - m);
+    den += w * p[s * (HD + 2) + 1];
+    num += w * p[s * (HD + 2) + 2 + j];
+  }
+  out[(int64_t)b * ldo + (int64_t)h * HD + j] = (half_t)(num / den);
+}
+
+// ---------------------------------------------------------------------------
+// Y[b, n] = sum_{i < nnz} X[b, h_i, :] . W[n, h_i, :] + bias[n] with W in the
+// (d, H, hd) layout of out_proj.weight: every output row gathers nnz segments
+// of hd contiguous values.  hd/8 lanes cover a segment, so a wavefront load
+// touches 64/(hd/8) heads; R output rows share the activation loads.
+// ---------------------------------------------------------------------------
+template <int B, int R, int HD>
+__global__ __launch_bounds__(256) void out_proj_rows_kernel(
+    const half_t* __restrict__ X, const half_t* __restrict__ W, const half_t* __restrict__ bias,
+    const int* __restrict__ head_idx, int nnz, int H, int N, half_t* __restrict__ Y) {
+  constexpr int PK = HD / 8;
+  constexpr int HPI = kWave / PK;  // heads per load instruction
+  const int lane = threadIdx.x & 63;
+  const int grp = lane / PK, sub = lane % PK;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int waves_per_block = blockDim.x >> 6;
+  const int ntasks = (N + R - 1) / R;
+  for (int task = blockIdx.x * waves_per_block + wave; task < ntasks;
+       task += gridDim.x * waves_per_block) {
+    const int n0 = task * R;
+    float acc[R][B];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int b = 0; b < B; ++b) acc[r][b] = 0.f;
+    for (int i0 = 0; i0 < nnz; i0 += HPI) {
+      const int i = i0 + grp;
+      int h = i < nnz ? head_idx[i] : -1;
+      const bool ok = h >= 0 && h < H;
+      if (!ok) h = 0;
+      const int64_t seg = (int64_t)h * HD + sub * 8;
+      half8_t w[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const int n = n0 + r < N ? n0 + r : N - 1;
+        w[r] = ok ? load8_stream(W + (int64_t)n * H * HD + seg) : zero8();
+      }
+#pragma unroll
+      for (int b = 0; b < B; ++b) {
+        const half8_t xv = load8(X + (int64_t)b * H * HD + seg);
+#pragma unroll
+        for (int r = 0; r < R; ++r) acc[r][b] = dot8_fast(w[r], xv, acc[r][b]);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int b = 0; b < B; ++b) {
+        const float v = butterfly_sum<kWave>(acc[r][b]);
+        const int n = n0 + r;
+        if (lane == 0 && n < N) Y[(int64_t)b * N + n] = (half_t)(v + (bias ? (float)bias[n] : 0.f));
+      }
+  }
+}
+
+}  // namespace dv

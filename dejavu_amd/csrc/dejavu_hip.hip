@@ -4,7 +4,9 @@
 #include "../../include/dejavu_hip.h"
 
 #include <hip/hip_runtime.h>
+#include <stdlib.h>
 
+#include "attention.hpp"
 #include "common.hpp"
 #include "gemv_cols.hpp"
 #include "gemv_rows.hpp"
@@ -100,12 +102,21 @@ int gather_rows_b(const half_t* x, const half_t* W, int64_t ldw, const half_t* b
 // ---- gathered column GEMV (fc2 / out_proj over transposed weights) ----------
 struct ColsPlan {
   int col_tiles, groups, rows_per_block;
+  bool fused;
 };
+
+int tuning_env(const char* name, int fallback) {
+  const char* v = getenv(name);
+  return v ? atoi(v) : fallback;
+}
 
 ColsPlan plan_cols(int N, int M) {
   ColsPlan p;
   p.col_tiles = (N + kColTile - 1) / kColTile;
-  const int target_blocks = compute_units() * 6;
+  static const int blocks_per_cu = tuning_env("DV_COLS_BLOCKS_PER_CU", 3);
+  static const int fused = tuning_env("DV_COLS_FUSED", 0);
+  p.fused = fused != 0;
+  const int target_blocks = compute_units() * blocks_per_cu;
   int groups = (target_blocks + p.col_tiles - 1) / p.col_tiles;
   int max_groups = (M + 15) / 16;  // at least 16 rows per workgroup
   if (max_groups < 1) max_groups = 1;
@@ -120,11 +131,34 @@ ColsPlan plan_cols(int N, int M) {
   return p;
 }
 
+// Workspace layout: completion counters first, at a fixed place, so that they
+// stay zero between launches of different shapes that share one workspace (the
+// kernels reset them; the partial sums behind them hold stale values).
+constexpr size_t kCounterBytes = 4096;
+constexpr int kMaxColTiles = (int)(kCounterBytes / sizeof(unsigned));
+
 size_t cols_workspace_bytes(int B, int N, int M) {
   const ColsPlan p = plan_cols(N, M);
-  size_t partial = (size_t)p.groups * B * N * sizeof(float);
-  partial = (partial + 255) & ~(size_t)255;
-  return partial + (size_t)p.col_tiles * sizeof(unsigned);
+  return kCounterBytes + (size_t)p.groups * B * N * sizeof(float);
+}
+
+template <int B, bool IDX64, bool BLOCKED>
+void launch_cols(const ColsPlan& p, const half_t* x, int64_t ldx, int x_expanded, const half_t* W,
+                 int64_t ldw, const half_t* bias, const void* idx, int blk, int N, int Z, int M,
+                 float* partial, unsigned* counters, half_t* y, hipStream_t s) {
+  dim3 grid(p.col_tiles, p.groups);
+  if (p.fused || p.groups == 1) {
+    hipLaunchKernelGGL((gather_cols_kernel<B, 8, IDX64, BLOCKED, true>), grid, dim3(256), 0, s, x,
+                       ldx, x_expanded, W, ldw, bias, idx, blk, N, Z, M, p.rows_per_block, partial,
+                       counters, y);
+  } else {
+    hipLaunchKernelGGL((gather_cols_kernel<B, 8, IDX64, BLOCKED, false>), grid, dim3(256), 0, s, x,
+                       ldx, x_expanded, W, ldw, bias, idx, blk, N, Z, M, p.rows_per_block, partial,
+                       counters, y);
+    const int64_t total = (int64_t)B * N;
+    hipLaunchKernelGGL(cols_reduce_kernel, dim3((unsigned)((total + 63) / 64)), dim3(256), 0, s,
+                       partial, bias, p.groups, B, N, y);
+  }
 }
 
 int gather_cols(const half_t* x, int64_t ldx, int x_expanded, const half_t* W, int64_t ldw,
@@ -133,17 +167,20 @@ int gather_cols(const half_t* x, int64_t ldx, int x_expanded, const half_t* W, i
   const ColsPlan p = plan_cols(N, M);
   if (workspace == nullptr || workspace_bytes < cols_workspace_bytes(B, N, M))
     return DV_ERR_WORKSPACE;
-  size_t partial_bytes = (size_t)p.groups * B * N * sizeof(float);
-  partial_bytes = (partial_bytes + 255) & ~(size_t)255;
-  float* partial = reinterpret_cast<float*>(workspace);
-  unsigned* counters =
-      reinterpret_cast<unsigned*>(reinterpret_cast<unsigned char*>(workspace) + partial_bytes);
-  dim3 grid(p.col_tiles, p.groups);
-#define DV_CASE(BB)                                                                               \
-  case BB:                                                                                        \
-    hipLaunchKernelGGL((gather_cols_kernel<BB, 8>), grid, dim3(256), 0, s, x, ldx, x_expanded, W, \
-                       ldw, bias, idx, idx_bytes, blk, N, Z, M, p.rows_per_block, partial,        \
-                       counters, y);                                                              \
+  if (p.col_tiles > kMaxColTiles) return DV_ERR_UNSUPPORTED;
+  unsigned* counters = reinterpret_cast<unsigned*>(workspace);
+  float* partial =
+      reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(workspace) + kCounterBytes);
+#define DV_ARGS p, x, ldx, x_expanded, W, ldw, bias, idx, blk, N, Z, M, partial, counters, y, s
+#define DV_CASE(BB)                                                   \
+  case BB:                                                            \
+    if (blk == 1) {                                                   \
+      if (idx_bytes == 8) launch_cols<BB, true, false>(DV_ARGS);      \
+      else launch_cols<BB, false, false>(DV_ARGS);                    \
+    } else {                                                          \
+      if (idx_bytes == 8) launch_cols<BB, true, true>(DV_ARGS);       \
+      else launch_cols<BB, false, true>(DV_ARGS);                     \
+    }                                                                 \
     break;
   switch (B) {
     DV_CASE(1) DV_CASE(2) DV_CASE(3) DV_CASE(4)
@@ -151,8 +188,27 @@ int gather_cols(const half_t* x, int64_t ldx, int x_expanded, const half_t* W, i
       return DV_ERR_UNSUPPORTED;
   }
 #undef DV_CASE
+#undef DV_ARGS
   return launch_status();
 }
+
+// ---- head-sparse attention ---------------------------------------------------
+template <int NBMAX>
+int launch_qkv(const half_t* x, const half_t* W, const half_t* bias, const int* head_idx,
+               const int* batch_idx, int nb, int d, int H, int hd, int nnz, half_t* y,
+               hipStream_t s) {
+  constexpr int R = 2, U = 4;
+  const int ntasks = nnz * 3 * (hd / R);
+  int blocks = (ntasks + 3) / 4;
+  const int cap = compute_units() * 8;
+  if (blocks > cap) blocks = cap;
+  if (blocks < 1) blocks = 1;
+  hipLaunchKernelGGL((qkv_sparse_kernel<NBMAX, R, U>), dim3(blocks), dim3(256), 0, s, x, W, bias,
+                     head_idx, batch_idx, nb, d, H, hd, nnz, y);
+  return launch_status();
+}
+
+inline int attn_splits(int n_len) { return n_len > 0 ? (n_len + kWave - 1) / kWave : 1; }
 
 }  // namespace
 
@@ -236,7 +292,7 @@ int dv_topk_f16(const void* logits, int B, int n, int k, void* idx_out, int idx_
 int dv_gather_gemv_f16(const void* x, const void* W, int64_t ldw, const void* bias,
                        const void* idx, int idx_bytes, int B, int N, int Z, int M, int act,
                        void* y, void* stream) {
-  if (!x || !W || !idx || !y || N <= 0 || Z <= 0 || M < 0 || !idx_ok(idx_bytes) ||
+  if (!x || !W || N <= 0 || Z <= 0 || M < 0 || !idx_ok(idx_bytes) || (M > 0 && (!idx || !y)) ||
       (act != DV_ACT_ID && act != DV_ACT_RELU))
     return DV_ERR_INVALID_ARG;
   if (B < 1 || B > 4) return DV_ERR_UNSUPPORTED;
@@ -264,7 +320,7 @@ int dv_gather_transposed_gemv_f16(const void* x, const void* W, int64_t ldw, con
                                   const void* idx, int idx_bytes, int B, int N, int Z, int M,
                                   void* y, void* workspace, size_t workspace_bytes,
                                   void* stream) {
-  if (!x || !W || !y || N <= 0 || Z <= 0 || M < 0 || !idx_ok(idx_bytes) || (M > 0 && !idx))
+  if (!W || !y || N <= 0 || Z <= 0 || M < 0 || !idx_ok(idx_bytes) || (M > 0 && (!idx || !x)))
     return DV_ERR_INVALID_ARG;
   if (B < 1 || B > 4) return DV_ERR_UNSUPPORTED;
   if (N % 8 || ldw % 8 || ldw < N || !aligned16(W)) return DV_ERR_ALIGNMENT;
@@ -272,6 +328,150 @@ int dv_gather_transposed_gemv_f16(const void* x, const void* W, int64_t ldw, con
                      ldw, reinterpret_cast<const half_t*>(bias), idx, idx_bytes, 1, B, N, Z, M,
                      reinterpret_cast<half_t*>(y), workspace, workspace_bytes,
                      reinterpret_cast<hipStream_t>(stream));
+}
+
+int dv_qkv_proj_sparse_f16(const void* x, const void* W, const void* bias, const void* head_idx,
+                           const void* batch_idx, int nb, int d, int H, int hd, int nnz, void* y,
+                           void* stream) {
+  if (!x || !W || !y || nb < 1 || d <= 0 || H <= 0 || nnz < 0 || (nnz > 0 && (!head_idx || !batch_idx)))
+    return DV_ERR_INVALID_ARG;
+  if (nb > 16 || (hd != 32 && hd != 64 && hd != 128)) return DV_ERR_UNSUPPORTED;
+  if (d % 8 || !aligned16(x) || !aligned16(W)) return DV_ERR_ALIGNMENT;
+  if (nnz == 0) return DV_OK;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const half_t* xx = reinterpret_cast<const half_t*>(x);
+  const half_t* ww = reinterpret_cast<const half_t*>(W);
+  const half_t* bb = reinterpret_cast<const half_t*>(bias);
+  const int* hi = reinterpret_cast<const int*>(head_idx);
+  const int* bi = reinterpret_cast<const int*>(batch_idx);
+  half_t* yy = reinterpret_cast<half_t*>(y);
+  if (nb == 1) return launch_qkv<1>(xx, ww, bb, hi, bi, nb, d, H, hd, nnz, yy, s);
+  if (nb == 2) return launch_qkv<2>(xx, ww, bb, hi, bi, nb, d, H, hd, nnz, yy, s);
+  if (nb <= 4) return launch_qkv<4>(xx, ww, bb, hi, bi, nb, d, H, hd, nnz, yy, s);
+  if (nb <= 8) return launch_qkv<8>(xx, ww, bb, hi, bi, nb, d, H, hd, nnz, yy, s);
+  return launch_qkv<16>(xx, ww, bb, hi, bi, nb, d, H, hd, nnz, yy, s);
+}
+
+int dv_kv_cache_copy_sparse_f16(const void* k, const void* v, int64_t ld_src, int nsrc,
+                                void* k_cache, void* v_cache, const void* head_idx,
+                                const void* seq_idx, int nnz, int nslots, const void* padding,
+                                int H, int hd, int S, void* stream) {
+  if ((!k_cache && !v_cache) || (k_cache && !k) || (v_cache && !v) || nsrc < 0 || nnz < 0 ||
+      nslots < 0 || H <= 0 || S <= 0 || (nnz > 0 && nslots > 0 && (!head_idx || !seq_idx)))
+    return DV_ERR_INVALID_ARG;
+  if (hd % 8 || hd > 1024 || hd <= 0) return DV_ERR_UNSUPPORTED;
+  if (nnz == 0 || nslots == 0 || nsrc == 0) return DV_OK;
+  hipLaunchKernelGGL(kv_cache_copy_kernel, dim3(nnz, nslots), dim3(hd), 0,
+                     reinterpret_cast<hipStream_t>(stream), reinterpret_cast<const half_t*>(k),
+                     reinterpret_cast<const half_t*>(v), ld_src, nsrc,
+                     reinterpret_cast<half_t*>(k_cache), reinterpret_cast<half_t*>(v_cache),
+                     reinterpret_cast<const int*>(head_idx), reinterpret_cast<const int*>(seq_idx),
+                     nslots, reinterpret_cast<const int*>(padding), H, hd, S);
+  return launch_status();
+}
+
+int dv_kv_append_f16(const void* k, const void* v, int64_t ld_src, void* k_cache, void* v_cache,
+                     const void* head_idx, int nheads, const void* lengths, int pos, int B, int H,
+                     int hd, int S, void* stream) {
+  if (!k || !v || !k_cache || !v_cache || nheads < 0 || B < 1 || H <= 0 || S <= 0)
+    return DV_ERR_INVALID_ARG;
+  if (hd % 8 || hd > 1024 || hd <= 0) return DV_ERR_UNSUPPORTED;
+  if (!lengths && (pos < 0 || pos >= S)) return DV_ERR_INVALID_ARG;
+  const int heads = head_idx ? nheads : H;
+  if (heads == 0) return DV_OK;
+  hipLaunchKernelGGL(kv_append_kernel, dim3(heads, B), dim3(hd), 0,
+                     reinterpret_cast<hipStream_t>(stream), reinterpret_cast<const half_t*>(k),
+                     reinterpret_cast<const half_t*>(v), ld_src, reinterpret_cast<half_t*>(k_cache),
+                     reinterpret_cast<half_t*>(v_cache), reinterpret_cast<const int*>(head_idx),
+                     reinterpret_cast<const int*>(lengths), pos, H, hd, S);
+  return launch_status();
+}
+
+size_t dv_decode_attention_workspace_bytes(int B, int nheads, int n_len, int hd) {
+  if (B < 1 || nheads < 0 || n_len < 0 || hd <= 0) return 0;
+  return (size_t)B * nheads * attn_splits(n_len) * (hd + 2) * sizeof(float);
+}
+
+int dv_decode_attention_f16(const void* q, int64_t ldq, const void* k_cache, const void* v_cache,
+                            const void* head_idx, int nheads, const void* lengths, int n_len,
+                            int B, int H, int hd, int S, float scale, void* out, int64_t ldo,
+                            void* workspace, size_t workspace_bytes, void* stream) {
+  if (!q || !k_cache || !v_cache || !out || nheads < 0 || B < 1 || H <= 0 || S <= 0 ||
+      n_len < 1 || n_len > S)
+    return DV_ERR_INVALID_ARG;
+  if (hd != 64 && hd != 128) return DV_ERR_UNSUPPORTED;
+  if (ldq % 8 || !aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache))
+    return DV_ERR_ALIGNMENT;
+  const int heads = head_idx ? nheads : H;
+  if (heads == 0) return DV_OK;
+  if (!workspace || workspace_bytes < dv_decode_attention_workspace_bytes(B, heads, n_len, hd))
+    return DV_ERR_WORKSPACE;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const int nsplit = attn_splits(n_len);
+  float* part = reinterpret_cast<float*>(workspace);
+  const half_t* qq = reinterpret_cast<const half_t*>(q);
+  const half_t* kc = reinterpret_cast<const half_t*>(k_cache);
+  const half_t* vc = reinterpret_cast<const half_t*>(v_cache);
+  const int* hi = reinterpret_cast<const int*>(head_idx);
+  const int* ln = reinterpret_cast<const int*>(lengths);
+  half_t* oo = reinterpret_cast<half_t*>(out);
+  dim3 grid(nsplit, heads, B);
+  if (hd == 128) {
+    hipLaunchKernelGGL((decode_attn_kernel<128>), grid, dim3(64), 0, s, qq, ldq, kc, vc, hi, ln,
+                       n_len, H, S, scale, nsplit, part);
+    hipLaunchKernelGGL((decode_attn_combine_kernel<128>), dim3(heads, B), dim3(128), 0, s, part,
+                       hi, H, nsplit, oo, ldo);
+  } else {
+    hipLaunchKernelGGL((decode_attn_kernel<64>), grid, dim3(64), 0, s, qq, ldq, kc, vc, hi, ln,
+                       n_len, H, S, scale, nsplit, part);
+    hipLaunchKernelGGL((decode_attn_combine_kernel<64>), dim3(heads, B), dim3(64), 0, s, part, hi,
+                       H, nsplit, oo, ldo);
+  }
+  return launch_status();
+}
+
+int dv_out_proj_sparse_f16(const void* x, const void* W, const void* bias, const void* head_idx,
+                           int nnz, int B, int H, int hd, int N, void* y, void* stream) {
+  if (!x || !W || !y || nnz < 0 || B < 1 || H <= 0 || N <= 0 || (nnz > 0 && !head_idx))
+    return DV_ERR_INVALID_ARG;
+  if (B > 4 || (hd != 64 && hd != 128)) return DV_ERR_UNSUPPORTED;
+  if (!aligned16(x) || !aligned16(W)) return DV_ERR_ALIGNMENT;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  constexpr int R = 4;
+  const int ntasks = (N + R - 1) / R;
+  int blocks = (ntasks + 3) / 4;
+  const int cap = compute_units() * 8;
+  if (blocks > cap) blocks = cap;
+#define DV_OP(BB, HH)                                                                          \
+  hipLaunchKernelGGL((out_proj_rows_kernel<BB, R, HH>), dim3(blocks), dim3(256), 0, s,          \
+                     reinterpret_cast<const half_t*>(x), reinterpret_cast<const half_t*>(W),   \
+                     reinterpret_cast<const half_t*>(bias), reinterpret_cast<const int*>(head_idx), \
+                     nnz, H, N, reinterpret_cast<half_t*>(y))
+  if (hd == 128) {
+    switch (B) { case 1: DV_OP(1, 128); break; case 2: DV_OP(2, 128); break; case 3: DV_OP(3, 128); break; default: DV_OP(4, 128); }
+  } else {
+    switch (B) { case 1: DV_OP(1, 64); break; case 2: DV_OP(2, 64); break; case 3: DV_OP(3, 64); break; default: DV_OP(4, 64); }
+  }
+#undef DV_OP
+  return launch_status();
+}
+
+size_t dv_out_proj_sparse_t_workspace_bytes(int B, int N, int nnz, int hd) {
+  if (B < 1 || N < 1 || nnz < 0 || hd < 1) return 0;
+  return cols_workspace_bytes(B, N, nnz * hd);
+}
+
+int dv_out_proj_sparse_t_f16(const void* x, const void* Wt, int64_t ldw, const void* bias,
+                             const void* head_idx, int nnz, int B, int H, int hd, int N, void* y,
+                             void* workspace, size_t workspace_bytes, void* stream) {
+  if (!x || !Wt || !y || nnz < 0 || B < 1 || H <= 0 || hd <= 0 || N <= 0 || (nnz > 0 && !head_idx))
+    return DV_ERR_INVALID_ARG;
+  if (B > 4) return DV_ERR_UNSUPPORTED;
+  if (N % 8 || ldw % 8 || ldw < N || !aligned16(Wt)) return DV_ERR_ALIGNMENT;
+  return gather_cols(reinterpret_cast<const half_t*>(x), (int64_t)H * hd, 1,
+                     reinterpret_cast<const half_t*>(Wt), ldw, reinterpret_cast<const half_t*>(bias),
+                     head_idx, 4, hd, B, N, H * hd, nnz * hd, reinterpret_cast<half_t*>(y),
+                     workspace, workspace_bytes, reinterpret_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

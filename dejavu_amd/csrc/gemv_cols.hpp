@@ -1,9 +1,9 @@
 // Column-wise ("transposed") gathered GEMV: Y[b, :] = sum_m x[b, m] * W[row(m), :] + bias.
 // Lanes own 8 adjacent output columns each and stream the gathered rows with
 // 128-bit loads; no cross-lane reduction is needed.  The M rows are split over
-// gridDim.y row groups; each group writes an fp32 partial and the last group
-// to finish a column tile sums the partials in a fixed order (deterministic,
-// no floating-point atomics) and adds the bias.
+// gridDim.y row groups; each group writes an fp32 partial, and the partials are
+// summed in a fixed order (deterministic, no floating-point atomics) either by
+// the last group to finish a column tile (FUSED) or by cols_reduce_kernel.
 #pragma once
 #include "common.hpp"
 
@@ -11,16 +11,26 @@ namespace dv {
 
 constexpr int kColTile = 8 * kWave;  // 512 columns per workgroup
 
-// Row mapping: with blk == 1, row(m) = idx[m] (sparse-MLP fc2 over W2^T).
-// With blk > 1, row(m) = idx[m / blk] * blk + m % blk (out_proj over
-// W_out^T, blk = head_dim, idx = active heads).
-// x_expanded == 0: X is (B, M), x[b, m];  == 1: X is (B, Z), x[b, row(m)].
-template <int B, int U>
+// Partials cross workgroups (and XCDs, whose L2s are not coherent with each
+// other): they are written and read with agent-scope accesses that go to the
+// device-wide coherence point, so no L2-wide write-back / invalidate is needed.
+__device__ __forceinline__ void store_agent(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_agent(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Row mapping: BLOCKED == false: row(m) = idx[m] (sparse-MLP fc2 over W2^T).
+// BLOCKED == true: row(m) = idx[m / blk] * blk + m % blk (out_proj over
+// W_out^T with blk = head_dim and idx = active heads).
+// x_expanded == 0: X is (B, M), x[b, m];  != 0: X is (B, Z), x[b, row(m)].
+template <int B, int U, bool IDX64, bool BLOCKED, bool FUSED>
 __global__ __launch_bounds__(256) void gather_cols_kernel(
     const half_t* __restrict__ X, int64_t ldx, int x_expanded, const half_t* __restrict__ W,
-    int64_t ldw, const half_t* __restrict__ bias, const void* __restrict__ idx, int idx_bytes,
-    int blk, int N, int Z, int M, int rows_per_block, float* __restrict__ partial,
-    unsigned* __restrict__ counters, half_t* __restrict__ Y) {
+    int64_t ldw, const half_t* __restrict__ bias, const void* __restrict__ idx, int blk, int N,
+    int Z, int M, int rows_per_block, float* __restrict__ partial, unsigned* __restrict__ counters,
+    half_t* __restrict__ Y) {
   __shared__ float red[4][B][kColTile];
   __shared__ int s_last;
 
@@ -32,6 +42,7 @@ __global__ __launch_bounds__(256) void gather_cols_kernel(
   const int G = gridDim.y;
   const int col = ct * kColTile + lane * 8;
   const bool col_ok = col < N;  // N % 8 == 0, so a lane is all-in or all-out
+  const half_t* wcol = W + (col_ok ? col : 0);
 
   const int rpw = (rows_per_block + 3) >> 2;
   const int m_begin = g * rows_per_block + wave * rpw;
@@ -45,36 +56,70 @@ __global__ __launch_bounds__(256) void gather_cols_kernel(
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[b][e] = 0.f;
 
-  for (int m0 = m_begin; m0 < m_end; m0 += U) {
-    half8_t w[U];
-    float xv[U][B];
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int m = m0 + u;
-      int64_t id = -1;
-      if (m < m_end) {
-        id = blk == 1 ? load_index(idx, idx_bytes, m)
-                      : load_index(idx, idx_bytes, m / blk) * blk + m % blk;
+  // 64 rows at a time: lane l fetches the row id and the activations of row
+  // mb + l once; the row loop then broadcasts them with readlane, so the
+  // weight loads are issued back to back without scalar-load stalls.
+  for (int mb = m_begin; mb < m_end; mb += kWave) {
+    const int m = mb + lane;
+    int rid = 0;
+    bool ok = false;
+    if (m < m_end) {
+      int64_t id;
+      if (BLOCKED) {
+        const int q = m / blk;
+        const int64_t h = IDX64 ? reinterpret_cast<const int64_t*>(idx)[q]
+                                : (int64_t) reinterpret_cast<const int32_t*>(idx)[q];
+        id = (h >= 0 && h < Z / blk) ? h * blk + (m - q * blk) : -1;
+      } else {
+        id = IDX64 ? reinterpret_cast<const int64_t*>(idx)[m]
+                   : (int64_t) reinterpret_cast<const int32_t*>(idx)[m];
       }
-      const bool ok = id >= 0 && id < Z;
-      w[u] = (ok && col_ok) ? load8_stream(W + id * ldw + col) : zero8();
-#pragma unroll
-      for (int b = 0; b < B; ++b)
-        xv[u][b] = ok ? (float)X[(int64_t)b * ldx + (x_expanded ? id : (int64_t)m)] : 0.f;
+      ok = id >= 0 && id < Z;
+      rid = ok ? (int)id : 0;
     }
+    float xl[B];
 #pragma unroll
-    for (int u = 0; u < U; ++u)
+    for (int b = 0; b < B; ++b)
+      xl[b] = ok ? (float)X[(int64_t)b * ldx + (x_expanded ? (int64_t)rid : (int64_t)m)] : 0.f;
+
+    const int cnt = (m_end - mb) < kWave ? (m_end - mb) : kWave;
+    int j = 0;
+    for (; j + U <= cnt; j += U) {
+      half8_t w[U];
 #pragma unroll
-      for (int b = 0; b < B; ++b)
+      for (int u = 0; u < U; ++u) {
+        const int r = __builtin_amdgcn_readlane(rid, j + u);
+        w[u] = load8_stream(wcol + (int64_t)r * ldw);
+      }
 #pragma unroll
-        for (int e = 0; e < 8; ++e) acc[b][e] = __builtin_fmaf((float)w[u][e], xv[u][b], acc[b][e]);
+      for (int u = 0; u < U; ++u) {
+#pragma unroll
+        for (int b = 0; b < B; ++b) {
+          const float xs = __builtin_bit_cast(
+              float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, xl[b]), j + u));
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[b][e] = __builtin_fmaf((float)w[u][e], xs, acc[b][e]);
+        }
+      }
+    }
+    for (; j < cnt; ++j) {
+      const int r = __builtin_amdgcn_readlane(rid, j);
+      const half8_t w = load8_stream(wcol + (int64_t)r * ldw);
+#pragma unroll
+      for (int b = 0; b < B; ++b) {
+        const float xs =
+            __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, xl[b]), j));
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[b][e] = __builtin_fmaf((float)w[e], xs, acc[b][e]);
+      }
+    }
   }
 
   // combine the four wavefronts of the workgroup
 #pragma unroll
   for (int b = 0; b < B; ++b)
 #pragma unroll
-    for (int e = 0; e < 8; ++e) red[wave][b][lane * 8 + e] = acc[b][e];
+    for (int e = 0; e < 8; ++e) red[wave][b][lane * 8 + e] = col_ok ? acc[b][e] : 0.f;
   __syncthreads();
 
   constexpr int PER_THREAD = B * kColTile / 256;
@@ -96,32 +141,88 @@ __global__ __launch_bounds__(256) void gather_cols_kernel(
     return;
   }
 
+  if (!FUSED) {
+#pragma unroll
+    for (int j = 0; j < PER_THREAD; ++j) {
+      const int o = j * 256 + tid;
+      const int b = o / kColTile, c = ct * kColTile + o % kColTile;
+      if (c < N) partial[((int64_t)g * B + b) * N + c] = sum[j];
+    }
+    return;
+  }
+
 #pragma unroll
   for (int j = 0; j < PER_THREAD; ++j) {
     const int o = j * 256 + tid;
     const int b = o / kColTile, c = ct * kColTile + o % kColTile;
-    if (c < N) partial[((int64_t)g * B + b) * N + c] = sum[j];
+    if (c < N) store_agent(&partial[((int64_t)g * B + b) * N + c], sum[j]);
   }
-  __threadfence();  // release the partials device-wide before signalling
+  // every wavefront waits for its own partial stores to be acknowledged, then
+  // the workgroup meets, then one thread signals completion
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
   if (tid == 0) {
-    const unsigned old = atomicAdd(&counters[ct], 1u);
+    const unsigned old =
+        __hip_atomic_fetch_add(&counters[ct], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     s_last = (old == (unsigned)(G - 1));
   }
   __syncthreads();
   if (!s_last) return;
-  __threadfence();  // acquire the other groups' partials
 #pragma unroll
   for (int j = 0; j < PER_THREAD; ++j) {
     const int o = j * 256 + tid;
     const int b = o / kColTile, c = ct * kColTile + o % kColTile;
     if (c < N) {
+      const float* p = partial + (int64_t)b * N + c;
+      const int64_t gstride = (int64_t)B * N;
       float s = 0.f;
-      for (int gg = 0; gg < G; ++gg) s += partial[((int64_t)gg * B + b) * N + c];
+      int gg = 0;
+      for (; gg + 8 <= G; gg += 8) {
+        float v[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) v[q] = load_agent(p + (gg + q) * gstride);
+#pragma unroll
+        for (int q = 0; q < 8; ++q) s += v[q];
+      }
+      for (; gg < G; ++gg) s += load_agent(p + gg * gstride);
       Y[(int64_t)b * N + c] = (half_t)(s + (bias ? (float)bias[c] : 0.f));
     }
   }
-  if (tid == 0) counters[ct] = 0;  // leave the counter ready for the next launch
+  if (tid == 0)
+    __hip_atomic_store(&counters[ct], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Second pass of the non-fused path: Y[b, c] = fp16(sum_g partial[g, b, c] + bias[c]).
+// A workgroup owns 64 outputs; its four wavefronts each add every fourth group
+// (ascending), and the four slice sums are combined in a fixed order.
+__global__ __launch_bounds__(256) void cols_reduce_kernel(const float* __restrict__ partial,
+                                                          const half_t* __restrict__ bias, int G,
+                                                          int B, int N, half_t* __restrict__ Y) {
+  __shared__ float red[4][kWave];
+  const int lane = threadIdx.x & 63;
+  const int slice = threadIdx.x >> 6;
+  const int64_t total = (int64_t)B * N;
+  const int64_t o = (int64_t)blockIdx.x * kWave + lane;
+  float s = 0.f;
+  if (o < total) {
+    const float* p = partial + o;
+    int gg = slice;
+    for (; gg + 28 < G; gg += 32) {
+      float v[8];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) v[q] = p[(int64_t)(gg + 4 * q) * total];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) s += v[q];
+    }
+    for (; gg < G; gg += 4) s += p[(int64_t)gg * total];
+  }
+  red[slice][lane] = s;
+  __syncthreads();
+  if (slice == 0 && o < total) {
+    const float r = (red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]);
+    Y[o] = (half_t)(r + (bias ? (float)bias[o % N] : 0.f));
+  }
 }
 
 }  // namespace dv

@@ -40,46 +40,59 @@ __global__ __launch_bounds__(THREADS) void topk_kernel(const half_t* __restrict_
   for (int i = 0; i < ITEMS / 2; ++i) key2[i] = 0u;  // padding never reaches a real key
   for (int b = 0; b < B; ++b) {
     const half_t* row = logits + (int64_t)b * n;
+    if (VEC) {
+      // all loads of a row are issued back to back; out-of-range groups read
+      // the (valid) start of the row and are masked afterwards
+      half8_t v[ITEMS / 8];
 #pragma unroll
-    for (int i = 0; i < ITEMS; i += 8) {
-      half8_t v = zero8();
-      bool have[8];
-      if (VEC) {
-        const bool in = base + i < n;
-        if (in) v = load8(row + base + i);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) have[e] = in;
-      } else {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          have[e] = base + i + e < n;
-          if (have[e]) v[e] = row[base + i + e];
-        }
+      for (int i = 0; i < ITEMS / 8; ++i) {
+        const int off = base + i * 8;
+        v[i] = load8(row + (off < n ? off : 0));
       }
 #pragma unroll
-      for (int e = 0; e < 8; e += 2) {
-        const unsigned lo = have[e] ? topk_key(v[e]) : 0u;
-        const unsigned hi = have[e + 1] ? topk_key(v[e + 1]) : 0u;
-        const unsigned old = key2[(i + e) / 2];
+      for (int i = 0; i < ITEMS / 8; ++i) {
+        const bool in = base + i * 8 < n;
+#pragma unroll
+        for (int e = 0; e < 8; e += 2) {
+          const unsigned lo = in ? topk_key(v[i][e]) : 0u;
+          const unsigned hi = in ? topk_key(v[i][e + 1]) : 0u;
+          const unsigned old = key2[(i * 8 + e) / 2];
+          const unsigned olo = old & 0xFFFFu, ohi = old >> 16;
+          key2[(i * 8 + e) / 2] = (lo > olo ? lo : olo) | ((hi > ohi ? hi : ohi) << 16);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < ITEMS; i += 2) {
+        const unsigned lo = base + i < n ? topk_key(row[base + i]) : 0u;
+        const unsigned hi = base + i + 1 < n ? topk_key(row[base + i + 1]) : 0u;
+        const unsigned old = key2[i / 2];
         const unsigned olo = old & 0xFFFFu, ohi = old >> 16;
-        key2[(i + e) / 2] = (lo > olo ? lo : olo) | ((hi > ohi ? hi : ohi) << 16);
+        key2[i / 2] = (lo > olo ? lo : olo) | ((hi > ohi ? hi : ohi) << 16);
       }
     }
   }
 
-  // largest T with count(key >= T) >= k
+  // largest T with count(key >= T) >= k.  Per thread the count is kept as two
+  // packed 16-bit counters: [key >= cand] = min(sat_sub(key, cand - 1), 1).
   unsigned T = 0u;
   for (int bit = 15; bit >= 0; --bit) {
     const unsigned cand = T | (1u << bit);
-    unsigned c = 0;
+    const unsigned cm1 = (cand - 1u) * 0x00010001u;  // cand - 1 in both halves
+    const unsigned one = 0x00010001u;
+    unsigned acc2 = 0u;
 #pragma unroll
     for (int i = 0; i < ITEMS / 2; ++i) {
-      // keep the keys packed across iterations (stops the unpacked halves from
-      // being hoisted out of the search loop into twice the registers)
-      asm volatile("" : "+v"(key2[i]));
-      c += (unsigned)__popcll(__ballot((key2[i] & 0xFFFFu) >= cand));
-      c += (unsigned)__popcll(__ballot((key2[i] >> 16) >= cand));
+      // written as instructions: the compiler otherwise expands the packed
+      // saturating form into per-half compares and selects
+      unsigned t;
+      asm volatile("v_pk_sub_u16 %0, %1, %2 clamp" : "=v"(t) : "v"(key2[i]), "v"(cm1));
+      asm volatile("v_pk_min_u16 %0, %1, %2" : "=v"(t) : "v"(t), "v"(one));
+      asm volatile("v_pk_add_u16 %0, %1, %2" : "=v"(acc2) : "v"(acc2), "v"(t));
     }
+    unsigned c = (acc2 & 0xFFFFu) + (acc2 >> 16);
+#pragma unroll
+    for (int off = kWave / 2; off >= 1; off >>= 1) c += __shfl_xor(c, off, kWave);
     const int buf = bit & 1;
     if (lane == 0) s_cnt[buf][wave] = c;
     __syncthreads();

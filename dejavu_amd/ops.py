@@ -186,3 +186,249 @@ def mlp_sparse(x, W1, W2t, idx, bias1=None, bias2=None):
     x = gather_gemv(x, W1, idx, bias1, activation="relu")
     x = gather_transposed_gemv(x, W2t, idx, bias2)
     return x
+
+
+# ---------------------------------------------------------------------------
+# head-sparse attention
+# ---------------------------------------------------------------------------
+def qkv_proj_sparse(x: torch.Tensor, weight: torch.Tensor, head_idx: torch.Tensor, batch_idx: torch.Tensor,
+                    bias: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """
+    Compute y = torch.einsum("bm,thdm->bthd", x, weight), but only for the active heads in @head_idx
+    and only for the batch indices in @batch_idx. Negative indices in batch_idx will be ignored.
+    :param x: input tensor, (batch_size, hidden_dim)
+    :param weight: weight matrix, (3, nheads, head_dim, hidden_dim)
+    :param head_idx: int32, (nnz,)
+    :param batch_idx: int32, (nnz, batch_size). Negative indices are ignored.
+    :param bias: indices, (3, nheads, head_dim)
+    :return: result tensor, (batch_size, 3, nheads, head_dim); entries of inactive heads /
+        skipped rows are uninitialised (or keep the content of ``out`` when it is given)
+    """
+    _require_device(x, weight, head_idx, batch_idx, bias)
+    three, nheads, head_dim, hidden_dim = weight.shape
+    assert three == 3
+    assert head_dim in [32, 64, 128]
+    assert hidden_dim % 128 == 0
+    batch_size, _ = x.shape
+    assert batch_size <= 16
+    assert x.shape == (batch_size, hidden_dim)
+    n_active = head_idx.shape[0]
+    assert n_active <= nheads
+    assert head_idx.shape == (n_active,)
+    assert head_idx.dtype == torch.int32
+    assert batch_idx.shape == (n_active, batch_size)
+    assert batch_idx.dtype == torch.int32
+    x = x.contiguous()
+    weight = weight.contiguous()
+    head_idx = head_idx.contiguous()
+    batch_idx = batch_idx.contiguous()
+    assert x.dtype == weight.dtype, f"Input and weight must have the same dtype, got {x.dtype} and {weight.dtype}"
+    assert x.dtype == torch.float16, "kernels are built for fp16"
+    if bias is not None:
+        bias = bias.contiguous()
+        assert bias.shape == (3, nheads, head_dim), "Incompatible dimensions in between weight and bias"
+        assert x.dtype == bias.dtype, f"Input and bias must have the same dtype, got {x.dtype} and {bias.dtype}"
+    if out is None:
+        out = torch.empty(batch_size, 3, nheads, head_dim, device=x.device, dtype=x.dtype)
+    else:
+        assert out.shape == (batch_size, 3, nheads, head_dim) and out.is_contiguous() and out.dtype == x.dtype
+    check(lib.dv_qkv_proj_sparse_f16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(head_idx), _ptr(batch_idx), batch_size,
+                                     hidden_dim, nheads, head_dim, n_active, _ptr(out), _stream()),
+          "dv_qkv_proj_sparse_f16")
+    return out
+
+
+def out_proj_sparse(x: torch.Tensor, weight: torch.Tensor, head_idx: torch.Tensor,
+                    bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """
+    Compute y = torch.einsum("bhd,nhd->bn", x, weight), but only for the active heads in @head_idx.
+    :param x: input tensor, (batch, nheads, head_dim)
+    :param weight: weight matrix, (hidden_dim, nheads, head_dim)
+    :param head_idx: int32, (nnz,)
+    :param bias: indices, (hidden_dim)
+    :return: result tensor, (batch, hidden_dim)
+    """
+    _require_device(x, weight, head_idx, bias)
+    hidden_dim, nheads, head_dim = weight.shape
+    assert head_dim in [32, 64, 128]
+    assert hidden_dim % 128 == 0
+    batch, _, _ = x.shape
+    assert x.shape == (batch, nheads, head_dim)
+    n_active = head_idx.shape[0]
+    assert head_idx.shape == (n_active,)
+    assert head_idx.dtype == torch.int32
+    assert batch <= 16
+    if batch > 4 or head_dim == 32:
+        raise NotImplementedError("out_proj_sparse kernels cover batch <= 4 and head_dim in {64, 128}")
+    x = x.contiguous()
+    weight = weight.contiguous()
+    assert x.dtype == weight.dtype, f"Input and weight must have the same dtype, got {x.dtype} and {weight.dtype}"
+    assert x.dtype == torch.float16, "kernels are built for fp16"
+    if bias is not None:
+        bias = bias.contiguous()
+        assert bias.shape == (hidden_dim,), "Incompatible dimensions in between weight and bias"
+        assert x.dtype == bias.dtype, f"Input and bias must have the same dtype, got {x.dtype} and {bias.dtype}"
+    head_idx = head_idx.contiguous()
+    output = torch.empty(batch, hidden_dim, device=x.device, dtype=x.dtype)
+    check(lib.dv_out_proj_sparse_f16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(head_idx), n_active, batch, nheads,
+                                     head_dim, hidden_dim, _ptr(output), _stream()), "dv_out_proj_sparse_f16")
+    return output
+
+
+def out_proj_sparse_t(x: torch.Tensor, weight_t: torch.Tensor, head_idx: torch.Tensor,
+                      bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Same result as ``out_proj_sparse`` from the transposed weight.
+
+    :param x: (batch, nheads, head_dim)
+    :param weight_t: (nheads * head_dim, hidden_dim) = out_proj.weight.t().contiguous(); the rows
+        of an active head are one contiguous block
+    """
+    _require_device(x, weight_t, head_idx, bias)
+    batch, nheads, head_dim = x.shape
+    rows, hidden_dim = weight_t.shape
+    assert rows == nheads * head_dim
+    assert head_idx.dtype == torch.int32
+    assert batch in [1, 2, 3, 4]
+    n_active = head_idx.shape[0]
+    x = x.contiguous()
+    if weight_t.stride(1) != 1:
+        weight_t = weight_t.contiguous()
+    assert x.dtype == weight_t.dtype == torch.float16
+    if bias is not None:
+        bias = bias.contiguous()
+        assert bias.shape == (hidden_dim,)
+    head_idx = head_idx.contiguous()
+    output = torch.empty(batch, hidden_dim, device=x.device, dtype=x.dtype)
+    nbytes = lib.dv_out_proj_sparse_t_workspace_bytes(batch, hidden_dim, n_active, head_dim)
+    ws = _workspace(x.device, nbytes)
+    check(lib.dv_out_proj_sparse_t_f16(_ptr(x), _ptr(weight_t), weight_t.stride(0), _ptr(bias), _ptr(head_idx),
+                                       n_active, batch, nheads, head_dim, hidden_dim, _ptr(output), _ptr(ws),
+                                       ws.numel(), _stream()), "dv_out_proj_sparse_t_f16")
+    return output
+
+
+def _cache_copy(k, v, k_cache, v_cache, head_idx, seqlen_idx, padding):
+    src = k if k is not None else v
+    _require_device(src, k_cache, v_cache, head_idx, seqlen_idx, padding)
+    nnz_seqlen, nheads, head_dim = src.shape
+    assert head_dim in [32, 64, 128]
+    assert nnz_seqlen <= 16
+    n_active = head_idx.shape[0]
+    assert n_active <= nheads
+    assert head_idx.shape == (n_active,)
+    assert head_idx.dtype == torch.int32
+    assert seqlen_idx.shape == (n_active, nnz_seqlen)
+    assert seqlen_idx.dtype == torch.int32
+    assert src.stride(2) == 1 and src.stride(1) == head_dim, "k / v must be (n, nheads, head_dim) with contiguous heads"
+    head_idx = head_idx.contiguous()
+    seqlen_idx = seqlen_idx.contiguous()
+    if padding is not None:
+        assert padding.shape == (1,)
+        assert padding.dtype == torch.int32
+    if k_cache is not None:
+        packsize = 8
+        assert k.dtype == torch.float16, "kernels are built for fp16"
+        _, _, _, seqlen, _ = k_cache.shape
+        assert k_cache.shape == (1, nheads, head_dim // packsize, seqlen, packsize)
+        assert k_cache.is_contiguous()
+        assert k.dtype == k_cache.dtype, f"k and k_cache must have the same dtype, got {k.dtype} and {k_cache.dtype}"
+    if v_cache is not None:
+        _, _, seqlen, _ = v_cache.shape
+        assert v_cache.shape == (1, nheads, seqlen, head_dim)
+        assert v_cache.is_contiguous()
+        assert v.dtype == v_cache.dtype, f"v and v_cache must have the same dtype, got {v.dtype} and {v_cache.dtype}"
+    if k is not None and v is not None:
+        assert k.stride(0) == v.stride(0)
+    check(lib.dv_kv_cache_copy_sparse_f16(_ptr(k), _ptr(v), src.stride(0), nnz_seqlen, _ptr(k_cache), _ptr(v_cache),
+                                          _ptr(head_idx), _ptr(seqlen_idx), n_active, nnz_seqlen, _ptr(padding),
+                                          nheads, head_dim, seqlen, _stream()), "dv_kv_cache_copy_sparse_f16")
+
+
+def k_cache_copy_sparse(k: torch.Tensor, k_cache: torch.Tensor, head_idx: torch.Tensor, seqlen_idx: torch.Tensor,
+                        padding: torch.Tensor = None) -> None:
+    """
+    :param k: input tensor, (nnz_seqlen, nheads, head_dim)
+    :param k_cache: input tensor, (1, nheads, headdim / PACKSIZE, seqlen, PACKSIZE), PACKSIZE = 8 (fp16)
+    :param head_idx: int32, (nnz,)
+    :param seqlen_idx: int32, (nnz, nnz_seqlen). Negative indices are ignored.
+    :param padding: int32, (1). Padding is added to indices in seqlen_idx before writing to k_cache
+    """
+    _cache_copy(k, None, k_cache, None, head_idx, seqlen_idx, padding)
+
+
+def v_cache_copy_sparse(v: torch.Tensor, v_cache: torch.Tensor, head_idx: torch.Tensor, seqlen_idx: torch.Tensor,
+                        padding: torch.Tensor = None) -> None:
+    """
+    :param v: input tensor, (nnz_seqlen, nheads, head_dim)
+    :param v_cache: input tensor, (1, nheads, seqlen, head_dim)
+    :param head_idx: int32, (nnz,)
+    :param seqlen_idx: int32, (nnz, nnz_seqlen). Negative indices are ignored.
+    :param padding: int32, (1). Padding is added to indices in seqlen_idx before writing to v_cache
+    """
+    _cache_copy(None, v, None, v_cache, head_idx, seqlen_idx, padding)
+
+
+def kv_cache_copy_sparse(k, v, k_cache, v_cache, head_idx, seqlen_idx, padding=None) -> None:
+    """Both cache copies in one launch."""
+    _cache_copy(k, v, k_cache, v_cache, head_idx, seqlen_idx, padding)
+
+
+def single_query_attention(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.Tensor],
+                           k_cache: torch.Tensor, v_cache: torch.Tensor,
+                           lengths_per_sample: Optional[torch.Tensor], timestep: int, rotary_emb_dim: int = 0,
+                           head_idx: Optional[torch.Tensor] = None, softmax_scale: Optional[float] = None,
+                           out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Decode attention with the call shape of ``ft_attention.single_query_attention``.
+
+    q, k, v: (B, H, hd) of the newest token (last dim contiguous); k_cache (B, H, hd/8, S, 8);
+    v_cache (B, H, S, hd).  k, v are written at position ``timestep`` (``lengths_per_sample[b]``
+    when given) and positions up to and including it are attended.  Pass ``k = v = None`` when the
+    caches already hold the newest token.  With ``head_idx`` (int32) only those heads are touched
+    and only their rows of the (B, H, hd) result are written.
+    """
+    _require_device(q, k, v, k_cache, v_cache, lengths_per_sample, head_idx)
+    assert rotary_emb_dim == 0, "OPT has no rotary embedding"
+    B, H, hd = q.shape
+    S = v_cache.shape[2]
+    assert q.dtype == torch.float16 and k_cache.dtype == torch.float16 and v_cache.dtype == torch.float16
+    assert v_cache.shape == (B, H, S, hd) and k_cache.shape == (B, H, hd // 8, S, 8)
+    assert k_cache.is_contiguous() and v_cache.is_contiguous()
+    assert q.stride(2) == 1 and q.stride(1) == hd
+    assert 0 <= timestep < S
+    nheads = 0
+    if head_idx is not None:
+        assert head_idx.dtype == torch.int32
+        head_idx = head_idx.contiguous()
+        nheads = head_idx.shape[0]
+    if lengths_per_sample is not None:
+        assert lengths_per_sample.dtype == torch.int32 and lengths_per_sample.shape == (B,)
+    if k is not None:
+        assert v is not None and k.shape == (B, H, hd) and v.shape == (B, H, hd)
+        assert k.stride(2) == 1 and k.stride(1) == hd and v.stride(2) == 1 and v.stride(1) == hd
+        assert k.stride(0) == v.stride(0)
+        check(lib.dv_kv_append_f16(_ptr(k), _ptr(v), k.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(head_idx),
+                                   nheads, _ptr(lengths_per_sample), timestep, B, H, hd, S, _stream()),
+              "dv_kv_append_f16")
+    if out is None:
+        out = torch.empty(B, H, hd, device=q.device, dtype=q.dtype)
+    n_len = S if lengths_per_sample is not None else timestep + 1
+    scale = float(hd ** -0.5 if softmax_scale is None else softmax_scale)
+    n_heads_ws = nheads if head_idx is not None else H
+    nbytes = lib.dv_decode_attention_workspace_bytes(B, n_heads_ws, n_len, hd)
+    ws = _attn_workspace(q.device, nbytes)
+    check(lib.dv_decode_attention_f16(_ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(head_idx), nheads,
+                                      _ptr(lengths_per_sample), n_len, B, H, hd, S, scale, _ptr(out), out.stride(0),
+                                      _ptr(ws), ws.numel(), _stream()), "dv_decode_attention_f16")
+    return out
+
+
+_attn_workspaces: dict = {}
+
+
+def _attn_workspace(device: torch.device, nbytes: int) -> torch.Tensor:
+    key = (device.type, device.index)
+    ws = _attn_workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _attn_workspaces[key] = ws
+    return ws

@@ -95,6 +95,88 @@ DV_API int dv_gather_transposed_gemv_f16(const void* x, const void* W, int64_t l
                                   void* y, void* workspace, size_t workspace_bytes,
                                   void* stream);
 
+/*
+ * QKV projection restricted to the active heads and the live window tokens:
+ *   y[b, t, h, :] = x[b, :] . W[t, h, :, :]^T + bias[t, h, :]
+ * for h = head_idx[i] and every b = batch_idx[i, s] >= 0.  Nothing is written
+ * for other heads / tokens (the reference leaves them uninitialised too).
+ * Replaces qkv_proj_sparse, Dejavu/src/ops/triton/attention_proj_sparse.py:110-194.
+ *   x (nb, d), nb <= 16; W (3, H, hd, d) contiguous; bias (3, H, hd) or NULL;
+ *   head_idx (nnz,) int32; batch_idx (nnz, nb) int32; y (nb, 3, H, hd);
+ *   hd in {32, 64, 128}.
+ */
+DV_API int dv_qkv_proj_sparse_f16(const void* x, const void* W, const void* bias,
+                                  const void* head_idx, const void* batch_idx, int nb, int d,
+                                  int H, int hd, int nnz, void* y, void* stream);
+
+/*
+ * Scatter of (re)computed keys / values into the caches:
+ *   k_cache[0, h, dp, s + pad, p] = k[s, h, dp*8 + p];  v_cache[0, h, s + pad, :] = v[s, h, :]
+ * for h = head_idx[i], s = seq_idx[i, slot] >= 0.  Either cache may be NULL.
+ * Replaces k_cache_copy_sparse / v_cache_copy_sparse,
+ * Dejavu/src/ops/triton/attention_proj_sparse.py:525-590 and 396-456.
+ *   k, v (nsrc, H, hd) with row stride ld_src; k_cache (1, H, hd/8, S, 8);
+ *   v_cache (1, H, S, hd); head_idx (nnz,) int32; seq_idx (nnz, nslots) int32;
+ *   padding: device int32[1] or NULL (= 0).
+ */
+DV_API int dv_kv_cache_copy_sparse_f16(const void* k, const void* v, int64_t ld_src, int nsrc,
+                                       void* k_cache, void* v_cache, const void* head_idx,
+                                       const void* seq_idx, int nnz, int nslots,
+                                       const void* padding, int H, int hd, int S, void* stream);
+
+/*
+ * Writes the newest token's k, v at position pos (or lengths[b]) of the caches,
+ * for all heads (head_idx NULL) or the listed ones.  This is the cache update
+ * that ft_attention.single_query_attention performs internally (call sites
+ * Dejavu/src/models/modules/mha_dejavu.py:1045-1053, 1439-1456).
+ *   k, v (B, H, hd) with batch stride ld_src; k_cache (B, H, hd/8, S, 8);
+ *   v_cache (B, H, S, hd); lengths: device int32[B] or NULL.
+ */
+DV_API int dv_kv_append_f16(const void* k, const void* v, int64_t ld_src, void* k_cache,
+                            void* v_cache, const void* head_idx, int nheads, const void* lengths,
+                            int pos, int B, int H, int hd, int S, void* stream);
+
+/*
+ * One-query attention over the fp16 KV cache for the listed heads (all if
+ * head_idx is NULL): out[b, h, :] = softmax(q[b, h] . K^T * scale) . V over
+ * positions [0, n_len) (or [0, lengths[b]] when lengths is given; then n_len
+ * is the upper bound S).  fp32 scores, softmax and accumulation.  Rows of
+ * `out` for unlisted heads are not written.  Replaces the attention part of
+ * ft_attention.single_query_attention (same call sites as dv_kv_append_f16).
+ *   q (B, H, hd) with batch stride ldq; out (B, H, hd) with batch stride ldo;
+ *   hd in {64, 128}; workspace: dv_decode_attention_workspace_bytes(...) bytes.
+ */
+DV_API size_t dv_decode_attention_workspace_bytes(int B, int nheads, int n_len, int hd);
+DV_API int dv_decode_attention_f16(const void* q, int64_t ldq, const void* k_cache,
+                                   const void* v_cache, const void* head_idx, int nheads,
+                                   const void* lengths, int n_len, int B, int H, int hd, int S,
+                                   float scale, void* out, int64_t ldo, void* workspace,
+                                   size_t workspace_bytes, void* stream);
+
+/*
+ * y[b, n] = sum_{h in head_idx} x[b, h, :] . W[n, h, :] + bias[n], weight in
+ * out_proj.weight's own (d, H, hd) layout.  Replaces out_proj_sparse,
+ * Dejavu/src/ops/triton/attention_proj_sparse.py:274-338.
+ *   x (B, H, hd) contiguous, B <= 4; W (N, H, hd) contiguous; head_idx int32.
+ */
+DV_API int dv_out_proj_sparse_f16(const void* x, const void* W, const void* bias,
+                                  const void* head_idx, int nnz, int B, int H, int hd, int N,
+                                  void* y, void* stream);
+
+/*
+ * Same result from the transposed weight Wt = W^T, (H*hd, N) with row stride
+ * ldw: the active heads become contiguous row blocks that stream like the fc2
+ * gather (the reference does the same for fc2 with fc2_weight_t,
+ * Dejavu/src/ops/fused_dense_sparse_dejavu.py:912-913).  Deterministic.
+ *   workspace: dv_out_proj_sparse_t_workspace_bytes(...) bytes, zero-filled
+ *   before first use (may be shared with dv_gather_transposed_gemv_f16).
+ */
+DV_API size_t dv_out_proj_sparse_t_workspace_bytes(int B, int N, int nnz, int hd);
+DV_API int dv_out_proj_sparse_t_f16(const void* x, const void* Wt, int64_t ldw, const void* bias,
+                                    const void* head_idx, int nnz, int B, int H, int hd, int N,
+                                    void* y, void* workspace, size_t workspace_bytes,
+                                    void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,206 @@
+"""GPU parity of the head-sparse attention operators against the CPU oracle
+(fp16 outputs within max-abs 2e-2 / relative L2 1e-3; cache copies bit-exact)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import dejavu_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS = 2e-2
+REL_L2 = 1e-3
+
+
+def assert_close(got, want, what=""):
+    got = np.asarray(got, dtype=np.float64)
+    want = np.asarray(want, dtype=np.float64)
+    max_abs = np.max(np.abs(got - want)) if got.size else 0.0
+    rel = np.linalg.norm(got - want) / max(np.linalg.norm(want), 1e-30)
+    assert max_abs <= MAX_ABS and rel <= REL_L2, f"{what}: max_abs={max_abs:.3e} rel_l2={rel:.3e}"
+
+
+def np16(t):
+    return t.detach().cpu().numpy()
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from dejavu_amd import ops as _ops
+
+    return _ops
+
+
+def randh(g, *shape, std=1.0):
+    return (torch.randn(*shape, generator=g) * std).half()
+
+
+# ------------------------------------------------------------------ QKV
+@pytest.mark.parametrize("H,hd,d,nb,nnz", [(12, 128, 12288, 16, 4), (12, 128, 1024, 1, 4), (6, 64, 768, 3, 2),
+                                           (8, 128, 1152, 5, 8), (8, 32, 512, 8, 3), (12, 128, 2048, 2, 12)])
+def test_qkv_proj_sparse(ops, H, hd, d, nb, nnz):
+    """First case is the shape of the reference's own self-check
+    (attention_proj_sparse.py:597-627): 12 heads, hidden 12288, 16 rows, 4 active heads,
+    a random permutation of the rows per head."""
+    g = torch.Generator().manual_seed(0)
+    x = randh(g, nb, d)
+    W = randh(g, 3, H, hd, d, std=0.02)
+    bias = randh(g, 3, H, hd)
+    head_idx = torch.randperm(H, generator=g)[:nnz].int()
+    batch_idx = torch.stack([torch.randperm(nb, generator=g) for _ in range(nnz)]).int()
+    print(f"case qkv H={H} hd={hd} d={d} nb={nb} nnz={nnz}", flush=True)
+    out = torch.full((nb, 3, H, hd), 7.0, dtype=torch.float16, device="cuda")
+    ops.qkv_proj_sparse(x.cuda(), W.cuda(), head_idx.cuda(), batch_idx.cuda(), bias.cuda(), out=out)
+    torch.cuda.synchronize()
+    ref = (torch.einsum("thdn,bn->bthd", W.float(), x.float()) + bias.float()).numpy()
+    hi = head_idx.long().numpy()
+    assert_close(np16(out)[:, :, hi], ref[:, :, hi], "qkv full rows")
+    others = [h for h in range(H) if h not in hi.tolist()]
+    assert np.all(np16(out)[:, :, others] == 7.0), "inactive heads must not be written"
+    # now with skipped rows: the oracle leaves them untouched
+    mask = torch.rand(nnz, nb, generator=g) < 0.4
+    bi2 = batch_idx.clone()
+    bi2[mask] = -1
+    out2 = torch.full((nb, 3, H, hd), 7.0, dtype=torch.float16, device="cuda")
+    ops.qkv_proj_sparse(x.cuda(), W.cuda(), head_idx.cuda(), bi2.cuda(), bias.cuda(), out=out2)
+    torch.cuda.synchronize()
+    want = O.qkv_proj_sparse(x.numpy(), W.numpy(), head_idx.numpy(), bi2.numpy(), bias.numpy(),
+                             out=np.full((nb, 3, H, hd), 7.0, dtype=np.float16))
+    assert_close(np16(out2), want, "qkv masked")
+    assert np.array_equal(np16(out2) == 7.0, want == 7.0), "written / untouched pattern differs"
+
+
+def test_qkv_proj_sparse_no_bias_and_empty(ops):
+    g = torch.Generator().manual_seed(1)
+    x = randh(g, 2, 256)
+    W = randh(g, 3, 4, 64, 256, std=0.05)
+    hi = torch.tensor([3, 0], dtype=torch.int32)
+    bi = torch.tensor([[0, 1], [1, -1]], dtype=torch.int32)
+    out = torch.zeros(2, 3, 4, 64, dtype=torch.float16, device="cuda")
+    ops.qkv_proj_sparse(x.cuda(), W.cuda(), hi.cuda(), bi.cuda(), None, out=out)
+    torch.cuda.synchronize()
+    assert_close(np16(out), O.qkv_proj_sparse(x.numpy(), W.numpy(), hi.numpy(), bi.numpy(), None), "no bias")
+    out3 = ops.qkv_proj_sparse(x.cuda(), W.cuda(), hi[:0].cuda(), bi[:0].cuda(), None)
+    assert out3.shape == (2, 3, 4, 64)
+    with pytest.raises(AssertionError):
+        ops.qkv_proj_sparse(x.cuda(), W.cuda(), hi.long().cuda(), bi.cuda(), None)  # int64 head_idx
+
+
+# ------------------------------------------------------------- out_proj
+@pytest.mark.parametrize("H,hd,d,B,nnz", [(12, 128, 12288, 2, 4), (12, 64, 768, 1, 4), (72, 128, 1152, 1, 24),
+                                          (8, 128, 520, 4, 3), (16, 128, 1024, 3, 16)])
+def test_out_proj_sparse_both_layouts(ops, H, hd, d, B, nnz):
+    g = torch.Generator().manual_seed(2)
+    if d % 128:
+        pytest.skip("reference asserts hidden_dim % 128 == 0") if False else None
+    x = randh(g, B, H, hd)
+    W = randh(g, d if d % 128 == 0 else 640, H, hd, std=0.02)
+    N = W.shape[0]
+    bias = randh(g, N)
+    head_idx = torch.randperm(H, generator=g)[:nnz].int()
+    print(f"case out_proj H={H} hd={hd} N={N} B={B} nnz={nnz}", flush=True)
+    want = O.out_proj_sparse(x.numpy(), W.numpy(), head_idx.numpy(), bias.numpy())
+    got = ops.out_proj_sparse(x.cuda(), W.cuda(), head_idx.cuda(), bias.cuda())
+    Wt = W.view(N, H * hd).t().contiguous().cuda()
+    got_t = ops.out_proj_sparse_t(x.cuda(), Wt, head_idx.cuda(), bias.cuda())
+    got_t2 = ops.out_proj_sparse_t(x.cuda(), Wt, head_idx.cuda(), bias.cuda())
+    torch.cuda.synchronize()
+    assert_close(np16(got), want, "out_proj (d,H,hd)")
+    assert_close(np16(got_t), want, "out_proj transposed")
+    assert torch.equal(got_t, got_t2)
+    dm = O.out_proj_head_masked(x.numpy(), W.numpy(), head_idx.numpy(), bias.numpy())
+    assert_close(np16(got_t), dm, "head-masked dense form")
+    # no heads selected: bias only
+    e = ops.out_proj_sparse_t(x.cuda(), Wt, head_idx[:0].cuda(), bias.cuda())
+    e2 = ops.out_proj_sparse(x.cuda(), W.cuda(), head_idx[:0].cuda(), bias.cuda())
+    torch.cuda.synchronize()
+    assert np.array_equal(np16(e), np.tile(bias.numpy(), (B, 1))) and np.array_equal(np16(e2), np16(e))
+
+
+# ----------------------------------------------------------- cache copy
+@pytest.mark.parametrize("hd", [64, 128])
+def test_cache_copy_sparse_bit_exact(ops, hd):
+    g = torch.Generator().manual_seed(3)
+    H, S, nb = 12, 48, 16
+    qkv = randh(g, nb, 3, H, hd)
+    head_idx = torch.randperm(H, generator=g)[:4].int()
+    seq_idx = torch.stack([torch.randperm(nb, generator=g) for _ in range(4)]).int()
+    seq_idx[torch.rand(4, nb, generator=g) < 0.5] = -1
+    padding = torch.tensor([16], dtype=torch.int32)
+    k_cache = torch.zeros(1, H, hd // 8, S, 8, dtype=torch.float16)
+    v_cache = torch.zeros(1, H, S, hd, dtype=torch.float16)
+    want_k = O.k_cache_copy_sparse(qkv[:, 1].numpy(), k_cache.numpy().copy(), head_idx.numpy(), seq_idx.numpy(), 16)
+    want_v = O.v_cache_copy_sparse(qkv[:, 2].numpy(), v_cache.numpy().copy(), head_idx.numpy(), seq_idx.numpy(), 16)
+    print(f"case cache copy hd={hd}", flush=True)
+    q = qkv.cuda()
+    kc, vc = k_cache.cuda(), v_cache.cuda()
+    ops.k_cache_copy_sparse(q[:, 1], kc, head_idx.cuda(), seq_idx.cuda(), padding.cuda())
+    ops.v_cache_copy_sparse(q[:, 2], vc, head_idx.cuda(), seq_idx.cuda(), padding.cuda())
+    kc2, vc2 = k_cache.cuda(), v_cache.cuda()
+    ops.kv_cache_copy_sparse(q[:, 1], q[:, 2], kc2, vc2, head_idx.cuda(), seq_idx.cuda(), padding.cuda())
+    torch.cuda.synchronize()
+    assert np.array_equal(np16(kc), want_k) and np.array_equal(np16(vc), want_v)
+    assert torch.equal(kc, kc2) and torch.equal(vc, vc2)
+    # without padding
+    kc3 = k_cache.cuda()
+    ops.k_cache_copy_sparse(q[:, 1], kc3, head_idx.cuda(), seq_idx.cuda())
+    torch.cuda.synchronize()
+    assert np.array_equal(np16(kc3), O.k_cache_copy_sparse(qkv[:, 1].numpy(), k_cache.numpy().copy(),
+                                                           head_idx.numpy(), seq_idx.numpy(), 0))
+
+
+# ------------------------------------------------------ decode attention
+@pytest.mark.parametrize("B,H,hd,S,t,nsel", [(1, 12, 128, 256, 200, 4), (2, 8, 64, 100, 99, 3), (1, 96, 128, 2048, 2047, 32),
+                                             (3, 4, 128, 70, 0, 4), (1, 6, 128, 130, 64, 2)])
+def test_single_query_attention(ops, B, H, hd, S, t, nsel):
+    g = torch.Generator().manual_seed(4)
+    q, k, v = (randh(g, B, H, hd) for _ in range(3))
+    kc = randh(g, B, H, S, hd)
+    vc = randh(g, B, H, S, hd)
+    from dejavu_amd.workloads import pack_k_cache
+
+    k_cache = pack_k_cache(kc)
+    print(f"case attention B={B} H={H} hd={hd} S={S} t={t} nsel={nsel}", flush=True)
+    head_idx = torch.randperm(H, generator=g)[:nsel].int()
+    # head-restricted
+    kcd, vcd = k_cache.cuda(), vc.cuda()
+    out = torch.full((B, H, hd), 3.0, dtype=torch.float16, device="cuda")
+    ops.single_query_attention(q.cuda(), k.cuda(), v.cuda(), kcd, vcd, None, t, head_idx=head_idx.cuda(), out=out)
+    torch.cuda.synchronize()
+    kn, vn = k_cache.numpy().copy(), vc.numpy().copy()
+    want = O.single_query_attention(q.numpy(), k.numpy(), v.numpy(), kn, vn, t, head_idx=head_idx.numpy())
+    hi = head_idx.long().numpy()
+    assert_close(np16(out)[:, hi], want[:, hi], "attention (selected heads)")
+    others = [h for h in range(H) if h not in hi.tolist()]
+    assert np.all(np16(out)[:, others] == 3.0)
+    assert np.array_equal(np16(kcd), kn) and np.array_equal(np16(vcd), vn), "cache append differs"
+    # all heads, as the dense path calls it
+    kcd, vcd = k_cache.cuda(), vc.cuda()
+    out_all = ops.single_query_attention(q.cuda(), k.cuda(), v.cuda(), kcd, vcd, None, t)
+    torch.cuda.synchronize()
+    kn, vn = k_cache.numpy().copy(), vc.numpy().copy()
+    want_all = O.single_query_attention(q.numpy(), k.numpy(), v.numpy(), kn, vn, t)
+    assert_close(np16(out_all), want_all, "attention (all heads)")
+    # cache already holds the newest token: no append
+    out_na = ops.single_query_attention(q.cuda(), None, None, kcd, vcd, None, t)
+    torch.cuda.synchronize()
+    assert torch.equal(out_na, out_all)
+
+
+def test_single_query_attention_lengths_per_sample(ops):
+    g = torch.Generator().manual_seed(5)
+    B, H, hd, S = 3, 4, 128, 160
+    q, k, v = (randh(g, B, H, hd) for _ in range(3))
+    kc = randh(g, B, H, S, hd)
+    vc = randh(g, B, H, S, hd)
+    from dejavu_amd.workloads import pack_k_cache
+
+    k_cache = pack_k_cache(kc)
+    lengths = torch.tensor([5, 159, 64], dtype=torch.int32)
+    kcd, vcd = k_cache.cuda(), vc.cuda()
+    out = ops.single_query_attention(q.cuda(), k.cuda(), v.cuda(), kcd, vcd, lengths.cuda(), 159)
+    torch.cuda.synchronize()
+    kn, vn = k_cache.numpy().copy(), vc.numpy().copy()
+    want = O.single_query_attention(q.numpy(), k.numpy(), v.numpy(), kn, vn, 159, lengths_per_sample=lengths.numpy())
+    assert_close(np16(out), want, "attention with lengths")
+    assert np.array_equal(np16(kcd), kn) and np.array_equal(np16(vcd), vn)

@@ -166,3 +166,17 @@ def test_reference_style_assertions(ops):
         ops.gather_gemv(x, W, idx)  # batch 5 not in 1..4
     with pytest.raises(AssertionError):
         ops.gather_gemv(x[:1].float(), W, idx)  # dtype mismatch
+
+
+def test_workspace_shared_across_shapes(ops):
+    """Consecutive fc2 calls with different split layouts share one scratch
+    buffer; stale partial sums of one shape must not disturb the next."""
+    g = torch.Generator().manual_seed(5)
+    W = (torch.randn(4096, 1024, generator=g) * 0.05).half().cuda()
+    for M, B in [(4096, 4), (96, 1), (4096, 1), (1024, 3), (4096, 2), (16, 1)]:
+        print(f"case workspace M={M} B={B}", flush=True)
+        idx = torch.randperm(4096, generator=g)[:M]
+        h = torch.randn(B, M, generator=g).half()
+        got = ops.gather_transposed_gemv(h.cuda(), W, idx.cuda(), None)
+        torch.cuda.synchronize()
+        assert_close(np16(got), O.gather_transposed_gemv(h.numpy(), W.cpu().numpy(), idx.numpy(), None), f"M={M} B={B}")
