@@ -135,6 +135,40 @@ __global__ void kv_cache_copy_kernel(const half_t* __restrict__ K, const half_t*
   if (v_cache) v_cache[((int64_t)h * S + dst) * hd + j] = V[src];
 }
 
+// One decode step of the skipped-head back-fill window.
+//   x_cache[counter, :] = x
+//   flush == 0: for i < nnz, h = head_idx[i], s <= counter:
+//                 batch_idx[i, s] = tracker[h, s];  tracker[h, s] = -1
+//   flush != 0: for every head h and s < 16: batch_idx[h, s] = s, tracker[h, s] = s
+// tracker is (H, 16) int32: tracker[h, s] == s while token s of the window has no
+// K/V for head h, -1 once it has.  Heads in head_idx are distinct.
+__global__ void window_step_kernel(const half_t* __restrict__ x, half_t* __restrict__ x_cache, int d,
+                                   int* __restrict__ tracker, const int* __restrict__ head_idx,
+                                   int nnz, int H, int counter, int flush,
+                                   int* __restrict__ batch_idx) {
+  const int tid = blockIdx.x * blockDim.x + threadIdx.x;
+  const int nthreads = gridDim.x * blockDim.x;
+  for (int j = tid; j < d; j += nthreads) x_cache[(int64_t)counter * d + j] = x[j];
+  if (flush) {
+    for (int o = tid; o < H * 16; o += nthreads) {
+      tracker[o] = o & 15;
+      batch_idx[o] = o & 15;
+    }
+  } else {
+    const int nb = counter + 1;
+    for (int o = tid; o < nnz * nb; o += nthreads) {
+      const int i = o / nb, s = o - i * nb;
+      const int h = head_idx[i];
+      if (h < 0 || h >= H) {
+        batch_idx[o] = -1;
+      } else {
+        batch_idx[o] = tracker[h * 16 + s];
+        tracker[h * 16 + s] = -1;
+      }
+    }
+  }
+}
+
 // Appends the newest token: for every batch row b and head (all, or head_idx):
 //   k_cache[b, h, :, pos_b, :] = K[b, h, :],  v_cache[b, h, pos_b, :] = V[b, h, :]
 // with pos_b = lengths[b] if lengths else pos.  K / V: (B, H, hd) with batch

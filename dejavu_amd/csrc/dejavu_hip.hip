@@ -370,6 +370,22 @@ int dv_kv_cache_copy_sparse_f16(const void* k, const void* v, int64_t ld_src, in
   return launch_status();
 }
 
+int dv_window_step_f16(const void* x, void* x_cache, int d, void* tracker, const void* head_idx,
+                       int nnz, int H, int counter, int flush, void* batch_idx, void* stream) {
+  if (!x || !x_cache || !tracker || !batch_idx || d <= 0 || H <= 0 || nnz < 0 || counter < 0 ||
+      counter > 15 || (!flush && nnz > 0 && !head_idx))
+    return DV_ERR_INVALID_ARG;
+  const int work = d > H * 16 ? d : H * 16;
+  int blocks = (work + 255) / 256;
+  if (blocks > 64) blocks = 64;
+  hipLaunchKernelGGL(window_step_kernel, dim3(blocks), dim3(256), 0,
+                     reinterpret_cast<hipStream_t>(stream), reinterpret_cast<const half_t*>(x),
+                     reinterpret_cast<half_t*>(x_cache), d, reinterpret_cast<int*>(tracker),
+                     reinterpret_cast<const int*>(head_idx), nnz, H, counter, flush,
+                     reinterpret_cast<int*>(batch_idx));
+  return launch_status();
+}
+
 int dv_kv_append_f16(const void* k, const void* v, int64_t ld_src, void* k_cache, void* v_cache,
                      const void* head_idx, int nheads, const void* lengths, int pos, int B, int H,
                      int hd, int S, void* stream) {

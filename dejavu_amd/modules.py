@@ -1,0 +1,361 @@
+"""Drop-in sparse MLP / sparse attention modules.
+
+Same constructor arguments, submodule names (``fc1``, ``fc2``, ``Wqkv``,
+``out_proj``, ``sp.fc0``, ``sp.fc1``) and ``forward`` signatures as the
+reference's modules, with the decode step running on the HIP kernels:
+
+  ParallelSP                Dejavu/src/ops/fused_dense_sparse_dejavu.py:33-76
+  ParallelFusedMLPDejavu    Dejavu/src/ops/fused_dense_sparse_dejavu.py:821-951
+  ParallelMHADejavu         Dejavu/src/models/modules/mha_dejavu.py:910-1075
+  ParallelMHASparseAttMlp   Dejavu/src/models/modules/mha_dejavu.py:1152-1511
+
+Single GPU: a process group of size 1 (or None) is accepted and the tensor
+parallel all-reduces of the reference are the identity.  The prompt phase
+(sequence length > 1) and layers that receive no prediction run dense through
+the library GEMM / attention of PyTorch, as the reference's do through cuBLAS.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Optional
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import ops
+from ._lib import check, lib
+
+
+def _world_size(process_group) -> int:
+    if process_group is None:
+        return 1
+    size = process_group.size() if callable(getattr(process_group, "size", None)) else int(process_group)
+    if size != 1:
+        raise NotImplementedError("this build runs the sparse decode path on one GPU (tensor parallel size 1)")
+    return size
+
+
+@dataclass
+class InferenceParams:
+    """Decode-time state shared by the layers (same fields as the
+    ``inference_params`` object the reference's modules read)."""
+
+    max_sequence_len: int
+    max_batch_size: int
+    sequence_len_offset: int = 0
+    batch_size_offset: int = 0
+    key_value_memory_dict: dict = field(default_factory=dict)
+    fused_ft_kernel: bool = True
+    lengths_per_sample: Optional[torch.Tensor] = None
+
+
+class ParallelSP(nn.Module):
+    """Low-rank sparsity predictor ``fc1(fc0(x))``, both linears bias-free."""
+
+    def __init__(self, layer_idx=None, embed_dim=None, low_rank_dim=None, out_dim=None, K=None,
+                 process_group=None, sequence_parallel=False, device=None, dtype=None) -> None:
+        super().__init__()
+        size = _world_size(process_group)
+        self.process_group = process_group
+        self.layer_idx = layer_idx
+        self.embed_dim = embed_dim
+        self.fc0 = nn.Linear(embed_dim, low_rank_dim, bias=False, device=device, dtype=dtype)
+        self.out = out_dim // size
+        self.fc1 = nn.Linear(low_rank_dim, out_dim, bias=False, device=device, dtype=dtype)
+        self.K = K // size
+
+    def forward(self, x):
+        """x: anything viewable as (embed_dim,) -> (out_dim,) logits, as the
+        reference; a (B, 1, embed_dim) batch gives (B, out_dim)."""
+        single = x.numel() == self.embed_dim
+        logits = ops.predictor_logits(x.reshape(-1, self.embed_dim), self.fc0.weight, self.fc1.weight)
+        return logits.view(-1) if single else logits
+
+    def topk(self, logits, k=None, dtype=torch.int64):
+        return ops.topk_indices(logits, self.K if k is None else k, dtype=dtype)
+
+
+class ParallelFusedMLPDejavu(nn.Module):
+    def __init__(self, in_features, hidden_features, sp_kwargs, out_features=None, activation="gelu_approx",
+                 layer_idx=None, process_group=None, bias1=True, bias2=True, sequence_parallel=True,
+                 checkpoint_lvl=0, heuristic="auto", device=None, dtype=None):
+        assert checkpoint_lvl in [0, 1, 2]
+        assert activation in ["gelu_approx", "relu"]
+        assert sp_kwargs != None, "sparse predictor parameters are not passed in."
+        super().__init__()
+        _world_size(process_group)
+        if out_features is None:
+            out_features = in_features
+        self.activation = activation
+        self.process_group = process_group
+        self.sequence_parallel = sequence_parallel
+        self.checkpoint_lvl = checkpoint_lvl
+        self.heuristic = heuristic
+        self.fc1 = nn.Linear(in_features, hidden_features, bias=bias1, device=device, dtype=dtype)
+        self.fc2 = nn.Linear(hidden_features, out_features, bias=bias2, device=device, dtype=dtype)
+        self.layer_idx = layer_idx
+        # fc2.weight transposed to (hidden, out) so that active neurons are contiguous rows;
+        # built on first sparse use, as the reference does
+        self.fc2_weight_t = None
+        self.sp = ParallelSP(layer_idx=layer_idx, device=device, dtype=dtype, process_group=process_group,
+                             sequence_parallel=sequence_parallel, **sp_kwargs)
+        self.sp_stream = None
+        self.event_mlp = None
+        self.event_mlp_sp = None
+
+    def _streams(self):
+        if self.sp_stream is None:
+            self.sp_stream = torch.cuda.Stream()
+            self.event_mlp = torch.cuda.Event(enable_timing=False, blocking=False)
+            self.event_mlp_sp = torch.cuda.Event(enable_timing=False, blocking=False)
+
+    def forward(self, x, residual, idx=None):
+        """x, residual: (B, 1, d) at decode (or (B, s, d) for the prompt).
+        idx: (K,) active neurons or None for the dense MLP.
+        Returns (out, mlp_logit); mlp_logit, the predictor output for the next
+        layer's MLP, only when decoding one token."""
+        self._streams()
+        curr_stream = torch.cuda.current_stream()
+        do_token_generation = x.size(1) == 1
+        if idx != None:
+            assert x.size(1) == 1
+            if self.activation != "relu":
+                raise NotImplementedError("the sparse MLP kernels fuse ReLU (OPT); gelu_approx runs dense only")
+            if self.fc2_weight_t is None:
+                self.fc2_weight_t = self.fc2.weight.t().contiguous()
+            out = ops.mlp_sparse(x.squeeze(1), self.fc1.weight, self.fc2_weight_t, idx, self.fc1.bias, self.fc2.bias)
+            out = out.unsqueeze(1)
+        else:
+            h = F.linear(x, self.fc1.weight, self.fc1.bias)
+            h = F.relu(h) if self.activation == "relu" else F.gelu(h, approximate="tanh")
+            out = F.linear(h, self.fc2.weight, self.fc2.bias)
+        curr_stream.record_event(self.event_mlp)
+        # (tensor parallel all-reduce of `out` is the identity on one GPU)
+        mlp_logit = None
+        with torch.cuda.stream(self.sp_stream):
+            self.sp_stream.wait_event(self.event_mlp)
+            if do_token_generation:
+                mlp_logit = self.sp(residual)
+            self.sp_stream.record_event(self.event_mlp_sp)
+        curr_stream.wait_event(self.event_mlp_sp)
+        return out, mlp_logit
+
+
+def _update_kv_cache(kv, inference_params, layer_idx):
+    """Prompt-phase cache fill.  kv: (B, s, 2, H, hd).  Creates / fills the
+    packed key cache (B, H, hd/8, S, 8) and the value cache (B, H, S, hd)
+    (Dejavu/src/models/modules/mha_dejavu.py:385-447, fused_ft_kernel layout)."""
+    B, s, _, H, hd = kv.shape
+    assert kv.dtype == torch.float16
+    if layer_idx not in inference_params.key_value_memory_dict:
+        k_cache = torch.zeros(inference_params.max_batch_size, H, hd // 8, inference_params.max_sequence_len, 8,
+                              dtype=kv.dtype, device=kv.device)
+        v_cache = torch.zeros(inference_params.max_batch_size, H, inference_params.max_sequence_len, hd,
+                              dtype=kv.dtype, device=kv.device)
+        inference_params.key_value_memory_dict[layer_idx] = (k_cache, v_cache)
+    k_cache, v_cache = inference_params.key_value_memory_dict[layer_idx]
+    b0 = inference_params.batch_size_offset
+    s0 = inference_params.sequence_len_offset
+    assert b0 + B <= v_cache.shape[0] and s0 + s <= v_cache.shape[2]
+    k_cache[b0:b0 + B, :, :, s0:s0 + s, :] = kv[:, :, 0].reshape(B, s, H, hd // 8, 8).permute(0, 2, 3, 1, 4)
+    v_cache[b0:b0 + B, :, s0:s0 + s, :] = kv[:, :, 1].permute(0, 2, 1, 3)
+    return kv
+
+
+class _MHABase(nn.Module):
+    """Shared dense / prompt machinery of the two attention modules."""
+
+    def _init_common(self, embed_dim, num_heads, process_group, bias, softmax_scale, causal, layer_idx,
+                     rotary_emb_dim, device, dtype):
+        _world_size(process_group)
+        assert rotary_emb_dim == 0, "OPT uses learned positions; rotary embedding is not built"
+        self.embed_dim = embed_dim
+        self.causal = causal
+        self.layer_idx = layer_idx
+        self.rotary_emb_dim = rotary_emb_dim
+        self.num_heads = num_heads
+        assert self.embed_dim % num_heads == 0, "self.kdim must be divisible by num_heads"
+        self.head_dim = self.embed_dim // num_heads
+        self.softmax_scale = softmax_scale
+        self.num_head_per_node = self.num_heads
+        self.Wqkv = nn.Linear(embed_dim, 3 * embed_dim, bias=bias, device=device, dtype=dtype)
+        self.out_proj = nn.Linear(embed_dim, embed_dim, device=device, dtype=dtype)
+        self.process_group = process_group
+        self.mlp_k = None
+        self.sp_stream = None
+
+    def _streams(self):
+        if self.sp_stream is None:
+            self.sp_stream = torch.cuda.Stream()
+            self.event_qkv = torch.cuda.Event(enable_timing=False, blocking=False)
+            self.event_out = torch.cuda.Event(enable_timing=False, blocking=False)
+            self.event_mlp_sp = torch.cuda.Event(enable_timing=False, blocking=False)
+            self.event_att_sp = torch.cuda.Event(enable_timing=False, blocking=False)
+
+    def _dense_context(self, qkv, inference_params):
+        """qkv: (B, s, 3, H, hd) -> context (B, s, H*hd) for the prompt or a dense decode step."""
+        B, s = qkv.shape[0], qkv.shape[1]
+        scale = self.softmax_scale
+        if inference_params is None or inference_params.sequence_len_offset == 0:
+            if inference_params is not None:
+                assert self.layer_idx is not None, "Generation requires layer_idx in the constructor"
+                _update_kv_cache(qkv[:, :, 1:], inference_params, self.layer_idx)
+            q, k, v = (t.transpose(1, 2) for t in qkv.unbind(dim=2))  # (B, H, s, hd)
+            causal = self.causal if inference_params is None else True
+            ctx = F.scaled_dot_product_attention(q, k, v, is_causal=causal and s > 1, scale=scale)
+            return ctx.transpose(1, 2).reshape(B, s, -1)
+        assert s == 1, "decode processes one token at a time"
+        k_cache, v_cache = inference_params.key_value_memory_dict[self.layer_idx]
+        b0 = inference_params.batch_size_offset
+        q, k, v = qkv[:, 0].unbind(dim=1)  # (B, H, hd) views
+        ctx = ops.single_query_attention(q, k, v, k_cache[b0:b0 + B], v_cache[b0:b0 + B],
+                                         inference_params.lengths_per_sample, inference_params.sequence_len_offset,
+                                         self.rotary_emb_dim, softmax_scale=scale)
+        return ctx.reshape(B, 1, -1)
+
+    def _mlp_topk(self, mlp_sp_logit, after_event):
+        """MLP top-k for this layer on the side stream, overlapping attention."""
+        mlp_idx = None
+        with torch.cuda.stream(self.sp_stream):
+            self.sp_stream.wait_event(after_event)
+            if mlp_sp_logit != None:
+                mlp_idx = ops.topk_indices(mlp_sp_logit, self.mlp_k)
+            self.sp_stream.record_event(self.event_mlp_sp)
+        return mlp_idx
+
+
+class ParallelMHADejavu(_MHABase):
+    """Dense attention + the MLP top-k (MLP-sparse-only model)."""
+
+    def __init__(self, embed_dim, num_heads, process_group=None, sp_kwargs=None, bias=True, dropout=0.0,
+                 softmax_scale=None, causal=False, layer_idx=None, rotary_emb_dim=0, rotary_emb_scale_base=0,
+                 use_flash_attn=False, checkpointing=False, sequence_parallel=True, device=None, dtype=None) -> None:
+        super().__init__()
+        self._init_common(embed_dim, num_heads, process_group, bias, softmax_scale, causal, layer_idx,
+                          rotary_emb_dim, device, dtype)
+
+    def forward(self, x, mlp_sp_logit=None, seqlen=None, inference_params=None, **kwargs):
+        """x: (B, s, d).  Returns (out, mlp_idx)."""
+        assert seqlen is None, "sequence-parallel input layout is not used for generation"
+        self._streams()
+        curr_stream = torch.cuda.current_stream()
+        qkv = self.Wqkv(x)
+        curr_stream.record_event(self.event_qkv)
+        mlp_idx = self._mlp_topk(mlp_sp_logit, self.event_qkv)
+        qkv = qkv.view(x.shape[0], x.shape[1], 3, self.num_heads, self.head_dim)
+        context = self._dense_context(qkv, inference_params)
+        out = self.out_proj(context)
+        curr_stream.wait_event(self.event_mlp_sp)
+        return out, mlp_idx
+
+
+class ParallelMHASparseAttMlp(_MHABase):
+    """Head-sparse attention; also runs both top-ks (this layer's MLP neurons,
+    next layer's heads) beside the main stream."""
+
+    WINDOW = 16
+
+    def __init__(self, embed_dim, num_heads, process_group=None, sp_kwargs=None, bias=True, dropout=0.0,
+                 softmax_scale=None, causal=False, layer_idx=None, rotary_emb_dim=0, rotary_emb_scale_base=0,
+                 use_flash_attn=False, checkpointing=False, sequence_parallel=True, device=None, dtype=None) -> None:
+        super().__init__()
+        assert sp_kwargs != None, "sparse predictor parameters are not passed in."
+        self._init_common(embed_dim, num_heads, process_group, bias, softmax_scale, causal, layer_idx,
+                          rotary_emb_dim, device, dtype)
+        self.sp_kwargs = sp_kwargs
+        self.sp = ParallelSP(layer_idx=layer_idx, device=device, dtype=dtype, process_group=process_group,
+                             sequence_parallel=sequence_parallel, **sp_kwargs)
+        self.att_k = self.sp.K
+        # LayerNorm outputs of the current 16-token window, to recompute K/V of skipped heads
+        self.x_cache = torch.zeros((self.WINDOW, embed_dim), dtype=torch.float16, device=device)
+        # tracker[h, s] == s while window token s has no K/V for head h, else -1
+        self.tracker = torch.arange(self.WINDOW, dtype=torch.int32, device=device).repeat(num_heads, 1)
+        self.counter = 0
+        self.cache_offset = None  # device int32[1]: cache position of window token 0
+        self.out_proj_weight_t = None
+        self._all_heads = None
+
+    def reset_window(self):
+        self.counter = 0
+        self.tracker.copy_(torch.arange(self.WINDOW, dtype=torch.int32, device=self.tracker.device)
+                           .repeat(self.num_heads, 1))
+
+    def _sparse_decode(self, x, head_idx, inference_params):
+        """x: (1, 1, d).  QKV for the active heads and the window tokens they
+        miss, cache scatter, attention over the active heads, out_proj."""
+        dev = x.device
+        assert x.dtype == torch.float16 and x.is_contiguous()
+        H, hd = self.num_heads, self.head_dim
+        flush = self.counter == self.WINDOW - 1
+        if flush:  # every 16th token all heads catch up
+            if self._all_heads is None:
+                self._all_heads = torch.arange(H, dtype=torch.int32, device=dev)
+            head_idx = self._all_heads
+        nnz = head_idx.shape[0]
+        nb = self.counter + 1
+        batch_idx = torch.empty(nnz, nb, dtype=torch.int32, device=dev)
+        stream = torch.cuda.current_stream().cuda_stream
+        check(lib.dv_window_step_f16(x.data_ptr(), self.x_cache.data_ptr(), self.embed_dim, self.tracker.data_ptr(),
+                                     head_idx.data_ptr(), nnz, H, self.counter, int(flush), batch_idx.data_ptr(),
+                                     stream), "dv_window_step_f16")
+        qkv = ops.qkv_proj_sparse(self.x_cache[:nb], self.Wqkv.weight.view(3, H, hd, self.embed_dim), head_idx,
+                                  batch_idx, None if self.Wqkv.bias is None else self.Wqkv.bias.view(3, H, hd))
+        self.counter += 1
+        return qkv, head_idx, batch_idx
+
+    def forward(self, x, residual, head_idx=None, mlp_sp_logit=None, seqlen=None, inference_params=None, **kwargs):
+        """x, residual: (B, s, d).  head_idx: (Hk,) int32 heads to compute, or None
+        for dense attention.  mlp_sp_logit: predictor logits for this layer's MLP.
+        Returns (out, mlp_idx, att_idx)."""
+        assert seqlen is None, "sequence-parallel input layout is not used for generation"
+        self._streams()
+        do_token_generation = x.size(1) == 1
+        if x.size(1) != 1:  # prompt: remember where the decode window starts
+            self.cache_offset = torch.tensor([x.size(1)], dtype=torch.int32, device=x.device)
+            self.reset_window()
+        curr_stream = torch.cuda.current_stream()
+        sparse = inference_params is not None and inference_params.sequence_len_offset > 0 and head_idx != None
+        if sparse:
+            assert x.size(1) == 1
+            assert x.size(0) == 1, "head-sparse decode keeps one back-fill window: batch size 1"
+            qkv, head_idx, batch_idx = self._sparse_decode(x, head_idx, inference_params)
+        else:
+            qkv = self.Wqkv(x)
+        curr_stream.record_event(self.event_qkv)
+        mlp_idx = self._mlp_topk(mlp_sp_logit, self.event_qkv)
+
+        if sparse:
+            k_cache, v_cache = inference_params.key_value_memory_dict[self.layer_idx]
+            b0 = inference_params.batch_size_offset
+            kc, vc = k_cache[b0:b0 + 1], v_cache[b0:b0 + 1]
+            if self.cache_offset is None:
+                self.cache_offset = torch.tensor([inference_params.sequence_len_offset - (self.counter - 1)],
+                                                 dtype=torch.int32, device=x.device)
+            ops.kv_cache_copy_sparse(qkv[:, 1], qkv[:, 2], kc, vc, head_idx, batch_idx, self.cache_offset)
+            # the caches now hold the newest token for the active heads
+            ctx = ops.single_query_attention(qkv[-1:, 0], None, None, kc, vc, inference_params.lengths_per_sample,
+                                             inference_params.sequence_len_offset, self.rotary_emb_dim,
+                                             head_idx=head_idx, softmax_scale=self.softmax_scale)
+            if self.out_proj_weight_t is None:
+                self.out_proj_weight_t = self.out_proj.weight.t().contiguous()
+            out = ops.out_proj_sparse_t(ctx, self.out_proj_weight_t, head_idx, self.out_proj.bias).unsqueeze(1)
+            if self.counter == self.WINDOW:  # window complete: start the next one
+                self.counter = 0
+                self.cache_offset += self.WINDOW
+        else:
+            qkv = qkv.view(x.shape[0], x.shape[1], 3, self.num_heads, self.head_dim)
+            context = self._dense_context(qkv, inference_params)
+            out = self.out_proj(context)
+        curr_stream.record_event(self.event_out)
+
+        att_idx = None
+        with torch.cuda.stream(self.sp_stream):
+            self.sp_stream.wait_event(self.event_out)
+            if do_token_generation:
+                att_sp_logit = self.sp(residual)
+                att_idx = ops.topk_indices(att_sp_logit, self.att_k, dtype=torch.int32)
+            self.sp_stream.record_event(self.event_att_sp)
+        curr_stream.wait_event(self.event_mlp_sp)
+        curr_stream.wait_event(self.event_att_sp)
+        return out, mlp_idx, att_idx

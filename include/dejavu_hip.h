@@ -125,6 +125,22 @@ DV_API int dv_kv_cache_copy_sparse_f16(const void* k, const void* v, int64_t ld_
                                        const void* padding, int H, int hd, int S, void* stream);
 
 /*
+ * One decode step of the skipped-head back-fill window: stores the step's
+ * LayerNorm output in the 16-row window buffer, returns for every active head
+ * which window tokens still lack K/V (-1 = already there) and marks them done;
+ * with flush != 0 (every 16th step) every head recomputes every window token
+ * and the tracker is re-armed.  Replaces ParallelTracker.get_batch_idx / update /
+ * reset and the x_cache write, Dejavu/src/models/modules/mha_dejavu.py:1124-1149,
+ * 1318-1329, 1355-1359.
+ *   x (d,) fp16; x_cache (16, d) fp16; tracker (H, 16) int32; head_idx (nnz,)
+ *   int32 (ignored when flushing); batch_idx out: (nnz, counter+1) int32, or
+ *   (H, 16) when flushing; 0 <= counter <= 15.
+ */
+DV_API int dv_window_step_f16(const void* x, void* x_cache, int d, void* tracker,
+                              const void* head_idx, int nnz, int H, int counter, int flush,
+                              void* batch_idx, void* stream);
+
+/*
  * Writes the newest token's k, v at position pos (or lengths[b]) of the caches,
  * for all heads (head_idx NULL) or the listed ones.  This is the cache update
  * that ft_attention.single_query_attention performs internally (call sites

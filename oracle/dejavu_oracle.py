@@ -489,3 +489,35 @@ def layer_norm(x, weight, bias, eps=1e-5):
     var = ((xf - mu) ** 2).mean(axis=-1, keepdims=True)
     y = (xf - mu) / np.sqrt(var + F32(eps))
     return (y * np.asarray(weight, F16).astype(F32) + np.asarray(bias, F16).astype(F32)).astype(F16)
+
+
+def sparse_attention_step_dense_kv(x_hist, Wqkv, bqkv, Wout, bout, head_idx, softmax_scale=None):
+    """Head-masked attention output for the newest token with K/V of EVERY past
+    token computed densely -- what the back-fill window must reproduce.
+
+    Closed form of ParallelMHASparseAttMlp.forward's decode branch
+    (Dejavu/src/models/modules/mha_dejavu.py:1283-1511) once all K/V of the
+    active heads are in the cache: q from the newest row of x_hist, K/V from
+    all rows, attention per active head (mha_dejavu.py:333-375), heads outside
+    head_idx zeroed before out_proj
+    (Decentralized_FM_alpha/modules/hf_opt_sparse_mlp_attention.py:365-373).
+    x_hist: (T, d) fp16 LayerNorm outputs; Wqkv: (3, H, hd, d); bqkv (3, H, hd);
+    Wout: (d, H, hd); bout (d,).  qkv and the context are rounded to fp16 as the
+    kernels store them.  Returns (out (d,) fp16, ctx (H, hd) fp16).
+    """
+    x_hist = np.asarray(x_hist, F16).astype(F32)
+    three, H, hd, d = Wqkv.shape
+    scale = F32(hd ** -0.5 if softmax_scale is None else softmax_scale)
+    ctx = np.zeros((H, hd), dtype=F16)
+    for h in [int(v) for v in np.asarray(head_idx)]:
+        w = np.asarray(Wqkv, F16)[:, h].astype(F32)  # (3, hd, d)
+        b = np.asarray(bqkv, F16)[:, h].astype(F32) if bqkv is not None else np.zeros((3, hd), F32)
+        q = (w[0] @ x_hist[-1] + b[0]).astype(F16).astype(F32)
+        K = (x_hist @ w[1].T + b[1]).astype(F16).astype(F32)
+        V = (x_hist @ w[2].T + b[2]).astype(F16).astype(F32)
+        s = (K @ q) * scale
+        p = np.exp(s - s.max())
+        p = p / p.sum(dtype=F32)
+        ctx[h] = (p @ V).astype(F16)
+    out = out_proj_sparse(ctx[None], Wout, head_idx, bout)[0]
+    return out, ctx
