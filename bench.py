@@ -1,0 +1,287 @@
+#!/usr/bin/env python3
+"""Benchmark of the sparse decode layer on one MI355X.
+
+A step = one pass of one sparse transformer block (head-sparse attention +
+sparse MLP + both predictors + top-ks + the two add/LayerNorms) over one decode
+token.  Default workload: the OPT-175B-shaped layer (d=12288, ffn=49152, 96
+heads x 128, K=4096 neurons, 32 heads, KV length 2048, batch 1), synthetic
+seeded weights.  Three distinct layers (weights, caches) are cycled so that no
+cache level can hold the working set; each layer's step is replayed from a HIP
+graph, and the next layer's head / neuron predictions are produced by the
+previous layer as in the model.
+
+Prints ONE JSON line (see README / DESIGN.md for the fields).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+N_LAYERS = 3
+
+
+def algorithmic_bytes(cfg, batch):
+    """Weight / KV bytes one layer step must read (fp16, counted once)."""
+    d, ffn, H, hd, r, K, Hk, S = (cfg[k] for k in ("d", "ffn", "H", "hd", "r", "K", "Hk", "S"))
+    return {
+        "qkv_sparse": 3 * Hk * hd * d * 2,
+        "decode_attn": 2 * Hk * S * hd * 2 * batch,
+        "out_proj_sparse": d * Hk * hd * 2,
+        "fc1_gather": K * d * 2,
+        "fc2_gather": K * d * 2,
+        "mlp_predictor": (d * r + r * ffn) * 2,
+        "head_predictor": (d * r + r * H) * 2,
+    }
+
+
+def build_layers(cfg, batch, device):
+    import torch
+
+    from dejavu_amd.block import create_sparse_block, init_block_synthetic
+    from dejavu_amd.modules import InferenceParams
+
+    d, ffn, H, hd, r, K, Hk, S = (cfg[k] for k in ("d", "ffn", "H", "hd", "r", "K", "Hk", "S"))
+    gen = torch.Generator(device=device)
+    gen.manual_seed(1234)
+
+    def randn(shape, std=1.0):
+        t = torch.empty(shape, dtype=torch.float32, device=device)
+        t.normal_(0.0, std, generator=gen)
+        return t.half()
+
+    layers = []
+    for l in range(N_LAYERS):
+        block = create_sparse_block(d, ffn, H, r, K, r, Hk, layer_idx=l, device=device)
+        init_block_synthetic(block, seed=l)
+        block.eval()
+        ip = InferenceParams(max_sequence_len=S, max_batch_size=batch, sequence_len_offset=S - 1)
+        ip.key_value_memory_dict[l] = (randn((batch, H, hd // 8, S, 8)), randn((batch, H, S, hd)))
+        # transposed copies the sparse path streams from (built lazily by the modules otherwise)
+        block.mlp.fc2_weight_t = block.mlp.fc2.weight.t().contiguous()
+        block.mixer.out_proj_weight_t = block.mixer.out_proj.weight.t().contiguous()
+        block.mixer.cache_offset = torch.tensor([S - 1], dtype=torch.int32, device=device)
+        layers.append(dict(block=block, ip=ip, hidden=randn((batch, 1, d)), residual=randn((batch, 1, d))))
+    # predictions travel from layer l to layer l+1 through fixed buffers
+    fresh = torch.arange(16, dtype=torch.int32, device=device).repeat(H, 1)
+    for l, L in enumerate(layers):
+        L["att_idx_in"] = torch.sort(torch.randperm(H, generator=gen, device=device)[:Hk]).values.int()
+        L["mlp_logit_in"] = randn((ffn,), 4.0)
+        L["fresh_tracker"] = fresh
+    for l, L in enumerate(layers):
+        nxt = layers[(l + 1) % N_LAYERS]
+        L["block"].mixer.att_idx_out = nxt["att_idx_in"]
+        L["block"].mlp.sp.logits_out = nxt["mlp_logit_in"]
+    return layers
+
+
+def layer_step(L):
+    """One decode step of one block in the state 'first token of a back-fill
+    window': every active head computes Q, K, V of the newest token."""
+    mixer = L["block"].mixer
+    mixer.counter = 0
+    mixer.tracker.copy_(L["fresh_tracker"])
+    return L["block"](L["hidden"], L["residual"], mixer_kwargs={"inference_params": L["ip"]},
+                      head_idx=L["att_idx_in"], mlp_sp_logit=L["mlp_logit_in"])
+
+
+def time_kernel(torch, fn, layers, iters=60):
+    """Average duration (us) of back-to-back launches bracketed by two HIP events
+    on the launch stream."""
+    for L in layers:
+        fn(L)
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for i in range(iters):
+        fn(layers[i % len(layers)])
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) * 1e3 / iters
+
+
+def kernel_table(torch, cfg, batch, layers):
+    """Per-kernel durations and achieved bandwidth, each launched alone."""
+    from dejavu_amd import ops
+
+    d, ffn, H, hd, K, Hk, S = (cfg[k] for k in ("d", "ffn", "H", "hd", "K", "Hk", "S"))
+    nbytes = algorithmic_bytes(cfg, batch)
+    dev = layers[0]["hidden"].device
+    x = layers[0]["hidden"].view(batch, d)
+    head_idx = layers[0]["att_idx_in"]
+    batch_idx = torch.zeros(Hk, 1, dtype=torch.int32, device=dev)
+    idx = ops.topk_indices(layers[0]["mlp_logit_in"], K)
+    h = ops.gather_gemv(x, layers[0]["block"].mlp.fc1.weight, idx, layers[0]["block"].mlp.fc1.bias, "relu")
+    qkv = torch.zeros(1, 3, H, hd, dtype=torch.float16, device=dev)
+    ctx = torch.zeros(batch, H, hd, dtype=torch.float16, device=dev)
+
+    def m(L):
+        return L["block"].mixer
+
+    def f(L):
+        return L["block"].mlp
+
+    fns = {
+        "qkv_sparse": lambda L: ops.qkv_proj_sparse(x[:1], m(L).Wqkv.weight.view(3, H, hd, d), head_idx, batch_idx,
+                                                    m(L).Wqkv.bias.view(3, H, hd), out=qkv),
+        "decode_attn": lambda L: ops.single_query_attention(qkv[:, 0], None, None, *L["ip"].key_value_memory_dict[
+            L["block"].mixer.layer_idx], None, S - 1, head_idx=head_idx, out=ctx),
+        "out_proj_sparse": lambda L: ops.out_proj_sparse_t(ctx, m(L).out_proj_weight_t, head_idx, m(L).out_proj.bias),
+        "fc1_gather": lambda L: ops.gather_gemv(x, f(L).fc1.weight, idx, f(L).fc1.bias, "relu"),
+        "fc2_gather": lambda L: ops.gather_transposed_gemv(h, f(L).fc2_weight_t, idx, f(L).fc2.bias),
+        "mlp_predictor": lambda L: ops.predictor_logits(x, f(L).sp.fc0.weight, f(L).sp.fc1.weight),
+        "head_predictor": lambda L: ops.predictor_logits(x, m(L).sp.fc0.weight, m(L).sp.fc1.weight),
+    }
+    table = {}
+    for name, fn in fns.items():
+        us = time_kernel(torch, fn, layers)
+        table[name] = {"us": round(us, 2), "MB": round(nbytes[name] / 1e6, 2),
+                       "GB/s": round(nbytes[name] / us / 1e3, 1),
+                       "frac": round(nbytes[name] / us / 1e3 / HBM_PEAK_GBPS, 4)}
+    return table
+
+
+def cpu_baseline(torch, cfg, batch, L, timed=15, warm=3):
+    """PyTorch CPU index_select + matmul form of the same layer step on the host cores."""
+    from oracle import cpu_baseline as C
+    from dejavu_amd.workloads import pack_k_cache  # noqa: F401
+
+    H, hd, S, d = cfg["H"], cfg["hd"], cfg["S"], cfg["d"]
+    m, f = L["block"].mixer, L["block"].mlp
+    k_cache, v_cache = L["ip"].key_value_memory_dict[m.layer_idx]
+    B = k_cache.shape[0]
+    t = {
+        "x": L["hidden"].view(batch, d).cpu(), "x2": L["hidden"].view(batch, d).cpu(),
+        "residual": L["residual"].view(batch, d).cpu(),
+        "Wqkv": m.Wqkv.weight.view(3, H, hd, d).cpu(), "bqkv": m.Wqkv.bias.view(3, H, hd).cpu(),
+        "Wout_t": m.out_proj_weight_t.cpu(), "bout": m.out_proj.bias.cpu(),
+        "k_cache_bhsd": k_cache.permute(0, 1, 3, 2, 4).reshape(B, H, S, hd).cpu(), "v_cache": v_cache.cpu(),
+        "W1": f.fc1.weight.cpu(), "b1": f.fc1.bias.cpu(), "W2t": f.fc2_weight_t.cpu(), "b2": f.fc2.bias.cpu(),
+        "mlp_Wa": f.sp.fc0.weight.cpu(), "mlp_Wb": f.sp.fc1.weight.cpu(),
+        "att_Wa": m.sp.fc0.weight.cpu(), "att_Wb": m.sp.fc1.weight.cpu(),
+        "K": cfg["K"], "Hk": cfg["Hk"], "S": S,
+    }
+    cores = torch.get_num_threads()
+    ts = []
+    with torch.no_grad():
+        for i in range(warm + timed):
+            t0 = time.perf_counter()
+            C.layer_step(t)
+            dt = time.perf_counter() - t0
+            if i >= warm:
+                ts.append(dt)
+    ts.sort()
+    med = ts[len(ts) // 2]
+    return {"value": round(med * 1e6, 1), "unit": "us/layer", "cores": cores, "kind": "port",
+            "sample": f"{timed} steps of the same layer (median; {warm} warm-up), torch {torch.__version__} "
+                      f"CPU index_select+matmul, fp32 compute from the same fp16 tensors"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=600)
+    ap.add_argument("--warmup", type=int, default=60)
+    ap.add_argument("--config", default="opt-175b")
+    ap.add_argument("--batch", type=int, default=1)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying HIP graphs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs the sparse decode layer on ONE GPU (no sharding); "
+              "use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from dejavu_amd.workloads import CONFIGS
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    torch.cuda.set_device(0)
+    cfg = CONFIGS[args.config]
+    batch = args.batch
+    assert batch == 1, "the head-sparse decode layer keeps one back-fill window (batch 1)"
+    device = torch.device("cuda:0")
+    layers = build_layers(cfg, batch, device)
+
+    with torch.no_grad():
+        # eager warm-up: allocates workspaces, sets kernel attributes
+        for _ in range(2):
+            for L in layers:
+                layer_step(L)
+        torch.cuda.synchronize()
+        graphs = []
+        if not args.no_graph:
+            for L in layers:
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    L["out"] = layer_step(L)
+                graphs.append(g)
+            torch.cuda.synchronize()
+
+        def run(i):
+            if graphs:
+                graphs[i % N_LAYERS].replay()
+            else:
+                layer_step(layers[i % N_LAYERS])
+
+        for i in range(args.warmup):
+            run(i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            run(i)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+
+        us_per_layer = elapsed / args.steps * 1e6
+        nbytes = algorithmic_bytes(cfg, batch)
+        layer_bytes = sum(nbytes.values())
+        table = kernel_table(torch, cfg, batch, layers)
+        dom = "qkv_sparse"  # largest share of the layer's bytes
+        roofline = {"bound": "hbm", "kernel": "qkv_sparse_kernel", "achieved": table[dom]["GB/s"],
+                    "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": table[dom]["frac"], "traffic": None,
+                    "bytes_per_launch": nbytes[dom], "us_per_launch": table[dom]["us"]}
+        cpu = None
+        if not args.no_cpu_baseline:
+            cpu = cpu_baseline(torch, cfg, batch, layers[0])
+
+    out = {
+        "metric": "us_per_layer, sparse MLP+attn decode, OPT-175B layer K=4096" if args.config == "opt-175b"
+        else f"us_per_layer, sparse MLP+attn decode, {args.config}",
+        "value": round(us_per_layer, 2),
+        "unit": "us/layer",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(us_per_layer / 1e3, 5),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": f"{args.config} sparse decode layer", "d": cfg["d"], "ffn": cfg["ffn"],
+                   "heads": cfg["H"], "head_dim": cfg["hd"], "K": cfg["K"], "active_heads": cfg["Hk"],
+                   "predictor_rank": cfg["r"], "kv_len": cfg["S"], "batch": batch,
+                   "layers_cycled": N_LAYERS, "hip_graph": not args.no_graph},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "layer": {"algorithmic_MB": round(layer_bytes / 1e6, 1), "GB/s": round(layer_bytes / us_per_layer / 1e3, 1),
+                  "frac_of_hbm_peak": round(layer_bytes / us_per_layer / 1e3 / HBM_PEAK_GBPS, 4),
+                  "tokens_per_s_per_layer": round(batch / (us_per_layer * 1e-6), 1)},
+        "kernels": table,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -49,6 +49,8 @@ SIGNATURES = {
         _c_int,
         [_c_ptr, _c_ptr, _c_i64, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_int,
          _c_int, _c_ptr]),
+    "dv_add_layer_norm_f16": (
+        _c_int, [_c_ptr, _c_ptr, _c_ptr, _c_ptr, ctypes.c_float, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr]),
     "dv_window_step_f16": (
         _c_int, [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr]),
     "dv_kv_append_f16": (

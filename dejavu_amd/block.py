@@ -1,0 +1,148 @@
+"""Pre-norm transformer block around the sparse attention and sparse MLP modules.
+
+Mirrors BlockMlpAttSparse / BlockDejavu of the reference
+(Dejavu/src/models/modules/block_dejavu.py:464-663 and 259-461): the block
+computes ``add -> LN -> mixer -> add -> LN -> mlp`` and returns both the MLP
+output and the residual stream, plus the predictions the next layer consumes
+(``next_mlp_sp_logit``, ``next_att_idx``).  Dropout / stochastic depth are
+inference no-ops and are not built.  The add + LayerNorm pairs run as one HIP
+kernel.
+"""
+from __future__ import annotations
+
+from functools import partial
+from typing import Optional
+
+import torch
+import torch.nn as nn
+from torch import Tensor
+
+from . import ops
+from .modules import ParallelFusedMLPDejavu, ParallelMHADejavu, ParallelMHASparseAttMlp
+
+
+def _add_norm(norm: nn.LayerNorm, hidden_states: Tensor, residual: Optional[Tensor]):
+    if hidden_states.is_cuda and hidden_states.dtype == torch.float16:
+        return ops.add_layer_norm(hidden_states, residual, norm.weight, norm.bias, norm.eps)
+    residual = hidden_states + residual if residual is not None else hidden_states
+    return norm(residual.to(dtype=norm.weight.dtype)), residual
+
+
+class BlockMlpAttSparse(nn.Module):
+    """Block whose mixer predicts heads for the next layer and whose MLP predicts
+    neurons for the next layer."""
+
+    def __init__(self, dim, mixer_cls=None, mlp_cls=None, norm_cls=nn.LayerNorm, dropout_cls=nn.Dropout,
+                 prenorm=True, resid_dropout1=0.0, resid_dropout2=0.0, drop_path1=0.0, drop_path2=0.0,
+                 fused_dropout_add_ln=False, return_residual=False, residual_in_fp32=False,
+                 sequence_parallel=False, mark_shared_params=False):
+        super().__init__()
+        assert prenorm == True, "Dejavu only support prenorm for now"
+        assert not residual_in_fp32, "the fused add + LayerNorm keeps the residual stream in fp16"
+        assert resid_dropout1 == 0.0 and resid_dropout2 == 0.0 and drop_path1 == 0.0 and drop_path2 == 0.0, \
+            "inference-only block: dropout / stochastic depth are not built"
+        assert mixer_cls is not None and mlp_cls is not None
+        self.prenorm = prenorm
+        self.mixer = mixer_cls(dim)
+        self.norm1 = norm_cls(dim)
+        self.mlp = mlp_cls(dim)
+        self.norm2 = norm_cls(dim)
+        # sp related
+        if hasattr(self.mlp, "sp"):
+            self.mixer.mlp_k = self.mlp.sp.K
+        if hasattr(self.mixer, "sp"):
+            self.mixer.att_k = self.mixer.sp.K
+
+    def forward(self, hidden_states: Tensor, residual: Optional[Tensor] = None, mixer_subset=None,
+                mixer_kwargs=None, head_idx=None, mlp_sp_logit=None):
+        """hidden_states: output of the previous block's MLP; residual: its
+        residual stream (None for the first block).  Returns
+        (hidden_states, residual, next_mlp_sp_logit, next_att_idx)."""
+        assert mixer_subset is None
+        hidden_states, residual = _add_norm(self.norm1, hidden_states, residual)
+        if mixer_kwargs is None:
+            mixer_kwargs = {}
+        hidden_states, mlp_idx, next_att_idx = self.mixer(hidden_states, residual=residual, head_idx=head_idx,
+                                                          mlp_sp_logit=mlp_sp_logit, **mixer_kwargs)
+        hidden_states, residual = _add_norm(self.norm2, hidden_states, residual)
+        hidden_states, next_mlp_sp_logit = self.mlp(hidden_states, residual, mlp_idx)
+        return hidden_states, residual, next_mlp_sp_logit, next_att_idx
+
+
+class BlockDejavu(nn.Module):
+    """Block with dense attention and a sparse MLP (block_dejavu.py:259-461)."""
+
+    def __init__(self, dim, mixer_cls=None, mlp_cls=None, norm_cls=nn.LayerNorm, prenorm=True, **unused):
+        super().__init__()
+        assert prenorm == True, "Dejavu only support prenorm for now"
+        assert mixer_cls is not None and mlp_cls is not None
+        self.mixer = mixer_cls(dim)
+        self.norm1 = norm_cls(dim)
+        self.mlp = mlp_cls(dim)
+        self.norm2 = norm_cls(dim)
+        if hasattr(self.mlp, "sp"):
+            self.mixer.mlp_k = self.mlp.sp.K
+
+    def forward(self, hidden_states: Tensor, residual: Optional[Tensor] = None, mixer_subset=None,
+                mixer_kwargs=None, mlp_sp_logit=None):
+        assert mixer_subset is None
+        hidden_states, residual = _add_norm(self.norm1, hidden_states, residual)
+        if mixer_kwargs is None:
+            mixer_kwargs = {}
+        hidden_states, mlp_idx = self.mixer(hidden_states, mlp_sp_logit=mlp_sp_logit, **mixer_kwargs)
+        hidden_states, residual = _add_norm(self.norm2, hidden_states, residual)
+        hidden_states, next_mlp_sp_logit = self.mlp(hidden_states, residual, mlp_idx)
+        return hidden_states, residual, next_mlp_sp_logit
+
+
+def create_sparse_block(d: int, ffn: int, num_heads: int, mlp_rank: int, mlp_K: int, att_rank: int, att_K: int,
+                        layer_idx: int, device="cuda", dtype=torch.float16, att_sparse: bool = True):
+    """One OPT-style block (ReLU MLP, biased projections) with both predictors,
+    assembled the way Dejavu/src/models/gpt_dejavu.py:168-305 wires create_mixer_cls /
+    create_mlp_cls / create_block."""
+    mlp_sp = {"embed_dim": d, "low_rank_dim": mlp_rank, "out_dim": ffn, "K": mlp_K}
+    mlp_cls = partial(ParallelFusedMLPDejavu, hidden_features=ffn, sp_kwargs=mlp_sp, activation="relu",
+                      layer_idx=layer_idx, process_group=None, sequence_parallel=False, device=device, dtype=dtype)
+    norm_cls = partial(nn.LayerNorm, eps=1e-5, device=device, dtype=dtype)
+    scale = (d // num_heads) ** -0.5
+    if att_sparse:
+        att_sp = {"embed_dim": d, "low_rank_dim": att_rank, "out_dim": num_heads, "K": att_K}
+        mixer_cls = partial(ParallelMHASparseAttMlp, num_heads=num_heads, process_group=None, sp_kwargs=att_sp,
+                            softmax_scale=scale, causal=True, layer_idx=layer_idx, sequence_parallel=False,
+                            device=device, dtype=dtype)
+        return BlockMlpAttSparse(d, mixer_cls, mlp_cls, norm_cls=norm_cls)
+    mixer_cls = partial(ParallelMHADejavu, num_heads=num_heads, process_group=None, softmax_scale=scale, causal=True,
+                        layer_idx=layer_idx, sequence_parallel=False, device=device, dtype=dtype)
+    return BlockDejavu(d, mixer_cls, mlp_cls, norm_cls=norm_cls)
+
+
+@torch.no_grad()
+def init_block_synthetic(block: nn.Module, seed: int) -> None:
+    """Seeded synthetic weights: projections ~ N(0, 0.02), fc1 bias ~ N(-0.1, 0.02), other
+    biases 0, predictors ~ N(0, 0.05), LayerNorm weight 1 / bias 0.  Drawn on the
+    parameters' own device."""
+    dev = next(block.parameters()).device
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed)
+
+    def fill(p, mean, std):
+        tmp = torch.empty(p.shape, dtype=torch.float32, device=dev)
+        tmp.normal_(mean, std, generator=gen)
+        p.copy_(tmp)
+
+    fill(block.mixer.Wqkv.weight, 0.0, 0.02)
+    block.mixer.Wqkv.bias.zero_()
+    fill(block.mixer.out_proj.weight, 0.0, 0.02)
+    block.mixer.out_proj.bias.zero_()
+    fill(block.mlp.fc1.weight, 0.0, 0.02)
+    fill(block.mlp.fc1.bias, -0.1, 0.02)
+    fill(block.mlp.fc2.weight, 0.0, 0.02)
+    block.mlp.fc2.bias.zero_()
+    fill(block.mlp.sp.fc0.weight, 0.0, 0.05)
+    fill(block.mlp.sp.fc1.weight, 0.0, 0.05)
+    if hasattr(block.mixer, "sp"):
+        fill(block.mixer.sp.fc0.weight, 0.0, 0.05)
+        fill(block.mixer.sp.fc1.weight, 0.0, 0.05)
+    for norm in (block.norm1, block.norm2):
+        norm.weight.fill_(1.0)
+        norm.bias.zero_()

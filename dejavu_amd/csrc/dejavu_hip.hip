@@ -10,6 +10,7 @@
 #include "common.hpp"
 #include "gemv_cols.hpp"
 #include "gemv_rows.hpp"
+#include "norm.hpp"
 #include "topk.hpp"
 
 using namespace dv;
@@ -488,6 +489,34 @@ int dv_out_proj_sparse_t_f16(const void* x, const void* Wt, int64_t ldw, const v
                      reinterpret_cast<const half_t*>(Wt), ldw, reinterpret_cast<const half_t*>(bias),
                      head_idx, 4, hd, B, N, H * hd, nnz * hd, reinterpret_cast<half_t*>(y),
                      workspace, workspace_bytes, reinterpret_cast<hipStream_t>(stream));
+}
+
+int dv_add_layer_norm_f16(const void* h, const void* residual, const void* gamma, const void* beta,
+                          float eps, int rows, int d, void* y, void* residual_out, void* stream) {
+  if (!h || !gamma || !beta || !y || rows < 0 || d <= 0) return DV_ERR_INVALID_ARG;
+  if (d % 8 || !aligned16(h) || !aligned16(y) || !aligned16(gamma) || !aligned16(beta) ||
+      (residual && !aligned16(residual)) || (residual_out && !aligned16(residual_out)))
+    return DV_ERR_ALIGNMENT;
+  if (d > 256 * 8 * 16) return DV_ERR_UNSUPPORTED;
+  if (rows == 0) return DV_OK;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+#define DV_LN(T, V)                                                                              \
+  hipLaunchKernelGGL((add_layer_norm_kernel<T, V>), dim3(rows), dim3(T), 0, s,                    \
+                     reinterpret_cast<const half_t*>(h), reinterpret_cast<const half_t*>(residual), \
+                     reinterpret_cast<const half_t*>(gamma), reinterpret_cast<const half_t*>(beta), \
+                     eps, d, reinterpret_cast<half_t*>(y), reinterpret_cast<half_t*>(residual_out))
+  if (d <= 256 * 8 * 1)
+    DV_LN(256, 1);
+  else if (d <= 256 * 8 * 2)
+    DV_LN(256, 2);
+  else if (d <= 256 * 8 * 4)
+    DV_LN(256, 4);
+  else if (d <= 256 * 8 * 8)
+    DV_LN(256, 8);
+  else
+    DV_LN(256, 16);
+#undef DV_LN
+  return launch_status();
 }
 
 }  // extern "C"

@@ -64,12 +64,15 @@ class ParallelSP(nn.Module):
         self.out = out_dim // size
         self.fc1 = nn.Linear(low_rank_dim, out_dim, bias=False, device=device, dtype=dtype)
         self.K = K // size
+        # optional caller-owned result buffer (fixed addresses for graph capture)
+        self.logits_out = None
 
     def forward(self, x):
         """x: anything viewable as (embed_dim,) -> (out_dim,) logits, as the
         reference; a (B, 1, embed_dim) batch gives (B, out_dim)."""
         single = x.numel() == self.embed_dim
-        logits = ops.predictor_logits(x.reshape(-1, self.embed_dim), self.fc0.weight, self.fc1.weight)
+        logits = ops.predictor_logits(x.reshape(-1, self.embed_dim), self.fc0.weight, self.fc1.weight,
+                                      out=self.logits_out)
         return logits.view(-1) if single else logits
 
     def topk(self, logits, k=None, dtype=torch.int64):
@@ -275,6 +278,8 @@ class ParallelMHASparseAttMlp(_MHABase):
         self.cache_offset = None  # device int32[1]: cache position of window token 0
         self.out_proj_weight_t = None
         self._all_heads = None
+        # optional caller-owned buffer for the predicted heads (fixed address for graph capture)
+        self.att_idx_out = None
 
     def reset_window(self):
         self.counter = 0
@@ -354,7 +359,7 @@ class ParallelMHASparseAttMlp(_MHABase):
             self.sp_stream.wait_event(self.event_out)
             if do_token_generation:
                 att_sp_logit = self.sp(residual)
-                att_idx = ops.topk_indices(att_sp_logit, self.att_k, dtype=torch.int32)
+                att_idx = ops.topk_indices(att_sp_logit, self.att_k, dtype=torch.int32, out=self.att_idx_out)
             self.sp_stream.record_event(self.event_att_sp)
         curr_stream.wait_event(self.event_mlp_sp)
         curr_stream.wait_event(self.event_att_sp)

@@ -64,7 +64,7 @@ def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
 # predictor + top-k
 # ---------------------------------------------------------------------------
 def predictor_logits(x: torch.Tensor, fc0_weight: torch.Tensor, fc1_weight: torch.Tensor,
-                     hidden: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     hidden: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``logits = fc1(fc0(x))`` for the bias-free low-rank predictor.
 
     x: (B, d) fp16, fc0_weight: (r, d), fc1_weight: (out, r) -> (B, out) fp16.
@@ -83,14 +83,19 @@ def predictor_logits(x: torch.Tensor, fc0_weight: torch.Tensor, fc1_weight: torc
         fc1_weight = fc1_weight.contiguous()
     if hidden is None:
         hidden = torch.empty(B, r, device=x.device, dtype=x.dtype)
-    logits = torch.empty(B, n_out, device=x.device, dtype=x.dtype)
+    if out is None:
+        logits = torch.empty(B, n_out, device=x.device, dtype=x.dtype)
+    else:
+        assert out.numel() == B * n_out and out.is_contiguous() and out.dtype == x.dtype
+        logits = out.view(B, n_out)
     check(lib.dv_predictor_logits_f16(_ptr(x), _ptr(fc0_weight), fc0_weight.stride(0), _ptr(fc1_weight),
                                       fc1_weight.stride(0), B, d, r, n_out, _ptr(hidden), _ptr(logits),
                                       _stream()), "dv_predictor_logits_f16")
     return logits
 
 
-def topk_indices(logits: torch.Tensor, k: int, dtype: torch.dtype = torch.int64) -> torch.Tensor:
+def topk_indices(logits: torch.Tensor, k: int, dtype: torch.dtype = torch.int64,
+                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Indices of the k largest logits (ties to the lower index), ascending.
 
     logits: (n,) or (B, n) fp16; for B > 1 a column is ranked by its maximum
@@ -105,7 +110,10 @@ def topk_indices(logits: torch.Tensor, k: int, dtype: torch.dtype = torch.int64)
     assert lg.dim() == 2
     B, n = lg.shape
     assert 0 <= k <= n, f"k={k} outside [0, {n}]"
-    out = torch.empty(k, device=lg.device, dtype=dtype)
+    if out is None:
+        out = torch.empty(k, device=lg.device, dtype=dtype)
+    else:
+        assert out.shape == (k,) and out.is_contiguous()
     check(lib.dv_topk_f16(_ptr(lg), B, n, k, _ptr(out), _idx_bytes(out), _stream()), "dv_topk_f16")
     return out
 
@@ -432,3 +440,28 @@ def _attn_workspace(device: torch.device, nbytes: int) -> torch.Tensor:
         ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
         _attn_workspaces[key] = ws
     return ws
+
+
+# ---------------------------------------------------------------------------
+# block glue
+# ---------------------------------------------------------------------------
+def add_layer_norm(hidden: torch.Tensor, residual: Optional[torch.Tensor], weight: torch.Tensor,
+                   bias: torch.Tensor, eps: float = 1e-5):
+    """``residual_out = hidden + residual`` (fp16) and ``LayerNorm(residual_out)``.
+
+    hidden / residual: (..., d) fp16.  Returns (normed, residual_out), both shaped like hidden.
+    """
+    _require_device(hidden, residual, weight, bias)
+    assert hidden.dtype == torch.float16 and weight.dtype == torch.float16 and bias.dtype == torch.float16
+    d = hidden.shape[-1]
+    assert weight.shape == (d,) and bias.shape == (d,)
+    hidden = hidden.contiguous()
+    if residual is not None:
+        assert residual.shape == hidden.shape and residual.dtype == hidden.dtype
+        residual = residual.contiguous()
+    rows = hidden.numel() // d
+    y = torch.empty_like(hidden)
+    r_out = torch.empty_like(hidden)
+    check(lib.dv_add_layer_norm_f16(_ptr(hidden), _ptr(residual), _ptr(weight.contiguous()), _ptr(bias.contiguous()),
+                                    float(eps), rows, d, _ptr(y), _ptr(r_out), _stream()), "dv_add_layer_norm_f16")
+    return y, r_out

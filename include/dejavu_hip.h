@@ -193,6 +193,20 @@ DV_API int dv_out_proj_sparse_t_f16(const void* x, const void* Wt, int64_t ldw, 
                                     void* y, void* workspace, size_t workspace_bytes,
                                     void* stream);
 
+/*
+ * Fused residual add + LayerNorm of the pre-norm block:
+ *   residual_out = fp16(h + residual)   (h alone when residual is NULL)
+ *   y = LayerNorm(residual_out) * gamma + beta, fp32 statistics, fp16 out.
+ * Replaces the unfused dropout(p=0) + add + nn.LayerNorm of
+ * Dejavu/src/models/modules/block_dejavu.py:575-584 and 626-634 (and the
+ * dropout_add_layer_norm extension call at :596-606, :648-658).
+ *   h, residual, y, residual_out: (rows, d) contiguous; gamma, beta (d,);
+ *   residual_out may be NULL; d % 8 == 0, d <= 32768.
+ */
+DV_API int dv_add_layer_norm_f16(const void* h, const void* residual, const void* gamma,
+                                 const void* beta, float eps, int rows, int d, void* y,
+                                 void* residual_out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -521,3 +521,39 @@ def sparse_attention_step_dense_kv(x_hist, Wqkv, bqkv, Wout, bout, head_idx, sof
         ctx[h] = (p @ V).astype(F16)
     out = out_proj_sparse(ctx[None], Wout, head_idx, bout)[0]
     return out, ctx
+
+
+def block_decode_step(p, hidden_states, residual, head_idx, mlp_sp_logit, k_cache, v_cache, timestep,
+                      residual2_override=None):
+    """One decode step of the pre-norm sparse block (batch 1), newest token only.
+
+    Dejavu/src/models/modules/block_dejavu.py:555-663: add -> LN1 -> mixer ->
+    add -> LN2 -> mlp, the mixer being ParallelMHASparseAttMlp.forward
+    (mha_dejavu.py:1283-1511) with every active head already up to date in the
+    cache, the mlp ParallelFusedMLPDejavu.forward
+    (fused_dense_sparse_dejavu.py:889-951).  ``p`` holds numpy fp16 arrays:
+    ln1_w, ln1_b, ln2_w, ln2_b, Wqkv (3,H,hd,d), bqkv, Wout (d,H,hd), bout, W1,
+    b1, W2t, b2, mlp_Wa, mlp_Wb, att_Wa, att_Wb and ints mlp_K, att_K.
+    hidden_states, residual: (1, d).  Caches are updated in place.
+    ``residual2_override`` (the device's own post-attention residual) can be
+    fed to the MLP predictor so that index sets are compared on identical input.
+    Returns dict(hidden, residual, next_mlp_logit, next_att_idx, mlp_idx, residual1, attn_out).
+    """
+    r1 = (np.asarray(hidden_states, F16).astype(F32) + np.asarray(residual, F16).astype(F32)).astype(F16) \
+        if residual is not None else np.asarray(hidden_states, F16)
+    x = layer_norm(r1, p["ln1_w"], p["ln1_b"])
+    H = p["Wqkv"].shape[1]
+    hi = np.asarray(head_idx, dtype=np.int32)
+    qkv = qkv_proj_sparse(x, p["Wqkv"], hi, np.zeros((len(hi), 1), dtype=np.int32), p["bqkv"])
+    ctx = single_query_attention(qkv[:, 0], qkv[:, 1], qkv[:, 2], k_cache, v_cache, timestep, head_idx=hi)
+    attn_out = out_proj_sparse(ctx, p["Wout"], hi, p["bout"])
+    mlp_idx = topk_lower_index(mlp_sp_logit, p["mlp_K"])
+    _, att_logit = predictor_logits(r1, p["att_Wa"], p["att_Wb"])
+    next_att_idx = topk_lower_index(att_logit[0], p["att_K"]).astype(np.int32)
+    r2 = (attn_out.astype(F32) + r1.astype(F32)).astype(F16)
+    x2 = layer_norm(r2, p["ln2_w"], p["ln2_b"])
+    hidden = mlp_sparse(x2, p["W1"], p["W2t"], mlp_idx, p["b1"], p["b2"])
+    r2_pred = r2 if residual2_override is None else np.asarray(residual2_override, F16)
+    _, next_mlp_logit = predictor_logits(r2_pred, p["mlp_Wa"], p["mlp_Wb"])
+    return dict(hidden=hidden, residual=r2, next_mlp_logit=next_mlp_logit[0], next_att_idx=next_att_idx,
+                mlp_idx=mlp_idx, residual1=r1, attn_out=attn_out)

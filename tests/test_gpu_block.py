@@ -1,0 +1,94 @@
+"""GPU parity of the fused add+LayerNorm kernel and of a whole sparse block
+decode step against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import dejavu_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def assert_close(got, want, what="", max_abs_tol=2e-2, rel_tol=1e-3):
+    got = np.asarray(got, dtype=np.float64)
+    want = np.asarray(want, dtype=np.float64)
+    max_abs = np.max(np.abs(got - want)) if got.size else 0.0
+    rel = np.linalg.norm(got - want) / max(np.linalg.norm(want), 1e-30)
+    assert max_abs <= max_abs_tol and rel <= rel_tol, f"{what}: max_abs={max_abs:.3e} rel_l2={rel:.3e}"
+
+
+def np16(t):
+    return t.detach().cpu().numpy()
+
+
+@pytest.mark.parametrize("rows,d", [(1, 768), (3, 4096), (1, 12288), (2, 9216), (5, 520), (1, 20480)])
+def test_add_layer_norm(rows, d):
+    from dejavu_amd import ops
+
+    g = torch.Generator().manual_seed(d)
+    h = torch.randn(rows, d, generator=g).half()
+    r = (torch.randn(rows, d, generator=g) * 3).half()
+    w = (1 + 0.1 * torch.randn(d, generator=g)).half()
+    b = (0.1 * torch.randn(d, generator=g)).half()
+    print(f"case add_layer_norm rows={rows} d={d}", flush=True)
+    y, r_out = ops.add_layer_norm(h.cuda(), r.cuda(), w.cuda(), b.cuda(), 1e-5)
+    y0, r0 = ops.add_layer_norm(h.cuda(), None, w.cuda(), b.cuda(), 1e-5)
+    torch.cuda.synchronize()
+    want_r = (h.float() + r.float()).half()
+    assert torch.equal(r_out.cpu(), want_r), "residual stream must be the fp16-rounded sum, bit for bit"
+    assert torch.equal(r0.cpu(), h)
+    assert_close(np16(y), O.layer_norm(want_r.numpy(), w.numpy(), b.numpy()), "add+LN")
+    assert_close(np16(y0), O.layer_norm(h.numpy(), w.numpy(), b.numpy()), "LN only")
+    ref = torch.nn.functional.layer_norm(want_r.float(), (d,), w.float(), b.float(), 1e-5).numpy()
+    assert_close(np16(y), ref, "add+LN vs torch fp32")
+
+
+def test_sparse_block_decode_step_matches_oracle():
+    from dejavu_amd.block import create_sparse_block, init_block_synthetic
+    from dejavu_amd.modules import InferenceParams
+    from dejavu_amd.workloads import pack_k_cache
+
+    d, ffn, H, r, K, Hk, S = 768, 3072, 12, 128, 1024, 4, 128
+    hd = d // H
+    block = create_sparse_block(d, ffn, H, r, K, r, Hk, layer_idx=2)
+    init_block_synthetic(block, seed=0)
+    with torch.no_grad():  # non-trivial LayerNorm parameters and biases
+        g = torch.Generator().manual_seed(9)
+        for n in (block.norm1, block.norm2):
+            n.weight.copy_((1 + 0.1 * torch.randn(d, generator=g)).half())
+            n.bias.copy_((0.1 * torch.randn(d, generator=g)).half())
+        block.mixer.Wqkv.bias.copy_((0.1 * torch.randn(3 * d, generator=g)).half())
+        block.mixer.out_proj.bias.copy_((0.1 * torch.randn(d, generator=g)).half())
+    g = torch.Generator().manual_seed(10)
+    t = S - 1
+    kc = torch.randn(1, H, S, hd, generator=g).half()
+    vc = torch.randn(1, H, S, hd, generator=g).half()
+    ip = InferenceParams(max_sequence_len=S, max_batch_size=1, sequence_len_offset=t)
+    ip.key_value_memory_dict[2] = (pack_k_cache(kc).cuda(), vc.cuda())
+    hs = torch.randn(1, 1, d, generator=g).half()
+    res = torch.randn(1, 1, d, generator=g).half()
+    head_idx = torch.sort(torch.randperm(H, generator=g)[:Hk]).values.int()
+    mlp_sp_logit = (torch.randn(ffn, generator=g) * 4).half()
+    print("case sparse block decode step", flush=True)
+    with torch.no_grad():
+        hidden, residual, next_logit, next_att = block(hs.cuda(), res.cuda(), mixer_kwargs={"inference_params": ip},
+                                                       head_idx=head_idx.cuda(), mlp_sp_logit=mlp_sp_logit.cuda())
+    torch.cuda.synchronize()
+    m, f = block.mixer, block.mlp
+    p = dict(ln1_w=np16(block.norm1.weight), ln1_b=np16(block.norm1.bias), ln2_w=np16(block.norm2.weight),
+             ln2_b=np16(block.norm2.bias), Wqkv=np16(m.Wqkv.weight).reshape(3, H, hd, d),
+             bqkv=np16(m.Wqkv.bias).reshape(3, H, hd), Wout=np16(m.out_proj.weight).reshape(d, H, hd),
+             bout=np16(m.out_proj.bias), W1=np16(f.fc1.weight), b1=np16(f.fc1.bias),
+             W2t=np.ascontiguousarray(np16(f.fc2.weight).T), b2=np16(f.fc2.bias), mlp_Wa=np16(f.sp.fc0.weight),
+             mlp_Wb=np16(f.sp.fc1.weight), att_Wa=np16(m.sp.fc0.weight), att_Wb=np16(m.sp.fc1.weight), mlp_K=K, att_K=Hk)
+    kn, vn = pack_k_cache(kc).numpy().copy(), vc.numpy().copy()
+    want = O.block_decode_step(p, hs.numpy()[0], res.numpy()[0], head_idx.numpy(), mlp_sp_logit.numpy(), kn, vn, t,
+                               residual2_override=np16(residual)[0])
+    assert_close(np16(residual)[0], want["residual"], "residual stream after attention")
+    assert_close(np16(hidden)[0], want["hidden"], "block output", max_abs_tol=3e-2, rel_tol=3e-3)
+    assert np.array_equal(np16(next_att).astype(np.int64), want["next_att_idx"].astype(np.int64)), "next heads differ"
+    assert np.array_equal(np16(next_logit).view(np.uint16), want["next_mlp_logit"].view(np.uint16)), \
+        "next-layer MLP logits not bit-exact"
+    kcd, vcd = ip.key_value_memory_dict[2]
+    assert np.array_equal(np16(vcd), vn), "value cache after the step differs"
+    assert_close(np16(kcd), kn, "key cache after the step")
