@@ -70,11 +70,9 @@ def build_layers(cfg, batch, device):
         block.mixer.cache_offset = torch.tensor([S - 1], dtype=torch.int32, device=device)
         layers.append(dict(block=block, ip=ip, hidden=randn((batch, 1, d)), residual=randn((batch, 1, d))))
     # predictions travel from layer l to layer l+1 through fixed buffers
-    fresh = torch.arange(16, dtype=torch.int32, device=device).repeat(H, 1)
     for l, L in enumerate(layers):
         L["att_idx_in"] = torch.sort(torch.randperm(H, generator=gen, device=device)[:Hk]).values.int()
         L["mlp_logit_in"] = randn((ffn,), 4.0)
-        L["fresh_tracker"] = fresh
     for l, L in enumerate(layers):
         nxt = layers[(l + 1) % N_LAYERS]
         L["block"].mixer.att_idx_out = nxt["att_idx_in"]
@@ -86,8 +84,7 @@ def layer_step(L):
     """One decode step of one block in the state 'first token of a back-fill
     window': every active head computes Q, K, V of the newest token."""
     mixer = L["block"].mixer
-    mixer.counter = 0
-    mixer.tracker.copy_(L["fresh_tracker"])
+    mixer.counter = 0  # the window step re-initialises the tracker at counter 0
     return L["block"](L["hidden"], L["residual"], mixer_kwargs={"inference_params": L["ip"]},
                       head_idx=L["att_idx_in"], mlp_sp_logit=L["mlp_logit_in"])
 
@@ -193,6 +190,10 @@ def main():
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying HIP graphs")
+    ap.add_argument("--single-stream", action="store_true", help="no side stream for predictors / top-k")
+    ap.add_argument("--layers-per-graph", type=int, default=3, choices=[1, 3])
+    ap.add_argument("--defer", action="store_true",
+                    help="let the MLP predictor of layer l run into layer l+1 (joined once per graph)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs the sparse decode layer on ONE GPU (no sharding); "
@@ -201,8 +202,10 @@ def main():
 
     import torch
 
+    import dejavu_amd.modules as dv_modules
     from dejavu_amd.workloads import CONFIGS
 
+    dv_modules.USE_SIDE_STREAM = not args.single_stream
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(1)
@@ -212,25 +215,42 @@ def main():
     assert batch == 1, "the head-sparse decode layer keeps one back-fill window (batch 1)"
     device = torch.device("cuda:0")
     layers = build_layers(cfg, batch, device)
+    defer = args.defer and (not args.single_stream) and args.layers_per_graph == N_LAYERS \
+        and not args.no_graph
+    for L in layers:
+        L["block"].mlp.defer_predictor_join = defer
 
     with torch.no_grad():
         # eager warm-up: allocates workspaces, sets kernel attributes
         for _ in range(2):
             for L in layers:
                 layer_step(L)
+            dv_modules.join_side_stream()
         torch.cuda.synchronize()
         graphs = []
-        if not args.no_graph:
+        if not args.no_graph and args.layers_per_graph == 1:
             for L in layers:
                 g = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(g):
                     L["out"] = layer_step(L)
                 graphs.append(g)
             torch.cuda.synchronize()
+        elif not args.no_graph:
+            assert args.steps % N_LAYERS == 0 and args.warmup % N_LAYERS == 0
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                for L in layers:
+                    L["out"] = layer_step(L)
+                dv_modules.join_side_stream()
+            graphs.append(g)
+            torch.cuda.synchronize()
 
         def run(i):
-            if graphs:
+            if len(graphs) == N_LAYERS:
                 graphs[i % N_LAYERS].replay()
+            elif graphs:
+                if i % N_LAYERS == 0:
+                    graphs[0].replay()
             else:
                 layer_step(layers[i % N_LAYERS])
 

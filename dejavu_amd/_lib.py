@@ -32,7 +32,9 @@ SIGNATURES = {
         _c_int,
         [_c_ptr, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr],
     ),
-    "dv_topk_f16": (_c_int, [_c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_ptr]),
+    "dv_topk_workspace_bytes": (_c_size, [_c_int]),
+    "dv_topk_f16": (_c_int, [_c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_ptr, _c_size, _c_ptr]),
+    "dv_topk_search_f16": (_c_int, [_c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_ptr]),
     "dv_gather_gemv_f16": (
         _c_int,
         [_c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr],
@@ -45,6 +47,15 @@ SIGNATURES = {
     ),
     "dv_qkv_proj_sparse_f16": (
         _c_int, [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr]),
+    "dv_qkv_proj_sparse_cache_f16": (
+        _c_int,
+        [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr,
+         _c_ptr, _c_int, _c_ptr]),
+    "dv_attention_out_proj_workspace_bytes": (_c_size, [_c_int, _c_int, _c_int, _c_int, _c_int]),
+    "dv_attention_out_proj_f16": (
+        _c_int,
+        [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int,
+         ctypes.c_float, _c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_size, _c_ptr]),
     "dv_kv_cache_copy_sparse_f16": (
         _c_int,
         [_c_ptr, _c_ptr, _c_i64, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_int,

@@ -20,13 +20,15 @@ namespace dv {
 // X (nb, d); W (3, H, hd, d) contiguous; Y (nb, 3, H, hd).  Rows of one (t, h)
 // are hd consecutive weight rows; a wavefront owns R of them at a time and
 // keeps one accumulator per live slot.  Nothing is written for dead slots or
-// unselected heads.
+// unselected heads.  With k_cache / v_cache given, the K and V rows are also
+// scattered into the caches at position (token + padding[0]).
 // ---------------------------------------------------------------------------
 template <int NBMAX, int R, int U>
 __global__ __launch_bounds__(256) void qkv_sparse_kernel(
     const half_t* __restrict__ X, const half_t* __restrict__ W, const half_t* __restrict__ bias,
     const int* __restrict__ head_idx, const int* __restrict__ batch_idx, int nb, int d, int H,
-    int hd, int nnz, half_t* __restrict__ Y) {
+    int hd, int nnz, half_t* __restrict__ Y, half_t* __restrict__ k_cache,
+    half_t* __restrict__ v_cache, const int* __restrict__ padding, int S) {
   constexpr int CH = 8 * kWave;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -102,7 +104,21 @@ __global__ __launch_bounds__(256) void qkv_sparse_kernel(
         for (int r = 0; r < R; ++r) {
           float v = butterfly_sum<kWave>(acc[r][s]);
           if (bias != nullptr) v += (float)bias[row0 + r];
-          if (lane == 0) Y[(int64_t)slot[s] * 3 * H * hd + row0 + r] = (half_t)v;
+          if (lane == 0) {
+            const half_t hv = (half_t)v;
+            Y[(int64_t)slot[s] * 3 * H * hd + row0 + r] = hv;
+            // optional fused cache scatter (same arithmetic as kv_cache_copy_kernel)
+            if (t != 0 && k_cache != nullptr) {
+              const int dst = slot[s] + (padding ? padding[0] : 0);
+              const int j = j0 + r;
+              if (dst >= 0 && dst < S) {
+                if (t == 1)
+                  k_cache[(((int64_t)h * (hd / 8) + j / 8) * S + dst) * 8 + (j & 7)] = hv;
+                else
+                  v_cache[((int64_t)h * S + dst) * hd + j] = hv;
+              }
+            }
+          }
         }
       }
     }
@@ -137,34 +153,42 @@ __global__ void kv_cache_copy_kernel(const half_t* __restrict__ K, const half_t*
 
 // One decode step of the skipped-head back-fill window.
 //   x_cache[counter, :] = x
-//   flush == 0: for i < nnz, h = head_idx[i], s <= counter:
-//                 batch_idx[i, s] = tracker[h, s];  tracker[h, s] = -1
 //   flush != 0: for every head h and s < 16: batch_idx[h, s] = s, tracker[h, s] = s
+//   flush == 0: (counter == 0: the tracker is first re-initialised, tracker[h, s] = s;
+//                a window always starts from that state)
+//               for i < nnz, h = head_idx[i], s <= counter:
+//                 batch_idx[i, s] = tracker[h, s];  tracker[h, s] = -1
 // tracker is (H, 16) int32: tracker[h, s] == s while token s of the window has no
-// K/V for head h, -1 once it has.  Heads in head_idx are distinct.
-__global__ void window_step_kernel(const half_t* __restrict__ x, half_t* __restrict__ x_cache, int d,
-                                   int* __restrict__ tracker, const int* __restrict__ head_idx,
-                                   int nnz, int H, int counter, int flush,
-                                   int* __restrict__ batch_idx) {
+// K/V for head h, -1 once it has.  Heads in head_idx are distinct.  Workgroup 0
+// owns the tracker (two phases separated by a barrier); all workgroups copy x.
+__global__ __launch_bounds__(256) void window_step_kernel(
+    const half_t* __restrict__ x, half_t* __restrict__ x_cache, int d, int* __restrict__ tracker,
+    const int* __restrict__ head_idx, int nnz, int H, int counter, int flush,
+    int* __restrict__ batch_idx) {
   const int tid = blockIdx.x * blockDim.x + threadIdx.x;
   const int nthreads = gridDim.x * blockDim.x;
   for (int j = tid; j < d; j += nthreads) x_cache[(int64_t)counter * d + j] = x[j];
+  if (blockIdx.x != 0) return;
   if (flush) {
-    for (int o = tid; o < H * 16; o += nthreads) {
+    for (int o = threadIdx.x; o < H * 16; o += blockDim.x) {
       tracker[o] = o & 15;
       batch_idx[o] = o & 15;
     }
-  } else {
-    const int nb = counter + 1;
-    for (int o = tid; o < nnz * nb; o += nthreads) {
-      const int i = o / nb, s = o - i * nb;
-      const int h = head_idx[i];
-      if (h < 0 || h >= H) {
-        batch_idx[o] = -1;
-      } else {
-        batch_idx[o] = tracker[h * 16 + s];
-        tracker[h * 16 + s] = -1;
-      }
+    return;
+  }
+  if (counter == 0) {
+    for (int o = threadIdx.x; o < H * 16; o += blockDim.x) tracker[o] = o & 15;
+    __syncthreads();
+  }
+  const int nb = counter + 1;
+  for (int o = threadIdx.x; o < nnz * nb; o += blockDim.x) {
+    const int i = o / nb, s = o - i * nb;
+    const int h = head_idx[i];
+    if (h < 0 || h >= H) {
+      batch_idx[o] = -1;
+    } else {
+      batch_idx[o] = tracker[h * 16 + s];
+      tracker[h * 16 + s] = -1;
     }
   }
 }
@@ -189,89 +213,101 @@ __global__ void kv_append_kernel(const half_t* __restrict__ K, const half_t* __r
 }
 
 // ---------------------------------------------------------------------------
-// One-query attention, one wavefront per (64-position split, head, batch row).
-// Lanes map to positions for q.K (each lane reads its position's hd/8 packets)
-// and to (row, 8-wide slice) for p.V.  All K and V loads of the split are
-// issued before any arithmetic.  Writes un-normalised partials
-//   part[(b, i, split)] = { max, sum, o[hd] }  (fp32)
+// One-query attention.  A workgroup of WAVES wavefronts handles WAVES*64 cached
+// positions of one (head, batch row); inside a wavefront lanes map to positions
+// for q.K (each lane reads its position's hd/8 packets) and to (row, 8-wide
+// slice) for p.V.  All K and V loads of a wavefront are issued before any
+// arithmetic.  The wavefronts are merged in LDS and the workgroup writes one
+// un-normalised partial  part[(b, i, split)] = { max, sum, o[hd] }  (fp32).
 // n_len = number of cached positions to attend (lengths[b] + 1 if lengths).
 // ---------------------------------------------------------------------------
-template <int HD>
-__global__ __launch_bounds__(64) void decode_attn_kernel(
+template <int HD, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void decode_attn_kernel(
     const half_t* __restrict__ Q, int64_t ldq, const half_t* __restrict__ k_cache,
     const half_t* __restrict__ v_cache, const int* __restrict__ head_idx,
     const int* __restrict__ lengths, int n_len, int H, int S, float scale, int nsplit,
     float* __restrict__ part) {
-  constexpr int PK = HD / 8;     // 16-byte packets per position / lanes per V row
-  constexpr int RPI = kWave / PK;  // V rows per load instruction
-  constexpr int VIT = kWave / RPI;  // V load instructions per split (= PK)
-  const int lane = threadIdx.x;
+  constexpr int PK = HD / 8;        // 16-byte packets per position / lanes per V row
+  constexpr int RPI = kWave / PK;   // V rows per load instruction
+  constexpr int VIT = kWave / RPI;  // V load instructions per wavefront (= PK)
+  __shared__ float s_m[WAVES], s_l[WAVES];
+  __shared__ float s_o[WAVES][HD];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
   const int split = blockIdx.x;
   const int i = blockIdx.y;
   const int b = blockIdx.z;
   const int h = head_idx ? head_idx[i] : i;
   const int len = lengths ? lengths[b] + 1 : n_len;
   float* out = part + (((int64_t)b * gridDim.y + i) * nsplit + split) * (HD + 2);
-  const int p0 = split * kWave;
-  if (h < 0 || h >= H || p0 >= len) {  // empty split: neutral element of the merge
-    if (lane == 0) {
-      out[0] = -INFINITY;
-      out[1] = 0.f;
-    }
-#pragma unroll
-    for (int e = lane; e < HD; e += kWave) out[2 + e] = 0.f;
-    return;
-  }
-  const int64_t bh = (int64_t)b * H + h;
-  const int pos = p0 + lane;
-  const bool pos_ok = pos < len;
-  const int pos_c = pos_ok ? pos : len - 1;  // clamp: always a valid address
-
-  // K packets of this lane's position
-  half8_t kp[PK];
-  const half_t* kbase = k_cache + (bh * PK * S + pos_c) * 8;
-#pragma unroll
-  for (int dp = 0; dp < PK; ++dp) kp[dp] = load8_stream(kbase + (int64_t)dp * S * 8);
-  // V rows: instruction it covers rows it*RPI + grp
-  const int grp = lane / PK, sub = lane % PK;
-  half8_t vv[VIT];
-#pragma unroll
-  for (int it = 0; it < VIT; ++it) {
-    int row = p0 + it * RPI + grp;
-    if (row >= len) row = len - 1;
-    vv[it] = load8_stream(v_cache + (bh * S + row) * HD + sub * 8);
-  }
-  // q (uniform across lanes)
-  const half_t* q = Q + (int64_t)b * ldq + (int64_t)h * HD;
-  float s = 0.f;
-#pragma unroll
-  for (int dp = 0; dp < PK; ++dp) s = dot8_fast(kp[dp], load8(q + dp * 8), s);
-  s = pos_ok ? s * scale : -INFINITY;
-  const float m = butterfly_max<kWave>(s);
-  const float p = pos_ok ? __expf(s - m) : 0.f;
-  const float l = butterfly_sum<kWave>(p);
-
+  const bool head_ok = h >= 0 && h < H;
+  const int p0 = (split * WAVES + wave) * kWave;
+  float m = -INFINITY, l = 0.f;
   float acc[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  const int grp = lane / PK, sub = lane % PK;
+  if (head_ok && p0 < len) {
+    const int64_t bh = (int64_t)b * H + h;
+    const int pos = p0 + lane;
+    const bool pos_ok = pos < len;
+    const int pos_c = pos_ok ? pos : len - 1;  // clamp: always a valid address
+    half8_t kp[PK];
+    const half_t* kbase = k_cache + (bh * PK * S + pos_c) * 8;
 #pragma unroll
-  for (int it = 0; it < VIT; ++it) {
-    const float pr = __shfl(p, it * RPI + grp, kWave);  // 0 for positions >= len
+    for (int dp = 0; dp < PK; ++dp) kp[dp] = load8_stream(kbase + (int64_t)dp * S * 8);
+    half8_t vv[VIT];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(pr, (float)vv[it][e], acc[e]);
-  }
+    for (int it = 0; it < VIT; ++it) {
+      int row = p0 + it * RPI + grp;
+      if (row >= len) row = len - 1;
+      vv[it] = load8_stream(v_cache + (bh * S + row) * HD + sub * 8);
+    }
+    const half_t* q = Q + (int64_t)b * ldq + (int64_t)h * HD;
+    float sc = 0.f;
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
+    for (int dp = 0; dp < PK; ++dp) sc = dot8_fast(kp[dp], load8(q + dp * 8), sc);
+    sc = pos_ok ? sc * scale : -INFINITY;
+    m = butterfly_max<kWave>(sc);
+    const float p = pos_ok ? __expf(sc - m) : 0.f;
+    l = butterfly_sum<kWave>(p);
 #pragma unroll
-    for (int off = PK; off < kWave; off <<= 1) acc[e] += __shfl_xor(acc[e], off, kWave);
+    for (int it = 0; it < VIT; ++it) {
+      const float pr = __shfl(p, it * RPI + grp, kWave);  // 0 for positions >= len
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(pr, (float)vv[it][e], acc[e]);
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+#pragma unroll
+      for (int off = PK; off < kWave; off <<= 1) acc[e] += __shfl_xor(acc[e], off, kWave);
+    }
   }
   if (lane == 0) {
-    out[0] = m;
-    out[1] = l;
+    s_m[wave] = m;
+    s_l[wave] = l;
   }
   if (grp == 0) {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) out[2 + sub * 8 + e] = acc[e];
+    for (int e = 0; e < 8; ++e) s_o[wave][sub * 8 + e] = acc[e];
+  }
+  __syncthreads();
+  // merge the wavefronts (empty ones carry max = -inf, sum = 0)
+  float M = -INFINITY;
+#pragma unroll
+  for (int w = 0; w < WAVES; ++w) M = fmaxf(M, s_m[w]);
+  for (int j = threadIdx.x; j < HD + 2; j += WAVES * kWave) {
+    float v = 0.f;
+    if (j == 0) {
+      v = M;
+    } else {
+#pragma unroll
+      for (int w = 0; w < WAVES; ++w) {
+        const float sw = s_m[w] == -INFINITY ? 0.f : __expf(s_m[w] - M);
+        v += sw * (j == 1 ? s_l[w] : s_o[w][j - 2]);
+      }
+    }
+    out[j] = v;
   }
 }
 
@@ -286,14 +322,31 @@ __global__ __launch_bounds__(HD) void decode_attn_combine_kernel(
   const int h = head_idx ? head_idx[i] : i;
   if (h < 0 || h >= H) return;
   const float* p = part + ((int64_t)b * gridDim.x + i) * nsplit * (HD + 2);
-  float m = -INFINITY;
-  for (int s = 0; s < nsplit; ++s) m = fmaxf(m, p[s * (HD + 2)]);
-  float num = 0.f, den = 0.f;
-  for (int s = 0; s < nsplit; ++s) {
-    const float ms = p[s * (HD + 2)];
-    const float w = ms == -INFINITY ? 0.f : __expf(ms - m);
-    den += w * p[s * (HD + 2) + 1];
-    num += w * p[s * (HD + 2) + 2 + j];
+  float m = -INFINITY, num = 0.f, den = 0.f;
+  for (int s0 = 0; s0 < nsplit; s0 += 8) {  // online merge, 8 splits' loads in flight
+    float ms[8], ls[8], os[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const bool ok = s0 + q < nsplit;
+      const float* ps = p + (int64_t)(ok ? s0 + q : s0) * (HD + 2);
+      ms[q] = ok ? ps[0] : -INFINITY;
+      ls[q] = ps[1];
+      os[q] = ps[2 + j];
+    }
+    float mc = m;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) mc = fmaxf(mc, ms[q]);
+    if (mc == -INFINITY) continue;
+    const float rescale = m == -INFINITY ? 0.f : __expf(m - mc);
+    num *= rescale;
+    den *= rescale;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const float w = ms[q] == -INFINITY ? 0.f : __expf(ms[q] - mc);
+      den += w * ls[q];
+      num += w * os[q];
+    }
+    m = mc;
   }
   out[(int64_t)b * ldo + (int64_t)h * HD + j] = (half_t)(num / den);
 }

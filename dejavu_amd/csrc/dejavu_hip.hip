@@ -197,7 +197,7 @@ int gather_cols(const half_t* x, int64_t ldx, int x_expanded, const half_t* W, i
 template <int NBMAX>
 int launch_qkv(const half_t* x, const half_t* W, const half_t* bias, const int* head_idx,
                const int* batch_idx, int nb, int d, int H, int hd, int nnz, half_t* y,
-               hipStream_t s) {
+               half_t* k_cache, half_t* v_cache, const int* padding, int S, hipStream_t s) {
   constexpr int R = 2, U = 4;
   const int ntasks = nnz * 3 * (hd / R);
   int blocks = (ntasks + 3) / 4;
@@ -205,11 +205,14 @@ int launch_qkv(const half_t* x, const half_t* W, const half_t* bias, const int* 
   if (blocks > cap) blocks = cap;
   if (blocks < 1) blocks = 1;
   hipLaunchKernelGGL((qkv_sparse_kernel<NBMAX, R, U>), dim3(blocks), dim3(256), 0, s, x, W, bias,
-                     head_idx, batch_idx, nb, d, H, hd, nnz, y);
+                     head_idx, batch_idx, nb, d, H, hd, nnz, y, k_cache, v_cache, padding, S);
   return launch_status();
 }
 
-inline int attn_splits(int n_len) { return n_len > 0 ? (n_len + kWave - 1) / kWave : 1; }
+constexpr int kAttnWaves = 4;  // wavefronts (x64 positions) per attention workgroup
+inline int attn_splits(int n_len) {
+  return n_len > 0 ? (n_len + kAttnWaves * kWave - 1) / (kAttnWaves * kWave) : 1;
+}
 
 }  // namespace
 
@@ -249,8 +252,50 @@ int dv_predictor_logits_f16(const void* x, const void* Wa, int64_t ldwa, const v
                         reinterpret_cast<half_t*>(logits), s);
 }
 
+size_t dv_topk_workspace_bytes(int n) { return n > 1024 ? 65536 * sizeof(unsigned) : 0; }
+
 int dv_topk_f16(const void* logits, int B, int n, int k, void* idx_out, int idx_bytes,
-                void* stream) {
+                void* workspace, size_t workspace_bytes, void* stream) {
+  if (!logits || B < 1 || n < 1 || k < 0 || k > n || !idx_ok(idx_bytes) || (k > 0 && !idx_out))
+    return DV_ERR_INVALID_ARG;
+  if (n > 65536) return DV_ERR_UNSUPPORTED;
+  if (k == 0) return DV_OK;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const half_t* lg = reinterpret_cast<const half_t*>(logits);
+  if (n <= 1024) {
+    hipLaunchKernelGGL(topk_small_kernel, dim3(1), dim3(256), 0, s, lg, B, n, k, idx_out, idx_bytes);
+    return launch_status();
+  }
+  if (n % 8 != 0) return DV_ERR_UNSUPPORTED;
+  if (!aligned16(logits)) return DV_ERR_ALIGNMENT;
+  if (!workspace || workspace_bytes < dv_topk_workspace_bytes(n) || !aligned16(workspace))
+    return DV_ERR_WORKSPACE;
+  unsigned* hist = reinterpret_cast<unsigned*>(workspace);
+  hipLaunchKernelGGL(topk_hist_kernel, dim3((n / 8 + 255) / 256), dim3(256), 0, s, lg, B, n, hist);
+#define DV_SEL(I) \
+  hipLaunchKernelGGL((topk_select_kernel<I>), dim3(1), dim3(1024), 0, s, lg, B, n, k, hist, idx_out, idx_bytes)
+  if (n <= 1024 * 8)
+    DV_SEL(8);
+  else if (n <= 1024 * 16)
+    DV_SEL(16);
+  else if (n <= 1024 * 24)
+    DV_SEL(24);
+  else if (n <= 1024 * 32)
+    DV_SEL(32);
+  else if (n <= 1024 * 40)
+    DV_SEL(40);
+  else if (n <= 1024 * 48)
+    DV_SEL(48);
+  else
+    DV_SEL(64);
+#undef DV_SEL
+  return launch_status();
+}
+
+// Single-launch variant without scratch memory (16-step bitwise search in one
+// workgroup); same result, slower for large n.
+int dv_topk_search_f16(const void* logits, int B, int n, int k, void* idx_out, int idx_bytes,
+                       void* stream) {
   if (!logits || B < 1 || n < 1 || k < 0 || k > n || !idx_ok(idx_bytes) || (k > 0 && !idx_out))
     return DV_ERR_INVALID_ARG;
   if (n > 65536) return DV_ERR_UNSUPPORTED;
@@ -331,10 +376,12 @@ int dv_gather_transposed_gemv_f16(const void* x, const void* W, int64_t ldw, con
                      reinterpret_cast<hipStream_t>(stream));
 }
 
-int dv_qkv_proj_sparse_f16(const void* x, const void* W, const void* bias, const void* head_idx,
-                           const void* batch_idx, int nb, int d, int H, int hd, int nnz, void* y,
-                           void* stream) {
-  if (!x || !W || !y || nb < 1 || d <= 0 || H <= 0 || nnz < 0 || (nnz > 0 && (!head_idx || !batch_idx)))
+int dv_qkv_proj_sparse_cache_f16(const void* x, const void* W, const void* bias,
+                                 const void* head_idx, const void* batch_idx, int nb, int d, int H,
+                                 int hd, int nnz, void* y, void* k_cache, void* v_cache,
+                                 const void* padding, int S, void* stream) {
+  if (!x || !W || !y || nb < 1 || d <= 0 || H <= 0 || nnz < 0 || (nnz > 0 && (!head_idx || !batch_idx)) ||
+      ((k_cache == nullptr) != (v_cache == nullptr)) || (k_cache && S <= 0))
     return DV_ERR_INVALID_ARG;
   if (nb > 16 || (hd != 32 && hd != 64 && hd != 128)) return DV_ERR_UNSUPPORTED;
   if (d % 8 || !aligned16(x) || !aligned16(W)) return DV_ERR_ALIGNMENT;
@@ -346,11 +393,23 @@ int dv_qkv_proj_sparse_f16(const void* x, const void* W, const void* bias, const
   const int* hi = reinterpret_cast<const int*>(head_idx);
   const int* bi = reinterpret_cast<const int*>(batch_idx);
   half_t* yy = reinterpret_cast<half_t*>(y);
-  if (nb == 1) return launch_qkv<1>(xx, ww, bb, hi, bi, nb, d, H, hd, nnz, yy, s);
-  if (nb == 2) return launch_qkv<2>(xx, ww, bb, hi, bi, nb, d, H, hd, nnz, yy, s);
-  if (nb <= 4) return launch_qkv<4>(xx, ww, bb, hi, bi, nb, d, H, hd, nnz, yy, s);
-  if (nb <= 8) return launch_qkv<8>(xx, ww, bb, hi, bi, nb, d, H, hd, nnz, yy, s);
-  return launch_qkv<16>(xx, ww, bb, hi, bi, nb, d, H, hd, nnz, yy, s);
+  half_t* kc = reinterpret_cast<half_t*>(k_cache);
+  half_t* vc = reinterpret_cast<half_t*>(v_cache);
+  const int* pad = reinterpret_cast<const int*>(padding);
+#define DV_QKV(NB) return launch_qkv<NB>(xx, ww, bb, hi, bi, nb, d, H, hd, nnz, yy, kc, vc, pad, S, s)
+  if (nb == 1) DV_QKV(1);
+  if (nb == 2) DV_QKV(2);
+  if (nb <= 4) DV_QKV(4);
+  if (nb <= 8) DV_QKV(8);
+  DV_QKV(16);
+#undef DV_QKV
+}
+
+int dv_qkv_proj_sparse_f16(const void* x, const void* W, const void* bias, const void* head_idx,
+                           const void* batch_idx, int nb, int d, int H, int hd, int nnz, void* y,
+                           void* stream) {
+  return dv_qkv_proj_sparse_cache_f16(x, W, bias, head_idx, batch_idx, nb, d, H, hd, nnz, y, nullptr,
+                                      nullptr, nullptr, 0, stream);
 }
 
 int dv_kv_cache_copy_sparse_f16(const void* k, const void* v, int64_t ld_src, int nsrc,
@@ -409,40 +468,119 @@ size_t dv_decode_attention_workspace_bytes(int B, int nheads, int n_len, int hd)
   return (size_t)B * nheads * attn_splits(n_len) * (hd + 2) * sizeof(float);
 }
 
-int dv_decode_attention_f16(const void* q, int64_t ldq, const void* k_cache, const void* v_cache,
-                            const void* head_idx, int nheads, const void* lengths, int n_len,
-                            int B, int H, int hd, int S, float scale, void* out, int64_t ldo,
-                            void* workspace, size_t workspace_bytes, void* stream) {
-  if (!q || !k_cache || !v_cache || !out || nheads < 0 || B < 1 || H <= 0 || S <= 0 ||
-      n_len < 1 || n_len > S)
-    return DV_ERR_INVALID_ARG;
-  if (hd != 64 && hd != 128) return DV_ERR_UNSUPPORTED;
-  if (ldq % 8 || !aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache))
-    return DV_ERR_ALIGNMENT;
-  const int heads = head_idx ? nheads : H;
-  if (heads == 0) return DV_OK;
-  if (!workspace || workspace_bytes < dv_decode_attention_workspace_bytes(B, heads, n_len, hd))
-    return DV_ERR_WORKSPACE;
-  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+namespace {
+int launch_attn_partials(const void* q, int64_t ldq, const void* k_cache, const void* v_cache,
+                         const void* head_idx, int heads, const void* lengths, int n_len, int B, int H,
+                         int hd, int S, float scale, float* part, hipStream_t s) {
   const int nsplit = attn_splits(n_len);
-  float* part = reinterpret_cast<float*>(workspace);
   const half_t* qq = reinterpret_cast<const half_t*>(q);
   const half_t* kc = reinterpret_cast<const half_t*>(k_cache);
   const half_t* vc = reinterpret_cast<const half_t*>(v_cache);
   const int* hi = reinterpret_cast<const int*>(head_idx);
   const int* ln = reinterpret_cast<const int*>(lengths);
-  half_t* oo = reinterpret_cast<half_t*>(out);
   dim3 grid(nsplit, heads, B);
-  if (hd == 128) {
-    hipLaunchKernelGGL((decode_attn_kernel<128>), grid, dim3(64), 0, s, qq, ldq, kc, vc, hi, ln,
-                       n_len, H, S, scale, nsplit, part);
+  if (hd == 128)
+    hipLaunchKernelGGL((decode_attn_kernel<128, kAttnWaves>), grid, dim3(kAttnWaves * 64), 0, s, qq,
+                       ldq, kc, vc, hi, ln, n_len, H, S, scale, nsplit, part);
+  else
+    hipLaunchKernelGGL((decode_attn_kernel<64, kAttnWaves>), grid, dim3(kAttnWaves * 64), 0, s, qq,
+                       ldq, kc, vc, hi, ln, n_len, H, S, scale, nsplit, part);
+  return launch_status();
+}
+
+int check_attn_args(const void* q, int64_t ldq, const void* k_cache, const void* v_cache, int nheads,
+                    int n_len, int B, int H, int hd, int S) {
+  if (!q || !k_cache || !v_cache || nheads < 0 || B < 1 || H <= 0 || S <= 0 || n_len < 1 || n_len > S)
+    return DV_ERR_INVALID_ARG;
+  if (hd != 64 && hd != 128) return DV_ERR_UNSUPPORTED;
+  if (ldq % 8 || !aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache)) return DV_ERR_ALIGNMENT;
+  return DV_OK;
+}
+}  // namespace
+
+int dv_decode_attention_f16(const void* q, int64_t ldq, const void* k_cache, const void* v_cache,
+                            const void* head_idx, int nheads, const void* lengths, int n_len,
+                            int B, int H, int hd, int S, float scale, void* out, int64_t ldo,
+                            void* workspace, size_t workspace_bytes, void* stream) {
+  int rc = check_attn_args(q, ldq, k_cache, v_cache, nheads, n_len, B, H, hd, S);
+  if (rc != DV_OK) return rc;
+  if (!out) return DV_ERR_INVALID_ARG;
+  const int heads = head_idx ? nheads : H;
+  if (heads == 0) return DV_OK;
+  if (!workspace || workspace_bytes < dv_decode_attention_workspace_bytes(B, heads, n_len, hd))
+    return DV_ERR_WORKSPACE;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  float* part = reinterpret_cast<float*>(workspace);
+  rc = launch_attn_partials(q, ldq, k_cache, v_cache, head_idx, heads, lengths, n_len, B, H, hd, S,
+                            scale, part, s);
+  if (rc != DV_OK) return rc;
+  const int nsplit = attn_splits(n_len);
+  const int* hi = reinterpret_cast<const int*>(head_idx);
+  half_t* oo = reinterpret_cast<half_t*>(out);
+  if (hd == 128)
     hipLaunchKernelGGL((decode_attn_combine_kernel<128>), dim3(heads, B), dim3(128), 0, s, part,
                        hi, H, nsplit, oo, ldo);
-  } else {
-    hipLaunchKernelGGL((decode_attn_kernel<64>), grid, dim3(64), 0, s, qq, ldq, kc, vc, hi, ln,
-                       n_len, H, S, scale, nsplit, part);
+  else
     hipLaunchKernelGGL((decode_attn_combine_kernel<64>), dim3(heads, B), dim3(64), 0, s, part, hi,
                        H, nsplit, oo, ldo);
+  return launch_status();
+}
+
+size_t dv_attention_out_proj_workspace_bytes(int B, int nheads, int n_len, int hd, int N) {
+  if (B < 1 || nheads < 0 || n_len < 0 || hd <= 0 || N < 1) return 0;
+  size_t a = dv_decode_attention_workspace_bytes(B, nheads, n_len, hd);
+  a = (a + 255) & ~(size_t)255;
+  return a + cols_workspace_bytes(B, N, nheads * hd);
+}
+
+int dv_attention_out_proj_f16(const void* q, int64_t ldq, const void* k_cache, const void* v_cache,
+                              const void* head_idx, int nheads, const void* lengths, int n_len,
+                              int B, int H, int hd, int S, float scale, const void* Wt, int64_t ldw,
+                              const void* bias, int N, void* y, void* workspace,
+                              size_t workspace_bytes, void* stream) {
+  int rc = check_attn_args(q, ldq, k_cache, v_cache, nheads, n_len, B, H, hd, S);
+  if (rc != DV_OK) return rc;
+  if (!head_idx || !Wt || !y || N <= 0) return DV_ERR_INVALID_ARG;
+  if (B > 4) return DV_ERR_UNSUPPORTED;
+  if (N % 8 || ldw % 8 || ldw < N || !aligned16(Wt)) return DV_ERR_ALIGNMENT;
+  if (!workspace || !aligned16(workspace) ||
+      workspace_bytes < dv_attention_out_proj_workspace_bytes(B, nheads, n_len, hd, N))
+    return DV_ERR_WORKSPACE;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  // layout: [counters + out_proj partial sums][attention partials]
+  const size_t cols_bytes = (cols_workspace_bytes(B, N, nheads * hd) + 255) & ~(size_t)255;
+  unsigned char* base = reinterpret_cast<unsigned char*>(workspace);
+  float* part = reinterpret_cast<float*>(base + cols_bytes);
+  if (nheads > 0) {
+    rc = launch_attn_partials(q, ldq, k_cache, v_cache, head_idx, nheads, lengths, n_len, B, H, hd, S,
+                              scale, part, s);
+    if (rc != DV_OK) return rc;
+  }
+  const int M = nheads * hd;
+  const ColsPlan p = plan_cols(N, M);
+  if (p.col_tiles > kMaxColTiles) return DV_ERR_UNSUPPORTED;
+  unsigned* counters = reinterpret_cast<unsigned*>(base);
+  float* partial = reinterpret_cast<float*>(base + kCounterBytes);
+  const half_t* ww = reinterpret_cast<const half_t*>(Wt);
+  const half_t* bb = reinterpret_cast<const half_t*>(bias);
+  half_t* yy = reinterpret_cast<half_t*>(y);
+  dim3 grid(p.col_tiles, p.groups);
+  const int nsplit = attn_splits(n_len);
+#define DV_AO(BB)                                                                                 \
+  hipLaunchKernelGGL((gather_cols_kernel<BB, 8, false, true, false, true>), grid, dim3(256), 0, s, \
+                     (const half_t*)nullptr, (int64_t)0, 1, ww, ldw, bb, head_idx, hd, N, H * hd, M, \
+                     p.rows_per_block, partial, counters, yy, part, nsplit)
+  switch (B) {
+    case 1: DV_AO(1); break;
+    case 2: DV_AO(2); break;
+    case 3: DV_AO(3); break;
+    default: DV_AO(4); break;
+  }
+#undef DV_AO
+  if (p.groups > 1) {
+    const int64_t total = (int64_t)B * N;
+    hipLaunchKernelGGL(cols_reduce_kernel, dim3((unsigned)((total + 63) / 64)), dim3(256), 0, s,
+                       partial, bb, p.groups, B, N, yy);
   }
   return launch_status();
 }
@@ -507,14 +645,14 @@ int dv_add_layer_norm_f16(const void* h, const void* residual, const void* gamma
                      eps, d, reinterpret_cast<half_t*>(y), reinterpret_cast<half_t*>(residual_out))
   if (d <= 256 * 8 * 1)
     DV_LN(256, 1);
-  else if (d <= 256 * 8 * 2)
-    DV_LN(256, 2);
-  else if (d <= 256 * 8 * 4)
-    DV_LN(256, 4);
-  else if (d <= 256 * 8 * 8)
-    DV_LN(256, 8);
+  else if (d <= 512 * 8 * 1)
+    DV_LN(512, 1);
+  else if (d <= 1024 * 8 * 1)
+    DV_LN(1024, 1);
+  else if (d <= 1024 * 8 * 2)
+    DV_LN(1024, 2);
   else
-    DV_LN(256, 16);
+    DV_LN(1024, 4);
 #undef DV_LN
   return launch_status();
 }

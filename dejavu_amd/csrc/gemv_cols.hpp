@@ -25,12 +25,16 @@ __device__ __forceinline__ float load_agent(const float* p) {
 // BLOCKED == true: row(m) = idx[m / blk] * blk + m % blk (out_proj over
 // W_out^T with blk = head_dim and idx = active heads).
 // x_expanded == 0: X is (B, M), x[b, m];  != 0: X is (B, Z), x[b, row(m)].
-template <int B, int U, bool IDX64, bool BLOCKED, bool FUSED>
+// ATTN (with BLOCKED): the activations are not read from X but merged on the
+// fly from the un-normalised attention partials { max, sum, o[blk] } of
+// decode_attn_kernel (attn_nsplit splits per head), rounded to fp16 as a
+// stored context vector would be.
+template <int B, int U, bool IDX64, bool BLOCKED, bool FUSED, bool ATTN = false>
 __global__ __launch_bounds__(256) void gather_cols_kernel(
     const half_t* __restrict__ X, int64_t ldx, int x_expanded, const half_t* __restrict__ W,
     int64_t ldw, const half_t* __restrict__ bias, const void* __restrict__ idx, int blk, int N,
     int Z, int M, int rows_per_block, float* __restrict__ partial, unsigned* __restrict__ counters,
-    half_t* __restrict__ Y) {
+    half_t* __restrict__ Y, const float* __restrict__ attn_part = nullptr, int attn_nsplit = 0) {
   __shared__ float red[4][B][kColTile];
   __shared__ int s_last;
 
@@ -78,9 +82,45 @@ __global__ __launch_bounds__(256) void gather_cols_kernel(
       rid = ok ? (int)id : 0;
     }
     float xl[B];
+    if (ATTN) {
+      const int nheads = M / blk;
+      const int q = ok ? m / blk : 0, jj = ok ? m - q * blk : 0;
 #pragma unroll
-    for (int b = 0; b < B; ++b)
-      xl[b] = ok ? (float)X[(int64_t)b * ldx + (x_expanded ? (int64_t)rid : (int64_t)m)] : 0.f;
+      for (int b = 0; b < B; ++b) {
+        const float* p = attn_part + ((int64_t)b * nheads + q) * attn_nsplit * (blk + 2);
+        float mx = -INFINITY, num = 0.f, den = 0.f;
+        for (int s0 = 0; s0 < attn_nsplit; s0 += 8) {  // online merge, 8 splits' loads in flight
+          float ms[8], ls[8], os[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            const bool in = s0 + u < attn_nsplit;
+            const float* ps = p + (int64_t)(in ? s0 + u : s0) * (blk + 2);
+            ms[u] = in ? ps[0] : -INFINITY;
+            ls[u] = ps[1];
+            os[u] = ps[2 + jj];
+          }
+          float mc = mx;
+#pragma unroll
+          for (int u = 0; u < 8; ++u) mc = fmaxf(mc, ms[u]);
+          if (mc == -INFINITY) continue;
+          const float rescale = mx == -INFINITY ? 0.f : __expf(mx - mc);
+          num *= rescale;
+          den *= rescale;
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            const float w = ms[u] == -INFINITY ? 0.f : __expf(ms[u] - mc);
+            den += w * ls[u];
+            num += w * os[u];
+          }
+          mx = mc;
+        }
+        xl[b] = ok ? (float)(half_t)(num / den) : 0.f;
+      }
+    } else {
+#pragma unroll
+      for (int b = 0; b < B; ++b)
+        xl[b] = ok ? (float)X[(int64_t)b * ldx + (x_expanded ? (int64_t)rid : (int64_t)m)] : 0.f;
+    }
 
     const int cnt = (m_end - mb) < kWave ? (m_end - mb) : kWave;
     int j = 0;

@@ -29,7 +29,13 @@ __global__ __launch_bounds__(THREADS) void add_layer_norm_kernel(
   __shared__ float scratch[THREADS / kWave];
   const int64_t row = blockIdx.x;
   const int nvec = d / 8;
-  half8_t v[MAXV];
+  half8_t v[MAXV], gm[MAXV], bt[MAXV];
+#pragma unroll
+  for (int j = 0; j < MAXV; ++j) {  // issued early: not needed until the last pass
+    const int i = threadIdx.x + j * THREADS;
+    gm[j] = i < nvec ? load8(gamma + i * 8) : zero8();
+    bt[j] = i < nvec ? load8(beta + i * 8) : zero8();
+  }
   float s = 0.f;
 #pragma unroll
   for (int j = 0; j < MAXV; ++j) {
@@ -66,8 +72,8 @@ __global__ __launch_bounds__(THREADS) void add_layer_norm_kernel(
   for (int j = 0; j < MAXV; ++j) {
     const int i = threadIdx.x + j * THREADS;
     if (i < nvec) {
-      const half8_t g = load8(gamma + i * 8);
-      const half8_t b = load8(beta + i * 8);
+      const half8_t g = gm[j];
+      const half8_t b = bt[j];
       half8_t o;
 #pragma unroll
       for (int e = 0; e < 8; ++e)

@@ -155,4 +155,215 @@ __global__ __launch_bounds__(THREADS) void topk_kernel(const half_t* __restrict_
   }
 }
 
+// ---------------------------------------------------------------------------
+// Small inputs (n <= 1024, e.g. attention heads): rank selection in one
+// workgroup.  Element i is selected iff fewer than k elements beat it, where j
+// beats i when key_j > key_i or (key_j == key_i and j < i); selected indices
+// are written in ascending order.  Same result as topk_kernel.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ void rank_select_emit(const unsigned* s_key, unsigned* s_sel, int n, int k,
+                                                 void* idx_out, int idx_bytes) {
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const unsigned ki = s_key[i];
+    int rank = 0;
+    for (int j = 0; j < n; ++j) {
+      const unsigned kj = s_key[j];
+      rank += (kj > ki) || (kj == ki && j < i);
+    }
+    s_sel[i] = rank < k ? 1u : 0u;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    if (s_sel[i]) {
+      int pos = 0;
+      for (int j = 0; j < i; ++j) pos += (int)s_sel[j];
+      if (idx_bytes == 8)
+        reinterpret_cast<int64_t*>(idx_out)[pos] = i;
+      else
+        reinterpret_cast<int32_t*>(idx_out)[pos] = i;
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void topk_small_kernel(const half_t* __restrict__ logits, int B, int n,
+                                                         int k, void* __restrict__ idx_out,
+                                                         int idx_bytes) {
+  __shared__ unsigned s_key[1024];
+  __shared__ unsigned s_sel[1024];
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    unsigned key = 0u;
+    for (int b = 0; b < B; ++b) {
+      const unsigned kk = topk_key(logits[(int64_t)b * n + i]);
+      key = kk > key ? kk : key;
+    }
+    s_key[i] = key;
+  }
+  __syncthreads();
+  rank_select_emit(s_key, s_sel, n, k, idx_out, idx_bytes);
+}
+
+// ---------------------------------------------------------------------------
+// Large inputs, two launches.
+//  1) topk_hist_kernel (many workgroups): hist[key] += 1 for every column's key
+//     (65536 bins, integer atomics => order-independent, deterministic).
+//  2) topk_select_kernel (one workgroup of 1024): scans the histogram from the
+//     top for the threshold key T (largest T with count(key >= T) >= k), clears
+//     the histogram for the next call, then emits the indices with key > T and
+//     the first k - count(key > T) indices with key == T, ascending, with one
+//     workgroup prefix sum.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void topk_hist_kernel(const half_t* __restrict__ logits, int B, int n,
+                                                        unsigned* __restrict__ hist) {
+  const int i0 = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+  if (i0 >= n) return;
+  unsigned key[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) key[e] = 0u;
+  for (int b = 0; b < B; ++b) {
+    const half8_t v = load8(logits + (int64_t)b * n + i0);  // n % 8 == 0
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const unsigned kk = topk_key(v[e]);
+      key[e] = kk > key[e] ? kk : key[e];
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) atomicAdd(&hist[key[e]], 1u);
+}
+
+template <int ITEMS>
+__global__ __launch_bounds__(1024) void topk_select_kernel(const half_t* __restrict__ logits, int B,
+                                                           int n, int k, unsigned* __restrict__ hist,
+                                                           void* __restrict__ idx_out, int idx_bytes) {
+  constexpr int THREADS = 1024, WAVES = THREADS / kWave, BINS = 65536 / THREADS;
+  __shared__ unsigned s_a[WAVES], s_b[WAVES];
+  __shared__ unsigned s_T, s_above;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+
+  // keys of this thread's columns (issued first, consumed last)
+  const int base = tid * ITEMS;
+  half8_t v[ITEMS / 8];
+#pragma unroll
+  for (int i = 0; i < ITEMS / 8; ++i) {
+    const int off = base + i * 8;
+    v[i] = load8(logits + (off < n ? off : 0));
+  }
+
+  // thread t owns the 64 bins [65536 - 64 (t + 1), 65536 - 64 t): descending key order
+  const int bin_lo = 65536 - BINS * (tid + 1);
+  const uint4* hv = reinterpret_cast<const uint4*>(hist + bin_lo);
+  unsigned mine = 0;
+#pragma unroll
+  for (int j = 0; j < BINS / 4; ++j) {
+    const uint4 c = hv[j];
+    mine += c.x + c.y + c.z + c.w;
+  }
+  // exclusive prefix (over descending keys) of the per-thread totals
+  unsigned inc = mine;
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {
+    const unsigned t2 = __shfl_up(inc, off, kWave);
+    if (lane >= off) inc += t2;
+  }
+  if (lane == kWave - 1) s_a[wave] = inc;
+  __syncthreads();
+  unsigned before = inc - mine;
+#pragma unroll
+  for (int w = 0; w < WAVES; ++w)
+    if (w < wave) before += s_a[w];
+  // the thread whose bins make the running count reach k owns the threshold:
+  // it walks its bins again, from the highest key down
+  if (k > 0 && before < (unsigned)k && before + mine >= (unsigned)k) {
+    unsigned run = before;
+    for (int j = BINS - 1; j >= 0; --j) {
+      const unsigned c = hist[bin_lo + j];
+      if (run < (unsigned)k && run + c >= (unsigned)k) {
+        s_T = (unsigned)(bin_lo + j);
+        s_above = run;  // count(key > T)
+      }
+      run += c;
+    }
+  }
+  __syncthreads();
+  {  // leave the histogram cleared for the next call
+    uint4* hz = reinterpret_cast<uint4*>(hist + bin_lo);
+    const uint4 z = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int j = 0; j < BINS / 4; ++j) hz[j] = z;
+  }
+  const unsigned T = s_T;
+  const unsigned need = (unsigned)k - s_above;
+
+  // B > 1: a column's key is the maximum over the rows
+  unsigned key[ITEMS];
+#pragma unroll
+  for (int i = 0; i < ITEMS / 8; ++i) {
+    const bool in = base + i * 8 < n;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) key[i * 8 + e] = in ? topk_key(v[i][e]) : 0u;
+  }
+  for (int b = 1; b < B; ++b) {
+#pragma unroll
+    for (int i = 0; i < ITEMS / 8; ++i) {
+      const int off = base + i * 8;
+      if (off < n) {
+        const half8_t w = load8(logits + (int64_t)b * n + off);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const unsigned kk = topk_key(w[e]);
+          key[i * 8 + e] = kk > key[i * 8 + e] ? kk : key[i * 8 + e];
+        }
+      }
+    }
+  }
+  unsigned gt = 0, eq = 0;
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    gt += key[i] > T;
+    eq += key[i] == T;
+  }
+  unsigned gt_inc = gt, eq_inc = eq;
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {
+    const unsigned g2 = __shfl_up(gt_inc, off, kWave);
+    const unsigned e2 = __shfl_up(eq_inc, off, kWave);
+    if (lane >= off) {
+      gt_inc += g2;
+      eq_inc += e2;
+    }
+  }
+  if (lane == kWave - 1) {
+    s_a[wave] = gt_inc;
+    s_b[wave] = eq_inc;
+  }
+  __syncthreads();
+  unsigned gt_before = gt_inc - gt, eq_before = eq_inc - eq;
+#pragma unroll
+  for (int w = 0; w < WAVES; ++w) {
+    if (w < wave) {
+      gt_before += s_a[w];
+      eq_before += s_b[w];
+    }
+  }
+  unsigned pos = gt_before + (eq_before < need ? eq_before : need);
+  unsigned eq_rank = eq_before;
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    bool take = key[i] > T;
+    if (key[i] == T) {
+      take = eq_rank < need;
+      ++eq_rank;
+    }
+    if (take) {
+      if (idx_bytes == 8)
+        reinterpret_cast<int64_t*>(idx_out)[pos] = base + i;
+      else
+        reinterpret_cast<int32_t*>(idx_out)[pos] = base + i;
+      ++pos;
+    }
+  }
+}
+
 }  // namespace dv

@@ -27,6 +27,38 @@ from . import ops
 from ._lib import check, lib
 
 
+# Side-stream overlap of predictor / top-k work with the main kernels.  Off = everything
+# is enqueued on the current stream in program order.
+USE_SIDE_STREAM = True
+
+_side_streams: dict = {}
+
+
+def side_stream(device=None) -> "torch.cuda.Stream":
+    """The one side stream (default priority) that all modules on a device share: predictors
+    and top-ks are enqueued on it in program order, so work handed from one module to the
+    next on that stream needs no event."""
+    dev = torch.cuda.current_device() if device is None else torch.device(device).index
+    if dev is None:
+        dev = torch.cuda.current_device()
+    st = _side_streams.get(dev)
+    if st is None:
+        st = torch.cuda.Stream(device=dev)
+        _side_streams[dev] = st
+    return st
+
+
+def join_side_stream() -> None:
+    """Makes the current stream wait for everything enqueued on the side stream so far.
+    Needed once at the end of a forward pass when predictor joins are deferred
+    (``ParallelFusedMLPDejavu.defer_predictor_join``), e.g. before a graph capture ends."""
+    if USE_SIDE_STREAM and _side_streams:
+        ev = torch.cuda.Event(enable_timing=False, blocking=False)
+        st = side_stream()
+        st.record_event(ev)
+        torch.cuda.current_stream().wait_event(ev)
+
+
 def _world_size(process_group) -> int:
     if process_group is None:
         return 1
@@ -106,10 +138,16 @@ class ParallelFusedMLPDejavu(nn.Module):
         self.sp_stream = None
         self.event_mlp = None
         self.event_mlp_sp = None
+        # When True, forward() returns while the predictor is still running on the side
+        # stream; the logits tensor carries its completion event (``_dv_ready``) and the
+        # next layer's attention module, which consumes it on the same side stream, needs
+        # no join.  Whoever reads the logits on another stream must wait for that event
+        # (or call join_side_stream()).  Off by default: forward() joins before returning.
+        self.defer_predictor_join = False
 
     def _streams(self):
         if self.sp_stream is None:
-            self.sp_stream = torch.cuda.Stream()
+            self.sp_stream = side_stream(self.fc1.weight.device)
             self.event_mlp = torch.cuda.Event(enable_timing=False, blocking=False)
             self.event_mlp_sp = torch.cuda.Event(enable_timing=False, blocking=False)
 
@@ -121,6 +159,19 @@ class ParallelFusedMLPDejavu(nn.Module):
         self._streams()
         curr_stream = torch.cuda.current_stream()
         do_token_generation = x.size(1) == 1
+        # The predictor only needs `residual`, so it streams its weights on the side
+        # stream while fc1 / fc2 run (the reference starts it after the MLP, to
+        # overlap the tensor-parallel all-reduce that one GPU does not have).
+        mlp_logit = None
+        side = do_token_generation and USE_SIDE_STREAM
+        if side:
+            curr_stream.record_event(self.event_mlp)
+            with torch.cuda.stream(self.sp_stream):
+                self.sp_stream.wait_event(self.event_mlp)
+                mlp_logit = self.sp(residual)
+                self.sp_stream.record_event(self.event_mlp_sp)
+        elif do_token_generation:
+            mlp_logit = self.sp(residual)
         if idx != None:
             assert x.size(1) == 1
             if self.activation != "relu":
@@ -133,15 +184,12 @@ class ParallelFusedMLPDejavu(nn.Module):
             h = F.linear(x, self.fc1.weight, self.fc1.bias)
             h = F.relu(h) if self.activation == "relu" else F.gelu(h, approximate="tanh")
             out = F.linear(h, self.fc2.weight, self.fc2.bias)
-        curr_stream.record_event(self.event_mlp)
         # (tensor parallel all-reduce of `out` is the identity on one GPU)
-        mlp_logit = None
-        with torch.cuda.stream(self.sp_stream):
-            self.sp_stream.wait_event(self.event_mlp)
-            if do_token_generation:
-                mlp_logit = self.sp(residual)
-            self.sp_stream.record_event(self.event_mlp_sp)
-        curr_stream.wait_event(self.event_mlp_sp)
+        if side:
+            if self.defer_predictor_join:
+                mlp_logit._dv_ready = self.event_mlp_sp
+            else:
+                curr_stream.wait_event(self.event_mlp_sp)
         return out, mlp_logit
 
 
@@ -187,14 +235,13 @@ class _MHABase(nn.Module):
         self.process_group = process_group
         self.mlp_k = None
         self.sp_stream = None
+        self._side_used = False
 
     def _streams(self):
         if self.sp_stream is None:
-            self.sp_stream = torch.cuda.Stream()
-            self.event_qkv = torch.cuda.Event(enable_timing=False, blocking=False)
-            self.event_out = torch.cuda.Event(enable_timing=False, blocking=False)
-            self.event_mlp_sp = torch.cuda.Event(enable_timing=False, blocking=False)
-            self.event_att_sp = torch.cuda.Event(enable_timing=False, blocking=False)
+            self.sp_stream = side_stream(self.Wqkv.weight.device)
+            self.event_in = torch.cuda.Event(enable_timing=False, blocking=False)
+            self.event_side = torch.cuda.Event(enable_timing=False, blocking=False)
 
     def _dense_context(self, qkv, inference_params):
         """qkv: (B, s, 3, H, hd) -> context (B, s, H*hd) for the prompt or a dense decode step."""
@@ -217,15 +264,41 @@ class _MHABase(nn.Module):
                                          self.rotary_emb_dim, softmax_scale=scale)
         return ctx.reshape(B, 1, -1)
 
-    def _mlp_topk(self, mlp_sp_logit, after_event):
-        """MLP top-k for this layer on the side stream, overlapping attention."""
-        mlp_idx = None
-        with torch.cuda.stream(self.sp_stream):
-            self.sp_stream.wait_event(after_event)
-            if mlp_sp_logit != None:
+    def _side_work(self, mlp_sp_logit, residual=None, att_sp=None, att_k=None, att_idx_out=None):
+        """Everything that does not depend on this layer's attention runs on the
+        side stream from the start of the forward: the head predictor + top-k for
+        the next layer (from the residual stream) and the MLP top-k for this layer
+        (from the previous layer's logits).  The caller joins with ``_join_side``
+        before returning."""
+        mlp_idx, att_idx = None, None
+        self._side_used = False
+        if mlp_sp_logit is None and att_sp is None:
+            return mlp_idx, att_idx
+        if not USE_SIDE_STREAM:
+            if att_sp is not None:
+                att_idx = ops.topk_indices(att_sp(residual), att_k, dtype=torch.int32, out=att_idx_out)
+            if mlp_sp_logit is not None:
                 mlp_idx = ops.topk_indices(mlp_sp_logit, self.mlp_k)
-            self.sp_stream.record_event(self.event_mlp_sp)
-        return mlp_idx
+            return mlp_idx, att_idx
+        self._side_used = True
+        torch.cuda.current_stream().record_event(self.event_in)
+        with torch.cuda.stream(self.sp_stream):
+            self.sp_stream.wait_event(self.event_in)
+            # logits handed over with a deferred join were produced on this same side
+            # stream (in order); a foreign producer stream needs its event waited on
+            ready = getattr(mlp_sp_logit, "_dv_ready", None) if mlp_sp_logit is not None else None
+            if ready is not None:
+                self.sp_stream.wait_event(ready)
+            if att_sp is not None:
+                att_idx = ops.topk_indices(att_sp(residual), att_k, dtype=torch.int32, out=att_idx_out)
+            if mlp_sp_logit is not None:
+                mlp_idx = ops.topk_indices(mlp_sp_logit, self.mlp_k)
+            self.sp_stream.record_event(self.event_side)
+        return mlp_idx, att_idx
+
+    def _join_side(self):
+        if self._side_used:
+            torch.cuda.current_stream().wait_event(self.event_side)
 
 
 class ParallelMHADejavu(_MHABase):
@@ -242,14 +315,12 @@ class ParallelMHADejavu(_MHABase):
         """x: (B, s, d).  Returns (out, mlp_idx)."""
         assert seqlen is None, "sequence-parallel input layout is not used for generation"
         self._streams()
-        curr_stream = torch.cuda.current_stream()
+        mlp_idx, _ = self._side_work(mlp_sp_logit)
         qkv = self.Wqkv(x)
-        curr_stream.record_event(self.event_qkv)
-        mlp_idx = self._mlp_topk(mlp_sp_logit, self.event_qkv)
         qkv = qkv.view(x.shape[0], x.shape[1], 3, self.num_heads, self.head_dim)
         context = self._dense_context(qkv, inference_params)
         out = self.out_proj(context)
-        curr_stream.wait_event(self.event_mlp_sp)
+        self._join_side()
         return out, mlp_idx
 
 
@@ -287,8 +358,8 @@ class ParallelMHASparseAttMlp(_MHABase):
                            .repeat(self.num_heads, 1))
 
     def _sparse_decode(self, x, head_idx, inference_params):
-        """x: (1, 1, d).  QKV for the active heads and the window tokens they
-        miss, cache scatter, attention over the active heads, out_proj."""
+        """x: (1, 1, d).  Window step, then QKV for the active heads and the window
+        tokens they miss; the K / V rows go straight into the caches."""
         dev = x.device
         assert x.dtype == torch.float16 and x.is_contiguous()
         H, hd = self.num_heads, self.head_dim
@@ -304,10 +375,17 @@ class ParallelMHASparseAttMlp(_MHABase):
         check(lib.dv_window_step_f16(x.data_ptr(), self.x_cache.data_ptr(), self.embed_dim, self.tracker.data_ptr(),
                                      head_idx.data_ptr(), nnz, H, self.counter, int(flush), batch_idx.data_ptr(),
                                      stream), "dv_window_step_f16")
+        k_cache, v_cache = inference_params.key_value_memory_dict[self.layer_idx]
+        b0 = inference_params.batch_size_offset
+        kc, vc = k_cache[b0:b0 + 1], v_cache[b0:b0 + 1]
+        if self.cache_offset is None:
+            self.cache_offset = torch.tensor([inference_params.sequence_len_offset - self.counter],
+                                             dtype=torch.int32, device=dev)
         qkv = ops.qkv_proj_sparse(self.x_cache[:nb], self.Wqkv.weight.view(3, H, hd, self.embed_dim), head_idx,
-                                  batch_idx, None if self.Wqkv.bias is None else self.Wqkv.bias.view(3, H, hd))
+                                  batch_idx, None if self.Wqkv.bias is None else self.Wqkv.bias.view(3, H, hd),
+                                  k_cache=kc, v_cache=vc, padding=self.cache_offset)
         self.counter += 1
-        return qkv, head_idx, batch_idx
+        return qkv, head_idx, kc, vc
 
     def forward(self, x, residual, head_idx=None, mlp_sp_logit=None, seqlen=None, inference_params=None, **kwargs):
         """x, residual: (B, s, d).  head_idx: (Hk,) int32 heads to compute, or None
@@ -319,48 +397,26 @@ class ParallelMHASparseAttMlp(_MHABase):
         if x.size(1) != 1:  # prompt: remember where the decode window starts
             self.cache_offset = torch.tensor([x.size(1)], dtype=torch.int32, device=x.device)
             self.reset_window()
-        curr_stream = torch.cuda.current_stream()
         sparse = inference_params is not None and inference_params.sequence_len_offset > 0 and head_idx != None
+        mlp_idx, att_idx = self._side_work(mlp_sp_logit, residual, self.sp if do_token_generation else None,
+                                           self.att_k, self.att_idx_out)
         if sparse:
             assert x.size(1) == 1
             assert x.size(0) == 1, "head-sparse decode keeps one back-fill window: batch size 1"
-            qkv, head_idx, batch_idx = self._sparse_decode(x, head_idx, inference_params)
-        else:
-            qkv = self.Wqkv(x)
-        curr_stream.record_event(self.event_qkv)
-        mlp_idx = self._mlp_topk(mlp_sp_logit, self.event_qkv)
-
-        if sparse:
-            k_cache, v_cache = inference_params.key_value_memory_dict[self.layer_idx]
-            b0 = inference_params.batch_size_offset
-            kc, vc = k_cache[b0:b0 + 1], v_cache[b0:b0 + 1]
-            if self.cache_offset is None:
-                self.cache_offset = torch.tensor([inference_params.sequence_len_offset - (self.counter - 1)],
-                                                 dtype=torch.int32, device=x.device)
-            ops.kv_cache_copy_sparse(qkv[:, 1], qkv[:, 2], kc, vc, head_idx, batch_idx, self.cache_offset)
+            qkv, head_idx, kc, vc = self._sparse_decode(x, head_idx, inference_params)
             # the caches now hold the newest token for the active heads
-            ctx = ops.single_query_attention(qkv[-1:, 0], None, None, kc, vc, inference_params.lengths_per_sample,
-                                             inference_params.sequence_len_offset, self.rotary_emb_dim,
-                                             head_idx=head_idx, softmax_scale=self.softmax_scale)
             if self.out_proj_weight_t is None:
                 self.out_proj_weight_t = self.out_proj.weight.t().contiguous()
-            out = ops.out_proj_sparse_t(ctx, self.out_proj_weight_t, head_idx, self.out_proj.bias).unsqueeze(1)
+            out = ops.attention_out_proj(qkv[-1:, 0], kc, vc, head_idx, inference_params.sequence_len_offset,
+                                         self.out_proj_weight_t, self.out_proj.bias,
+                                         inference_params.lengths_per_sample, self.softmax_scale).unsqueeze(1)
             if self.counter == self.WINDOW:  # window complete: start the next one
                 self.counter = 0
                 self.cache_offset += self.WINDOW
         else:
+            qkv = self.Wqkv(x)
             qkv = qkv.view(x.shape[0], x.shape[1], 3, self.num_heads, self.head_dim)
             context = self._dense_context(qkv, inference_params)
             out = self.out_proj(context)
-        curr_stream.record_event(self.event_out)
-
-        att_idx = None
-        with torch.cuda.stream(self.sp_stream):
-            self.sp_stream.wait_event(self.event_out)
-            if do_token_generation:
-                att_sp_logit = self.sp(residual)
-                att_idx = ops.topk_indices(att_sp_logit, self.att_k, dtype=torch.int32, out=self.att_idx_out)
-            self.sp_stream.record_event(self.event_att_sp)
-        curr_stream.wait_event(self.event_mlp_sp)
-        curr_stream.wait_event(self.event_att_sp)
+        self._join_side()
         return out, mlp_idx, att_idx

@@ -94,8 +94,22 @@ def predictor_logits(x: torch.Tensor, fc0_weight: torch.Tensor, fc1_weight: torc
     return logits
 
 
+_topk_workspaces: dict = {}
+
+
+def _topk_workspace(device: torch.device) -> torch.Tensor:
+    """Zero-initialised 65536-bin histogram per device; the kernels hand it back zeroed.
+    Top-k calls that share it must not overlap."""
+    key = (device.type, device.index)
+    ws = _topk_workspaces.get(key)
+    if ws is None:
+        ws = torch.zeros(65536, dtype=torch.int32, device=device)
+        _topk_workspaces[key] = ws
+    return ws
+
+
 def topk_indices(logits: torch.Tensor, k: int, dtype: torch.dtype = torch.int64,
-                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                 out: Optional[torch.Tensor] = None, single_launch: bool = False) -> torch.Tensor:
     """Indices of the k largest logits (ties to the lower index), ascending.
 
     logits: (n,) or (B, n) fp16; for B > 1 a column is ranked by its maximum
@@ -114,7 +128,12 @@ def topk_indices(logits: torch.Tensor, k: int, dtype: torch.dtype = torch.int64,
         out = torch.empty(k, device=lg.device, dtype=dtype)
     else:
         assert out.shape == (k,) and out.is_contiguous()
-    check(lib.dv_topk_f16(_ptr(lg), B, n, k, _ptr(out), _idx_bytes(out), _stream()), "dv_topk_f16")
+    if single_launch or (n > 1024 and n % 8 != 0):
+        check(lib.dv_topk_search_f16(_ptr(lg), B, n, k, _ptr(out), _idx_bytes(out), _stream()), "dv_topk_search_f16")
+        return out
+    ws = _topk_workspace(lg.device) if n > 1024 else None
+    check(lib.dv_topk_f16(_ptr(lg), B, n, k, _ptr(out), _idx_bytes(out), _ptr(ws), 0 if ws is None else ws.numel() * 4,
+                          _stream()), "dv_topk_f16")
     return out
 
 
@@ -200,7 +219,9 @@ def mlp_sparse(x, W1, W2t, idx, bias1=None, bias2=None):
 # head-sparse attention
 # ---------------------------------------------------------------------------
 def qkv_proj_sparse(x: torch.Tensor, weight: torch.Tensor, head_idx: torch.Tensor, batch_idx: torch.Tensor,
-                    bias: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    bias: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+                    k_cache: Optional[torch.Tensor] = None, v_cache: Optional[torch.Tensor] = None,
+                    padding: Optional[torch.Tensor] = None) -> torch.Tensor:
     """
     Compute y = torch.einsum("bm,thdm->bthd", x, weight), but only for the active heads in @head_idx
     and only for the batch indices in @batch_idx. Negative indices in batch_idx will be ignored.
@@ -209,6 +230,9 @@ def qkv_proj_sparse(x: torch.Tensor, weight: torch.Tensor, head_idx: torch.Tenso
     :param head_idx: int32, (nnz,)
     :param batch_idx: int32, (nnz, batch_size). Negative indices are ignored.
     :param bias: indices, (3, nheads, head_dim)
+    :param k_cache, v_cache, padding: optional; when given, the computed K / V rows are also scattered
+        into the caches exactly as ``k_cache_copy_sparse`` / ``v_cache_copy_sparse`` would with
+        ``seqlen_idx = batch_idx`` (one launch instead of three)
     :return: result tensor, (batch_size, 3, nheads, head_dim); entries of inactive heads /
         skipped rows are uninitialised (or keep the content of ``out`` when it is given)
     """
@@ -240,9 +264,20 @@ def qkv_proj_sparse(x: torch.Tensor, weight: torch.Tensor, head_idx: torch.Tenso
         out = torch.empty(batch_size, 3, nheads, head_dim, device=x.device, dtype=x.dtype)
     else:
         assert out.shape == (batch_size, 3, nheads, head_dim) and out.is_contiguous() and out.dtype == x.dtype
-    check(lib.dv_qkv_proj_sparse_f16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(head_idx), _ptr(batch_idx), batch_size,
-                                     hidden_dim, nheads, head_dim, n_active, _ptr(out), _stream()),
-          "dv_qkv_proj_sparse_f16")
+    S = 0
+    if k_cache is not None:
+        assert v_cache is not None
+        _require_device(k_cache, v_cache, padding)
+        S = v_cache.shape[2]
+        assert v_cache.shape == (1, nheads, S, head_dim) and k_cache.shape == (1, nheads, head_dim // 8, S, 8)
+        assert k_cache.is_contiguous() and v_cache.is_contiguous()
+        assert k_cache.dtype == x.dtype and v_cache.dtype == x.dtype
+        if padding is not None:
+            assert padding.shape == (1,) and padding.dtype == torch.int32
+    check(lib.dv_qkv_proj_sparse_cache_f16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(head_idx), _ptr(batch_idx),
+                                           batch_size, hidden_dim, nheads, head_dim, n_active, _ptr(out),
+                                           _ptr(k_cache), _ptr(v_cache), _ptr(padding), S, _stream()),
+          "dv_qkv_proj_sparse_cache_f16")
     return out
 
 
@@ -465,3 +500,42 @@ def add_layer_norm(hidden: torch.Tensor, residual: Optional[torch.Tensor], weigh
     check(lib.dv_add_layer_norm_f16(_ptr(hidden), _ptr(residual), _ptr(weight.contiguous()), _ptr(bias.contiguous()),
                                     float(eps), rows, d, _ptr(y), _ptr(r_out), _stream()), "dv_add_layer_norm_f16")
     return y, r_out
+
+
+def attention_out_proj(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, head_idx: torch.Tensor,
+                       timestep: int, weight_t: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                       lengths_per_sample: Optional[torch.Tensor] = None,
+                       softmax_scale: Optional[float] = None) -> torch.Tensor:
+    """``out_proj_sparse_t(single_query_attention(q, ...), weight_t, head_idx, bias)`` in two launches,
+    without writing the context vector: the out_proj kernel merges the attention splits itself.
+
+    q: (B, H, hd); caches already hold the newest token; weight_t: (H*hd, d).  Returns (B, d).
+    """
+    _require_device(q, k_cache, v_cache, head_idx, weight_t, bias, lengths_per_sample)
+    B, H, hd = q.shape
+    S = v_cache.shape[2]
+    rows, N = weight_t.shape
+    assert rows == H * hd and head_idx.dtype == torch.int32 and B in [1, 2, 3, 4]
+    assert q.dtype == k_cache.dtype == v_cache.dtype == weight_t.dtype == torch.float16
+    assert v_cache.shape == (B, H, S, hd) and k_cache.shape == (B, H, hd // 8, S, 8)
+    assert k_cache.is_contiguous() and v_cache.is_contiguous() and q.stride(2) == 1 and q.stride(1) == hd
+    assert 0 <= timestep < S
+    if weight_t.stride(1) != 1:
+        weight_t = weight_t.contiguous()
+    head_idx = head_idx.contiguous()
+    nheads = head_idx.shape[0]
+    if bias is not None:
+        bias = bias.contiguous()
+        assert bias.shape == (N,)
+    if lengths_per_sample is not None:
+        assert lengths_per_sample.dtype == torch.int32 and lengths_per_sample.shape == (B,)
+    n_len = S if lengths_per_sample is not None else timestep + 1
+    scale = float(hd ** -0.5 if softmax_scale is None else softmax_scale)
+    out = torch.empty(B, N, device=q.device, dtype=q.dtype)
+    nbytes = lib.dv_attention_out_proj_workspace_bytes(B, nheads, n_len, hd, N)
+    ws = _workspace(q.device, nbytes)
+    check(lib.dv_attention_out_proj_f16(_ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(head_idx), nheads,
+                                        _ptr(lengths_per_sample), n_len, B, H, hd, S, scale, _ptr(weight_t),
+                                        weight_t.stride(0), _ptr(bias), N, _ptr(out), _ptr(ws), ws.numel(),
+                                        _stream()), "dv_attention_out_proj_f16")
+    return out

@@ -66,9 +66,19 @@ DV_API int dv_predictor_logits_f16(const void* x, const void* Wa, int64_t ldwa, 
  * B rows.  Replaces Tensor.topk(k, sorted=False) at
  * Dejavu/src/models/modules/mha_dejavu.py:1069, 1369, 1506-1507.
  *   logits (B, n) fp16; idx_out (k,) int32/int64.  n <= 65536, 0 <= k <= n.
+ * dv_topk_f16: n <= 1024 is ranked in one workgroup; larger n (n % 8 == 0)
+ *   builds a 65536-bin key histogram with many workgroups, then one workgroup
+ *   reads the threshold off it.  workspace: dv_topk_workspace_bytes(n) bytes,
+ *   zero-filled before first use (the call leaves it zeroed); calls sharing it
+ *   must not overlap.
+ * dv_topk_search_f16: same result in a single launch without scratch memory
+ *   (16-step bitwise threshold search in one workgroup).
  */
+DV_API size_t dv_topk_workspace_bytes(int n);
 DV_API int dv_topk_f16(const void* logits, int B, int n, int k, void* idx_out, int idx_bytes,
-                void* stream);
+                       void* workspace, size_t workspace_bytes, void* stream);
+DV_API int dv_topk_search_f16(const void* logits, int B, int n, int k, void* idx_out,
+                              int idx_bytes, void* stream);
 
 /*
  * y = act(x . W[idx]^T + bias[idx]).  Replaces gather_gemv,
@@ -108,6 +118,19 @@ DV_API int dv_gather_transposed_gemv_f16(const void* x, const void* W, int64_t l
 DV_API int dv_qkv_proj_sparse_f16(const void* x, const void* W, const void* bias,
                                   const void* head_idx, const void* batch_idx, int nb, int d,
                                   int H, int hd, int nnz, void* y, void* stream);
+
+/*
+ * dv_qkv_proj_sparse_f16 with the cache scatter of dv_kv_cache_copy_sparse_f16
+ * fused into its epilogue: K and V rows are also written to
+ * k_cache[0, h, :, token + padding[0], :] / v_cache[0, h, token + padding[0], :].
+ * (qkv_proj_sparse followed by k_cache_copy_sparse + v_cache_copy_sparse with
+ * seqlen_idx = batch_idx, Dejavu/src/models/modules/mha_dejavu.py:1333-1352, 1425-1438.)
+ *   k_cache (1, H, hd/8, S, 8), v_cache (1, H, S, hd): both or neither NULL.
+ */
+DV_API int dv_qkv_proj_sparse_cache_f16(const void* x, const void* W, const void* bias,
+                                        const void* head_idx, const void* batch_idx, int nb, int d,
+                                        int H, int hd, int nnz, void* y, void* k_cache,
+                                        void* v_cache, const void* padding, int S, void* stream);
 
 /*
  * Scatter of (re)computed keys / values into the caches:
@@ -168,6 +191,23 @@ DV_API int dv_decode_attention_f16(const void* q, int64_t ldq, const void* k_cac
                                    const void* lengths, int n_len, int B, int H, int hd, int S,
                                    float scale, void* out, int64_t ldo, void* workspace,
                                    size_t workspace_bytes, void* stream);
+
+/*
+ * dv_decode_attention_f16 followed by dv_out_proj_sparse_t_f16 without
+ * materialising the context: the out_proj kernel merges the attention split
+ * partials while it loads its activations.  Same arithmetic (the merged
+ * context is rounded to fp16 as a stored one would be).
+ *   head_idx (nheads,) int32, required; Wt (H*hd, N) row stride ldw; y (B, N);
+ *   B <= 4; workspace: dv_attention_out_proj_workspace_bytes(...) bytes whose
+ *   first 4 KiB are zero before first use.
+ */
+DV_API size_t dv_attention_out_proj_workspace_bytes(int B, int nheads, int n_len, int hd, int N);
+DV_API int dv_attention_out_proj_f16(const void* q, int64_t ldq, const void* k_cache,
+                                     const void* v_cache, const void* head_idx, int nheads,
+                                     const void* lengths, int n_len, int B, int H, int hd, int S,
+                                     float scale, const void* Wt, int64_t ldw, const void* bias,
+                                     int N, void* y, void* workspace, size_t workspace_bytes,
+                                     void* stream);
 
 /*
  * y[b, n] = sum_{h in head_idx} x[b, h, :] . W[n, h, :] + bias[n], weight in

@@ -204,3 +204,45 @@ def test_single_query_attention_lengths_per_sample(ops):
     want = O.single_query_attention(q.numpy(), k.numpy(), v.numpy(), kn, vn, 159, lengths_per_sample=lengths.numpy())
     assert_close(np16(out), want, "attention with lengths")
     assert np.array_equal(np16(kcd), kn) and np.array_equal(np16(vcd), vn)
+
+
+def test_fused_qkv_cache_and_attention_out_proj_match_separate_ops(ops):
+    """The fused entry points (QKV + cache scatter; attention + out_proj without a
+    stored context) must reproduce the separate operators."""
+    from dejavu_amd.workloads import pack_k_cache
+
+    g = torch.Generator().manual_seed(6)
+    H, hd, d, S, nb, nnz = 12, 128, 1024, 300, 5, 4
+    x = randh(g, nb, d)
+    W = randh(g, 3, H, hd, d, std=0.03)
+    bias = randh(g, 3, H, hd, std=0.1)
+    head_idx = torch.sort(torch.randperm(H, generator=g)[:nnz]).values.int()
+    batch_idx = torch.stack([torch.arange(nb) for _ in range(nnz)]).int()
+    batch_idx[torch.rand(nnz, nb, generator=g) < 0.4] = -1
+    batch_idx[:, -1] = nb - 1  # newest token always live
+    padding = torch.tensor([S - nb], dtype=torch.int32)
+    kc0 = pack_k_cache(randh(g, 1, H, S, hd))
+    vc0 = randh(g, 1, H, S, hd)
+    print("case fused qkv+cache / attention+out_proj", flush=True)
+    # separate
+    kc_a, vc_a = kc0.cuda(), vc0.cuda()
+    qkv_a = torch.zeros(nb, 3, H, hd, dtype=torch.float16, device="cuda")
+    ops.qkv_proj_sparse(x.cuda(), W.cuda(), head_idx.cuda(), batch_idx.cuda(), bias.cuda(), out=qkv_a)
+    ops.kv_cache_copy_sparse(qkv_a[:, 1], qkv_a[:, 2], kc_a, vc_a, head_idx.cuda(), batch_idx.cuda(), padding.cuda())
+    ctx = ops.single_query_attention(qkv_a[-1:, 0], None, None, kc_a, vc_a, None, S - 1, head_idx=head_idx.cuda())
+    Wt = randh(g, H * hd, d, std=0.03).cuda()
+    bo = randh(g, d, std=0.1).cuda()
+    out_a = ops.out_proj_sparse_t(ctx, Wt, head_idx.cuda(), bo)
+    # fused
+    kc_b, vc_b = kc0.cuda(), vc0.cuda()
+    qkv_b = torch.zeros(nb, 3, H, hd, dtype=torch.float16, device="cuda")
+    ops.qkv_proj_sparse(x.cuda(), W.cuda(), head_idx.cuda(), batch_idx.cuda(), bias.cuda(), out=qkv_b,
+                        k_cache=kc_b, v_cache=vc_b, padding=padding.cuda())
+    out_b = ops.attention_out_proj(qkv_b[-1:, 0], kc_b, vc_b, head_idx.cuda(), S - 1, Wt, bo)
+    torch.cuda.synchronize()
+    assert torch.equal(qkv_a, qkv_b) and torch.equal(kc_a, kc_b) and torch.equal(vc_a, vc_b)
+    assert torch.equal(out_a, out_b), "fused attention+out_proj must be bit-identical to the separate ops"
+    want_ctx = O.single_query_attention(np16(qkv_a)[-1:, 0], np16(qkv_a)[-1:, 1], np16(qkv_a)[-1:, 2], kc0.numpy().copy()
+                                        if False else np16(kc_a).copy(), np16(vc_a).copy(), S - 1, head_idx=head_idx.numpy())
+    want = O.out_proj_sparse(want_ctx, np16(Wt).T.reshape(d, H, hd), head_idx.numpy(), np16(bo))
+    assert_close(np16(out_b), want, "fused vs oracle")

@@ -84,18 +84,27 @@ def test_topk_random_and_ties(ops, n):
     for name, x in cases.items():
         for k in sorted({0, 1, n // 3, n - 1, n}):
             print(f"case topk n={n} {name} k={k}", flush=True)
+            want = O.topk_lower_index(x, k)
             for dt in (torch.int64, torch.int32):
                 got = ops.topk_indices(torch.from_numpy(x).cuda(), k, dtype=dt)
                 torch.cuda.synchronize()
-                assert np.array_equal(np16(got).astype(np.int64), O.topk_lower_index(x, k)), (name, k)
+                assert np.array_equal(np16(got).astype(np.int64), want), (name, k)
+            got = ops.topk_indices(torch.from_numpy(x).cuda(), k, single_launch=True)
+            torch.cuda.synchronize()
+            assert np.array_equal(np16(got), want), ("single launch", name, k)
 
 
 def test_topk_batched_scores(ops):
     g = np.random.default_rng(3)
     L = (g.standard_normal((8, 16384)) * 4).astype(np.float16)
-    got = ops.topk_indices(torch.from_numpy(L).cuda(), 4096)
+    for single in (False, True):
+        got = ops.topk_indices(torch.from_numpy(L).cuda(), 4096, single_launch=single)
+        torch.cuda.synchronize()
+        assert np.array_equal(np16(got), O.topk_lower_index(L, 4096))
+    Ls = L[:3, :96].copy()
+    got = ops.topk_indices(torch.from_numpy(Ls).cuda(), 32, dtype=torch.int32)
     torch.cuda.synchronize()
-    assert np.array_equal(np16(got), O.topk_lower_index(L, 4096))
+    assert np.array_equal(np16(got).astype(np.int64), O.topk_lower_index(Ls, 32))
 
 
 # ----------------------------------------------------------------- sparse MLP
