@@ -8,6 +8,7 @@
 
 #include "attention.hpp"
 #include "common.hpp"
+#include "gemm_mfma.hpp"
 #include "gemv_cols.hpp"
 #include "gemv_rows.hpp"
 #include "norm.hpp"
@@ -193,6 +194,104 @@ int gather_cols(const half_t* x, int64_t ldx, int x_expanded, const half_t* W, i
   return launch_status();
 }
 
+// ---- batched gathered GEMMs on the matrix cores (5 <= B <= 64) -------------------
+template <int BT, bool IDX64, bool RELU>
+int launch_rows_mfma(const half_t* x, const half_t* W, int64_t ldw, const half_t* bias, const void* idx,
+                     int B, int N, int Z, int M, half_t* y, hipStream_t s) {
+  auto kern = gather_rows_mfma_kernel<BT, IDX64, RELU>;
+  const size_t lds = (size_t)4 * 32 * kMfmaLdsRow * sizeof(half_t);
+  static bool granted = false;
+  if (!granted) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return DV_ERR_UNSUPPORTED;
+    granted = true;
+  }
+  const int ntasks = (M + 31) / 32;
+  int blocks = (ntasks + 3) / 4;
+  const int cap = compute_units() * 2;
+  if (blocks > cap) blocks = cap;
+  if (blocks < 1) blocks = 1;
+  hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), lds, s, x, W, bias, idx, B, N, ldw, Z, M, y);
+  return launch_status();
+}
+
+int gather_rows_mfma(const half_t* x, const half_t* W, int64_t ldw, const half_t* bias, const void* idx,
+                     int idx_bytes, int B, int N, int Z, int M, int act, half_t* y, hipStream_t s) {
+  const bool relu = act == DV_ACT_RELU, i64 = idx_bytes == 8;
+#define DV_RM(BT)                                                                              \
+  (relu ? (i64 ? launch_rows_mfma<BT, true, true>(x, W, ldw, bias, idx, B, N, Z, M, y, s)        \
+               : launch_rows_mfma<BT, false, true>(x, W, ldw, bias, idx, B, N, Z, M, y, s))      \
+        : (i64 ? launch_rows_mfma<BT, true, false>(x, W, ldw, bias, idx, B, N, Z, M, y, s)       \
+               : launch_rows_mfma<BT, false, false>(x, W, ldw, bias, idx, B, N, Z, M, y, s)))
+  if (B <= 32) return DV_RM(1);
+  return DV_RM(2);
+#undef DV_RM
+}
+
+struct ColsMfmaPlan {
+  int col_tiles, groups, rows_per_block;
+};
+
+ColsMfmaPlan plan_cols_mfma(int N, int M) {
+  ColsMfmaPlan p;
+  p.col_tiles = (N + kMfmaColTile - 1) / kMfmaColTile;
+  const int target_blocks = compute_units() * 3;
+  int groups = (target_blocks + p.col_tiles - 1) / p.col_tiles;
+  const int max_groups = M > 32 ? (M + 31) / 32 : 1;
+  if (groups > max_groups) groups = max_groups;
+  if (groups < 1) groups = 1;
+  int rpb = (M + groups - 1) / groups;
+  rpb = (rpb + 31) & ~31;
+  if (rpb < 32) rpb = 32;
+  p.rows_per_block = rpb;
+  p.groups = M > 0 ? (M + rpb - 1) / rpb : 1;
+  return p;
+}
+
+size_t cols_mfma_workspace_bytes(int B, int N, int M) {
+  const ColsMfmaPlan p = plan_cols_mfma(N, M);
+  return kCounterBytes + (size_t)p.groups * B * N * sizeof(float);
+}
+
+template <int BT, bool IDX64, bool BLOCKED>
+void launch_cols_mfma(const ColsMfmaPlan& p, const half_t* h, int64_t ldh, int x_expanded, const half_t* W,
+                      int64_t ldw, const half_t* bias, const void* idx, int blk, int B, int N, int Z, int M,
+                      float* partial, half_t* y, hipStream_t s) {
+  hipLaunchKernelGGL((gather_cols_mfma_kernel<BT, IDX64, BLOCKED>), dim3(p.col_tiles, p.groups), dim3(256), 0,
+                     s, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M, p.rows_per_block, partial, y);
+  if (p.groups > 1) {
+    const int64_t total = (int64_t)B * N;
+    hipLaunchKernelGGL(cols_reduce_kernel, dim3((unsigned)((total + 63) / 64)), dim3(256), 0, s, partial,
+                       bias, p.groups, B, N, y);
+  }
+}
+
+int gather_cols_mfma(const half_t* h, int64_t ldh, int x_expanded, const half_t* W, int64_t ldw,
+                     const half_t* bias, const void* idx, int idx_bytes, int blk, int B, int N, int Z, int M,
+                     half_t* y, void* workspace, size_t workspace_bytes, hipStream_t s) {
+  const ColsMfmaPlan p = plan_cols_mfma(N, M);
+  if (workspace == nullptr || workspace_bytes < cols_mfma_workspace_bytes(B, N, M)) return DV_ERR_WORKSPACE;
+  float* partial = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(workspace) + kCounterBytes);
+  const bool i64 = idx_bytes == 8, blocked = blk != 1;
+#define DV_CM(BT)                                                                                        \
+  do {                                                                                                   \
+    if (blocked) {                                                                                       \
+      if (i64) launch_cols_mfma<BT, true, true>(p, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M, partial, y, s);   \
+      else launch_cols_mfma<BT, false, true>(p, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M, partial, y, s);      \
+    } else {                                                                                             \
+      if (i64) launch_cols_mfma<BT, true, false>(p, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M, partial, y, s);  \
+      else launch_cols_mfma<BT, false, false>(p, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M, partial, y, s);     \
+    }                                                                                                    \
+  } while (0)
+  if (B <= 32)
+    DV_CM(1);
+  else
+    DV_CM(2);
+#undef DV_CM
+  return launch_status();
+}
+
 // ---- head-sparse attention ---------------------------------------------------
 template <int NBMAX>
 int launch_qkv(const half_t* x, const half_t* W, const half_t* bias, const int* head_idx,
@@ -252,7 +351,11 @@ int dv_predictor_logits_f16(const void* x, const void* Wa, int64_t ldwa, const v
                         reinterpret_cast<half_t*>(logits), s);
 }
 
-size_t dv_topk_workspace_bytes(int n) { return n > 1024 ? 65536 * sizeof(unsigned) : 0; }
+size_t dv_topk_workspace_bytes(int n) {
+  if (n <= 1024) return 0;
+  const int blocks = (n + kTopkItemsPerBlock - 1) / kTopkItemsPerBlock;
+  return (size_t)(kTopkCountsOff + 2 * blocks) * sizeof(unsigned);
+}
 
 int dv_topk_f16(const void* logits, int B, int n, int k, void* idx_out, int idx_bytes,
                 void* workspace, size_t workspace_bytes, void* stream) {
@@ -270,25 +373,11 @@ int dv_topk_f16(const void* logits, int B, int n, int k, void* idx_out, int idx_
   if (!aligned16(logits)) return DV_ERR_ALIGNMENT;
   if (!workspace || workspace_bytes < dv_topk_workspace_bytes(n) || !aligned16(workspace))
     return DV_ERR_WORKSPACE;
-  unsigned* hist = reinterpret_cast<unsigned*>(workspace);
-  hipLaunchKernelGGL(topk_hist_kernel, dim3((n / 8 + 255) / 256), dim3(256), 0, s, lg, B, n, hist);
-#define DV_SEL(I) \
-  hipLaunchKernelGGL((topk_select_kernel<I>), dim3(1), dim3(1024), 0, s, lg, B, n, k, hist, idx_out, idx_bytes)
-  if (n <= 1024 * 8)
-    DV_SEL(8);
-  else if (n <= 1024 * 16)
-    DV_SEL(16);
-  else if (n <= 1024 * 24)
-    DV_SEL(24);
-  else if (n <= 1024 * 32)
-    DV_SEL(32);
-  else if (n <= 1024 * 40)
-    DV_SEL(40);
-  else if (n <= 1024 * 48)
-    DV_SEL(48);
-  else
-    DV_SEL(64);
-#undef DV_SEL
+  unsigned* ws = reinterpret_cast<unsigned*>(workspace);
+  const int blocks = (n + kTopkItemsPerBlock - 1) / kTopkItemsPerBlock;
+  hipLaunchKernelGGL(topk_hist_kernel, dim3(blocks), dim3(256), 0, s, lg, B, n, ws);
+  hipLaunchKernelGGL(topk_count_kernel, dim3(blocks), dim3(256), 0, s, lg, B, n, k, ws);
+  hipLaunchKernelGGL(topk_emit_kernel, dim3(blocks), dim3(256), 0, s, lg, B, n, ws, idx_out, idx_bytes);
   return launch_status();
 }
 
@@ -341,7 +430,7 @@ int dv_gather_gemv_f16(const void* x, const void* W, int64_t ldw, const void* bi
   if (!x || !W || N <= 0 || Z <= 0 || M < 0 || !idx_ok(idx_bytes) || (M > 0 && (!idx || !y)) ||
       (act != DV_ACT_ID && act != DV_ACT_RELU))
     return DV_ERR_INVALID_ARG;
-  if (B < 1 || B > 4) return DV_ERR_UNSUPPORTED;
+  if (B < 1 || B > 64) return DV_ERR_UNSUPPORTED;
   if (N % 8 || ldw % 8 || ldw < N || !aligned16(x) || !aligned16(W)) return DV_ERR_ALIGNMENT;
   if (M == 0) return DV_OK;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
@@ -349,6 +438,7 @@ int dv_gather_gemv_f16(const void* x, const void* W, int64_t ldw, const void* bi
   const half_t* ww = reinterpret_cast<const half_t*>(W);
   const half_t* bb = reinterpret_cast<const half_t*>(bias);
   half_t* yy = reinterpret_cast<half_t*>(y);
+  if (B > 4) return gather_rows_mfma(xx, ww, ldw, bb, idx, idx_bytes, B, N, Z, M, act, yy, s);
   switch (B) {
     case 1: return gather_rows_b<1>(xx, ww, ldw, bb, idx, idx_bytes, N, Z, M, act, yy, s);
     case 2: return gather_rows_b<2>(xx, ww, ldw, bb, idx, idx_bytes, N, Z, M, act, yy, s);
@@ -359,7 +449,7 @@ int dv_gather_gemv_f16(const void* x, const void* W, int64_t ldw, const void* bi
 
 size_t dv_gather_transposed_gemv_workspace_bytes(int B, int N, int M) {
   if (B < 1 || N < 1 || M < 0) return 0;
-  return cols_workspace_bytes(B, N, M);
+  return B > 4 ? cols_mfma_workspace_bytes(B, N, M) : cols_workspace_bytes(B, N, M);
 }
 
 int dv_gather_transposed_gemv_f16(const void* x, const void* W, int64_t ldw, const void* bias,
@@ -368,8 +458,13 @@ int dv_gather_transposed_gemv_f16(const void* x, const void* W, int64_t ldw, con
                                   void* stream) {
   if (!W || !y || N <= 0 || Z <= 0 || M < 0 || !idx_ok(idx_bytes) || (M > 0 && (!idx || !x)))
     return DV_ERR_INVALID_ARG;
-  if (B < 1 || B > 4) return DV_ERR_UNSUPPORTED;
+  if (B < 1 || B > 64) return DV_ERR_UNSUPPORTED;
   if (N % 8 || ldw % 8 || ldw < N || !aligned16(W)) return DV_ERR_ALIGNMENT;
+  if (B > 4)
+    return gather_cols_mfma(reinterpret_cast<const half_t*>(x), M, 0, reinterpret_cast<const half_t*>(W),
+                            ldw, reinterpret_cast<const half_t*>(bias), idx, idx_bytes, 1, B, N, Z, M,
+                            reinterpret_cast<half_t*>(y), workspace, workspace_bytes,
+                            reinterpret_cast<hipStream_t>(stream));
   return gather_cols(reinterpret_cast<const half_t*>(x), M, 0, reinterpret_cast<const half_t*>(W),
                      ldw, reinterpret_cast<const half_t*>(bias), idx, idx_bytes, 1, B, N, Z, M,
                      reinterpret_cast<half_t*>(y), workspace, workspace_bytes,
@@ -613,7 +708,7 @@ int dv_out_proj_sparse_f16(const void* x, const void* W, const void* bias, const
 
 size_t dv_out_proj_sparse_t_workspace_bytes(int B, int N, int nnz, int hd) {
   if (B < 1 || N < 1 || nnz < 0 || hd < 1) return 0;
-  return cols_workspace_bytes(B, N, nnz * hd);
+  return B > 4 ? cols_mfma_workspace_bytes(B, N, nnz * hd) : cols_workspace_bytes(B, N, nnz * hd);
 }
 
 int dv_out_proj_sparse_t_f16(const void* x, const void* Wt, int64_t ldw, const void* bias,
@@ -621,8 +716,13 @@ int dv_out_proj_sparse_t_f16(const void* x, const void* Wt, int64_t ldw, const v
                              void* workspace, size_t workspace_bytes, void* stream) {
   if (!x || !Wt || !y || nnz < 0 || B < 1 || H <= 0 || hd <= 0 || N <= 0 || (nnz > 0 && !head_idx))
     return DV_ERR_INVALID_ARG;
-  if (B > 4) return DV_ERR_UNSUPPORTED;
+  if (B > 64) return DV_ERR_UNSUPPORTED;
   if (N % 8 || ldw % 8 || ldw < N || !aligned16(Wt)) return DV_ERR_ALIGNMENT;
+  if (B > 4)
+    return gather_cols_mfma(reinterpret_cast<const half_t*>(x), (int64_t)H * hd, 1,
+                            reinterpret_cast<const half_t*>(Wt), ldw, reinterpret_cast<const half_t*>(bias),
+                            head_idx, 4, hd, B, N, H * hd, nnz * hd, reinterpret_cast<half_t*>(y), workspace,
+                            workspace_bytes, reinterpret_cast<hipStream_t>(stream));
   return gather_cols(reinterpret_cast<const half_t*>(x), (int64_t)H * hd, 1,
                      reinterpret_cast<const half_t*>(Wt), ldw, reinterpret_cast<const half_t*>(bias),
                      head_idx, 4, hd, B, N, H * hd, nnz * hd, reinterpret_cast<half_t*>(y),

@@ -1,0 +1,228 @@
+// Batched (5 <= B <= 64) gathered GEMMs on the matrix cores.  The gathered weight
+// rows are streamed with coalesced 128-bit loads into LDS and read back in the
+// operand layout of v_mfma_f32_32x32x16_f16; the batch is padded to tiles of 32.
+//
+// Operand layout of the 32x32x16 fp16 MFMA (64 lanes): lane l holds, for the A
+// operand, 8 consecutive-k values of row (l % 32), k-group (l / 32); for the B
+// operand 8 k values of column (l % 32), same k-group; the 32x32 fp32 result has
+// 16 values per lane: value v is row 8*(v/4) + 4*(l/32) + (v%4), column l % 32.
+#pragma once
+#include "common.hpp"
+
+namespace dv {
+
+__device__ __forceinline__ float16_t mfma_32x32x16(half8_t a, half8_t b, float16_t c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+
+// ---------------------------------------------------------------------------
+// fc1: Y[b, m] = act( sum_n X[b, n] * W[idx[m], n] + bias[idx[m]] ), fp16 out.
+// A wavefront owns 32 gathered rows; per K-chunk of KC = 256 columns it copies
+// its 32 x 256 weight tile to its private LDS region (2 rows per load
+// instruction, 512 contiguous bytes each), then issues KC/16 MFMAs per batch
+// tile with the rows as the A operand and X^T as the B operand.
+// N % 8 == 0, ldw % 8 == 0.  BT = batch tiles of 32 (B <= 32 * BT).
+// ---------------------------------------------------------------------------
+constexpr int kMfmaKC = 256;            // columns per staged chunk
+constexpr int kMfmaRowPad = 8;          // halfs of padding per LDS row (bank spread)
+constexpr int kMfmaLdsRow = kMfmaKC + kMfmaRowPad;
+
+template <int BT, bool IDX64, bool RELU>
+__global__ __launch_bounds__(256) void gather_rows_mfma_kernel(
+    const half_t* __restrict__ X, const half_t* __restrict__ W, const half_t* __restrict__ bias,
+    const void* __restrict__ idx, int B, int N, int64_t ldw, int Z, int M, half_t* __restrict__ Y) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  half_t* tile = reinterpret_cast<half_t*>(smem_raw) + (size_t)wave * 32 * kMfmaLdsRow;
+  const int waves_per_block = blockDim.x >> 6;
+  const int ntasks = (M + 31) / 32;
+  const int half_id = lane >> 5;  // which of the two rows a load instruction covers / k-group
+  const int l32 = lane & 31;
+
+  for (int t = blockIdx.x * waves_per_block + wave; t < ntasks; t += gridDim.x * waves_per_block) {
+    // row id of output row (t*32 + l32), shared by lanes l32 and l32 + 32
+    const int m_mine = t * 32 + l32;
+    int64_t id = -1;
+    if (m_mine < M)
+      id = IDX64 ? reinterpret_cast<const int64_t*>(idx)[m_mine]
+                 : (int64_t) reinterpret_cast<const int32_t*>(idx)[m_mine];
+    const bool ok_mine = id >= 0 && id < Z;
+    const int rid_mine = ok_mine ? (int)id : 0;
+
+    float16_t acc[BT];
+#pragma unroll
+    for (int bt = 0; bt < BT; ++bt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[bt][v] = 0.f;
+
+    for (int k0 = 0; k0 < N; k0 += kMfmaKC) {
+      // stage 32 rows x KC columns: instruction r2 covers rows 2*r2 + half_id
+      half8_t stage[16];
+      const int col = k0 + l32 * 8;
+#pragma unroll
+      for (int r2 = 0; r2 < 16; ++r2) {
+        const int row = 2 * r2 + half_id;
+        const int rid = __shfl(rid_mine, row, kWave);
+        const bool ok = __shfl((int)ok_mine, row, kWave) != 0;
+        stage[r2] = (ok && col < N) ? load8_stream(W + (int64_t)rid * ldw + col) : zero8();
+      }
+#pragma unroll
+      for (int r2 = 0; r2 < 16; ++r2)
+        store8(tile + (2 * r2 + half_id) * kMfmaLdsRow + l32 * 8, stage[r2]);
+      // the tile is private to this wavefront, whose LDS accesses complete in order: a
+      // wavefront-scope fence (compiler ordering only) is all the synchronisation needed
+      __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int ks = 0; ks < kMfmaKC / 16; ++ks) {
+        const int kk = k0 + ks * 16 + half_id * 8;
+        const half8_t a = load8(tile + l32 * kMfmaLdsRow + ks * 16 + half_id * 8);
+#pragma unroll
+        for (int bt = 0; bt < BT; ++bt) {
+          const int b = bt * 32 + l32;
+          const half8_t xb = (b < B && kk < N) ? load8(X + (int64_t)b * N + kk) : zero8();
+          acc[bt] = mfma_32x32x16(a, xb, acc[bt]);
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");  // reads done before the tile is overwritten
+      __builtin_amdgcn_wave_barrier();
+    }
+    // epilogue: value v of lane l is row 8*(v/4) + 4*half_id + v%4, batch column bt*32 + l32
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int row = 8 * (v / 4) + 4 * half_id + (v % 4);
+      const int m = t * 32 + row;
+      const int rid = __shfl(rid_mine, row, kWave);
+      const bool ok = __shfl((int)ok_mine, row, kWave) != 0;
+      const float bv = (bias != nullptr && ok) ? (float)bias[rid] : 0.f;
+#pragma unroll
+      for (int bt = 0; bt < BT; ++bt) {
+        const int b = bt * 32 + l32;
+        float val = acc[bt][v] + bv;
+        if (RELU) val = relu_f(val);
+        if (!ok) val = 0.f;
+        if (m < M && b < B) Y[(int64_t)b * M + m] = (half_t)val;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// fc2 / out_proj over a transposed weight: Y[b, n] = sum_m H[b, m] * W[row(m), n].
+// The contraction index m runs over gathered ROWS, so the weight tile must be
+// transposed on its way to the MFMA: a workgroup copies 32 gathered rows x 512
+// columns into LDS (one full 1 KiB row segment per wavefront load), then every
+// wavefront reads, for its four 32-column sub-tiles, the A operand W^T (n x m)
+// with 16-bit LDS reads, and multiplies by H^T (m x b) loaded straight from
+// memory.  Partial sums over the row groups (gridDim.y) go to `partial`
+// [(g * B + b) * N + n] and are reduced by cols_reduce_kernel; with one group
+// the result (+ bias) is written directly.
+// Row mapping as gather_cols_kernel: BLOCKED ? idx[m / blk] * blk + m % blk : idx[m];
+// x_expanded: H is (B, Z) indexed by row(m) instead of (B, M) indexed by m.
+// ---------------------------------------------------------------------------
+constexpr int kMfmaColTile = 512;
+constexpr int kMfmaColLdsRow = kMfmaColTile + 8;
+
+template <int BT, bool IDX64, bool BLOCKED>
+__global__ __launch_bounds__(256) void gather_cols_mfma_kernel(
+    const half_t* __restrict__ H, int64_t ldh, int x_expanded, const half_t* __restrict__ W,
+    int64_t ldw, const half_t* __restrict__ bias, const void* __restrict__ idx, int blk, int B, int N,
+    int Z, int M, int rows_per_block, float* __restrict__ partial, half_t* __restrict__ Y) {
+  __shared__ __attribute__((aligned(16))) half_t tile[32 * kMfmaColLdsRow];
+  __shared__ int s_rid[32];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int half_id = lane >> 5, l32 = lane & 31;
+  const int ct = blockIdx.x, g = blockIdx.y, G = gridDim.y;
+  const int col0 = ct * kMfmaColTile;
+  const int m_begin = g * rows_per_block;
+  int m_end = m_begin + rows_per_block;
+  if (m_end > M) m_end = M;
+
+  float16_t acc[4][BT];
+#pragma unroll
+  for (int s = 0; s < 4; ++s)
+#pragma unroll
+    for (int bt = 0; bt < BT; ++bt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[s][bt][v] = 0.f;
+
+  for (int mb = m_begin; mb < m_end; mb += 32) {
+    __syncthreads();  // previous tile fully consumed
+    if (tid < 32) {
+      const int m = mb + tid;
+      int64_t id = -1;
+      if (m < m_end) {
+        if (BLOCKED) {
+          const int q = m / blk;
+          const int64_t h = IDX64 ? reinterpret_cast<const int64_t*>(idx)[q]
+                                  : (int64_t) reinterpret_cast<const int32_t*>(idx)[q];
+          id = (h >= 0 && h < Z / blk) ? h * blk + (m - q * blk) : -1;
+        } else {
+          id = IDX64 ? reinterpret_cast<const int64_t*>(idx)[m]
+                     : (int64_t) reinterpret_cast<const int32_t*>(idx)[m];
+        }
+      }
+      s_rid[tid] = (id >= 0 && id < Z) ? (int)id : -1;
+    }
+    __syncthreads();
+    // wavefront w copies rows w, w+4, ..: one 1 KiB row segment per load instruction
+    half8_t stage[8];
+    const int col = col0 + lane * 8;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const int rid = s_rid[wave + 4 * r];
+      stage[r] = (rid >= 0 && col < N) ? load8_stream(W + (int64_t)rid * ldw + col) : zero8();
+    }
+#pragma unroll
+    for (int r = 0; r < 8; ++r) store8(tile + (wave + 4 * r) * kMfmaColLdsRow + lane * 8, stage[r]);
+    __syncthreads();
+    // two K = 16 steps over the 32 staged rows
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      const int mk = ks * 16 + half_id * 8;  // first of this lane's 8 staged rows
+      half8_t hb[BT];
+#pragma unroll
+      for (int bt = 0; bt < BT; ++bt) {
+        const int b = bt * 32 + l32;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int rid = s_rid[mk + j];
+          const int m = mb + mk + j;
+          hb[bt][j] = (b < B && rid >= 0) ? H[(int64_t)b * ldh + (x_expanded ? (int64_t)rid : (int64_t)m)]
+                                         : (half_t)0.f;
+        }
+      }
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const int n_local = (wave * 4 + s) * 32 + l32;  // this lane's column inside the tile
+        half8_t a;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) a[j] = tile[(mk + j) * kMfmaColLdsRow + n_local];
+#pragma unroll
+        for (int bt = 0; bt < BT; ++bt) acc[s][bt] = mfma_32x32x16(a, hb[bt], acc[s][bt]);
+      }
+    }
+  }
+  // result rows are columns n of the tile, result columns are batch entries
+#pragma unroll
+  for (int s = 0; s < 4; ++s)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int n = col0 + (wave * 4 + s) * 32 + 8 * (v / 4) + 4 * half_id + (v % 4);
+#pragma unroll
+      for (int bt = 0; bt < BT; ++bt) {
+        const int b = bt * 32 + l32;
+        if (n < N && b < B) {
+          if (G == 1)
+            Y[(int64_t)b * N + n] = (half_t)(acc[s][bt][v] + (bias ? (float)bias[n] : 0.f));
+          else
+            partial[((int64_t)g * B + b) * N + n] = acc[s][bt][v];
+        }
+      }
+    }
+}
+
+}  // namespace dv

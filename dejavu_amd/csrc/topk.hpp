@@ -203,22 +203,29 @@ __global__ __launch_bounds__(256) void topk_small_kernel(const half_t* __restric
 }
 
 // ---------------------------------------------------------------------------
-// Large inputs, two launches.
-//  1) topk_hist_kernel (many workgroups): hist[key] += 1 for every column's key
-//     (65536 bins, integer atomics => order-independent, deterministic).
-//  2) topk_select_kernel (one workgroup of 1024): scans the histogram from the
-//     top for the threshold key T (largest T with count(key >= T) >= k), clears
-//     the histogram for the next call, then emits the indices with key > T and
-//     the first k - count(key > T) indices with key == T, ascending, with one
-//     workgroup prefix sum.
+// Large inputs: three launches, every one spread over many workgroups.
+//  1) topk_hist_kernel: fine[key] += 1 (65536 bins) and coarse[key >> 8] += 1
+//     (256 bins) for every column's key.  Integer atomics: order-independent.
+//  2) topk_count_kernel: every workgroup reads the threshold key T (largest T
+//     with count(key >= T) >= k) off the two histograms -- 256 coarse bins, then
+//     the 256 fine bins of the crossing coarse bin -- and counts its own columns
+//     above / at T.  Workgroup 0 also publishes T and the number of ties to take.
+//  3) topk_emit_kernel: every workgroup sums the counts of the workgroups before
+//     it, emits its indices with key > T and those of the first `need` columns
+//     with key == T (ascending, exact positions), and clears its slice of the
+//     histograms for the next call.
+// Workspace layout (u32): fine[65536] coarse[256] meta[2] = {T, need} counts[2*WG].
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void topk_hist_kernel(const half_t* __restrict__ logits, int B, int n,
-                                                        unsigned* __restrict__ hist) {
-  const int i0 = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
-  if (i0 >= n) return;
-  unsigned key[8];
+constexpr int kTopkItemsPerBlock = 256 * 8;
+constexpr int kTopkFine = 65536, kTopkCoarse = 256;
+constexpr int kTopkMetaOff = kTopkFine + kTopkCoarse;
+constexpr int kTopkCountsOff = kTopkMetaOff + 2;
+
+__device__ __forceinline__ void topk_load_keys(const half_t* __restrict__ logits, int B, int n, int i0,
+                                               unsigned key[8]) {
 #pragma unroll
   for (int e = 0; e < 8; ++e) key[e] = 0u;
+  if (i0 >= n) return;
   for (int b = 0; b < B; ++b) {
     const half8_t v = load8(logits + (int64_t)b * n + i0);  // n % 8 == 0
 #pragma unroll
@@ -227,143 +234,151 @@ __global__ __launch_bounds__(256) void topk_hist_kernel(const half_t* __restrict
       key[e] = kk > key[e] ? kk : key[e];
     }
   }
-#pragma unroll
-  for (int e = 0; e < 8; ++e) atomicAdd(&hist[key[e]], 1u);
 }
 
-template <int ITEMS>
-__global__ __launch_bounds__(1024) void topk_select_kernel(const half_t* __restrict__ logits, int B,
-                                                           int n, int k, unsigned* __restrict__ hist,
-                                                           void* __restrict__ idx_out, int idx_bytes) {
-  constexpr int THREADS = 1024, WAVES = THREADS / kWave, BINS = 65536 / THREADS;
-  __shared__ unsigned s_a[WAVES], s_b[WAVES];
-  __shared__ unsigned s_T, s_above;
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-
-  // keys of this thread's columns (issued first, consumed last)
-  const int base = tid * ITEMS;
-  half8_t v[ITEMS / 8];
+__global__ __launch_bounds__(256) void topk_hist_kernel(const half_t* __restrict__ logits, int B, int n,
+                                                        unsigned* __restrict__ ws) {
+  // the 256 coarse bins are hot (most logits share a few exponents): aggregate them in
+  // LDS and add each non-empty bin to memory once per workgroup
+  __shared__ unsigned s_coarse[kTopkCoarse];
+  s_coarse[threadIdx.x] = 0u;
+  __syncthreads();
+  const int i0 = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+  if (i0 < n) {
+    unsigned key[8];
+    topk_load_keys(logits, B, n, i0, key);
 #pragma unroll
-  for (int i = 0; i < ITEMS / 8; ++i) {
-    const int off = base + i * 8;
-    v[i] = load8(logits + (off < n ? off : 0));
+    for (int e = 0; e < 8; ++e) {
+      atomicAdd(&ws[key[e]], 1u);
+      atomicAdd(&s_coarse[key[e] >> 8], 1u);
+    }
   }
+  __syncthreads();
+  const unsigned c = s_coarse[threadIdx.x];
+  if (c != 0u) atomicAdd(&ws[kTopkFine + threadIdx.x], c);
+}
 
-  // thread t owns the 64 bins [65536 - 64 (t + 1), 65536 - 64 t): descending key order
-  const int bin_lo = 65536 - BINS * (tid + 1);
-  const uint4* hv = reinterpret_cast<const uint4*>(hist + bin_lo);
-  unsigned mine = 0;
-#pragma unroll
-  for (int j = 0; j < BINS / 4; ++j) {
-    const uint4 c = hv[j];
-    mine += c.x + c.y + c.z + c.w;
-  }
-  // exclusive prefix (over descending keys) of the per-thread totals
-  unsigned inc = mine;
+// Inclusive prefix sum over the 256 threads of a workgroup (s_w: 4 words of LDS).
+__device__ __forceinline__ unsigned block256_inclusive_scan(unsigned v, unsigned* s_w) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
   for (int off = 1; off < kWave; off <<= 1) {
-    const unsigned t2 = __shfl_up(inc, off, kWave);
-    if (lane >= off) inc += t2;
+    const unsigned t = __shfl_up(v, off, kWave);
+    if (lane >= off) v += t;
   }
-  if (lane == kWave - 1) s_a[wave] = inc;
+  __syncthreads();  // s_w may still be read from a previous scan
+  if (lane == kWave - 1) s_w[wave] = v;
   __syncthreads();
-  unsigned before = inc - mine;
-#pragma unroll
-  for (int w = 0; w < WAVES; ++w)
-    if (w < wave) before += s_a[w];
-  // the thread whose bins make the running count reach k owns the threshold:
-  // it walks its bins again, from the highest key down
-  if (k > 0 && before < (unsigned)k && before + mine >= (unsigned)k) {
-    unsigned run = before;
-    for (int j = BINS - 1; j >= 0; --j) {
-      const unsigned c = hist[bin_lo + j];
-      if (run < (unsigned)k && run + c >= (unsigned)k) {
-        s_T = (unsigned)(bin_lo + j);
-        s_above = run;  // count(key > T)
-      }
-      run += c;
-    }
-  }
-  __syncthreads();
-  {  // leave the histogram cleared for the next call
-    uint4* hz = reinterpret_cast<uint4*>(hist + bin_lo);
-    const uint4 z = {0u, 0u, 0u, 0u};
-#pragma unroll
-    for (int j = 0; j < BINS / 4; ++j) hz[j] = z;
-  }
-  const unsigned T = s_T;
-  const unsigned need = (unsigned)k - s_above;
+  for (int w = 0; w < wave; ++w) v += s_w[w];
+  return v;
+}
 
-  // B > 1: a column's key is the maximum over the rows
-  unsigned key[ITEMS];
-#pragma unroll
-  for (int i = 0; i < ITEMS / 8; ++i) {
-    const bool in = base + i * 8 < n;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) key[i * 8 + e] = in ? topk_key(v[i][e]) : 0u;
+// Threshold from the histograms; all 256 threads return the same (T, above).
+__device__ __forceinline__ void topk_find_threshold(const unsigned* __restrict__ ws, unsigned k,
+                                                    unsigned* s_w, unsigned* s_pair, unsigned& T,
+                                                    unsigned& above) {
+  const int t = threadIdx.x;
+  // coarse bins in descending key order: thread t owns bin 255 - t
+  const unsigned c = ws[kTopkFine + 255 - t];
+  const unsigned cinc = block256_inclusive_scan(c, s_w);
+  if (cinc - c < k && cinc >= k) {
+    s_pair[0] = 255u - t;  // crossing coarse bin
+    s_pair[1] = cinc - c;  // columns in higher coarse bins
   }
-  for (int b = 1; b < B; ++b) {
+  __syncthreads();
+  const unsigned cstar = s_pair[0], above_c = s_pair[1];
+  const unsigned f = ws[cstar * 256 + 255 - t];
+  const unsigned finc = block256_inclusive_scan(f, s_w);
+  const unsigned k2 = k - above_c;
+  if (finc - f < k2 && finc >= k2) {
+    s_pair[2] = cstar * 256 + 255 - t;
+    s_pair[3] = above_c + finc - f;
+  }
+  __syncthreads();
+  T = s_pair[2];
+  above = s_pair[3];
+}
+
+__global__ __launch_bounds__(256) void topk_count_kernel(const half_t* __restrict__ logits, int B, int n,
+                                                         int k, unsigned* __restrict__ ws) {
+  __shared__ unsigned s_w[4], s_pair[4], s_gt[4], s_eq[4];
+  unsigned key[8];
+  const int i0 = (blockIdx.x * 256 + threadIdx.x) * 8;
+  topk_load_keys(logits, B, n, i0, key);  // issued before the histogram reads
+  unsigned T, above;
+  topk_find_threshold(ws, (unsigned)k, s_w, s_pair, T, above);
+  unsigned gt = 0, eq = 0;
 #pragma unroll
-    for (int i = 0; i < ITEMS / 8; ++i) {
-      const int off = base + i * 8;
-      if (off < n) {
-        const half8_t w = load8(logits + (int64_t)b * n + off);
+  for (int e = 0; e < 8; ++e) {
+    gt += key[e] > T;
+    eq += key[e] == T;
+  }
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const unsigned kk = topk_key(w[e]);
-          key[i * 8 + e] = kk > key[i * 8 + e] ? kk : key[i * 8 + e];
-        }
-      }
+  for (int off = kWave / 2; off >= 1; off >>= 1) {
+    gt += __shfl_xor(gt, off, kWave);
+    eq += __shfl_xor(eq, off, kWave);
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) {
+    s_gt[wave] = gt;
+    s_eq[wave] = eq;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    ws[kTopkCountsOff + 2 * blockIdx.x] = s_gt[0] + s_gt[1] + s_gt[2] + s_gt[3];
+    ws[kTopkCountsOff + 2 * blockIdx.x + 1] = s_eq[0] + s_eq[1] + s_eq[2] + s_eq[3];
+    if (blockIdx.x == 0) {
+      ws[kTopkMetaOff] = T;
+      ws[kTopkMetaOff + 1] = (unsigned)k - above;  // ties to take, lowest index first
     }
+  }
+}
+
+__global__ __launch_bounds__(256) void topk_emit_kernel(const half_t* __restrict__ logits, int B, int n,
+                                                        unsigned* __restrict__ ws,
+                                                        void* __restrict__ idx_out, int idx_bytes) {
+  __shared__ unsigned s_w[4], s_base[2];
+  unsigned key[8];
+  const int i0 = (blockIdx.x * 256 + threadIdx.x) * 8;
+  topk_load_keys(logits, B, n, i0, key);
+  const unsigned T = ws[kTopkMetaOff], need = ws[kTopkMetaOff + 1];
+  // columns above / at T in the workgroups before this one
+  if (threadIdx.x < 2) {
+    unsigned acc = 0;
+    for (int w = 0; w < (int)blockIdx.x; ++w) acc += ws[kTopkCountsOff + 2 * w + threadIdx.x];
+    s_base[threadIdx.x] = acc;
   }
   unsigned gt = 0, eq = 0;
 #pragma unroll
-  for (int i = 0; i < ITEMS; ++i) {
-    gt += key[i] > T;
-    eq += key[i] == T;
+  for (int e = 0; e < 8; ++e) {
+    gt += key[e] > T;
+    eq += key[e] == T;
   }
-  unsigned gt_inc = gt, eq_inc = eq;
-#pragma unroll
-  for (int off = 1; off < kWave; off <<= 1) {
-    const unsigned g2 = __shfl_up(gt_inc, off, kWave);
-    const unsigned e2 = __shfl_up(eq_inc, off, kWave);
-    if (lane >= off) {
-      gt_inc += g2;
-      eq_inc += e2;
-    }
-  }
-  if (lane == kWave - 1) {
-    s_a[wave] = gt_inc;
-    s_b[wave] = eq_inc;
-  }
+  const unsigned gt_inc = block256_inclusive_scan(gt, s_w);
+  const unsigned eq_inc = block256_inclusive_scan(eq, s_w);
   __syncthreads();
-  unsigned gt_before = gt_inc - gt, eq_before = eq_inc - eq;
-#pragma unroll
-  for (int w = 0; w < WAVES; ++w) {
-    if (w < wave) {
-      gt_before += s_a[w];
-      eq_before += s_b[w];
-    }
-  }
+  const unsigned gt_before = s_base[0] + gt_inc - gt;
+  const unsigned eq_before = s_base[1] + eq_inc - eq;
   unsigned pos = gt_before + (eq_before < need ? eq_before : need);
   unsigned eq_rank = eq_before;
 #pragma unroll
-  for (int i = 0; i < ITEMS; ++i) {
-    bool take = key[i] > T;
-    if (key[i] == T) {
+  for (int e = 0; e < 8; ++e) {
+    bool take = key[e] > T;
+    if (key[e] == T) {
       take = eq_rank < need;
       ++eq_rank;
     }
     if (take) {
       if (idx_bytes == 8)
-        reinterpret_cast<int64_t*>(idx_out)[pos] = base + i;
+        reinterpret_cast<int64_t*>(idx_out)[pos] = i0 + e;
       else
-        reinterpret_cast<int32_t*>(idx_out)[pos] = base + i;
+        reinterpret_cast<int32_t*>(idx_out)[pos] = i0 + e;
       ++pos;
     }
   }
+  // clear the histograms for the next call (nobody reads them in this kernel)
+  const int nthreads = gridDim.x * 256;
+  for (int j = blockIdx.x * 256 + threadIdx.x; j < kTopkFine + kTopkCoarse; j += nthreads) ws[j] = 0u;
 }
 
 }  // namespace dv

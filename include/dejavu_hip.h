@@ -67,10 +67,11 @@ DV_API int dv_predictor_logits_f16(const void* x, const void* Wa, int64_t ldwa, 
  * Dejavu/src/models/modules/mha_dejavu.py:1069, 1369, 1506-1507.
  *   logits (B, n) fp16; idx_out (k,) int32/int64.  n <= 65536, 0 <= k <= n.
  * dv_topk_f16: n <= 1024 is ranked in one workgroup; larger n (n % 8 == 0)
- *   builds a 65536-bin key histogram with many workgroups, then one workgroup
- *   reads the threshold off it.  workspace: dv_topk_workspace_bytes(n) bytes,
- *   zero-filled before first use (the call leaves it zeroed); calls sharing it
- *   must not overlap.
+ *   takes three launches spread over many workgroups: key histograms, the
+ *   threshold read off them plus per-workgroup counts, then the ordered
+ *   emission.  workspace: dv_topk_workspace_bytes(n) bytes, zero-filled before
+ *   first use (the call leaves the histograms zeroed); calls sharing it must
+ *   not overlap.
  * dv_topk_search_f16: same result in a single launch without scratch memory
  *   (16-step bitwise threshold search in one workgroup).
  */
@@ -84,7 +85,9 @@ DV_API int dv_topk_search_f16(const void* logits, int B, int n, int k, void* idx
  * y = act(x . W[idx]^T + bias[idx]).  Replaces gather_gemv,
  * Dejavu/src/ops/triton/gather_gemv.py:198-254.
  *   x (B, N); W (Z, N) row stride ldw; bias (Z,) or NULL; idx (M,);
- *   y (B, M) fp16.  1 <= B <= 4 (the reference's own limit).
+ *   y (B, M) fp16.  1 <= B <= 64: B <= 4 (the reference's own limit) runs as a
+ *   bandwidth-bound GEMV on the vector ALUs; 5 <= B <= 64 stages the gathered
+ *   rows through LDS into 32x32x16 fp16 MFMA tiles.
  */
 DV_API int dv_gather_gemv_f16(const void* x, const void* W, int64_t ldw, const void* bias,
                        const void* idx, int idx_bytes, int B, int N, int Z, int M, int act,
@@ -95,7 +98,7 @@ DV_API int dv_gather_gemv_f16(const void* x, const void* W, int64_t ldw, const v
  * Dejavu/src/ops/triton/gather_gemv.py:572-644 (deterministic: fixed-order
  * split over row groups instead of floating-point atomics).
  *   x (B, M); W (Z, N) row stride ldw; bias (N,) or NULL; idx (M,);
- *   y (B, N) fp16.  1 <= B <= 4.
+ *   y (B, N) fp16.  1 <= B <= 64 (vector ALUs up to 4, MFMA tiles above).
  *   workspace: dv_gather_transposed_gemv_workspace_bytes(B, N, M) bytes,
  *   zero-filled before its first use; calls sharing it must not overlap.
  */
