@@ -199,7 +199,7 @@ template <int BT, bool IDX64, bool RELU>
 int launch_rows_mfma(const half_t* x, const half_t* W, int64_t ldw, const half_t* bias, const void* idx,
                      int B, int N, int Z, int M, half_t* y, hipStream_t s) {
   auto kern = gather_rows_mfma_kernel<BT, IDX64, RELU>;
-  const size_t lds = (size_t)4 * 32 * kMfmaLdsRow * sizeof(half_t);
+  const size_t lds = (size_t)kMfmaWaves * 2 * kMfmaRows * kMfmaLdsRow * sizeof(half_t);
   static bool granted = false;
   if (!granted) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -207,12 +207,11 @@ int launch_rows_mfma(const half_t* x, const half_t* W, int64_t ldw, const half_t
       return DV_ERR_UNSUPPORTED;
     granted = true;
   }
-  const int ntasks = (M + 31) / 32;
-  int blocks = (ntasks + 3) / 4;
-  const int cap = compute_units() * 2;
+  int blocks = (M + kMfmaRows - 1) / kMfmaRows;
+  const int cap = compute_units() * 4;
   if (blocks > cap) blocks = cap;
   if (blocks < 1) blocks = 1;
-  hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), lds, s, x, W, bias, idx, B, N, ldw, Z, M, y);
+  hipLaunchKernelGGL(kern, dim3(blocks), dim3(kMfmaWaves * 64), lds, s, x, W, bias, idx, B, N, ldw, Z, M, y);
   return launch_status();
 }
 
@@ -224,8 +223,9 @@ int gather_rows_mfma(const half_t* x, const half_t* W, int64_t ldw, const half_t
                : launch_rows_mfma<BT, false, true>(x, W, ldw, bias, idx, B, N, Z, M, y, s))      \
         : (i64 ? launch_rows_mfma<BT, true, false>(x, W, ldw, bias, idx, B, N, Z, M, y, s)       \
                : launch_rows_mfma<BT, false, false>(x, W, ldw, bias, idx, B, N, Z, M, y, s)))
-  if (B <= 32) return DV_RM(1);
-  return DV_RM(2);
+  if (B <= 16) return DV_RM(1);
+  if (B <= 32) return DV_RM(2);
+  return DV_RM(4);
 #undef DV_RM
 }
 
@@ -233,10 +233,11 @@ struct ColsMfmaPlan {
   int col_tiles, groups, rows_per_block;
 };
 
-ColsMfmaPlan plan_cols_mfma(int N, int M) {
+ColsMfmaPlan plan_cols_mfma(int B, int N, int M) {
   ColsMfmaPlan p;
   p.col_tiles = (N + kMfmaColTile - 1) / kMfmaColTile;
-  const int target_blocks = compute_units() * 3;
+  // every row group writes a (B, N) fp32 partial: fewer, longer groups as the batch grows
+  const int target_blocks = compute_units() * (B <= 8 ? 3 : (B <= 16 ? 2 : 1));
   int groups = (target_blocks + p.col_tiles - 1) / p.col_tiles;
   const int max_groups = M > 32 ? (M + 31) / 32 : 1;
   if (groups > max_groups) groups = max_groups;
@@ -250,7 +251,7 @@ ColsMfmaPlan plan_cols_mfma(int N, int M) {
 }
 
 size_t cols_mfma_workspace_bytes(int B, int N, int M) {
-  const ColsMfmaPlan p = plan_cols_mfma(N, M);
+  const ColsMfmaPlan p = plan_cols_mfma(B, N, M);
   return kCounterBytes + (size_t)p.groups * B * N * sizeof(float);
 }
 
@@ -270,7 +271,7 @@ void launch_cols_mfma(const ColsMfmaPlan& p, const half_t* h, int64_t ldh, int x
 int gather_cols_mfma(const half_t* h, int64_t ldh, int x_expanded, const half_t* W, int64_t ldw,
                      const half_t* bias, const void* idx, int idx_bytes, int blk, int B, int N, int Z, int M,
                      half_t* y, void* workspace, size_t workspace_bytes, hipStream_t s) {
-  const ColsMfmaPlan p = plan_cols_mfma(N, M);
+  const ColsMfmaPlan p = plan_cols_mfma(B, N, M);
   if (workspace == nullptr || workspace_bytes < cols_mfma_workspace_bytes(B, N, M)) return DV_ERR_WORKSPACE;
   float* partial = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(workspace) + kCounterBytes);
   const bool i64 = idx_bytes == 8, blocked = blk != 1;

@@ -15,34 +15,44 @@ __device__ __forceinline__ float16_t mfma_32x32x16(half8_t a, half8_t b, float16
   return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
 }
 
+__device__ __forceinline__ float4_t mfma_16x16x32(half8_t a, half8_t b, float4_t c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+
 // ---------------------------------------------------------------------------
 // fc1: Y[b, m] = act( sum_n X[b, n] * W[idx[m], n] + bias[idx[m]] ), fp16 out.
-// A wavefront owns 32 gathered rows; per K-chunk of KC = 256 columns it copies
-// its 32 x 256 weight tile to its private LDS region (2 rows per load
-// instruction, 512 contiguous bytes each), then issues KC/16 MFMAs per batch
-// tile with the rows as the A operand and X^T as the B operand.
-// N % 8 == 0, ldw % 8 == 0.  BT = batch tiles of 32 (B <= 32 * BT).
+// A workgroup of 8 wavefronts owns 16 gathered rows and splits the N columns
+// into chunks of KC = 256: wavefront w takes chunks w, w + 8, ...  Per chunk it
+// copies its 16 x 256 weight tile to a private LDS region with coalesced loads
+// (2 rows per instruction, 512 contiguous bytes each), then issues KC/32
+// v_mfma_f32_16x16x32_f16 per batch tile of 16, rows as the A operand
+// (lane: row l % 16, k-group l / 16, 8 consecutive k) and X^T as the B operand
+// (lane: batch column l % 16, same k-group).  Result layout: value v of lane l
+// is row 4 * (l / 16) + v, column l % 16.  The 8 partial tiles are summed
+// through LDS in wavefront order.  N % 8 == 0, ldw % 8 == 0, B <= 16 * BT.
 // ---------------------------------------------------------------------------
 constexpr int kMfmaKC = 256;            // columns per staged chunk
 constexpr int kMfmaRowPad = 8;          // halfs of padding per LDS row (bank spread)
 constexpr int kMfmaLdsRow = kMfmaKC + kMfmaRowPad;
+constexpr int kMfmaWaves = 8;
+constexpr int kMfmaRows = 16;
 
 template <int BT, bool IDX64, bool RELU>
-__global__ __launch_bounds__(256) void gather_rows_mfma_kernel(
+__global__ __launch_bounds__(kMfmaWaves * 64) void gather_rows_mfma_kernel(
     const half_t* __restrict__ X, const half_t* __restrict__ W, const half_t* __restrict__ bias,
     const void* __restrict__ idx, int B, int N, int64_t ldw, int Z, int M, half_t* __restrict__ Y) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  half_t* tile = reinterpret_cast<half_t*>(smem_raw) + (size_t)wave * 32 * kMfmaLdsRow;
-  const int waves_per_block = blockDim.x >> 6;
-  const int ntasks = (M + 31) / 32;
-  const int half_id = lane >> 5;  // which of the two rows a load instruction covers / k-group
-  const int l32 = lane & 31;
+  half_t* tile = reinterpret_cast<half_t*>(smem_raw) + (size_t)wave * 2 * kMfmaRows * kMfmaLdsRow;
+  float* red = reinterpret_cast<float*>(smem_raw);  // reused after the main loop
+  const int l16 = lane & 15, kg = lane >> 4;  // MFMA operand coordinates
+  const int l32 = lane & 31, half_id = lane >> 5;  // staging coordinates
+  const int nchunks = (N + kMfmaKC - 1) / kMfmaKC;
 
-  for (int t = blockIdx.x * waves_per_block + wave; t < ntasks; t += gridDim.x * waves_per_block) {
-    // row id of output row (t*32 + l32), shared by lanes l32 and l32 + 32
-    const int m_mine = t * 32 + l32;
+  for (int t = blockIdx.x; t * kMfmaRows < M; t += gridDim.x) {
+    // row id of output row (t*16 + l16), replicated over the four 16-lane groups
+    const int m_mine = t * kMfmaRows + l16;
     int64_t id = -1;
     if (m_mine < M)
       id = IDX64 ? reinterpret_cast<const int64_t*>(idx)[m_mine]
@@ -50,61 +60,80 @@ __global__ __launch_bounds__(256) void gather_rows_mfma_kernel(
     const bool ok_mine = id >= 0 && id < Z;
     const int rid_mine = ok_mine ? (int)id : 0;
 
-    float16_t acc[BT];
+    float4_t acc[BT];
 #pragma unroll
-    for (int bt = 0; bt < BT; ++bt)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[bt][v] = 0.f;
+    for (int bt = 0; bt < BT; ++bt) acc[bt] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    for (int k0 = 0; k0 < N; k0 += kMfmaKC) {
-      // stage 32 rows x KC columns: instruction r2 covers rows 2*r2 + half_id
-      half8_t stage[16];
-      const int col = k0 + l32 * 8;
+    // two chunks (c and c + 8) are staged per iteration: 16 loads in flight per lane
+    for (int c = wave; c < nchunks; c += 2 * kMfmaWaves) {
+      half8_t stage[2][8];
 #pragma unroll
-      for (int r2 = 0; r2 < 16; ++r2) {
-        const int row = 2 * r2 + half_id;
-        const int rid = __shfl(rid_mine, row, kWave);
-        const bool ok = __shfl((int)ok_mine, row, kWave) != 0;
-        stage[r2] = (ok && col < N) ? load8_stream(W + (int64_t)rid * ldw + col) : zero8();
+      for (int u = 0; u < 2; ++u) {
+        const int col = (c + u * kMfmaWaves) * kMfmaKC + l32 * 8;
+#pragma unroll
+        for (int r2 = 0; r2 < 8; ++r2) {
+          const int row = 2 * r2 + half_id;
+          const int rid = __shfl(rid_mine, row, kWave);
+          const bool ok = __shfl((int)ok_mine, row, kWave) != 0;
+          stage[u][r2] = (ok && col < N) ? load8_stream(W + (int64_t)rid * ldw + col) : zero8();
+        }
       }
 #pragma unroll
-      for (int r2 = 0; r2 < 16; ++r2)
-        store8(tile + (2 * r2 + half_id) * kMfmaLdsRow + l32 * 8, stage[r2]);
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int r2 = 0; r2 < 8; ++r2)
+          store8(tile + (u * kMfmaRows + 2 * r2 + half_id) * kMfmaLdsRow + l32 * 8, stage[u][r2]);
       // the tile is private to this wavefront, whose LDS accesses complete in order: a
       // wavefront-scope fence (compiler ordering only) is all the synchronisation needed
       __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
       __builtin_amdgcn_wave_barrier();
 #pragma unroll
-      for (int ks = 0; ks < kMfmaKC / 16; ++ks) {
-        const int kk = k0 + ks * 16 + half_id * 8;
-        const half8_t a = load8(tile + l32 * kMfmaLdsRow + ks * 16 + half_id * 8);
+      for (int u = 0; u < 2; ++u) {
+        const int k0 = (c + u * kMfmaWaves) * kMfmaKC;
+        if (k0 < N) {
 #pragma unroll
-        for (int bt = 0; bt < BT; ++bt) {
-          const int b = bt * 32 + l32;
-          const half8_t xb = (b < B && kk < N) ? load8(X + (int64_t)b * N + kk) : zero8();
-          acc[bt] = mfma_32x32x16(a, xb, acc[bt]);
+          for (int ks = 0; ks < kMfmaKC / 32; ++ks) {
+            const int kk = k0 + ks * 32 + kg * 8;
+            const half8_t a = load8(tile + (u * kMfmaRows + l16) * kMfmaLdsRow + ks * 32 + kg * 8);
+#pragma unroll
+            for (int bt = 0; bt < BT; ++bt) {
+              const int b = bt * 16 + l16;
+              const half8_t xb = (b < B && kk < N) ? load8(X + (int64_t)b * N + kk) : zero8();
+              acc[bt] = mfma_16x16x32(a, xb, acc[bt]);
+            }
+          }
         }
       }
       __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");  // reads done before the tile is overwritten
       __builtin_amdgcn_wave_barrier();
     }
-    // epilogue: value v of lane l is row 8*(v/4) + 4*half_id + v%4, batch column bt*32 + l32
+    // sum the 8 wavefronts' partial tiles (fixed order) and finish
+    __syncthreads();  // every wavefront is done with its staging region
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int row = 8 * (v / 4) + 4 * half_id + (v % 4);
-      const int m = t * 32 + row;
-      const int rid = __shfl(rid_mine, row, kWave);
-      const bool ok = __shfl((int)ok_mine, row, kWave) != 0;
-      const float bv = (bias != nullptr && ok) ? (float)bias[rid] : 0.f;
+    for (int bt = 0; bt < BT; ++bt)
 #pragma unroll
-      for (int bt = 0; bt < BT; ++bt) {
-        const int b = bt * 32 + l32;
-        float val = acc[bt][v] + bv;
-        if (RELU) val = relu_f(val);
-        if (!ok) val = 0.f;
-        if (m < M && b < B) Y[(int64_t)b * M + m] = (half_t)val;
-      }
+      for (int v = 0; v < 4; ++v) red[((wave * BT + bt) * 4 + v) * 64 + lane] = acc[bt][v];
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+      for (int bt = 0; bt < BT; ++bt)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          float val = 0.f;
+#pragma unroll
+          for (int w = 0; w < kMfmaWaves; ++w) val += red[((w * BT + bt) * 4 + v) * 64 + lane];
+          const int row = 4 * kg + v;
+          const int m = t * kMfmaRows + row;
+          const int rid = __shfl(rid_mine, row, kWave);
+          const bool ok = __shfl((int)ok_mine, row, kWave) != 0;
+          val += (bias != nullptr && ok) ? (float)bias[rid] : 0.f;
+          if (RELU) val = relu_f(val);
+          if (!ok) val = 0.f;
+          const int b = bt * 16 + l16;
+          if (m < M && b < B) Y[(int64_t)b * M + m] = (half_t)val;
+        }
     }
+    __syncthreads();  // red is staging memory again
   }
 }
 
@@ -140,6 +169,9 @@ __global__ __launch_bounds__(256) void gather_cols_mfma_kernel(
   const int m_begin = g * rows_per_block;
   int m_end = m_begin + rows_per_block;
   if (m_end > M) m_end = M;
+  // 128-bit loads of H need 8-element alignment of every (b, first row) pair
+  const bool h_vec_ok = (ldh % 8 == 0) && ((reinterpret_cast<uintptr_t>(H) & 15u) == 0) &&
+                        (x_expanded ? (blk % 8 == 0) : true);
 
   float16_t acc[4][BT];
 #pragma unroll
@@ -184,9 +216,19 @@ __global__ __launch_bounds__(256) void gather_cols_mfma_kernel(
     for (int ks = 0; ks < 2; ++ks) {
       const int mk = ks * 16 + half_id * 8;  // first of this lane's 8 staged rows
       half8_t hb[BT];
+      // the 8 staged rows of this lane are 8 consecutive entries of H[b, :] when the
+      // gather is compact (or one head block of the expanded layout): one 128-bit load
+      const int rid0 = s_rid[mk];
+      const int64_t h0 = x_expanded ? (int64_t)rid0 : (int64_t)(mb + mk);
+      const bool vec = h_vec_ok && rid0 >= 0 && s_rid[mk + 7] >= 0 && mb + mk + 8 <= m_end &&
+                       (!x_expanded || s_rid[mk + 7] == rid0 + 7);
 #pragma unroll
       for (int bt = 0; bt < BT; ++bt) {
         const int b = bt * 32 + l32;
+        if (vec) {
+          hb[bt] = b < B ? load8(H + (int64_t)b * ldh + h0) : zero8();
+          continue;
+        }
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const int rid = s_rid[mk + j];
