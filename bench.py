@@ -26,6 +26,10 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0
 N_LAYERS = 3
+# HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (scaled by a 1 GiB copy; see profiles/layer_opt175b_pmc_traffic.md).  Not measurable from inside
+# this script, so only reported for the shape it was taken on.
+MEASURED_TRAFFIC_BYTES = {("opt-175b", 1, "qkv_sparse"): 302.42e6 + 0.06e6}
 
 
 def algorithmic_bytes(cfg, batch):
@@ -192,6 +196,8 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying HIP graphs")
     ap.add_argument("--single-stream", action="store_true", help="no side stream for predictors / top-k")
     ap.add_argument("--layers-per-graph", type=int, default=3, choices=[1, 3])
+    ap.add_argument("--pmc-calibration", action="store_true",
+                    help="also run a plain 1 GiB device copy (known traffic) for counter calibration")
     ap.add_argument("--defer", action="store_true",
                     help="let the MLP predictor of layer l run into layer l+1 (joined once per graph)")
     args = ap.parse_args()
@@ -263,13 +269,22 @@ def main():
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - t0
 
+        if args.pmc_calibration:
+            src = torch.empty(1 << 30, dtype=torch.uint8, device=device)
+            dst = torch.empty_like(src)
+            for _ in range(3):
+                dst.copy_(src)
+            torch.cuda.synchronize()
+            del src, dst
+
         us_per_layer = elapsed / args.steps * 1e6
         nbytes = algorithmic_bytes(cfg, batch)
         layer_bytes = sum(nbytes.values())
         table = kernel_table(torch, cfg, batch, layers)
         dom = "qkv_sparse"  # largest share of the layer's bytes
         roofline = {"bound": "hbm", "kernel": "qkv_sparse_kernel", "achieved": table[dom]["GB/s"],
-                    "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": table[dom]["frac"], "traffic": None,
+                    "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": table[dom]["frac"],
+                    "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, batch, dom)),
                     "bytes_per_launch": nbytes[dom], "us_per_launch": table[dom]["us"]}
         cpu = None
         if not args.no_cpu_baseline:
