@@ -17,7 +17,7 @@ import torch
 import torch.nn as nn
 from torch import Tensor
 
-from . import ops
+from . import fused_layer, ops
 from .modules import ParallelFusedMLPDejavu, ParallelMHADejavu, ParallelMHASparseAttMlp
 
 
@@ -52,6 +52,9 @@ class BlockMlpAttSparse(nn.Module):
             self.mixer.mlp_k = self.mlp.sp.K
         if hasattr(self.mixer, "sp"):
             self.mixer.att_k = self.mixer.sp.K
+        # ordinary head-sparse decode steps run as one fused call (nine launches); set to
+        # False to always go through the modules' own forwards
+        self.use_fused_layer = True
 
     def forward(self, hidden_states: Tensor, residual: Optional[Tensor] = None, mixer_subset=None,
                 mixer_kwargs=None, head_idx=None, mlp_sp_logit=None):
@@ -59,6 +62,9 @@ class BlockMlpAttSparse(nn.Module):
         residual stream (None for the first block).  Returns
         (hidden_states, residual, next_mlp_sp_logit, next_att_idx)."""
         assert mixer_subset is None
+        ip = None if mixer_kwargs is None else mixer_kwargs.get("inference_params")
+        if self.use_fused_layer and fused_layer.eligible(self, hidden_states, residual, head_idx, mlp_sp_logit, ip):
+            return fused_layer.sparse_layer_decode(self, hidden_states, residual, head_idx, mlp_sp_logit, ip)
         hidden_states, residual = _add_norm(self.norm1, hidden_states, residual)
         if mixer_kwargs is None:
             mixer_kwargs = {}

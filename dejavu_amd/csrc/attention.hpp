@@ -24,19 +24,20 @@ namespace dv {
 // scattered into the caches at position (token + padding[0]).
 // ---------------------------------------------------------------------------
 template <int NBMAX, int R, int U>
-__global__ __launch_bounds__(256) void qkv_sparse_kernel(
+__device__ __forceinline__ void qkv_sparse_body(
     const half_t* __restrict__ X, const half_t* __restrict__ W, const half_t* __restrict__ bias,
     const int* __restrict__ head_idx, const int* __restrict__ batch_idx, int nb, int d, int H,
     int hd, int nnz, half_t* __restrict__ Y, half_t* __restrict__ k_cache,
-    half_t* __restrict__ v_cache, const int* __restrict__ padding, int S) {
+    half_t* __restrict__ v_cache, const int* __restrict__ padding, int S, int block_id,
+    int nblocks) {
   constexpr int CH = 8 * kWave;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int waves_per_block = blockDim.x >> 6;
   const int groups_per_head = hd / R;  // hd % R == 0 (checked on the host)
   const int ntasks = nnz * 3 * groups_per_head;
-  for (int task = blockIdx.x * waves_per_block + wave; task < ntasks;
-       task += gridDim.x * waves_per_block) {
+  for (int task = block_id * waves_per_block + wave; task < ntasks;
+       task += nblocks * waves_per_block) {
     const int i = task / (3 * groups_per_head);
     const int rem = task - i * 3 * groups_per_head;
     const int t = rem / groups_per_head;
@@ -125,6 +126,16 @@ __global__ __launch_bounds__(256) void qkv_sparse_kernel(
   }
 }
 
+template <int NBMAX, int R, int U>
+__global__ __launch_bounds__(256) void qkv_sparse_kernel(
+    const half_t* __restrict__ X, const half_t* __restrict__ W, const half_t* __restrict__ bias,
+    const int* __restrict__ head_idx, const int* __restrict__ batch_idx, int nb, int d, int H,
+    int hd, int nnz, half_t* __restrict__ Y, half_t* __restrict__ k_cache,
+    half_t* __restrict__ v_cache, const int* __restrict__ padding, int S) {
+  qkv_sparse_body<NBMAX, R, U>(X, W, bias, head_idx, batch_idx, nb, d, H, hd, nnz, Y, k_cache, v_cache,
+                               padding, S, blockIdx.x, gridDim.x);
+}
+
 // ---------------------------------------------------------------------------
 // For i < nnz, h = head_idx[i], every slot with s = seq_idx[i, slot] >= 0:
 //   k_cache[0, h, dp, s + pad, p] = K[s, h, dp*8 + p]      (if k_cache != null)
@@ -161,14 +172,11 @@ __global__ void kv_cache_copy_kernel(const half_t* __restrict__ K, const half_t*
 // tracker is (H, 16) int32: tracker[h, s] == s while token s of the window has no
 // K/V for head h, -1 once it has.  Heads in head_idx are distinct.  Workgroup 0
 // owns the tracker (two phases separated by a barrier); all workgroups copy x.
-__global__ __launch_bounds__(256) void window_step_kernel(
-    const half_t* __restrict__ x, half_t* __restrict__ x_cache, int d, int* __restrict__ tracker,
-    const int* __restrict__ head_idx, int nnz, int H, int counter, int flush,
-    int* __restrict__ batch_idx) {
-  const int tid = blockIdx.x * blockDim.x + threadIdx.x;
-  const int nthreads = gridDim.x * blockDim.x;
-  for (int j = tid; j < d; j += nthreads) x_cache[(int64_t)counter * d + j] = x[j];
-  if (blockIdx.x != 0) return;
+// Tracker part, executed by ONE workgroup (any size).
+__device__ __forceinline__ void window_tracker_step(int* __restrict__ tracker,
+                                                    const int* __restrict__ head_idx, int nnz, int H,
+                                                    int counter, int flush,
+                                                    int* __restrict__ batch_idx) {
   if (flush) {
     for (int o = threadIdx.x; o < H * 16; o += blockDim.x) {
       tracker[o] = o & 15;
@@ -191,6 +199,17 @@ __global__ __launch_bounds__(256) void window_step_kernel(
       tracker[h * 16 + s] = -1;
     }
   }
+}
+
+__global__ __launch_bounds__(256) void window_step_kernel(
+    const half_t* __restrict__ x, half_t* __restrict__ x_cache, int d, int* __restrict__ tracker,
+    const int* __restrict__ head_idx, int nnz, int H, int counter, int flush,
+    int* __restrict__ batch_idx) {
+  const int tid = blockIdx.x * blockDim.x + threadIdx.x;
+  const int nthreads = gridDim.x * blockDim.x;
+  for (int j = tid; j < d; j += nthreads) x_cache[(int64_t)counter * d + j] = x[j];
+  if (blockIdx.x != 0) return;
+  window_tracker_step(tracker, head_idx, nnz, H, counter, flush, batch_idx);
 }
 
 // Appends the newest token: for every batch row b and head (all, or head_idx):
@@ -222,11 +241,11 @@ __global__ void kv_append_kernel(const half_t* __restrict__ K, const half_t* __r
 // n_len = number of cached positions to attend (lengths[b] + 1 if lengths).
 // ---------------------------------------------------------------------------
 template <int HD, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void decode_attn_kernel(
+__device__ __forceinline__ void decode_attn_body(
     const half_t* __restrict__ Q, int64_t ldq, const half_t* __restrict__ k_cache,
     const half_t* __restrict__ v_cache, const int* __restrict__ head_idx,
     const int* __restrict__ lengths, int n_len, int H, int S, float scale, int nsplit,
-    float* __restrict__ part) {
+    float* __restrict__ part, int split, int i, int b, int nheads) {
   constexpr int PK = HD / 8;        // 16-byte packets per position / lanes per V row
   constexpr int RPI = kWave / PK;   // V rows per load instruction
   constexpr int VIT = kWave / RPI;  // V load instructions per wavefront (= PK)
@@ -234,12 +253,9 @@ __global__ __launch_bounds__(WAVES * 64) void decode_attn_kernel(
   __shared__ float s_o[WAVES][HD];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int split = blockIdx.x;
-  const int i = blockIdx.y;
-  const int b = blockIdx.z;
   const int h = head_idx ? head_idx[i] : i;
   const int len = lengths ? lengths[b] + 1 : n_len;
-  float* out = part + (((int64_t)b * gridDim.y + i) * nsplit + split) * (HD + 2);
+  float* out = part + (((int64_t)b * nheads + i) * nsplit + split) * (HD + 2);
   const bool head_ok = h >= 0 && h < H;
   const int p0 = (split * WAVES + wave) * kWave;
   float m = -INFINITY, l = 0.f;
@@ -309,6 +325,16 @@ __global__ __launch_bounds__(WAVES * 64) void decode_attn_kernel(
     }
     out[j] = v;
   }
+}
+
+template <int HD, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void decode_attn_kernel(
+    const half_t* __restrict__ Q, int64_t ldq, const half_t* __restrict__ k_cache,
+    const half_t* __restrict__ v_cache, const int* __restrict__ head_idx,
+    const int* __restrict__ lengths, int n_len, int H, int S, float scale, int nsplit,
+    float* __restrict__ part) {
+  decode_attn_body<HD, WAVES>(Q, ldq, k_cache, v_cache, head_idx, lengths, n_len, H, S, scale, nsplit, part,
+                              blockIdx.x, blockIdx.y, blockIdx.z, gridDim.y);
 }
 
 // out[b, h, :] = sum_s o_s * exp(m_s - m) / sum_s l_s * exp(m_s - m).  Grid (heads, B), HD threads.

@@ -11,6 +11,7 @@
 #include "gemm_mfma.hpp"
 #include "gemv_cols.hpp"
 #include "gemv_rows.hpp"
+#include "layer_fused.hpp"
 #include "norm.hpp"
 #include "topk.hpp"
 
@@ -755,6 +756,208 @@ int dv_add_layer_norm_f16(const void* h, const void* residual, const void* gamma
   else
     DV_LN(1024, 4);
 #undef DV_LN
+  return launch_status();
+}
+
+namespace {
+struct LayerPlan {
+  size_t off_topk, off_x, off_res1, off_attn_out, off_x2, off_qkv, off_batch_idx, off_hp_hidden,
+      off_mp_hidden, off_h, off_head_logits, off_attn_part, off_cols_part, total;
+  int nsplit;
+  ColsPlan out_cols, fc2_cols;
+};
+
+inline size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
+
+LayerPlan plan_layer(const dvSparseLayerArgs& a) {
+  LayerPlan p;
+  size_t o = 0;
+  p.off_topk = o;  // zero-initialised region first
+  o = align_up(o + dv_topk_workspace_bytes(a.ffn > 1024 ? a.ffn : 2048));
+  p.off_x = o;            o = align_up(o + (size_t)a.d * 2);
+  p.off_res1 = o;         o = align_up(o + (size_t)a.d * 2);
+  p.off_attn_out = o;     o = align_up(o + (size_t)a.d * 2);
+  p.off_x2 = o;           o = align_up(o + (size_t)a.d * 2);
+  p.off_qkv = o;          o = align_up(o + (size_t)16 * 3 * a.H * a.hd * 2);
+  p.off_batch_idx = o;    o = align_up(o + (size_t)a.H * 16 * 4);
+  p.off_hp_hidden = o;    o = align_up(o + (size_t)a.r_att * 2);
+  p.off_mp_hidden = o;    o = align_up(o + (size_t)a.r_mlp * 2);
+  p.off_h = o;            o = align_up(o + (size_t)a.K * 2);
+  p.off_head_logits = o;  o = align_up(o + (size_t)a.H * 2);
+  p.nsplit = attn_splits(a.n_len > 0 ? a.S : 1);  // sized for the full cache
+  p.off_attn_part = o;    o = align_up(o + (size_t)a.Hk * p.nsplit * (a.hd + 2) * 4);
+  p.out_cols = plan_cols(a.d, a.Hk * a.hd);
+  p.fc2_cols = plan_cols(a.d, a.K);
+  const int g = p.out_cols.groups > p.fc2_cols.groups ? p.out_cols.groups : p.fc2_cols.groups;
+  p.off_cols_part = o;    o = align_up(o + (size_t)g * a.d * 4);
+  p.total = o;
+  return p;
+}
+
+int check_layer_args(const dvSparseLayerArgs& a) {
+  if (!a.hidden || !a.ln1_w || !a.ln1_b || !a.ln2_w || !a.ln2_b || !a.Wqkv || !a.Wout_t || !a.att_Wa ||
+      !a.att_Wb || !a.W1 || !a.W2t || !a.mlp_Wa || !a.mlp_Wb || !a.head_idx || !a.mlp_logit_in ||
+      !a.cache_offset || !a.k_cache || !a.v_cache || !a.x_cache || !a.tracker || !a.hidden_out ||
+      !a.residual_out || !a.mlp_logit_out || !a.att_idx_out || !a.mlp_idx_out || !a.workspace)
+    return DV_ERR_INVALID_ARG;
+  if (a.d <= 0 || a.ffn <= 0 || a.H <= 0 || a.Hk < 1 || a.Hk > a.H || a.att_k < 1 || a.att_k > a.H ||
+      a.K < 1 || a.K > a.ffn || a.r_att <= 0 || a.r_mlp <= 0 || a.S <= 0 || a.n_len < 1 || a.n_len > a.S ||
+      a.counter < 0 || a.counter > 14)
+    return DV_ERR_INVALID_ARG;
+  if ((a.hd != 64 && a.hd != 128) || a.H * a.hd != a.d || a.H > 1024 || a.ffn > 65536 || a.ffn <= 1024 ||
+      a.d > 1024 * 8 * 4 || (size_t)a.d * 2 > 160 * 1024)
+    return DV_ERR_UNSUPPORTED;
+  if (a.d % 8 || a.ffn % 8 || a.r_att % 8 || a.r_mlp % 8) return DV_ERR_ALIGNMENT;
+  return DV_OK;
+}
+}  // namespace
+
+size_t dv_sparse_layer_workspace_bytes(const dvSparseLayerArgs* args) {
+  if (!args || args->d <= 0 || args->ffn <= 0 || args->H <= 0 || args->Hk < 1 || args->K < 1) return 0;
+  return plan_layer(*args).total;
+}
+
+int dv_sparse_layer_decode_f16(const dvSparseLayerArgs* args, void* stream) {
+  if (!args) return DV_ERR_INVALID_ARG;
+  const dvSparseLayerArgs& a = *args;
+  int rc = check_layer_args(a);
+  if (rc != DV_OK) return rc;
+  const LayerPlan p = plan_layer(a);
+  if (a.workspace_bytes < p.total || !aligned16(a.workspace)) return DV_ERR_WORKSPACE;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  unsigned char* ws = reinterpret_cast<unsigned char*>(a.workspace);
+  auto H16 = [&](size_t off) { return reinterpret_cast<half_t*>(ws + off); };
+  auto CH = [](const void* q) { return reinterpret_cast<const half_t*>(q); };
+  unsigned* topk_ws = reinterpret_cast<unsigned*>(ws + p.off_topk);
+  int* batch_idx = reinterpret_cast<int*>(ws + p.off_batch_idx);
+  float* attn_part = reinterpret_cast<float*>(ws + p.off_attn_part);
+  float* cols_part = reinterpret_cast<float*>(ws + p.off_cols_part);
+  half_t* x = H16(p.off_x);
+  half_t* res1 = H16(p.off_res1);
+  half_t* attn_out = H16(p.off_attn_out);
+  half_t* x2 = H16(p.off_x2);
+  half_t* qkv = H16(p.off_qkv);
+  half_t* hp_hidden = H16(p.off_hp_hidden);
+  half_t* mp_hidden = H16(p.off_mp_hidden);
+  half_t* hbuf = H16(p.off_h);
+  half_t* head_logits = H16(p.off_head_logits);
+  half_t* x_cache = reinterpret_cast<half_t*>(a.x_cache);
+  const int* head_idx = reinterpret_cast<const int*>(a.head_idx);
+  const int cus = compute_units();
+  const int nb = a.counter + 1;
+  const int topk_blocks = (a.ffn + kTopkItemsPerBlock - 1) / kTopkItemsPerBlock;
+
+  // L1: add + LayerNorm 1 + window step
+  {
+#define DV_L1(V)                                                                                      \
+  hipLaunchKernelGGL((layer_l1_kernel<V>), dim3(1), dim3(kLnThreads), 0, s, CH(a.hidden), CH(a.residual), \
+                     CH(a.ln1_w), CH(a.ln1_b), a.eps1, a.d, x, res1, x_cache + (size_t)a.counter * a.d, \
+                     reinterpret_cast<int*>(a.tracker), head_idx, a.Hk, a.H, a.counter, batch_idx)
+    if (a.d <= kLnThreads * 8) DV_L1(1);
+    else if (a.d <= kLnThreads * 16) DV_L1(2);
+    else DV_L1(4);
+#undef DV_L1
+  }
+  // L2: QKV + cache scatter | head predictor fc0 | key histogram of this layer's MLP logits
+  {
+    QkvArgs q{x_cache, CH(a.Wqkv), CH(a.bqkv), head_idx, batch_idx, nb, a.d, a.H, a.hd, a.Hk, qkv,
+              reinterpret_cast<half_t*>(a.k_cache), reinterpret_cast<half_t*>(a.v_cache),
+              reinterpret_cast<const int*>(a.cache_offset), a.S};
+    const int ntasks = a.Hk * 3 * (a.hd / 2);
+    int nq = (ntasks + 3) / 4;
+    if (nq > cus * 8) nq = cus * 8;
+    CanonArgs hp0{res1, CH(a.att_Wa), (int64_t)a.d, a.r_att, a.d, hp_hidden};
+    const int rw0 = a.d <= 1024 ? 4 : 1;
+    const int nh = ((a.r_att + rw0 - 1) / rw0 + 3) / 4;
+    const dim3 grid(nq + nh + topk_blocks);
+#define DV_L2(NB)                                                                                 \
+  hipLaunchKernelGGL((layer_l2_kernel<NB>), grid, dim3(256), 0, s, q, nq, hp0, nh, CH(a.mlp_logit_in), \
+                     a.ffn, topk_ws)
+    if (nb == 1) DV_L2(1);
+    else if (nb == 2) DV_L2(2);
+    else if (nb <= 4) DV_L2(4);
+    else if (nb <= 8) DV_L2(8);
+    else DV_L2(16);
+#undef DV_L2
+  }
+  // L3: attention partials | head predictor fc1 | top-k threshold and counts
+  const int nsplit = attn_splits(a.n_len);
+  {
+    AttnArgs at{qkv + (size_t)a.counter * 3 * a.H * a.hd, (int64_t)3 * a.H * a.hd,
+                reinterpret_cast<const half_t*>(a.k_cache), reinterpret_cast<const half_t*>(a.v_cache),
+                head_idx, a.n_len, a.H, a.S, nsplit, a.Hk, a.softmax_scale, attn_part};
+    CanonArgs hp1{hp_hidden, CH(a.att_Wb), (int64_t)a.r_att, a.H, a.r_att, head_logits};
+    const int na = nsplit * a.Hk;
+    const int rw1 = a.r_att <= 1024 ? 4 : 1;
+    const int nh1 = ((a.H + rw1 - 1) / rw1 + 3) / 4;
+    const dim3 grid(na + nh1 + topk_blocks);
+    if (a.hd == 128)
+      hipLaunchKernelGGL((layer_l3_kernel<128>), grid, dim3(256), 0, s, at, na, hp1, nh1, CH(a.mlp_logit_in),
+                         a.ffn, a.K, topk_ws);
+    else
+      hipLaunchKernelGGL((layer_l3_kernel<64>), grid, dim3(256), 0, s, at, na, hp1, nh1, CH(a.mlp_logit_in),
+                         a.ffn, a.K, topk_ws);
+  }
+  // L4 + L5: out_proj from the attention partials | head top-k | top-k emission; split reduction
+  {
+    const ColsPlan& c = p.out_cols;
+    OutProjArgs o{CH(a.Wout_t), (int64_t)a.d, CH(a.bout), head_idx, a.hd, a.d, a.H * a.hd, a.Hk * a.hd,
+                  c.rows_per_block, c.col_tiles, c.groups, cols_part, attn_out, attn_part, nsplit};
+    const int no = c.col_tiles * c.groups;
+    hipLaunchKernelGGL(layer_l4_kernel, dim3(no + 1 + topk_blocks), dim3(256), 0, s, o, no, head_logits, a.H,
+                       a.att_k, reinterpret_cast<int*>(a.att_idx_out), CH(a.mlp_logit_in), a.ffn, topk_ws,
+                       reinterpret_cast<int64_t*>(a.mlp_idx_out), topk_blocks);
+    if (c.groups > 1)
+      hipLaunchKernelGGL(cols_reduce_kernel, dim3((unsigned)((a.d + 63) / 64)), dim3(256), 0, s, cols_part,
+                         CH(a.bout), c.groups, 1, a.d, attn_out);
+  }
+  // L6: add + LayerNorm 2
+  {
+    half_t* res2 = reinterpret_cast<half_t*>(a.residual_out);
+#define DV_L6(V)                                                                                    \
+  hipLaunchKernelGGL((add_layer_norm_kernel<kLnThreads, V>), dim3(1), dim3(kLnThreads), 0, s, attn_out, \
+                     res1, CH(a.ln2_w), CH(a.ln2_b), a.eps2, a.d, x2, res2)
+    if (a.d <= kLnThreads * 8) DV_L6(1);
+    else if (a.d <= kLnThreads * 16) DV_L6(2);
+    else DV_L6(4);
+#undef DV_L6
+  }
+  const half_t* res2 = reinterpret_cast<const half_t*>(a.residual_out);
+  const int64_t* mlp_idx = reinterpret_cast<const int64_t*>(a.mlp_idx_out);
+  // L7: fc1 gather | MLP predictor fc0
+  {
+    RowsArgs f{x2, CH(a.W1), CH(a.b1), mlp_idx, a.d, (int64_t)a.d, a.ffn, a.K, hbuf};
+    int nf = ((a.K + 1) / 2 + 3) / 4;
+    if (nf > cus * 8) nf = cus * 8;
+    CanonArgs mp0{res2, CH(a.mlp_Wa), (int64_t)a.d, a.r_mlp, a.d, mp_hidden};
+    const int rw0 = a.d <= 1024 ? 4 : 1;
+    const int nm = ((a.r_mlp + rw0 - 1) / rw0 + 3) / 4;
+    const size_t lds = (size_t)a.d * sizeof(half_t);
+    static size_t lds_granted = 48 * 1024;
+    if (lds > lds_granted) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(layer_l7_kernel),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+        return DV_ERR_UNSUPPORTED;
+      lds_granted = lds;
+    }
+    hipLaunchKernelGGL(layer_l7_kernel, dim3(nf + nm), dim3(256), lds, s, f, nf, mp0, nm);
+  }
+  // L8 + L9: fc2 gather | MLP predictor fc1, then the split reduction
+  {
+    const ColsPlan& c = p.fc2_cols;
+    ColsArgs cc{hbuf, CH(a.W2t), (int64_t)a.d, mlp_idx, a.d, a.ffn, a.K, c.rows_per_block, c.col_tiles, c.groups,
+                cols_part, reinterpret_cast<half_t*>(a.hidden_out), CH(a.b2)};
+    CanonArgs mp1{mp_hidden, CH(a.mlp_Wb), (int64_t)a.r_mlp, a.ffn, a.r_mlp,
+                  reinterpret_cast<half_t*>(a.mlp_logit_out)};
+    const int rw1 = a.r_mlp <= 1024 ? 4 : 1;
+    int nm = ((a.ffn + rw1 - 1) / rw1 + 3) / 4;
+    if (nm > cus * 16) nm = cus * 16;
+    const int nf = c.col_tiles * c.groups;
+    hipLaunchKernelGGL(layer_l8_kernel, dim3(nf + nm), dim3(256), 0, s, cc, nf, mp1, nm);
+    if (c.groups > 1)
+      hipLaunchKernelGGL(cols_reduce_kernel, dim3((unsigned)((a.d + 63) / 64)), dim3(256), 0, s, cols_part,
+                         CH(a.b2), c.groups, 1, a.d, reinterpret_cast<half_t*>(a.hidden_out));
+  }
   return launch_status();
 }
 

@@ -29,21 +29,19 @@ __device__ __forceinline__ float load_agent(const float* p) {
 // fly from the un-normalised attention partials { max, sum, o[blk] } of
 // decode_attn_kernel (attn_nsplit splits per head), rounded to fp16 as a
 // stored context vector would be.
-template <int B, int U, bool IDX64, bool BLOCKED, bool FUSED, bool ATTN = false>
-__global__ __launch_bounds__(256) void gather_cols_kernel(
+template <int B, int U, bool IDX64, bool BLOCKED, bool FUSED, bool ATTN>
+__device__ __forceinline__ void gather_cols_body(
     const half_t* __restrict__ X, int64_t ldx, int x_expanded, const half_t* __restrict__ W,
     int64_t ldw, const half_t* __restrict__ bias, const void* __restrict__ idx, int blk, int N,
     int Z, int M, int rows_per_block, float* __restrict__ partial, unsigned* __restrict__ counters,
-    half_t* __restrict__ Y, const float* __restrict__ attn_part = nullptr, int attn_nsplit = 0) {
+    half_t* __restrict__ Y, const float* __restrict__ attn_part, int attn_nsplit, int ct, int g,
+    int G) {
   __shared__ float red[4][B][kColTile];
   __shared__ int s_last;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int ct = blockIdx.x;
-  const int g = blockIdx.y;
-  const int G = gridDim.y;
   const int col = ct * kColTile + lane * 8;
   const bool col_ok = col < N;  // N % 8 == 0, so a lane is all-in or all-out
   const half_t* wcol = W + (col_ok ? col : 0);
@@ -231,6 +229,17 @@ __global__ __launch_bounds__(256) void gather_cols_kernel(
   }
   if (tid == 0)
     __hip_atomic_store(&counters[ct], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <int B, int U, bool IDX64, bool BLOCKED, bool FUSED, bool ATTN = false>
+__global__ __launch_bounds__(256) void gather_cols_kernel(
+    const half_t* __restrict__ X, int64_t ldx, int x_expanded, const half_t* __restrict__ W,
+    int64_t ldw, const half_t* __restrict__ bias, const void* __restrict__ idx, int blk, int N,
+    int Z, int M, int rows_per_block, float* __restrict__ partial, unsigned* __restrict__ counters,
+    half_t* __restrict__ Y, const float* __restrict__ attn_part = nullptr, int attn_nsplit = 0) {
+  gather_cols_body<B, U, IDX64, BLOCKED, FUSED, ATTN>(X, ldx, x_expanded, W, ldw, bias, idx, blk, N, Z, M,
+                                                     rows_per_block, partial, counters, Y, attn_part,
+                                                     attn_nsplit, blockIdx.x, blockIdx.y, gridDim.y);
 }
 
 // Second pass of the non-fused path: Y[b, c] = fp16(sum_g partial[g, b, c] + bias[c]).

@@ -19,9 +19,9 @@ namespace dv {
 // Requires n % 8 == 0 and ldw % 8 == 0.
 // ---------------------------------------------------------------------------
 template <int LANES, int B, int U>
-__global__ __launch_bounds__(256) void canonical_gemv_kernel(
+__device__ __forceinline__ void canonical_gemv_body(
     const half_t* __restrict__ X, const half_t* __restrict__ W, int64_t ldw, int rows, int n,
-    half_t* __restrict__ Y) {
+    half_t* __restrict__ Y, int block_id, int nblocks) {
   constexpr int RW = kWave / LANES;  // rows per wavefront pass
   constexpr int CH = 8 * LANES;      // elements per chunk
   const int lane = threadIdx.x & 63;
@@ -30,7 +30,7 @@ __global__ __launch_bounds__(256) void canonical_gemv_kernel(
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int waves_per_block = blockDim.x >> 6;
   const int ntasks = (rows + RW - 1) / RW;
-  for (int t = blockIdx.x * waves_per_block + wave; t < ntasks; t += gridDim.x * waves_per_block) {
+  for (int t = block_id * waves_per_block + wave; t < ntasks; t += nblocks * waves_per_block) {
     const int row = t * RW + grp;
     const bool valid = row < rows;
     const half_t* wr = W + (int64_t)(valid ? row : 0) * ldw + sub * 8;
@@ -67,6 +67,13 @@ __global__ __launch_bounds__(256) void canonical_gemv_kernel(
   }
 }
 
+template <int LANES, int B, int U>
+__global__ __launch_bounds__(256) void canonical_gemv_kernel(
+    const half_t* __restrict__ X, const half_t* __restrict__ W, int64_t ldw, int rows, int n,
+    half_t* __restrict__ Y) {
+  canonical_gemv_body<LANES, B, U>(X, W, ldw, rows, n, Y, blockIdx.x, gridDim.x);
+}
+
 // ---------------------------------------------------------------------------
 // Y[b, m] = act( sum_i W[idx[m], i] * X[b, i] + bias[idx[m]] ), fp16 out.
 // One wavefront owns R gathered rows at a time (R independent load streams);
@@ -74,12 +81,10 @@ __global__ __launch_bounds__(256) void canonical_gemv_kernel(
 // instead of a wild read.  Requires n % 8 == 0 and ldw % 8 == 0.
 // ---------------------------------------------------------------------------
 template <int B, int R, int U, bool RELU>
-__global__ __launch_bounds__(256) void gather_rows_kernel(
+__device__ __forceinline__ void gather_rows_body(
     const half_t* __restrict__ X, const half_t* __restrict__ W, const half_t* __restrict__ bias,
     const void* __restrict__ idx, int idx_bytes, int n, int64_t ldw, int Z, int M,
-    half_t* __restrict__ Y) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  half_t* xs = reinterpret_cast<half_t*>(smem_raw);
+    half_t* __restrict__ Y, half_t* xs, int block_id, int nblocks) {
   for (int i = threadIdx.x * 8; i < B * n; i += blockDim.x * 8) store8(xs + i, load8(X + i));
   __syncthreads();
 
@@ -88,7 +93,7 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int waves_per_block = blockDim.x >> 6;
   const int ntasks = (M + R - 1) / R;
-  for (int t = blockIdx.x * waves_per_block + wave; t < ntasks; t += gridDim.x * waves_per_block) {
+  for (int t = block_id * waves_per_block + wave; t < ntasks; t += nblocks * waves_per_block) {
     const half_t* wr[R];
     bool valid[R];
     int64_t rid[R];
@@ -150,6 +155,16 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(
       }
     }
   }
+}
+
+template <int B, int R, int U, bool RELU>
+__global__ __launch_bounds__(256) void gather_rows_kernel(
+    const half_t* __restrict__ X, const half_t* __restrict__ W, const half_t* __restrict__ bias,
+    const void* __restrict__ idx, int idx_bytes, int n, int64_t ldw, int Z, int M,
+    half_t* __restrict__ Y) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  gather_rows_body<B, R, U, RELU>(X, W, bias, idx, idx_bytes, n, ldw, Z, M, Y,
+                                  reinterpret_cast<half_t*>(smem_raw), blockIdx.x, gridDim.x);
 }
 
 }  // namespace dv

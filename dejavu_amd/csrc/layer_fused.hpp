@@ -1,0 +1,198 @@
+// One decode step of a whole sparse block in nine launches.  Kernels that are
+// independent of each other share a launch ("roles" picked by workgroup index),
+// so the small latency-bound pieces (LayerNorm, window step, predictors, top-k)
+// run beside the bandwidth-bound ones instead of each paying a launch of its own.
+// The role bodies are the very same device functions as the stand-alone kernels.
+//
+//  L1  add+LayerNorm 1 + back-fill window step
+//  L2  QKV (+ cache scatter) of the active heads       | head predictor fc0 | key histogram of the MLP logits
+//  L3  attention partials over the active heads        | head predictor fc1 | top-k threshold + counts
+//  L4  out_proj over W_out^T, merging the attention    | head top-k         | top-k emission
+//      partials on the fly
+//  L5  split reduction (+ bias)
+//  L6  add+LayerNorm 2
+//  L7  fc1 gather (+bias, ReLU)                         | MLP predictor fc0
+//  L8  fc2 gather                                       | MLP predictor fc1
+//  L9  split reduction (+ bias)
+#pragma once
+#include "attention.hpp"
+#include "common.hpp"
+#include "gemv_cols.hpp"
+#include "gemv_rows.hpp"
+#include "norm.hpp"
+#include "topk.hpp"
+
+namespace dv {
+
+constexpr int kLnThreads = 1024;
+
+// ---- L1 -------------------------------------------------------------------
+template <int MAXV>
+__global__ __launch_bounds__(kLnThreads) void layer_l1_kernel(
+    const half_t* __restrict__ hidden, const half_t* __restrict__ residual,
+    const half_t* __restrict__ gamma, const half_t* __restrict__ beta, float eps, int d,
+    half_t* __restrict__ x, half_t* __restrict__ residual1, half_t* __restrict__ x_cache_row,
+    int* __restrict__ tracker, const int* __restrict__ head_idx, int nnz, int H, int counter,
+    int* __restrict__ batch_idx) {
+  add_layer_norm_body<kLnThreads, MAXV>(hidden, residual, gamma, beta, eps, d, x, residual1, x_cache_row, 0);
+  window_tracker_step(tracker, head_idx, nnz, H, counter, 0, batch_idx);
+}
+
+// ---- L2 -------------------------------------------------------------------
+struct QkvArgs {
+  const half_t* X;  // window buffer rows [0, nb)
+  const half_t* W;
+  const half_t* bias;
+  const int* head_idx;
+  const int* batch_idx;
+  int nb, d, H, hd, nnz;
+  half_t* Y;
+  half_t* k_cache;
+  half_t* v_cache;
+  const int* padding;
+  int S;
+};
+
+struct CanonArgs {
+  const half_t* X;
+  const half_t* W;
+  int64_t ldw;
+  int rows, n;
+  half_t* Y;
+};
+
+// canonical GEMV role with the lane count the fixed summation order prescribes for n
+__device__ __forceinline__ void canonical_role(const CanonArgs& c, int block_id, int nblocks) {
+  if (c.n <= 1024)
+    canonical_gemv_body<16, 1, 8>(c.X, c.W, c.ldw, c.rows, c.n, c.Y, block_id, nblocks);
+  else
+    canonical_gemv_body<64, 1, 8>(c.X, c.W, c.ldw, c.rows, c.n, c.Y, block_id, nblocks);
+}
+
+template <int NBMAX>
+__global__ __launch_bounds__(256) void layer_l2_kernel(QkvArgs q, int nblk_qkv, CanonArgs hp0, int nblk_hp0,
+                                                       const half_t* __restrict__ mlp_logits, int ffn,
+                                                       unsigned* __restrict__ topk_ws) {
+  const int bid = blockIdx.x;
+  if (bid < nblk_qkv) {
+    qkv_sparse_body<NBMAX, 2, 4>(q.X, q.W, q.bias, q.head_idx, q.batch_idx, q.nb, q.d, q.H, q.hd, q.nnz, q.Y,
+                                 q.k_cache, q.v_cache, q.padding, q.S, bid, nblk_qkv);
+  } else if (bid < nblk_qkv + nblk_hp0) {
+    canonical_role(hp0, bid - nblk_qkv, nblk_hp0);
+  } else {
+    topk_hist_body(mlp_logits, 1, ffn, topk_ws, bid - nblk_qkv - nblk_hp0);
+  }
+}
+
+// ---- L3 -------------------------------------------------------------------
+struct AttnArgs {
+  const half_t* Q;
+  int64_t ldq;
+  const half_t* k_cache;
+  const half_t* v_cache;
+  const int* head_idx;
+  int n_len, H, S, nsplit, nheads;
+  float scale;
+  float* part;
+};
+
+template <int HD>
+__global__ __launch_bounds__(256) void layer_l3_kernel(AttnArgs a, int nblk_attn, CanonArgs hp1, int nblk_hp1,
+                                                       const half_t* __restrict__ mlp_logits, int ffn,
+                                                       int K, unsigned* __restrict__ topk_ws) {
+  const int bid = blockIdx.x;
+  if (bid < nblk_attn) {
+    const int split = bid % a.nsplit, i = bid / a.nsplit;
+    decode_attn_body<HD, 4>(a.Q, a.ldq, a.k_cache, a.v_cache, a.head_idx, nullptr, a.n_len, a.H, a.S, a.scale,
+                            a.nsplit, a.part, split, i, 0, a.nheads);
+  } else if (bid < nblk_attn + nblk_hp1) {
+    canonical_role(hp1, bid - nblk_attn, nblk_hp1);
+  } else {
+    topk_count_body(mlp_logits, 1, ffn, K, topk_ws, bid - nblk_attn - nblk_hp1);
+  }
+}
+
+// ---- L4 -------------------------------------------------------------------
+struct OutProjArgs {
+  const half_t* W;
+  int64_t ldw;
+  const half_t* bias;
+  const int* head_idx;
+  int hd, N, Z, M, rows_per_block, col_tiles, groups;
+  float* partial;
+  half_t* Y;
+  const float* attn_part;
+  int nsplit;
+};
+
+__global__ __launch_bounds__(256) void layer_l4_kernel(OutProjArgs o, int nblk_out,
+                                                       const half_t* __restrict__ head_logits, int H,
+                                                       int att_k, int* __restrict__ att_idx_out,
+                                                       const half_t* __restrict__ mlp_logits, int ffn,
+                                                       unsigned* __restrict__ topk_ws,
+                                                       int64_t* __restrict__ mlp_idx_out, int nblk_emit) {
+  const int bid = blockIdx.x;
+  if (bid < nblk_out) {
+    const int ct = bid % o.col_tiles, g = bid / o.col_tiles;
+    gather_cols_body<1, 8, false, true, false, true>(nullptr, 0, 1, o.W, o.ldw, o.bias, o.head_idx, o.hd, o.N,
+                                                     o.Z, o.M, o.rows_per_block, o.partial, nullptr, o.Y,
+                                                     o.attn_part, o.nsplit, ct, g, o.groups);
+  } else if (bid == nblk_out) {
+    // head top-k for the next layer (rank selection, one workgroup)
+    __shared__ unsigned s_key[1024];
+    __shared__ unsigned s_sel[1024];
+    for (int j = threadIdx.x; j < H; j += blockDim.x) s_key[j] = topk_key(head_logits[j]);
+    __syncthreads();
+    rank_select_emit(s_key, s_sel, H, att_k, att_idx_out, 4);
+  } else {
+    topk_emit_body(mlp_logits, 1, ffn, topk_ws, mlp_idx_out, 8, bid - nblk_out - 1, nblk_emit);
+  }
+}
+
+// ---- L7 / L8 --------------------------------------------------------------
+struct RowsArgs {
+  const half_t* X;
+  const half_t* W;
+  const half_t* bias;
+  const int64_t* idx;
+  int n;
+  int64_t ldw;
+  int Z, M;
+  half_t* Y;
+};
+
+__global__ __launch_bounds__(256) void layer_l7_kernel(RowsArgs f, int nblk_fc1, CanonArgs mp0, int nblk_mp0) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  const int bid = blockIdx.x;
+  if (bid < nblk_fc1) {
+    gather_rows_body<1, 2, 4, true>(f.X, f.W, f.bias, f.idx, 8, f.n, f.ldw, f.Z, f.M, f.Y,
+                                    reinterpret_cast<half_t*>(smem_raw), bid, nblk_fc1);
+  } else {
+    canonical_role(mp0, bid - nblk_fc1, nblk_mp0);
+  }
+}
+
+struct ColsArgs {
+  const half_t* X;
+  const half_t* W;
+  int64_t ldw;
+  const int64_t* idx;
+  int N, Z, M, rows_per_block, col_tiles, groups;
+  float* partial;
+  half_t* Y;
+  const half_t* bias;
+};
+
+__global__ __launch_bounds__(256) void layer_l8_kernel(ColsArgs c, int nblk_fc2, CanonArgs mp1, int nblk_mp1) {
+  const int bid = blockIdx.x;
+  if (bid < nblk_fc2) {
+    const int ct = bid % c.col_tiles, g = bid / c.col_tiles;
+    gather_cols_body<1, 8, true, false, false, false>(c.X, c.M, 0, c.W, c.ldw, c.bias, c.idx, 1, c.N, c.Z, c.M,
+                                                      c.rows_per_block, c.partial, nullptr, c.Y, nullptr, 0, ct,
+                                                      g, c.groups);
+  } else {
+    canonical_role(mp1, bid - nblk_fc2, nblk_mp1);
+  }
+}
+
+}  // namespace dv

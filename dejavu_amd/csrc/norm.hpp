@@ -21,13 +21,13 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
 }
 
 // MAXV: 8-element vectors held per thread; requires d % 8 == 0 and d <= THREADS * 8 * MAXV.
+// Y2 (optional) receives a second copy of the normalised row (the back-fill window buffer).
 template <int THREADS, int MAXV>
-__global__ __launch_bounds__(THREADS) void add_layer_norm_kernel(
+__device__ __forceinline__ void add_layer_norm_body(
     const half_t* __restrict__ H, const half_t* __restrict__ R, const half_t* __restrict__ gamma,
     const half_t* __restrict__ beta, float eps, int d, half_t* __restrict__ Y,
-    half_t* __restrict__ Rout) {
+    half_t* __restrict__ Rout, half_t* __restrict__ Y2, int64_t row) {
   __shared__ float scratch[THREADS / kWave];
-  const int64_t row = blockIdx.x;
   const int nvec = d / 8;
   half8_t v[MAXV], gm[MAXV], bt[MAXV];
 #pragma unroll
@@ -79,8 +79,17 @@ __global__ __launch_bounds__(THREADS) void add_layer_norm_kernel(
       for (int e = 0; e < 8; ++e)
         o[e] = (half_t)(((float)v[j][e] - mean) * rstd * (float)g[e] + (float)b[e]);
       store8(Y + row * d + i * 8, o);
+      if (Y2 != nullptr) store8(Y2 + row * d + i * 8, o);
     }
   }
+}
+
+template <int THREADS, int MAXV>
+__global__ __launch_bounds__(THREADS) void add_layer_norm_kernel(
+    const half_t* __restrict__ H, const half_t* __restrict__ R, const half_t* __restrict__ gamma,
+    const half_t* __restrict__ beta, float eps, int d, half_t* __restrict__ Y,
+    half_t* __restrict__ Rout) {
+  add_layer_norm_body<THREADS, MAXV>(H, R, gamma, beta, eps, d, Y, Rout, nullptr, blockIdx.x);
 }
 
 }  // namespace dv

@@ -236,14 +236,14 @@ __device__ __forceinline__ void topk_load_keys(const half_t* __restrict__ logits
   }
 }
 
-__global__ __launch_bounds__(256) void topk_hist_kernel(const half_t* __restrict__ logits, int B, int n,
-                                                        unsigned* __restrict__ ws) {
+__device__ __forceinline__ void topk_hist_body(const half_t* __restrict__ logits, int B, int n,
+                                               unsigned* __restrict__ ws, int block_id) {
   // the 256 coarse bins are hot (most logits share a few exponents): aggregate them in
   // LDS and add each non-empty bin to memory once per workgroup
   __shared__ unsigned s_coarse[kTopkCoarse];
   s_coarse[threadIdx.x] = 0u;
   __syncthreads();
-  const int i0 = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+  const int i0 = (block_id * 256 + threadIdx.x) * 8;
   if (i0 < n) {
     unsigned key[8];
     topk_load_keys(logits, B, n, i0, key);
@@ -256,6 +256,11 @@ __global__ __launch_bounds__(256) void topk_hist_kernel(const half_t* __restrict
   __syncthreads();
   const unsigned c = s_coarse[threadIdx.x];
   if (c != 0u) atomicAdd(&ws[kTopkFine + threadIdx.x], c);
+}
+
+__global__ __launch_bounds__(256) void topk_hist_kernel(const half_t* __restrict__ logits, int B, int n,
+                                                        unsigned* __restrict__ ws) {
+  topk_hist_body(logits, B, n, ws, blockIdx.x);
 }
 
 // Inclusive prefix sum over the 256 threads of a workgroup (s_w: 4 words of LDS).
@@ -299,11 +304,11 @@ __device__ __forceinline__ void topk_find_threshold(const unsigned* __restrict__
   above = s_pair[3];
 }
 
-__global__ __launch_bounds__(256) void topk_count_kernel(const half_t* __restrict__ logits, int B, int n,
-                                                         int k, unsigned* __restrict__ ws) {
+__device__ __forceinline__ void topk_count_body(const half_t* __restrict__ logits, int B, int n, int k,
+                                                unsigned* __restrict__ ws, int block_id) {
   __shared__ unsigned s_w[4], s_pair[4], s_gt[4], s_eq[4];
   unsigned key[8];
-  const int i0 = (blockIdx.x * 256 + threadIdx.x) * 8;
+  const int i0 = (block_id * 256 + threadIdx.x) * 8;
   topk_load_keys(logits, B, n, i0, key);  // issued before the histogram reads
   unsigned T, above;
   topk_find_threshold(ws, (unsigned)k, s_w, s_pair, T, above);
@@ -325,27 +330,32 @@ __global__ __launch_bounds__(256) void topk_count_kernel(const half_t* __restric
   }
   __syncthreads();
   if (threadIdx.x == 0) {
-    ws[kTopkCountsOff + 2 * blockIdx.x] = s_gt[0] + s_gt[1] + s_gt[2] + s_gt[3];
-    ws[kTopkCountsOff + 2 * blockIdx.x + 1] = s_eq[0] + s_eq[1] + s_eq[2] + s_eq[3];
-    if (blockIdx.x == 0) {
+    ws[kTopkCountsOff + 2 * block_id] = s_gt[0] + s_gt[1] + s_gt[2] + s_gt[3];
+    ws[kTopkCountsOff + 2 * block_id + 1] = s_eq[0] + s_eq[1] + s_eq[2] + s_eq[3];
+    if (block_id == 0) {
       ws[kTopkMetaOff] = T;
       ws[kTopkMetaOff + 1] = (unsigned)k - above;  // ties to take, lowest index first
     }
   }
 }
 
-__global__ __launch_bounds__(256) void topk_emit_kernel(const half_t* __restrict__ logits, int B, int n,
-                                                        unsigned* __restrict__ ws,
-                                                        void* __restrict__ idx_out, int idx_bytes) {
+__global__ __launch_bounds__(256) void topk_count_kernel(const half_t* __restrict__ logits, int B, int n,
+                                                         int k, unsigned* __restrict__ ws) {
+  topk_count_body(logits, B, n, k, ws, blockIdx.x);
+}
+
+__device__ __forceinline__ void topk_emit_body(const half_t* __restrict__ logits, int B, int n,
+                                               unsigned* __restrict__ ws, void* __restrict__ idx_out,
+                                               int idx_bytes, int block_id, int nblocks) {
   __shared__ unsigned s_w[4], s_base[2];
   unsigned key[8];
-  const int i0 = (blockIdx.x * 256 + threadIdx.x) * 8;
+  const int i0 = (block_id * 256 + threadIdx.x) * 8;
   topk_load_keys(logits, B, n, i0, key);
   const unsigned T = ws[kTopkMetaOff], need = ws[kTopkMetaOff + 1];
   // columns above / at T in the workgroups before this one
   if (threadIdx.x < 2) {
     unsigned acc = 0;
-    for (int w = 0; w < (int)blockIdx.x; ++w) acc += ws[kTopkCountsOff + 2 * w + threadIdx.x];
+    for (int w = 0; w < block_id; ++w) acc += ws[kTopkCountsOff + 2 * w + threadIdx.x];
     s_base[threadIdx.x] = acc;
   }
   unsigned gt = 0, eq = 0;
@@ -377,8 +387,14 @@ __global__ __launch_bounds__(256) void topk_emit_kernel(const half_t* __restrict
     }
   }
   // clear the histograms for the next call (nobody reads them in this kernel)
-  const int nthreads = gridDim.x * 256;
-  for (int j = blockIdx.x * 256 + threadIdx.x; j < kTopkFine + kTopkCoarse; j += nthreads) ws[j] = 0u;
+  const int nthreads = nblocks * 256;
+  for (int j = block_id * 256 + threadIdx.x; j < kTopkFine + kTopkCoarse; j += nthreads) ws[j] = 0u;
+}
+
+__global__ __launch_bounds__(256) void topk_emit_kernel(const half_t* __restrict__ logits, int B, int n,
+                                                        unsigned* __restrict__ ws,
+                                                        void* __restrict__ idx_out, int idx_bytes) {
+  topk_emit_body(logits, B, n, ws, idx_out, idx_bytes, blockIdx.x, gridDim.x);
 }
 
 }  // namespace dv

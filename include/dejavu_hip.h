@@ -250,6 +250,61 @@ DV_API int dv_add_layer_norm_f16(const void* h, const void* residual, const void
                                  const void* beta, float eps, int rows, int d, void* y,
                                  void* residual_out, void* stream);
 
+/*
+ * One decode step (batch 1, one new token) of a whole sparse block in nine
+ * launches: add+LayerNorm 1, back-fill window step, QKV of the active heads with
+ * cache scatter, attention, out_proj, add+LayerNorm 2, the sparse MLP, and beside
+ * them the MLP top-k for this layer and both predictors (+ head top-k) for the
+ * next layer.  Same arithmetic, kernel bodies and results as the separate entry
+ * points called in the order of BlockMlpAttSparse.forward,
+ * Dejavu/src/models/modules/block_dejavu.py:555-663 (mixer:
+ * Dejavu/src/models/modules/mha_dejavu.py:1283-1511, mlp:
+ * Dejavu/src/ops/fused_dense_sparse_dejavu.py:889-951).
+ * Steps that flush the window (every 16th token, all heads and all 16 tokens)
+ * are not taken by this entry point: callers run them through the separate ones.
+ */
+typedef struct dvSparseLayerArgs {
+  /* shapes */
+  int d, ffn, H, hd;      /* hidden, MLP width, heads, head_dim (64 or 128)            */
+  int r_att, r_mlp;       /* predictor ranks                                           */
+  int K, Hk, att_k;       /* active neurons; heads computed now; heads predicted next  */
+  int S;                  /* KV cache capacity                                         */
+  int counter;            /* window position of this token, 0..14                      */
+  int n_len;              /* cached positions to attend, newest token included         */
+  float eps1, eps2, softmax_scale;
+  /* inputs (device, fp16 unless stated) */
+  const void* hidden;     /* (d,) output of the previous block's MLP                   */
+  const void* residual;   /* (d,) residual stream, or NULL for the first block         */
+  const void *ln1_w, *ln1_b, *ln2_w, *ln2_b;
+  const void* Wqkv;       /* (3, H, hd, d)                                             */
+  const void* bqkv;       /* (3, H, hd) or NULL                                        */
+  const void* Wout_t;     /* (H*hd, d): out_proj.weight transposed                     */
+  const void* bout;       /* (d,) or NULL                                              */
+  const void *att_Wa, *att_Wb; /* (r_att, d), (H, r_att)                               */
+  const void *W1, *b1;    /* (ffn, d), (ffn,) or NULL                                  */
+  const void *W2t, *b2;   /* (ffn, d): fc2.weight transposed; (d,) or NULL             */
+  const void *mlp_Wa, *mlp_Wb; /* (r_mlp, d), (ffn, r_mlp)                             */
+  const void* head_idx;   /* (Hk,) int32 heads to compute                              */
+  const void* mlp_logit_in; /* (ffn,) predictor logits for THIS layer's MLP            */
+  const void* cache_offset; /* int32[1]: cache position of window token 0             */
+  /* state, updated in place */
+  void *k_cache, *v_cache; /* (1, H, hd/8, S, 8), (1, H, S, hd)                        */
+  void* x_cache;          /* (16, d) LayerNorm-1 outputs of the window                 */
+  void* tracker;          /* (H, 16) int32                                             */
+  /* outputs */
+  void* hidden_out;       /* (d,) MLP output                                           */
+  void* residual_out;     /* (d,) residual stream after attention                      */
+  void* mlp_logit_out;    /* (ffn,) logits for the NEXT layer's MLP                    */
+  void* att_idx_out;      /* (att_k,) int32 heads for the NEXT layer                   */
+  void* mlp_idx_out;      /* (K,) int64 neurons used by this layer                     */
+  /* scratch: dv_sparse_layer_workspace_bytes() bytes, zero-filled before first use */
+  void* workspace;
+  size_t workspace_bytes;
+} dvSparseLayerArgs;
+
+DV_API size_t dv_sparse_layer_workspace_bytes(const dvSparseLayerArgs* args);
+DV_API int dv_sparse_layer_decode_f16(const dvSparseLayerArgs* args, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

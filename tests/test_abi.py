@@ -23,10 +23,13 @@ def test_header_declares_symbols():
 def test_library_exports_every_declared_symbol():
     from dejavu_amd import _lib
 
+    from dejavu_amd import fused_layer  # noqa: F401  (binds the struct-taking entry points)
+
+    struct_entry_points = {"dv_sparse_layer_workspace_bytes", "dv_sparse_layer_decode_f16"}
     for name in declared_symbols():
         assert hasattr(_lib.lib, name), f"{name} declared in the header but not exported"
-        assert name in _lib.SIGNATURES, f"{name} has no ctypes signature"
-    assert set(_lib.SIGNATURES) == set(declared_symbols())
+        assert name in _lib.SIGNATURES or name in struct_entry_points, f"{name} has no ctypes signature"
+    assert set(_lib.SIGNATURES) | struct_entry_points == set(declared_symbols())
     assert _lib.lib.dv_version() >= 100
     assert _lib.lib.dv_error_string(0) == b"ok"
 

@@ -92,3 +92,57 @@ def test_sparse_block_decode_step_matches_oracle():
     kcd, vcd = ip.key_value_memory_dict[2]
     assert np.array_equal(np16(vcd), vn), "value cache after the step differs"
     assert_close(np16(kcd), kn, "key cache after the step")
+
+
+@pytest.mark.parametrize("d,H,ffn,r", [(768, 12, 3072, 128), (1024, 8, 4096, 1000)])
+def test_fused_layer_equals_module_by_module_path(d, H, ffn, r):
+    """The nine-launch fused block step and the module-by-module path run the same kernel
+    bodies: outputs, predictions, caches and window state must agree bit for bit over a
+    whole back-fill window (the flush step falls back to the modules in both)."""
+    import copy
+
+    from dejavu_amd.block import create_sparse_block, init_block_synthetic
+    from dejavu_amd.modules import InferenceParams
+    from dejavu_amd.workloads import pack_k_cache
+
+    K, Hk, S = 512, 3, 96
+    hd = d // H
+    blk_a = create_sparse_block(d, ffn, H, r, K, r, Hk, layer_idx=0)
+    init_block_synthetic(blk_a, seed=3)
+    with torch.no_grad():
+        g = torch.Generator().manual_seed(11)
+        for n in (blk_a.norm1, blk_a.norm2):
+            n.weight.copy_((1 + 0.1 * torch.randn(d, generator=g)).half())
+            n.bias.copy_((0.1 * torch.randn(d, generator=g)).half())
+        blk_a.mixer.Wqkv.bias.copy_((0.1 * torch.randn(3 * d, generator=g)).half())
+    blk_b = copy.deepcopy(blk_a)
+    blk_a.use_fused_layer, blk_b.use_fused_layer = True, False
+    g = torch.Generator().manual_seed(12)
+    t0 = 40
+    kc = pack_k_cache(torch.randn(1, H, S, hd, generator=g).half())
+    vc = torch.randn(1, H, S, hd, generator=g).half()
+    ips = []
+    for _ in range(2):
+        ip = InferenceParams(max_sequence_len=S, max_batch_size=1, sequence_len_offset=t0)
+        ip.key_value_memory_dict[0] = (kc.clone().cuda(), vc.clone().cuda())
+        ips.append(ip)
+    for step in range(20):
+        hs = torch.randn(1, 1, d, generator=g).half().cuda()
+        res = torch.randn(1, 1, d, generator=g).half().cuda()
+        head_idx = torch.sort(torch.randperm(H, generator=g)[:Hk]).values.int().cuda()
+        logit = (torch.randn(ffn, generator=g) * 4).half().cuda()
+        print(f"case fused vs modules d={d} step={step} counter={blk_a.mixer.counter}", flush=True)
+        outs = []
+        with torch.no_grad():
+            for blk, ip in ((blk_a, ips[0]), (blk_b, ips[1])):
+                outs.append(blk(hs, res, mixer_kwargs={"inference_params": ip}, head_idx=head_idx, mlp_sp_logit=logit))
+        torch.cuda.synchronize()
+        for name, xa, xb in zip(("hidden", "residual", "next_logit", "next_att_idx"), outs[0], outs[1]):
+            assert torch.equal(xa.reshape(-1), xb.reshape(-1)), f"step {step}: {name} differs"
+        assert blk_a.mixer.counter == blk_b.mixer.counter
+        assert torch.equal(blk_a.mixer.tracker, blk_b.mixer.tracker) and torch.equal(blk_a.mixer.x_cache[:max(1, blk_a.mixer.counter)],
+                                                                                     blk_b.mixer.x_cache[:max(1, blk_b.mixer.counter)])
+        for ca, cb in zip(ips[0].key_value_memory_dict[0], ips[1].key_value_memory_dict[0]):
+            assert torch.equal(ca, cb), f"step {step}: caches differ"
+        for ip in ips:
+            ip.sequence_len_offset += 1

@@ -168,11 +168,11 @@ def test_gather_gemv_edge_cases(ops):
 
 
 def test_reference_style_assertions(ops):
-    x = torch.zeros(5, 64, dtype=torch.float16, device="cuda")
+    x = torch.zeros(65, 64, dtype=torch.float16, device="cuda")
     W = torch.zeros(128, 64, dtype=torch.float16, device="cuda")
     idx = torch.arange(8, device="cuda")
     with pytest.raises(AssertionError):
-        ops.gather_gemv(x, W, idx)  # batch 5 not in 1..4
+        ops.gather_gemv(x, W, idx)  # batch 65 is beyond the supported 1..64
     with pytest.raises(AssertionError):
         ops.gather_gemv(x[:1].float(), W, idx)  # dtype mismatch
 
