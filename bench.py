@@ -222,7 +222,7 @@ def main():
     device = torch.device("cuda:0")
     layers = build_layers(cfg, batch, device)
     defer = args.defer and (not args.single_stream) and args.layers_per_graph == N_LAYERS \
-        and not args.no_graph
+        and not args.no_graph and args.steps % N_LAYERS == 0 and args.warmup % N_LAYERS == 0
     for L in layers:
         L["block"].mlp.defer_predictor_join = defer
 
@@ -234,6 +234,10 @@ def main():
             dv_modules.join_side_stream()
         torch.cuda.synchronize()
         graphs = []
+        # a graph of all three layers can only be replayed whole: fall back to one graph per
+        # layer when the step counts are not multiples of three, so exactly --steps steps run
+        if args.steps % N_LAYERS or args.warmup % N_LAYERS:
+            args.layers_per_graph = 1
         if not args.no_graph and args.layers_per_graph == 1:
             for L in layers:
                 g = torch.cuda.CUDAGraph()
@@ -242,7 +246,6 @@ def main():
                 graphs.append(g)
             torch.cuda.synchronize()
         elif not args.no_graph:
-            assert args.steps % N_LAYERS == 0 and args.warmup % N_LAYERS == 0
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g):
                 for L in layers:
@@ -307,7 +310,8 @@ def main():
         "config": {"workload": f"{args.config} sparse decode layer", "d": cfg["d"], "ffn": cfg["ffn"],
                    "heads": cfg["H"], "head_dim": cfg["hd"], "K": cfg["K"], "active_heads": cfg["Hk"],
                    "predictor_rank": cfg["r"], "kv_len": cfg["S"], "batch": batch,
-                   "layers_cycled": N_LAYERS, "hip_graph": not args.no_graph},
+                   "layers_cycled": N_LAYERS, "hip_graph": not args.no_graph,
+                   "layers_per_graph": 0 if args.no_graph else args.layers_per_graph},
         "roofline": roofline,
         "cpu_baseline": cpu,
         "layer": {"algorithmic_MB": round(layer_bytes / 1e6, 1), "GB/s": round(layer_bytes / us_per_layer / 1e3, 1),

@@ -105,21 +105,16 @@ int gather_rows_b(const half_t* x, const half_t* W, int64_t ldw, const half_t* b
 // ---- gathered column GEMV (fc2 / out_proj over transposed weights) ----------
 struct ColsPlan {
   int col_tiles, groups, rows_per_block;
-  bool fused;
 };
 
-int tuning_env(const char* name, int fallback) {
-  const char* v = getenv(name);
-  return v ? atoi(v) : fallback;
-}
+// Three workgroups per compute unit measured best for the split over gathered
+// rows; the partial sums are combined by a second, deterministic pass.
+constexpr int kColsBlocksPerCu = 3;
 
 ColsPlan plan_cols(int N, int M) {
   ColsPlan p;
   p.col_tiles = (N + kColTile - 1) / kColTile;
-  static const int blocks_per_cu = tuning_env("DV_COLS_BLOCKS_PER_CU", 3);
-  static const int fused = tuning_env("DV_COLS_FUSED", 0);
-  p.fused = fused != 0;
-  const int target_blocks = compute_units() * blocks_per_cu;
+  const int target_blocks = compute_units() * kColsBlocksPerCu;
   int groups = (target_blocks + p.col_tiles - 1) / p.col_tiles;
   int max_groups = (M + 15) / 16;  // at least 16 rows per workgroup
   if (max_groups < 1) max_groups = 1;
@@ -150,7 +145,7 @@ void launch_cols(const ColsPlan& p, const half_t* x, int64_t ldx, int x_expanded
                  int64_t ldw, const half_t* bias, const void* idx, int blk, int N, int Z, int M,
                  float* partial, unsigned* counters, half_t* y, hipStream_t s) {
   dim3 grid(p.col_tiles, p.groups);
-  if (p.fused || p.groups == 1) {
+  if (p.groups == 1) {
     hipLaunchKernelGGL((gather_cols_kernel<B, 8, IDX64, BLOCKED, true>), grid, dim3(256), 0, s, x,
                        ldx, x_expanded, W, ldw, bias, idx, blk, N, Z, M, p.rows_per_block, partial,
                        counters, y);
