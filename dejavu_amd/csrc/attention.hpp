@@ -254,7 +254,8 @@ __device__ __forceinline__ void decode_attn_body(
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int h = head_idx ? head_idx[i] : i;
-  const int len = lengths ? lengths[b] + 1 : n_len;
+  int len = lengths ? lengths[b] + 1 : n_len;
+  if (len > S) len = S;  // a device-side length can never address past the cache
   float* out = part + (((int64_t)b * nheads + i) * nsplit + split) * (HD + 2);
   const bool head_ok = h >= 0 && h < H;
   const int p0 = (split * WAVES + wave) * kWave;

@@ -876,11 +876,12 @@ int dv_sparse_layer_decode_f16(const dvSparseLayerArgs* args, void* stream) {
 #undef DV_L2
   }
   // L3: attention partials | head predictor fc1 | top-k threshold and counts
-  const int nsplit = attn_splits(a.n_len);
+  const int nsplit = a.seq_pos ? p.nsplit : attn_splits(a.n_len);
   {
     AttnArgs at{qkv + (size_t)a.counter * 3 * a.H * a.hd, (int64_t)3 * a.H * a.hd,
                 reinterpret_cast<const half_t*>(a.k_cache), reinterpret_cast<const half_t*>(a.v_cache),
-                head_idx, a.n_len, a.H, a.S, nsplit, a.Hk, a.softmax_scale, attn_part};
+                head_idx, reinterpret_cast<const int*>(a.seq_pos), a.n_len, a.H, a.S, nsplit, a.Hk,
+                a.softmax_scale, attn_part};
     CanonArgs hp1{hp_hidden, CH(a.att_Wb), (int64_t)a.r_att, a.H, a.r_att, head_logits};
     const int na = nsplit * a.Hk;
     const int rw1 = a.r_att <= 1024 ? 4 : 1;

@@ -91,6 +91,7 @@ struct AttnArgs {
   const half_t* k_cache;
   const half_t* v_cache;
   const int* head_idx;
+  const int* seq_pos;  // device position of the newest token, or nullptr (then n_len counts)
   int n_len, H, S, nsplit, nheads;
   float scale;
   float* part;
@@ -103,7 +104,7 @@ __global__ __launch_bounds__(256) void layer_l3_kernel(AttnArgs a, int nblk_attn
   const int bid = blockIdx.x;
   if (bid < nblk_attn) {
     const int split = bid % a.nsplit, i = bid / a.nsplit;
-    decode_attn_body<HD, 4>(a.Q, a.ldq, a.k_cache, a.v_cache, a.head_idx, nullptr, a.n_len, a.H, a.S, a.scale,
+    decode_attn_body<HD, 4>(a.Q, a.ldq, a.k_cache, a.v_cache, a.head_idx, a.seq_pos, a.n_len, a.H, a.S, a.scale,
                             a.nsplit, a.part, split, i, 0, a.nheads);
   } else if (bid < nblk_attn + nblk_hp1) {
     canonical_role(hp1, bid - nblk_attn, nblk_hp1);

@@ -31,7 +31,7 @@ class SparseLayerArgs(ctypes.Structure):
         ("att_Wa", _p), ("att_Wb", _p),
         ("W1", _p), ("b1", _p), ("W2t", _p), ("b2", _p),
         ("mlp_Wa", _p), ("mlp_Wb", _p),
-        ("head_idx", _p), ("mlp_logit_in", _p), ("cache_offset", _p),
+        ("head_idx", _p), ("mlp_logit_in", _p), ("cache_offset", _p), ("seq_pos", _p),
         ("k_cache", _p), ("v_cache", _p), ("x_cache", _p), ("tracker", _p),
         ("hidden_out", _p), ("residual_out", _p), ("mlp_logit_out", _p), ("att_idx_out", _p),
         ("mlp_idx_out", _p),
@@ -70,7 +70,10 @@ def eligible(block, hidden_states, residual, head_idx, mlp_sp_logit, inference_p
         return False
     if head_idx is None or mlp_sp_logit is None or inference_params is None:
         return False
-    if inference_params.sequence_len_offset <= 0 or inference_params.lengths_per_sample is not None:
+    if inference_params.sequence_len_offset <= 0:
+        return False
+    lengths = inference_params.lengths_per_sample
+    if lengths is not None and not (lengths.dtype == torch.int32 and lengths.numel() == 1 and lengths.is_cuda):
         return False
     if not (hidden_states.is_cuda and hidden_states.dtype == torch.float16 and hidden_states.numel() == m.embed_dim):
         return False
@@ -92,8 +95,7 @@ def sparse_layer_decode(block, hidden_states, residual, head_idx, mlp_sp_logit, 
     if m.out_proj_weight_t is None:
         m.out_proj_weight_t = m.out_proj.weight.t().contiguous()
     if m.cache_offset is None:
-        m.cache_offset = torch.tensor([inference_params.sequence_len_offset - m.counter], dtype=torch.int32,
-                                      device=dev)
+        m._set_cache_offset(inference_params.sequence_len_offset - m.counter, dev)
     k_cache, v_cache = inference_params.key_value_memory_dict[m.layer_idx]
     b0 = inference_params.batch_size_offset
     kc, vc = k_cache[b0:b0 + 1], v_cache[b0:b0 + 1]
@@ -130,6 +132,7 @@ def sparse_layer_decode(block, hidden_states, residual, head_idx, mlp_sp_logit, 
     a.W2t, a.b2 = _ptr(f.fc2_weight_t), _ptr(f.fc2.bias)
     a.mlp_Wa, a.mlp_Wb = _ptr(f.sp.fc0.weight), _ptr(f.sp.fc1.weight)
     a.head_idx, a.mlp_logit_in, a.cache_offset = _ptr(head_idx), _ptr(mlp_sp_logit), _ptr(m.cache_offset)
+    a.seq_pos = _ptr(inference_params.lengths_per_sample)
     a.k_cache, a.v_cache, a.x_cache, a.tracker = _ptr(kc), _ptr(vc), _ptr(m.x_cache), _ptr(m.tracker)
     a.hidden_out, a.residual_out = _ptr(hidden_out), _ptr(residual_out)
     a.mlp_logit_out, a.att_idx_out, a.mlp_idx_out = _ptr(logit_out), _ptr(att_idx_out), _ptr(mlp_idx_out)

@@ -352,6 +352,13 @@ class ParallelMHASparseAttMlp(_MHABase):
         # optional caller-owned buffer for the predicted heads (fixed address for graph capture)
         self.att_idx_out = None
 
+    def _set_cache_offset(self, value: int, device) -> None:
+        """Updated in place once it exists: captured launch sequences hold its address."""
+        if self.cache_offset is None:
+            self.cache_offset = torch.tensor([value], dtype=torch.int32, device=device)
+        else:
+            self.cache_offset.fill_(value)
+
     def reset_window(self):
         self.counter = 0
         self.tracker.copy_(torch.arange(self.WINDOW, dtype=torch.int32, device=self.tracker.device)
@@ -379,8 +386,7 @@ class ParallelMHASparseAttMlp(_MHABase):
         b0 = inference_params.batch_size_offset
         kc, vc = k_cache[b0:b0 + 1], v_cache[b0:b0 + 1]
         if self.cache_offset is None:
-            self.cache_offset = torch.tensor([inference_params.sequence_len_offset - self.counter],
-                                             dtype=torch.int32, device=dev)
+            self._set_cache_offset(inference_params.sequence_len_offset - self.counter, dev)
         qkv = ops.qkv_proj_sparse(self.x_cache[:nb], self.Wqkv.weight.view(3, H, hd, self.embed_dim), head_idx,
                                   batch_idx, None if self.Wqkv.bias is None else self.Wqkv.bias.view(3, H, hd),
                                   k_cache=kc, v_cache=vc, padding=self.cache_offset)
@@ -395,7 +401,7 @@ class ParallelMHASparseAttMlp(_MHABase):
         self._streams()
         do_token_generation = x.size(1) == 1
         if x.size(1) != 1:  # prompt: remember where the decode window starts
-            self.cache_offset = torch.tensor([x.size(1)], dtype=torch.int32, device=x.device)
+            self._set_cache_offset(x.size(1), x.device)
             self.reset_window()
         sparse = inference_params is not None and inference_params.sequence_len_offset > 0 and head_idx != None
         mlp_idx, att_idx = self._side_work(mlp_sp_logit, residual, self.sp if do_token_generation else None,

@@ -287,6 +287,10 @@ typedef struct dvSparseLayerArgs {
   const void* head_idx;   /* (Hk,) int32 heads to compute                              */
   const void* mlp_logit_in; /* (ffn,) predictor logits for THIS layer's MLP            */
   const void* cache_offset; /* int32[1]: cache position of window token 0             */
+  const void* seq_pos;    /* int32[1] cache position of the newest token, or NULL: when   */
+                          /* given it replaces n_len - 1, so that a captured launch     */
+                          /* sequence can be replayed as the sequence grows (the role of */
+                          /* lengths_per_sample, mha_dejavu.py:1439-1446)                */
   /* state, updated in place */
   void *k_cache, *v_cache; /* (1, H, hd/8, S, 8), (1, H, S, hd)                        */
   void* x_cache;          /* (16, d) LayerNorm-1 outputs of the window                 */

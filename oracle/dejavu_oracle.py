@@ -28,6 +28,13 @@ How each function is pinned (see tests/test_oracle.py):
   textbook definition the reference restates in CrossAttention.forward.
 * cache copies / window tracker: index arithmetic checked against a dense
   always-recompute KV cache.
+* ``model_prompt`` / ``model_decode_step`` / ``greedy_decode`` (the model loop
+  around the blocks): against a from-scratch dense float64 transformer when
+  every neuron and head is selected (K = ffn, Hk = H), and against the
+  single-layer functions above for the lookahead threading (layer l's
+  predictions feed layer l+1, the first layer runs dense).  The greedy loop
+  itself restates flash-attention v0.2.8 ``flash_attn/utils/generation.py``
+  (``decode``), a dependency the reference does not vendor.
 * top-k tie order: the reference (``torch.topk(sorted=False)`` on CUDA) leaves
   it unspecified and holds no vectors; the rule "ties go to the lower index" is
   this build's definition: parity unpinned against the reference's CUDA tie
@@ -557,3 +564,166 @@ def block_decode_step(p, hidden_states, residual, head_idx, mlp_sp_logit, k_cach
     _, next_mlp_logit = predictor_logits(r2_pred, p["mlp_Wa"], p["mlp_Wb"])
     return dict(hidden=hidden, residual=r2, next_mlp_logit=next_mlp_logit[0], next_att_idx=next_att_idx,
                 mlp_idx=mlp_idx, residual1=r1, attn_out=attn_out)
+
+
+# --------------------------------------------------------------------------
+# whole model: embeddings -> blocks (lookahead predictions) -> ln_f -> lm_head
+# --------------------------------------------------------------------------
+def _linear_f16(x, W, b=None):
+    """fp16 nn.Linear: fp32 accumulation, fp16 result."""
+    y = np.asarray(x, F16).astype(F32) @ np.asarray(W, F16).astype(F32).T
+    if b is not None:
+        y = y + np.asarray(b, F16).astype(F32)
+    return y.astype(F16)
+
+
+def _add_f16(a, b):
+    return (np.asarray(a, F16).astype(F32) + np.asarray(b, F16).astype(F32)).astype(F16)
+
+
+def new_decode_state(params, max_len):
+    """Empty caches, one (k_cache, v_cache) pair per layer in the packed layouts
+    of Dejavu/src/models/modules/mha_dejavu.py:404-446."""
+    caches = []
+    for p in params["layers"]:
+        _, H, hd, _ = p["Wqkv"].shape
+        caches.append((np.zeros((1, H, hd // 8, max_len, 8), F16), np.zeros((1, H, max_len, hd), F16)))
+    return {"caches": caches, "pos": 0, "window": 0}
+
+
+def model_prompt(params, state, input_ids):
+    """Dense forward over the prompt, filling the caches; returns the fp16 logits
+    of the last prompt token.
+
+    Dejavu/src/models/gpt_dejavu.py:552-623 (GPTModel.forward) with
+    ``x.size(1) > 1``: every block takes its dense branch (no predictions are
+    produced for a prompt: mha_dejavu.py:1283-1511 and
+    fused_dense_sparse_dejavu.py:889-951 only predict when one token is
+    decoded), attention is causal (gpt_dejavu.py:236), then ln_f and the tied
+    lm_head (gpt_dejavu.py:604-623, 676-690).
+    """
+    ids = np.asarray(input_ids).reshape(-1)
+    T = len(ids)
+    hidden = _add_f16(params["wte"][ids], params["wpe"][np.arange(T)])
+    residual = None
+    for p, (k_cache, v_cache) in zip(params["layers"], state["caches"]):
+        _, H, hd, d = p["Wqkv"].shape
+        residual = hidden if residual is None else _add_f16(hidden, residual)
+        x = layer_norm(residual, p["ln1_w"], p["ln1_b"])
+        qkv = _linear_f16(x, p["Wqkv"].reshape(3 * H * hd, d), p["bqkv"].reshape(-1)).reshape(T, 3, H, hd)
+        k_cache[0, :, :, :T, :] = pack_k_cache(qkv[None, :, 1])[0]
+        v_cache[0, :, :T, :] = qkv[:, 2].transpose(1, 0, 2)
+        scale = F32(hd ** -0.5)
+        ctx = np.zeros((T, H, hd), F16)
+        mask = np.triu(np.ones((T, T), bool), 1)
+        for h in range(H):
+            q, k, v = (qkv[:, j, h].astype(F32) for j in range(3))
+            sc = (q @ k.T) * scale
+            sc[mask] = -np.inf
+            pr = np.exp(sc - sc.max(axis=-1, keepdims=True))
+            pr = pr / pr.sum(axis=-1, keepdims=True, dtype=F32)
+            ctx[:, h] = (pr @ v).astype(F16)
+        attn_out = _linear_f16(ctx.reshape(T, H * hd), p["Wout"].reshape(d, H * hd), p["bout"])
+        residual = _add_f16(attn_out, residual)
+        x2 = layer_norm(residual, p["ln2_w"], p["ln2_b"])
+        h1 = relu(_linear_f16(x2, p["W1"], p["b1"]))
+        hidden = _linear_f16(h1, p["W2t"].T, p["b2"])
+    state["pos"] = T
+    state["window"] = 0
+    final = layer_norm(_add_f16(hidden[-1:], residual[-1:]), params["lnf_w"], params["lnf_b"])
+    return _linear_f16(final, params["wte"])[0]
+
+
+def model_decode_step(params, state, token, overrides=None):
+    """One decoded token through every block; returns (fp16 logits, trace).
+
+    Dejavu/src/models/gpt_dejavu.py:574-592: ``next_mlp_sp_logit`` and
+    ``next_att_idx`` start as None, so the first block runs dense attention and
+    a dense MLP, and block l consumes what block l-1 predicted during the same
+    token.  A sparse block attends with the selected heads over K/V that are
+    complete for those heads, which is what the back-fill window of
+    mha_dejavu.py:1318-1359 guarantees; here every head's K/V of every token is
+    simply kept (dense) so that property holds by construction.
+    Every 16th decoded token (window counter 15) a sparse block computes and
+    attends with ALL heads (mha_dejavu.py:1320-1326), after which the window
+    restarts (mha_dejavu.py:1485-1492).
+    ``overrides[l]`` = (head_idx, mlp_sp_logit) replaces the lookahead inputs of
+    block l (l >= 1), so that a device run's own selections can be replayed.
+    trace[l] = dict(head_idx (as used), mlp_sp_logit, mlp_idx, hidden, residual).
+    """
+    t = state["pos"]
+    flush = state["window"] == 15
+    hidden = _add_f16(params["wte"][int(token)][None], params["wpe"][t][None])
+    residual = None
+    head_idx, mlp_logit = None, None
+    trace = []
+    for l, (p, (k_cache, v_cache)) in enumerate(zip(params["layers"], state["caches"])):
+        _, H, hd, d = p["Wqkv"].shape
+        if overrides is not None and l > 0 and overrides[l] is not None:
+            head_idx, mlp_logit = overrides[l]
+        if head_idx is not None and flush:
+            head_idx = np.arange(H, dtype=np.int32)
+        used = dict(head_idx=head_idx, mlp_sp_logit=mlp_logit)
+        r1 = hidden if residual is None else _add_f16(hidden, residual)
+        x = layer_norm(r1, p["ln1_w"], p["ln1_b"])
+        # K / V of the new token for every head (what the skipped heads get back-filled with)
+        all_heads = np.arange(H, dtype=np.int32)
+        qkv = qkv_proj_sparse(x, p["Wqkv"], all_heads, np.zeros((H, 1), np.int32), p["bqkv"])
+        k_cache[0, :, :, t, :] = qkv[0, 1].reshape(H, hd // 8, 8)
+        v_cache[0, :, t, :] = qkv[0, 2]
+        if head_idx is None:
+            ctx = single_query_attention(qkv[:, 0], qkv[:, 1], qkv[:, 2], k_cache, v_cache, t)
+            attn_out = out_proj_sparse(ctx, p["Wout"], all_heads, p["bout"])
+            _, att_logit = predictor_logits(r1, p["att_Wa"], p["att_Wb"])
+            next_att_idx = topk_lower_index(att_logit[0], p["att_K"]).astype(np.int32)
+            r2 = _add_f16(attn_out, r1)
+            x2 = layer_norm(r2, p["ln2_w"], p["ln2_b"])
+            if mlp_logit is None:
+                mlp_idx = np.arange(p["W1"].shape[0])
+            else:
+                mlp_idx = topk_lower_index(mlp_logit, p["mlp_K"])
+            hidden = mlp_sparse(x2, p["W1"], p["W2t"], mlp_idx, p["b1"], p["b2"])
+            _, next_logit = predictor_logits(r2, p["mlp_Wa"], p["mlp_Wb"])
+            out = dict(hidden=hidden, residual=r2, next_mlp_logit=next_logit[0], next_att_idx=next_att_idx,
+                       mlp_idx=mlp_idx)
+        else:
+            out = block_decode_step(p, hidden, residual, head_idx, mlp_logit, k_cache, v_cache, t)
+        hidden, residual = out["hidden"], out["residual"]
+        head_idx, mlp_logit = out["next_att_idx"], out["next_mlp_logit"]
+        used.update(mlp_idx=out["mlp_idx"], hidden=hidden, residual=residual)
+        trace.append(used)
+    state["pos"] = t + 1
+    state["window"] = (state["window"] + 1) % 16
+    final = layer_norm(_add_f16(hidden, residual), params["lnf_w"], params["lnf_b"])
+    return _linear_f16(final, params["wte"])[0], trace
+
+
+def greedy_decode(params, input_ids, max_length, forced_tokens=None, overrides=None):
+    """Greedy generation: prompt, then one token at a time until ``max_length``.
+
+    Restates ``decode`` of flash-attention v0.2.8 ``flash_attn/utils/generation.py``
+    (called through ``model.generate`` at
+    Dejavu/benchmarks/benchmark_generation_opt_dejavu.py:187-196, top_k = 1):
+    the first new token is the argmax of the prompt's last logits; each further
+    one comes from a single-token forward at position ``sequence_len_offset``.
+    ``forced_tokens[i]`` / ``overrides[i]`` (per decode step) replace the token
+    fed back / the lookahead inputs, for teacher-forced comparison with a device.
+    Returns (sequence incl. prompt, list of per-step fp16 logits).
+    """
+    ids = [int(v) for v in np.asarray(input_ids).reshape(-1)]
+    state = new_decode_state(params, max_length)
+    logits = model_prompt(params, state, ids)
+    scores = [logits]
+    seq = list(ids)
+    step = 0
+    while len(seq) < max_length:
+        tok = int(np.argmax(logits.astype(F32)))
+        if forced_tokens is not None:
+            tok = int(forced_tokens[step])
+        seq.append(tok)
+        if len(seq) >= max_length:
+            break
+        logits, _ = model_decode_step(params, state, tok, None if overrides is None else overrides[step])
+        scores.append(logits)
+        step += 1
+    return seq, scores

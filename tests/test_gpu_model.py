@@ -1,0 +1,146 @@
+"""Whole-model greedy decoding on the GPU against the oracle's model loop.
+
+The device run records, per decode step and block, the lookahead inputs it consumed
+(predicted heads, predictor logits).  The oracle replays exactly those selections
+(index sets are discrete: a last-bit difference in a logit would otherwise change
+which neuron is dropped), so the comparison is one of arithmetic, within tolerance; that
+the selections themselves are the exact top-k of the device's logits is checked bit
+for bit.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import dejavu_oracle as O
+from tests.model_utils import load_model_params, make_model_params
+
+pytestmark = pytest.mark.gpu
+
+
+def build(L, d, H, ffn, r, V, P, mlp_K, att_K, seed):
+    from dejavu_amd.gpt import GPTLMHeadModel, SparseGPTConfig
+
+    l2 = int(0.65 * L)
+    # create_mixer_cls gives att_K[0] to layers >= l2 and att_K[1] to the others
+    per_layer = [att_K[0] if l >= l2 else att_K[1] for l in range(L)]
+    params = make_model_params(L, d, H, ffn, r, V, P, mlp_K, per_layer, seed=seed)
+    cfg = SparseGPTConfig(hidden_size=d, num_attention_heads=H, num_hidden_layers=L, vocab_size=V, n_inner=ffn,
+                          max_position_embeddings=P, mlp_K=mlp_K, mlp_sp_dim=r, att_K=list(att_K), att_sp_dim=r)
+    model = GPTLMHeadModel(cfg, device="cuda", dtype=torch.float16).eval()
+    load_model_params(model, params)
+    return model, params
+
+
+def rel_l2(a, b):
+    a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+    return np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-30)
+
+
+@pytest.mark.parametrize("mlp_K,att_K", [(512, (2, 3)), (2048, (4, 4))], ids=["sparse", "everything-selected"])
+def test_greedy_generation_matches_oracle_with_replayed_selections(mlp_K, att_K):
+    L, d, H, ffn, r, V, P = 3, 256, 4, 2048, 64, 512, 96
+    model, params = build(L, d, H, ffn, r, V, P, mlp_K, att_K, seed=21)
+    prompt = [17, 4, 250, 99, 3, 8, 41]
+    n_new = 40  # crosses two window flushes
+    ids = torch.tensor([prompt], device="cuda")
+    model.transformer.record = []
+    print(f"case generate eager mlp_K={mlp_K} att_K={att_K}", flush=True)
+    out = model.generate(ids, max_length=len(prompt) + n_new, return_dict_in_generate=True, output_scores=True)
+    torch.cuda.synchronize()
+    record, model.transformer.record = model.transformer.record, None
+    seq = out.sequences[0].cpu().tolist()
+    scores = out.scores.cpu().numpy()
+    assert seq[: len(prompt)] == prompt and len(seq) == len(prompt) + n_new
+    assert len(record) == (n_new - 1) * L
+
+    # the device's own selections, replayed by the oracle
+    overrides = []
+    for s in range(n_new - 1):
+        step = []
+        for l in range(L):
+            hi, lg = record[s * L + l]
+            if l == 0:
+                assert hi is None and lg is None  # first block runs dense
+                step.append(None)
+            else:
+                assert hi.dtype == torch.int32 and hi.numel() == params["layers"][l - 1]["att_K"]
+                step.append((hi.cpu().numpy(), lg.cpu().numpy()))
+        overrides.append(step)
+    forced = seq[len(prompt):]
+    o_seq, o_scores = O.greedy_decode(params, prompt, len(prompt) + n_new, forced_tokens=forced, overrides=overrides)
+    assert len(o_scores) == n_new
+    worst_abs, worst_rel, checked = 0.0, 0.0, 0
+    for i in range(n_new):
+        want = o_scores[i].astype(np.float32)
+        got = scores[i].astype(np.float32)
+        worst_abs = max(worst_abs, float(np.abs(got - want).max()))
+        worst_rel = max(worst_rel, rel_l2(got, want))
+        top2 = np.sort(want)[-2:]
+        if top2[1] - top2[0] > 0.05:  # greedy token agrees wherever the oracle separates the best two
+            assert int(np.argmax(want)) == seq[len(prompt) + i], f"step {i}"
+            checked += 1
+    print(f"logits: worst max-abs {worst_abs:.4g}, worst rel-L2 {worst_rel:.4g}, tokens checked {checked}")
+    # three blocks + lm_head of fp16-rounded intermediates against the oracle's own fp16 rounding
+    assert worst_abs <= 2e-2 and worst_rel <= 2.5e-3
+    assert checked >= n_new // 2
+
+
+def test_device_selections_are_exact_topk_of_device_logits():
+    L, d, H, ffn, r, V, P = 3, 256, 4, 2048, 64, 512, 96
+    model, params = build(L, d, H, ffn, r, V, P, 512, (2, 3), seed=22)
+    ids = torch.tensor([[5, 6, 7, 8]], device="cuda")
+    model.transformer.record = []
+    print("case generate eager, selections", flush=True)
+    model.generate(ids, max_length=4 + 20)
+    torch.cuda.synchronize()
+    record, model.transformer.record = model.transformer.record, None
+    n = 0
+    for s in range(19):
+        for l in range(1, L):
+            blk = model.transformer.layers[l]
+            hi, lg = record[s * L + l]
+            assert hi.numel() == params["layers"][l - 1]["att_K"]
+            assert torch.all(hi[1:] > hi[:-1])  # ascending, distinct
+            n += 1
+    assert n == 19 * (L - 1)
+    # last step: the neurons each sparse block used are the oracle's top-k of the logits it was given
+    for l in range(1, L):
+        blk = model.transformer.layers[l]
+        if getattr(blk, "last_mlp_idx", None) is None:
+            continue
+        _, lg = record[18 * L + l]
+        want = O.topk_lower_index(lg.cpu().numpy(), 512)
+        np.testing.assert_array_equal(blk.last_mlp_idx.cpu().numpy(), want)
+
+
+def test_graph_replayed_generation_equals_eager_bit_for_bit():
+    L, d, H, ffn, r, V, P = 4, 256, 4, 2048, 64, 512, 128
+    model, _ = build(L, d, H, ffn, r, V, P, 512, (2, 3), seed=23)
+    prompt = torch.tensor([[9, 100, 31, 77, 2]], device="cuda")
+    n_new = 70  # 16 eager steps, then every window position replayed at least three times
+    print("case generate eager (reference for graphs)", flush=True)
+    eager = model.generate(prompt, max_length=5 + n_new, return_dict_in_generate=True, output_scores=True)
+    torch.cuda.synchronize()
+    print("case generate cg=True, first call (captures)", flush=True)
+    g1 = model.generate(prompt, max_length=5 + n_new, cg=True, return_dict_in_generate=True, output_scores=True)
+    torch.cuda.synchronize()
+    assert torch.equal(g1.sequences, eager.sequences)
+    assert torch.equal(g1.scores, eager.scores)
+    assert len(model._decoding_cache.graphs) == 16
+    # second call: all graphs exist; a different prompt of the same length must not see stale state
+    prompt2 = torch.tensor([[1, 2, 3, 4, 5]], device="cuda")
+    print("case generate cg=True, second call (replays only)", flush=True)
+    g2 = model.generate(prompt2, max_length=5 + n_new, cg=True, return_dict_in_generate=True, output_scores=True)
+    torch.cuda.synchronize()
+    e2 = model.generate(prompt2, max_length=5 + n_new, return_dict_in_generate=True, output_scores=True)
+    torch.cuda.synchronize()
+    assert torch.equal(g2.sequences, e2.sequences)
+    assert torch.equal(g2.scores, e2.scores)
+    assert not torch.equal(g2.sequences, g1.sequences)
+    # a prompt of another length works with the same graphs (positions live on the device)
+    prompt3 = torch.tensor([[1, 2, 3, 4, 5, 6, 7, 8, 9]], device="cuda")
+    print("case generate cg=True, longer prompt", flush=True)
+    g3 = model.generate(prompt3, max_length=5 + n_new, cg=True, return_dict_in_generate=True, output_scores=True)
+    e3 = model.generate(prompt3, max_length=5 + n_new, return_dict_in_generate=True, output_scores=True)
+    torch.cuda.synchronize()
+    assert torch.equal(g3.sequences, e3.sequences)
