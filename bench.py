@@ -185,6 +185,74 @@ def cpu_baseline(torch, cfg, batch, L, timed=15, warm=3):
                       f"CPU index_select+matmul, fp32 compute from the same fp16 tensors"}
 
 
+def decode_bench(args):
+    """End-to-end greedy generation of a 40-layer OPT-13B-shaped model (all layers but the
+    first head- and MLP-sparse): 128-token prompt, 256 new tokens, decode steps replayed from
+    HIP graphs.  A step here is one generated token; prints its own JSON line."""
+    import torch
+
+    from dejavu_amd.block import init_block_synthetic
+    from dejavu_amd.gpt import GPTLMHeadModel, SparseGPTConfig
+    from dejavu_amd.workloads import CONFIGS
+
+    cfg = CONFIGS["opt-13b"]
+    layers, vocab, prompt_len, new_tokens = args.decode_layers, 50272, 128, args.steps
+    torch.cuda.set_device(0)
+    conf = SparseGPTConfig(hidden_size=cfg["d"], num_attention_heads=cfg["H"], num_hidden_layers=layers,
+                           vocab_size=vocab, n_inner=cfg["ffn"], max_position_embeddings=2048, mlp_K=cfg["K"],
+                           mlp_sp_dim=cfg["r"], att_K=[cfg["Hk"], cfg["Hk"]], att_sp_dim=cfg["r"],
+                           pad_vocab_size_multiple=8)
+    model = GPTLMHeadModel(conf, device="cuda", dtype=torch.float16).eval()
+    with torch.no_grad():
+        gen = torch.Generator(device="cuda")
+        gen.manual_seed(7)
+        for l, blk in enumerate(model.transformer.layers):
+            init_block_synthetic(blk, seed=100 + l)
+        for emb in (model.transformer.embeddings.word_embeddings, model.transformer.embeddings.position_embeddings):
+            tmp = torch.empty(emb.weight.shape, dtype=torch.float32, device="cuda")
+            tmp.normal_(0.0, 0.02, generator=gen)
+            emb.weight.copy_(tmp)
+        model.tie_weights()
+        ids = torch.randint(0, vocab, (1, prompt_len), generator=gen, device="cuda")
+        max_length = prompt_len + new_tokens
+
+        def run(cg, length=max_length):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            out = model.generate(ids, max_length=length, cg=cg, vocab_size=vocab)
+            torch.cuda.synchronize()
+            return time.perf_counter() - t0, out
+
+        for _ in range(max(1, args.warmup)):
+            run(True)  # first call captures the 16 graphs
+        t_total, seq_cg = min((run(True) for _ in range(3)), key=lambda r: r[0])
+        t_prompt, _ = min((run(True, prompt_len + 1) for _ in range(3)), key=lambda r: r[0])
+        t_eager, seq_eager = run(False)
+    same = bool(torch.equal(seq_cg, seq_eager))
+    decode_s = t_total - t_prompt
+    steps = new_tokens - 1
+    d, ffn, H, hd, r, K, Hk = (cfg[k] for k in ("d", "ffn", "H", "hd", "r", "K", "Hk"))
+    sparse_layer = (3 * Hk * hd * d + d * Hk * hd + 2 * K * d + d * r + r * ffn + d * r + r * H) * 2
+    dense_layer = (4 * d * d + 2 * d * ffn + d * r + r * ffn + d * r + r * H) * 2
+    token_bytes = dense_layer + (layers - 1) * sparse_layer + vocab * d * 2
+    out = {
+        "metric": "tokens_per_s, greedy decode, OPT-13B-shaped 40-layer sparse model, batch 1",
+        "value": round(steps / decode_s, 2), "unit": "tokens/s", "n_gpus": 1, "steps": new_tokens,
+        "warmup": args.warmup, "ms_per_step": round(decode_s / steps * 1e3, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "opt-13b-shaped greedy decode", "layers": layers, "d": d, "ffn": ffn, "heads": H,
+                   "K": K, "active_heads": Hk, "vocab": vocab, "prompt": prompt_len, "new_tokens": new_tokens,
+                   "hip_graphs": 16},
+        "prompt_ms": round(t_prompt * 1e3, 2), "total_ms": round(t_total * 1e3, 2),
+        "eager_total_ms": round(t_eager * 1e3, 2), "graph_equals_eager": same,
+        "us_per_layer": round(decode_s / steps / layers * 1e6, 2),
+        "weight_MB_per_token": round(token_bytes / 1e6, 1),
+        "GB/s": round(token_bytes * steps / decode_s / 1e9, 1),
+        "frac_of_hbm_peak": round(token_bytes * steps / decode_s / 1e9 / HBM_PEAK_GBPS, 4),
+    }
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -200,6 +268,10 @@ def main():
                     help="also run a plain 1 GiB device copy (known traffic) for counter calibration")
     ap.add_argument("--defer", action="store_true",
                     help="let the MLP predictor of layer l run into layer l+1 (joined once per graph)")
+    ap.add_argument("--workload", default="layer", choices=["layer", "decode"],
+                    help="layer: the headline sparse decode layer; decode: end-to-end greedy generation "
+                         "(40-layer OPT-13B shape, --steps = new tokens, default 256)")
+    ap.add_argument("--decode-layers", type=int, default=40)
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs the sparse decode layer on ONE GPU (no sharding); "
@@ -211,6 +283,10 @@ def main():
     import dejavu_amd.modules as dv_modules
     from dejavu_amd.workloads import CONFIGS
 
+    if args.workload == "decode":
+        if args.steps == 600:
+            args.steps, args.warmup = 256, 1
+        return decode_bench(args)
     dv_modules.USE_SIDE_STREAM = not args.single_stream
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)

@@ -13,6 +13,7 @@
 #include "gemv_rows.hpp"
 #include "layer_fused.hpp"
 #include "norm.hpp"
+#include "qkv_mfma.hpp"
 #include "topk.hpp"
 
 using namespace dv;
@@ -305,6 +306,19 @@ int launch_qkv(const half_t* x, const half_t* W, const half_t* bias, const int* 
   return launch_status();
 }
 
+// More than eight window tokens: one pass on the matrix cores covers all 16 slots at a cost
+// that does not grow with the number of live ones (measured break-even at 6..8 tokens).
+inline bool qkv_use_mfma(int nb, int d) { return nb > 8 && d % 64 == 0; }
+
+int launch_qkv_mfma(const half_t* x, const half_t* W, const half_t* bias, const int* head_idx,
+                    const int* batch_idx, int nb, int d, int H, int hd, int nnz, half_t* y,
+                    half_t* k_cache, half_t* v_cache, const int* padding, int S, hipStream_t s) {
+  const int ntasks = nnz * 3 * (hd / 16);
+  hipLaunchKernelGGL((qkv_window_mfma_kernel<kQkvMfmaWaves, kQkvMfmaUnroll>), dim3(ntasks), dim3(kQkvMfmaWaves * 64), 0, s,
+                     x, W, bias, head_idx, batch_idx, nb, d, H, hd, nnz, y, k_cache, v_cache, padding, S);
+  return launch_status();
+}
+
 constexpr int kAttnWaves = 4;  // wavefronts (x64 positions) per attention workgroup
 inline int attn_splits(int n_len) {
   return n_len > 0 ? (n_len + kAttnWaves * kWave - 1) / (kAttnWaves * kWave) : 1;
@@ -488,6 +502,8 @@ int dv_qkv_proj_sparse_cache_f16(const void* x, const void* W, const void* bias,
   half_t* kc = reinterpret_cast<half_t*>(k_cache);
   half_t* vc = reinterpret_cast<half_t*>(v_cache);
   const int* pad = reinterpret_cast<const int*>(padding);
+  if (qkv_use_mfma(nb, d))
+    return launch_qkv_mfma(xx, ww, bb, hi, bi, nb, d, H, hd, nnz, yy, kc, vc, pad, S, s);
 #define DV_QKV(NB) return launch_qkv<NB>(xx, ww, bb, hi, bi, nb, d, H, hd, nnz, yy, kc, vc, pad, S, s)
   if (nb == 1) DV_QKV(1);
   if (nb == 2) DV_QKV(2);
@@ -858,9 +874,11 @@ int dv_sparse_layer_decode_f16(const dvSparseLayerArgs* args, void* stream) {
     QkvArgs q{x_cache, CH(a.Wqkv), CH(a.bqkv), head_idx, batch_idx, nb, a.d, a.H, a.hd, a.Hk, qkv,
               reinterpret_cast<half_t*>(a.k_cache), reinterpret_cast<half_t*>(a.v_cache),
               reinterpret_cast<const int*>(a.cache_offset), a.S};
+    const bool mfma = qkv_use_mfma(nb, a.d);
     const int ntasks = a.Hk * 3 * (a.hd / 2);
     int nq = (ntasks + 3) / 4;
     if (nq > cus * 8) nq = cus * 8;
+    if (mfma) nq = a.Hk * 3 * (a.hd / 16);
     CanonArgs hp0{res1, CH(a.att_Wa), (int64_t)a.d, a.r_att, a.d, hp_hidden};
     const int rw0 = a.d <= 1024 ? 4 : 1;
     const int nh = ((a.r_att + rw0 - 1) / rw0 + 3) / 4;
@@ -868,7 +886,8 @@ int dv_sparse_layer_decode_f16(const dvSparseLayerArgs* args, void* stream) {
 #define DV_L2(NB)                                                                                 \
   hipLaunchKernelGGL((layer_l2_kernel<NB>), grid, dim3(256), 0, s, q, nq, hp0, nh, CH(a.mlp_logit_in), \
                      a.ffn, topk_ws)
-    if (nb == 1) DV_L2(1);
+    if (mfma) DV_L2(0);
+    else if (nb == 1) DV_L2(1);
     else if (nb == 2) DV_L2(2);
     else if (nb <= 4) DV_L2(4);
     else if (nb <= 8) DV_L2(8);

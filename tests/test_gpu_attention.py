@@ -37,7 +37,10 @@ def randh(g, *shape, std=1.0):
 
 # ------------------------------------------------------------------ QKV
 @pytest.mark.parametrize("H,hd,d,nb,nnz", [(12, 128, 12288, 16, 4), (12, 128, 1024, 1, 4), (6, 64, 768, 3, 2),
-                                           (8, 128, 1152, 5, 8), (8, 32, 512, 8, 3), (12, 128, 2048, 2, 12)])
+                                           (8, 128, 1152, 5, 8), (8, 32, 512, 8, 3), (12, 128, 2048, 2, 12),
+                                           # more than 8 rows: matrix-core kernel (d % 64 == 0) or its fallback
+                                           (8, 64, 1024, 12, 3), (5, 64, 320, 9, 5), (4, 32, 128, 16, 2),
+                                           (6, 128, 1096, 16, 3)])
 def test_qkv_proj_sparse(ops, H, hd, d, nb, nnz):
     """First case is the shape of the reference's own self-check
     (attention_proj_sparse.py:597-627): 12 heads, hidden 12288, 16 rows, 4 active heads,
@@ -206,13 +209,14 @@ def test_single_query_attention_lengths_per_sample(ops):
     assert np.array_equal(np16(kcd), kn) and np.array_equal(np16(vcd), vn)
 
 
-def test_fused_qkv_cache_and_attention_out_proj_match_separate_ops(ops):
+@pytest.mark.parametrize("nb", [5, 13])
+def test_fused_qkv_cache_and_attention_out_proj_match_separate_ops(ops, nb):
     """The fused entry points (QKV + cache scatter; attention + out_proj without a
     stored context) must reproduce the separate operators."""
     from dejavu_amd.workloads import pack_k_cache
 
     g = torch.Generator().manual_seed(6)
-    H, hd, d, S, nb, nnz = 12, 128, 1024, 300, 5, 4
+    H, hd, d, S, nnz = 12, 128, 1024, 300, 4
     x = randh(g, nb, d)
     W = randh(g, 3, H, hd, d, std=0.03)
     bias = randh(g, 3, H, hd, std=0.1)
