@@ -39,8 +39,8 @@ def randh(g, *shape, std=1.0):
 @pytest.mark.parametrize("H,hd,d,nb,nnz", [(12, 128, 12288, 16, 4), (12, 128, 1024, 1, 4), (6, 64, 768, 3, 2),
                                            (8, 128, 1152, 5, 8), (8, 32, 512, 8, 3), (12, 128, 2048, 2, 12),
                                            # more than 8 rows: matrix-core kernel (d % 64 == 0) or its fallback
-                                           (8, 64, 1024, 12, 3), (5, 64, 320, 9, 5), (4, 32, 128, 16, 2),
-                                           (6, 128, 1096, 16, 3)])
+                                           (8, 64, 1024, 12, 3), (5, 64, 384, 9, 5), (4, 32, 128, 16, 2),
+                                           (6, 128, 640, 16, 3)])
 def test_qkv_proj_sparse(ops, H, hd, d, nb, nnz):
     """First case is the shape of the reference's own self-check
     (attention_proj_sparse.py:597-627): 12 heads, hidden 12288, 16 rows, 4 active heads,
@@ -71,6 +71,29 @@ def test_qkv_proj_sparse(ops, H, hd, d, nb, nnz):
                              out=np.full((nb, 3, H, hd), 7.0, dtype=np.float16))
     assert_close(np16(out2), want, "qkv masked")
     assert np.array_equal(np16(out2) == 7.0, want == 7.0), "written / untouched pattern differs"
+
+
+def test_qkv_many_rows_with_hidden_size_not_a_multiple_of_64(ops):
+    """Straight through the C ABI (the Python operator keeps the reference's d % 128 == 0
+    precondition): 16 window rows with d % 64 != 0 take the per-row kernel."""
+    from dejavu_amd._lib import check, lib
+
+    g = torch.Generator().manual_seed(3)
+    H, hd, d, nb, nnz = 4, 64, 328, 16, 3
+    x, W, bias = randh(g, nb, d), randh(g, 3, H, hd, d, std=0.05), randh(g, 3, H, hd)
+    head_idx = torch.tensor([3, 0, 2], dtype=torch.int32)
+    batch_idx = torch.stack([torch.arange(nb) for _ in range(nnz)]).int()
+    batch_idx[torch.rand(nnz, nb, generator=g) < 0.3] = -1
+    out = torch.full((nb, 3, H, hd), 7.0, dtype=torch.float16, device="cuda")
+    xd, Wd, bd, hd_, bi = x.cuda(), W.cuda(), bias.cuda(), head_idx.cuda(), batch_idx.cuda()
+    print("case qkv C ABI d=328 nb=16", flush=True)
+    check(lib.dv_qkv_proj_sparse_f16(xd.data_ptr(), Wd.data_ptr(), bd.data_ptr(), hd_.data_ptr(), bi.data_ptr(), nb, d,
+                                     H, hd, nnz, out.data_ptr(), torch.cuda.current_stream().cuda_stream), "qkv")
+    torch.cuda.synchronize()
+    want = O.qkv_proj_sparse(x.numpy(), W.numpy(), head_idx.numpy(), batch_idx.numpy(), bias.numpy(),
+                             out=np.full((nb, 3, H, hd), 7.0, dtype=np.float16))
+    assert_close(np16(out), want, "qkv d=328")
+    assert np.array_equal(np16(out) == 7.0, want == 7.0)
 
 
 def test_qkv_proj_sparse_no_bias_and_empty(ops):
