@@ -6,9 +6,17 @@ sparse MLP + both predictors + top-ks + the two add/LayerNorms) over one decode
 token.  Default workload: the OPT-175B-shaped layer (d=12288, ffn=49152, 96
 heads x 128, K=4096 neurons, 32 heads, KV length 2048, batch 1), synthetic
 seeded weights.  Three distinct layers (weights, caches) are cycled so that no
-cache level can hold the working set; each layer's step is replayed from a HIP
-graph, and the next layer's head / neuron predictions are produced by the
-previous layer as in the model.
+cache level can hold the working set, and the next layer's neuron predictions
+are produced by the previous layer as in the model.
+
+The steps walk through whole 16-token back-fill windows: at window position c a
+layer also recomputes K / V of the window tokens its active heads skipped, and
+position 15 is the flush step that brings every head up to date.  The active
+heads are re-drawn at random for every (layer, position) -- no correlation
+between consecutive tokens, the most back-fill work a window can have.
+``--window start`` times only the first position of a window (no back-fill).
+Steps are replayed from HIP graphs (one graph of 3 layers x 16 positions when the
+step counts are multiples of 48, one graph per (layer, position) otherwise).
 
 Prints ONE JSON line (see README / DESIGN.md for the fields).
 """
@@ -26,6 +34,7 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0
 N_LAYERS = 3
+WINDOW = 16
 # HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (scaled by a 1 GiB copy; see profiles/layer_opt175b_pmc_traffic.md).  Not measurable from inside
 # this script, so only reported for the shape it was taken on.
@@ -44,6 +53,12 @@ def algorithmic_bytes(cfg, batch):
         "mlp_predictor": (d * r + r * ffn) * 2,
         "head_predictor": (d * r + r * H) * 2,
     }
+
+
+def flush_step_bytes(cfg, batch):
+    """Bytes of the step that closes a window: QKV, KV and out_proj of ALL heads."""
+    d, ffn, H, hd, r, K, S = (cfg[k] for k in ("d", "ffn", "H", "hd", "r", "K", "S"))
+    return (3 * H * hd * d + 2 * H * S * hd * batch + d * H * hd + 2 * K * d + d * r + r * ffn + d * r + r * H) * 2
 
 
 def build_layers(cfg, batch, device):
@@ -77,6 +92,10 @@ def build_layers(cfg, batch, device):
     for l, L in enumerate(layers):
         L["att_idx_in"] = torch.sort(torch.randperm(H, generator=gen, device=device)[:Hk]).values.int()
         L["mlp_logit_in"] = randn((ffn,), 4.0)
+        # active heads per window position, independent draws
+        L["heads"] = [torch.sort(torch.randperm(H, generator=gen, device=device)[:Hk]).values.int()
+                      for _ in range(WINDOW)]
+        L["S"] = S
     for l, L in enumerate(layers):
         nxt = layers[(l + 1) % N_LAYERS]
         L["block"].mixer.att_idx_out = nxt["att_idx_in"]
@@ -86,11 +105,26 @@ def build_layers(cfg, batch, device):
 
 def layer_step(L):
     """One decode step of one block in the state 'first token of a back-fill
-    window': every active head computes Q, K, V of the newest token."""
+    window': every active head computes Q, K, V of the newest token only."""
     mixer = L["block"].mixer
     mixer.counter = 0  # the window step re-initialises the tracker at counter 0
+    L["ip"].sequence_len_offset = L["S"] - 1  # mixer.cache_offset must hold S - 1 (set by the caller)
     return L["block"](L["hidden"], L["residual"], mixer_kwargs={"inference_params": L["ip"]},
                       head_idx=L["att_idx_in"], mlp_sp_logit=L["mlp_logit_in"])
+
+
+def window_step(L, c):
+    """Decode step at window position c (0..15) of a window that occupies the last 16 cache
+    positions; heads drawn for this (layer, position).  Position 15 flushes the window."""
+    mixer = L["block"].mixer
+    S = L["S"]
+    if c == 0:
+        mixer.counter = 0
+        mixer.cache_offset.fill_(S - WINDOW)
+    assert mixer.counter == c
+    L["ip"].sequence_len_offset = S - WINDOW + c
+    return L["block"](L["hidden"], L["residual"], mixer_kwargs={"inference_params": L["ip"]},
+                      head_idx=L["heads"][c], mlp_sp_logit=L["mlp_logit_in"])
 
 
 def time_kernel(torch, fn, layers, iters=60):
@@ -256,18 +290,20 @@ def decode_bench(args):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=600)
-    ap.add_argument("--warmup", type=int, default=60)
+    ap.add_argument("--steps", type=int, default=None, help="default 960 (20 windows of 3 layers x 16 positions)")
+    ap.add_argument("--warmup", type=int, default=None, help="default 96")
+    ap.add_argument("--window", default="cycle", choices=["cycle", "start"],
+                    help="cycle: steps walk through whole 16-token back-fill windows; "
+                         "start: only the first position of a window (no back-fill)")
     ap.add_argument("--config", default="opt-175b")
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying HIP graphs")
     ap.add_argument("--single-stream", action="store_true", help="no side stream for predictors / top-k")
-    ap.add_argument("--layers-per-graph", type=int, default=3, choices=[1, 3])
+    ap.add_argument("--graph-per-step", action="store_true",
+                    help="one HIP graph per step even when the step counts allow one graph per schedule period")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (known traffic) for counter calibration")
-    ap.add_argument("--defer", action="store_true",
-                    help="let the MLP predictor of layer l run into layer l+1 (joined once per graph)")
     ap.add_argument("--workload", default="layer", choices=["layer", "decode"],
                     help="layer: the headline sparse decode layer; decode: end-to-end greedy generation "
                          "(40-layer OPT-13B shape, --steps = new tokens, default 256)")
@@ -284,9 +320,11 @@ def main():
     from dejavu_amd.workloads import CONFIGS
 
     if args.workload == "decode":
-        if args.steps == 600:
-            args.steps, args.warmup = 256, 1
+        args.steps = 256 if args.steps is None else args.steps
+        args.warmup = 1 if args.warmup is None else args.warmup
         return decode_bench(args)
+    args.steps = 960 if args.steps is None else args.steps
+    args.warmup = 96 if args.warmup is None else args.warmup
     dv_modules.USE_SIDE_STREAM = not args.single_stream
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
@@ -297,56 +335,70 @@ def main():
     assert batch == 1, "the head-sparse decode layer keeps one back-fill window (batch 1)"
     device = torch.device("cuda:0")
     layers = build_layers(cfg, batch, device)
-    defer = args.defer and (not args.single_stream) and args.layers_per_graph == N_LAYERS \
-        and not args.no_graph and args.steps % N_LAYERS == 0 and args.warmup % N_LAYERS == 0
-    for L in layers:
-        L["block"].mlp.defer_predictor_join = defer
+    cycle = args.window == "cycle"
+    period = N_LAYERS * (WINDOW if cycle else 1)
 
-    with torch.no_grad():
-        # eager warm-up: allocates workspaces, sets kernel attributes
-        for _ in range(2):
-            for L in layers:
-                layer_step(L)
+    def step_fn(i):
+        """i-th step of the repeating schedule: positions outermost, layers innermost."""
+        if cycle:
+            c, l = divmod(i % period, N_LAYERS)
+            return window_step(layers[l], c)
+        return layer_step(layers[i % N_LAYERS])
+
+    def capture(first, count):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for i in range(first, first + count):
+                step_fn(i)
             dv_modules.join_side_stream()
-        torch.cuda.synchronize()
-        graphs = []
-        # a graph of all three layers can only be replayed whole: fall back to one graph per
-        # layer when the step counts are not multiples of three, so exactly --steps steps run
-        if args.steps % N_LAYERS or args.warmup % N_LAYERS:
-            args.layers_per_graph = 1
-        if not args.no_graph and args.layers_per_graph == 1:
-            for L in layers:
-                g = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(g):
-                    L["out"] = layer_step(L)
-                graphs.append(g)
-            torch.cuda.synchronize()
-        elif not args.no_graph:
-            g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g):
-                for L in layers:
-                    L["out"] = layer_step(L)
-                dv_modules.join_side_stream()
-            graphs.append(g)
-            torch.cuda.synchronize()
+        return g
 
-        def run(i):
-            if len(graphs) == N_LAYERS:
-                graphs[i % N_LAYERS].replay()
-            elif graphs:
-                if i % N_LAYERS == 0:
-                    graphs[0].replay()
-            else:
-                layer_step(layers[i % N_LAYERS])
-
-        for i in range(args.warmup):
+    def timed(run, steps, warmup):
+        for i in range(warmup):
             run(i)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for i in range(args.steps):
+        for i in range(steps):
             run(i)
         torch.cuda.synchronize()
-        elapsed = time.perf_counter() - t0
+        return (time.perf_counter() - t0) / steps * 1e6
+
+    with torch.no_grad():
+        if not cycle:
+            for L in layers:
+                L["block"].mixer.cache_offset.fill_(cfg["S"] - 1)
+        # eager warm-up: allocates workspaces, sets kernel attributes (every window position once)
+        for i in range(2 * period):
+            step_fn(i)
+        dv_modules.join_side_stream()
+        torch.cuda.synchronize()
+        whole = args.steps % period == 0 and args.warmup % period == 0 and not args.graph_per_step
+        if args.no_graph:
+            us_per_layer = timed(step_fn, args.steps, args.warmup)
+            graph_mode = "none"
+        elif whole:
+            g = capture(0, period)
+            torch.cuda.synchronize()
+            us_per_layer = timed(lambda i: g.replay() if i % period == 0 else None, args.steps, args.warmup)
+            graph_mode = f"one graph of {period} steps"
+        else:
+            graphs = [capture(i, 1) for i in range(period)]
+            torch.cuda.synchronize()
+            us_per_layer = timed(lambda i: graphs[i % period].replay(), args.steps, args.warmup)
+            graph_mode = "one graph per step"
+
+        # the same three layers at the first position of a window only (no back-fill work)
+        window_start_us = None
+        if cycle and not args.no_graph:
+            cycle = False
+            for L in layers:
+                L["block"].mixer.cache_offset.fill_(cfg["S"] - 1)
+            for i in range(N_LAYERS):
+                step_fn(i)
+            g0 = capture(0, N_LAYERS)
+            torch.cuda.synchronize()
+            window_start_us = timed(lambda i: g0.replay() if i % N_LAYERS == 0 else None, 300, 30)
+            cycle = True
 
         if args.pmc_calibration:
             src = torch.empty(1 << 30, dtype=torch.uint8, device=device)
@@ -356,9 +408,11 @@ def main():
             torch.cuda.synchronize()
             del src, dst
 
-        us_per_layer = elapsed / args.steps * 1e6
         nbytes = algorithmic_bytes(cfg, batch)
-        layer_bytes = sum(nbytes.values())
+        start_bytes = sum(nbytes.values())
+        # a window = 15 steps with the predicted heads + 1 flush step with all heads
+        layer_bytes = (15 * start_bytes + flush_step_bytes(cfg, batch)) / 16 if args.window == "cycle" \
+            else start_bytes
         table = kernel_table(torch, cfg, batch, layers)
         dom = "qkv_sparse"  # largest share of the layer's bytes
         roofline = {"bound": "hbm", "kernel": "qkv_sparse_kernel", "achieved": table[dom]["GB/s"],
@@ -383,13 +437,18 @@ def main():
         "vs_baseline": None,
         "dtype": "f16",
         "data": "synthetic",
-        "config": {"workload": f"{args.config} sparse decode layer", "d": cfg["d"], "ffn": cfg["ffn"],
+        "config": {"workload": f"{args.config} sparse decode layer, batch 1, " + (
+            "steps walk 16-token back-fill windows (heads re-drawn every token, flush step included)"
+            if args.window == "cycle" else "first position of a back-fill window"), "d": cfg["d"], "ffn": cfg["ffn"],
                    "heads": cfg["H"], "head_dim": cfg["hd"], "K": cfg["K"], "active_heads": cfg["Hk"],
                    "predictor_rank": cfg["r"], "kv_len": cfg["S"], "batch": batch,
-                   "layers_cycled": N_LAYERS, "hip_graph": not args.no_graph,
-                   "layers_per_graph": 0 if args.no_graph else args.layers_per_graph},
+                   "layers_cycled": N_LAYERS, "window": args.window, "hip_graph": graph_mode},
         "roofline": roofline,
         "cpu_baseline": cpu,
+        "window_start": None if window_start_us is None else {
+            "us_per_layer": round(window_start_us, 2), "algorithmic_MB": round(start_bytes / 1e6, 1),
+            "GB/s": round(start_bytes / window_start_us / 1e3, 1),
+            "frac_of_hbm_peak": round(start_bytes / window_start_us / 1e3 / HBM_PEAK_GBPS, 4)},
         "layer": {"algorithmic_MB": round(layer_bytes / 1e6, 1), "GB/s": round(layer_bytes / us_per_layer / 1e3, 1),
                   "frac_of_hbm_peak": round(layer_bytes / us_per_layer / 1e3 / HBM_PEAK_GBPS, 4),
                   "tokens_per_s_per_layer": round(batch / (us_per_layer * 1e-6), 1)},
