@@ -287,6 +287,68 @@ def decode_bench(args):
     print(json.dumps(out))
 
 
+def mlp_bench(args):
+    """Sparse MLP block (predictor + union top-k + fc1 + fc2) at batch sizes 1..64: batches up to
+    4 stream the gathered rows through the vector ALUs, larger ones through LDS into MFMA tiles.
+    Prints its own JSON line; a step is one block step at the given batch."""
+    import torch
+
+    from dejavu_amd import ops
+    from dejavu_amd.workloads import CONFIGS, make_mlp
+
+    cfg = CONFIGS[args.config]
+    d, ffn, r, K = cfg["d"], cfg["ffn"], cfg["r"], cfg["K"]
+    torch.cuda.set_device(0)
+    sets = [make_mlp(cfg, batch=64, device="cuda", seed=s) for s in range(N_LAYERS)]
+    weight_bytes = 2 * K * d * 2
+    pred_bytes = (d * r + r * ffn) * 2
+    results = {}
+    with torch.no_grad():
+        for B in args.batches:
+            def step(t, B=B):
+                x, res = t["x2"][:B], t["residual"][:B]
+                logits = ops.predictor_logits(res, t["mlp_Wa"], t["mlp_Wb"])
+                idx = ops.topk_indices(logits, K)
+                return ops.mlp_sparse(x, t["W1"], t["W2t"], idx, t["b1"], t["b2"])
+
+            def mlp_only(t, B=B):
+                return ops.mlp_sparse(t["x2"][:B], t["W1"], t["W2t"], t["idx"], t["b1"], t["b2"])
+
+            for t in sets:
+                t["idx"] = ops.topk_indices(ops.predictor_logits(t["residual"][:B], t["mlp_Wa"], t["mlp_Wb"]), K)
+                step(t)
+            torch.cuda.synchronize()
+            out = {}
+            for name, fn, nbytes in (("block", step, weight_bytes + pred_bytes * ((B + 7) // 8)),
+                                     ("fc1_fc2", mlp_only, weight_bytes)):
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    for t in sets:
+                        fn(t)
+                for _ in range(5):
+                    g.replay()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                reps = max(1, args.steps // N_LAYERS)
+                for _ in range(reps):
+                    g.replay()
+                torch.cuda.synchronize()
+                us = (time.perf_counter() - t0) / (reps * N_LAYERS) * 1e6
+                out[name] = {"us": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1),
+                             "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
+            out["fc1_fc2"]["TFLOP/s"] = round(2.0 * B * (weight_bytes / 2) / out["fc1_fc2"]["us"] / 1e6, 2)
+            out["tokens_per_s"] = round(B / (out["block"]["us"] * 1e-6), 1)
+            out["path"] = "vector ALU gather-GEMV" if B <= 4 else "LDS-staged MFMA tiles"
+            results[str(B)] = out
+    print(json.dumps({
+        "metric": f"us per sparse MLP block step, {args.config} shape, K={K}", "unit": "us/step", "n_gpus": 1,
+        "steps": args.steps, "dtype": "f16", "data": "synthetic", "higher_is_better": False,
+        "config": {"workload": f"{args.config} sparse MLP block, batch sweep", "d": d, "ffn": ffn, "K": K,
+                   "predictor_rank": r, "weight_sets_cycled": N_LAYERS, "hip_graph": True},
+        "algorithmic_MB": {"fc1_fc2": round(weight_bytes / 1e6, 2), "predictor_per_8_rows": round(pred_bytes / 1e6, 2)},
+        "batches": results}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -304,7 +366,9 @@ def main():
                     help="one HIP graph per step even when the step counts allow one graph per schedule period")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy (known traffic) for counter calibration")
-    ap.add_argument("--workload", default="layer", choices=["layer", "decode"],
+    ap.add_argument("--batches", type=int, nargs="+", default=[1, 4, 8, 16, 32],
+                    help="batch sizes of --workload mlp")
+    ap.add_argument("--workload", default="layer", choices=["layer", "decode", "mlp"],
                     help="layer: the headline sparse decode layer; decode: end-to-end greedy generation "
                          "(40-layer OPT-13B shape, --steps = new tokens, default 256)")
     ap.add_argument("--decode-layers", type=int, default=40)
@@ -323,6 +387,9 @@ def main():
         args.steps = 256 if args.steps is None else args.steps
         args.warmup = 1 if args.warmup is None else args.warmup
         return decode_bench(args)
+    if args.workload == "mlp":
+        args.steps = 300 if args.steps is None else args.steps
+        return mlp_bench(args)
     args.steps = 960 if args.steps is None else args.steps
     args.warmup = 96 if args.warmup is None else args.warmup
     dv_modules.USE_SIDE_STREAM = not args.single_stream
