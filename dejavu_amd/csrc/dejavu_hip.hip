@@ -233,15 +233,18 @@ struct ColsMfmaPlan {
 ColsMfmaPlan plan_cols_mfma(int B, int N, int M) {
   ColsMfmaPlan p;
   p.col_tiles = (N + kMfmaColTile - 1) / kMfmaColTile;
-  // every row group writes a (B, N) fp32 partial: fewer, longer groups as the batch grows
-  const int target_blocks = compute_units() * (B <= 8 ? 3 : (B <= 16 ? 2 : 1));
-  int groups = (target_blocks + p.col_tiles - 1) / p.col_tiles;
-  const int max_groups = M > 32 ? (M + 31) / 32 : 1;
+  // Every row group writes a (B, N) fp32 partial that a second pass reads back, so few, long
+  // groups win: each wavefront (128 columns of one group) keeps 16 KiB of weights in flight
+  // and three to four of them per compute unit measured best for batch 8..64.
+  const int waves_per_cu = B <= 8 ? 4 : 3;
+  const int col_waves = (N + kMfmaColWave - 1) / kMfmaColWave;
+  int groups = (compute_units() * waves_per_cu + col_waves - 1) / col_waves;
+  const int max_groups = M > kMfmaColRows ? (M + kMfmaColRows - 1) / kMfmaColRows : 1;
   if (groups > max_groups) groups = max_groups;
   if (groups < 1) groups = 1;
   int rpb = (M + groups - 1) / groups;
-  rpb = (rpb + 31) & ~31;
-  if (rpb < 32) rpb = 32;
+  rpb = (rpb + kMfmaColRows - 1) / kMfmaColRows * kMfmaColRows;
+  if (rpb < kMfmaColRows) rpb = kMfmaColRows;
   p.rows_per_block = rpb;
   p.groups = M > 0 ? (M + rpb - 1) / rpb : 1;
   return p;
@@ -252,11 +255,11 @@ size_t cols_mfma_workspace_bytes(int B, int N, int M) {
   return kCounterBytes + (size_t)p.groups * B * N * sizeof(float);
 }
 
-template <int BT, bool IDX64, bool BLOCKED>
+template <int BT, bool IDX64, bool BLOCKED, bool HVEC>
 void launch_cols_mfma(const ColsMfmaPlan& p, const half_t* h, int64_t ldh, int x_expanded, const half_t* W,
                       int64_t ldw, const half_t* bias, const void* idx, int blk, int B, int N, int Z, int M,
                       float* partial, half_t* y, hipStream_t s) {
-  hipLaunchKernelGGL((gather_cols_mfma_kernel<BT, IDX64, BLOCKED>), dim3(p.col_tiles, p.groups), dim3(256), 0,
+  hipLaunchKernelGGL((gather_cols_mfma_kernel<BT, IDX64, BLOCKED, HVEC>), dim3(p.col_tiles, p.groups), dim3(256), 0,
                      s, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M, p.rows_per_block, partial, y);
   if (p.groups > 1) {
     const int64_t total = (int64_t)B * N;
@@ -272,20 +275,29 @@ int gather_cols_mfma(const half_t* h, int64_t ldh, int x_expanded, const half_t*
   if (workspace == nullptr || workspace_bytes < cols_mfma_workspace_bytes(B, N, M)) return DV_ERR_WORKSPACE;
   float* partial = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(workspace) + kCounterBytes);
   const bool i64 = idx_bytes == 8, blocked = blk != 1;
-#define DV_CM(BT)                                                                                        \
-  do {                                                                                                   \
-    if (blocked) {                                                                                       \
-      if (i64) launch_cols_mfma<BT, true, true>(p, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M, partial, y, s);   \
-      else launch_cols_mfma<BT, false, true>(p, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M, partial, y, s);      \
-    } else {                                                                                             \
-      if (i64) launch_cols_mfma<BT, true, false>(p, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M, partial, y, s);  \
-      else launch_cols_mfma<BT, false, false>(p, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M, partial, y, s);     \
-    }                                                                                                    \
+  const bool hvec = M % 8 == 0 && ldh % 8 == 0 && aligned16(h) && (!x_expanded || blk % 8 == 0);
+#define DV_ARGS p, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M, partial, y, s
+#define DV_CM3(BT, I64, BLK)                                   \
+  do {                                                         \
+    if (hvec) launch_cols_mfma<BT, I64, BLK, true>(DV_ARGS);   \
+    else launch_cols_mfma<BT, I64, BLK, false>(DV_ARGS);       \
+  } while (0)
+#define DV_CM(BT)                                  \
+  do {                                             \
+    if (blocked) {                                 \
+      if (i64) DV_CM3(BT, true, true);             \
+      else DV_CM3(BT, false, true);                \
+    } else {                                       \
+      if (i64) DV_CM3(BT, true, false);            \
+      else DV_CM3(BT, false, false);               \
+    }                                              \
   } while (0)
   if (B <= 32)
     DV_CM(1);
   else
     DV_CM(2);
+#undef DV_CM3
+#undef DV_ARGS
 #undef DV_CM
   return launch_status();
 }

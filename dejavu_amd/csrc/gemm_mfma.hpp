@@ -142,38 +142,66 @@ __global__ __launch_bounds__(kMfmaWaves * 64) void gather_rows_mfma_kernel(
 // ---------------------------------------------------------------------------
 // fc2 / out_proj over a transposed weight: Y[b, n] = sum_m H[b, m] * W[row(m), n].
 // The contraction index m runs over gathered ROWS, so the weight tile must be
-// transposed on its way to the MFMA: a workgroup copies 32 gathered rows x 512
-// columns into LDS (one full 1 KiB row segment per wavefront load), then every
-// wavefront reads, for its four 32-column sub-tiles, the A operand W^T (n x m)
-// with 16-bit LDS reads, and multiplies by H^T (m x b) loaded straight from
-// memory.  Partial sums over the row groups (gridDim.y) go to `partial`
+// transposed on its way to the MFMA.  Every wavefront works on its own: it owns
+// 128 of the workgroup's 512 columns and walks the workgroup's row group 64 rows
+// at a time.  Per step it copies 64 rows x 128 columns (sixteen loads of 4 rows x
+// 256 contiguous bytes) through registers into a private LDS tile, issues the
+// loads of the NEXT step, and only then consumes the tile: for each of its four
+// 32-column sub-tiles the A operand W^T (n x m) is gathered with 16-bit LDS
+// reads and multiplied by H^T (m x b), which comes straight from memory.  No
+// workgroup barrier is needed; the weight stream stays in flight during the
+// MFMAs.  Partial sums over the row groups (gridDim.y) go to `partial`
 // [(g * B + b) * N + n] and are reduced by cols_reduce_kernel; with one group
 // the result (+ bias) is written directly.
 // Row mapping as gather_cols_kernel: BLOCKED ? idx[m / blk] * blk + m % blk : idx[m];
 // x_expanded: H is (B, Z) indexed by row(m) instead of (B, M) indexed by m.
+// HVEC: H is read with 128-bit loads; the host guarantees M % 8 == 0, ldh % 8 == 0, a
+// 16-byte aligned H and, for the expanded layout, blk % 8 == 0 (groups of 8 rows never
+// straddle a block).  Otherwise H is gathered element by element.
 // ---------------------------------------------------------------------------
-constexpr int kMfmaColTile = 512;
-constexpr int kMfmaColLdsRow = kMfmaColTile + 8;
+constexpr int kMfmaColTile = 512;               // columns per workgroup
+constexpr int kMfmaColWave = 128;               // columns per wavefront
+constexpr int kMfmaColLdsRow = kMfmaColWave + 8;  // halfs per LDS tile row (bank spread)
+constexpr int kMfmaColRows = 64;                // rows per step
 
-template <int BT, bool IDX64, bool BLOCKED>
+template <int BT, bool IDX64, bool BLOCKED, bool HVEC>
 __global__ __launch_bounds__(256) void gather_cols_mfma_kernel(
     const half_t* __restrict__ H, int64_t ldh, int x_expanded, const half_t* __restrict__ W,
     int64_t ldw, const half_t* __restrict__ bias, const void* __restrict__ idx, int blk, int B, int N,
     int Z, int M, int rows_per_block, float* __restrict__ partial, half_t* __restrict__ Y) {
-  __shared__ __attribute__((aligned(16))) half_t tile[32 * kMfmaColLdsRow];
-  __shared__ int s_rid[32];
+  __shared__ __attribute__((aligned(16))) half_t tiles[4][kMfmaColRows * kMfmaColLdsRow];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  half_t* tile = tiles[wave];
   const int half_id = lane >> 5, l32 = lane & 31;
+  const int lrow = lane >> 4, lcol = (lane & 15) * 8;  // staging coordinates: 4 rows x 16 pieces of 8 columns
   const int ct = blockIdx.x, g = blockIdx.y, G = gridDim.y;
-  const int col0 = ct * kMfmaColTile;
+  const int col0 = ct * kMfmaColTile + wave * kMfmaColWave;
+  const bool col_ok = col0 + lcol < N;  // N % 8 == 0
   const int m_begin = g * rows_per_block;
   int m_end = m_begin + rows_per_block;
   if (m_end > M) m_end = M;
-  // 128-bit loads of H need 8-element alignment of every (b, first row) pair
-  const bool h_vec_ok = (ldh % 8 == 0) && ((reinterpret_cast<uintptr_t>(H) & 15u) == 0) &&
-                        (x_expanded ? (blk % 8 == 0) : true);
+  const bool any_rows = m_begin < m_end;
+  // Every load below is unconditional (addresses clamped to something valid, results
+  // masked afterwards): with a fixed number of loads per step the compiler can wait for
+  // the older H loads while the newer weight loads stay in flight.
+  // raw index word of row (mb + lane); rows past the group re-read its first row
+  auto fetch_index = [&](int mb) -> int64_t {
+    if (!any_rows) return -1;
+    int m = mb + lane;
+    if (m >= m_end) m = m_begin;
+    if (BLOCKED) m /= blk;
+    return IDX64 ? reinterpret_cast<const int64_t*>(idx)[m]
+                 : (int64_t) reinterpret_cast<const int32_t*>(idx)[m];
+  };
+  // weight row of row (mb + lane), or -1
+  auto to_row = [&](int mb, int64_t raw) -> int {
+    const int m = mb + lane;
+    int64_t id = raw;
+    if (BLOCKED) id = (raw >= 0 && raw < Z / blk) ? raw * blk + (m % blk) : -1;
+    return (m < m_end && id >= 0 && id < Z) ? (int)id : -1;
+  };
 
   float16_t acc[4][BT];
 #pragma unroll
@@ -183,79 +211,107 @@ __global__ __launch_bounds__(256) void gather_cols_mfma_kernel(
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[s][bt][v] = 0.f;
 
-  for (int mb = m_begin; mb < m_end; mb += 32) {
-    __syncthreads();  // previous tile fully consumed
-    if (tid < 32) {
-      const int m = mb + tid;
-      int64_t id = -1;
-      if (m < m_end) {
-        if (BLOCKED) {
-          const int q = m / blk;
-          const int64_t h = IDX64 ? reinterpret_cast<const int64_t*>(idx)[q]
-                                  : (int64_t) reinterpret_cast<const int32_t*>(idx)[q];
-          id = (h >= 0 && h < Z / blk) ? h * blk + (m - q * blk) : -1;
-        } else {
-          id = IDX64 ? reinterpret_cast<const int64_t*>(idx)[m]
-                     : (int64_t) reinterpret_cast<const int32_t*>(idx)[m];
+  constexpr int NQ = kMfmaColRows / 4;   // weight load instructions per step
+  constexpr int KS = kMfmaColRows / 16;  // MFMA k-steps per step
+  half8_t stage[NQ];
+  unsigned stage_ok = 0;  // bit q: stage[q] holds a real row
+  const int wcol = col_ok ? col0 + lcol : 0;
+
+  auto load_stage = [&](int rid_all) {
+    stage_ok = 0;
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+      const int rid = __shfl(rid_all, q * 4 + lrow, kWave);
+      stage[q] = load8_stream(W + (int64_t)(rid >= 0 ? rid : 0) * ldw + wcol);
+      stage_ok |= (unsigned)(rid >= 0 && col_ok) << q;
+    }
+  };
+  auto store_stage = [&]() {
+    // reads of the previous step are done before the tile is overwritten (same wavefront:
+    // LDS operations complete in order, the fences only stop compiler reordering)
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int q = 0; q < NQ; ++q)
+      store8(tile + (q * 4 + lrow) * kMfmaColLdsRow + lcol, ((stage_ok >> q) & 1u) ? stage[q] : zero8());
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  };
+  half8_t hb[KS][BT];
+  auto load_h = [&](int mb, int rid_cur) {
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int mk = ks * 16 + half_id * 8;  // first of this lane's 8 rows
+      if (HVEC) {
+        // the lane's 8 rows are 8 consecutive entries of H[b, :] (compact gather, or one head
+        // block of the expanded layout): one 128-bit load.  Rows without a valid id carry
+        // zero weights, so whatever (finite) value H holds there contributes nothing.
+        const int rid0 = __shfl(rid_cur, mk, kWave);
+        int64_t h0 = x_expanded ? (int64_t)(rid0 >= 0 ? rid0 : 0) : (int64_t)(mb + mk);
+        if (!x_expanded && h0 + 8 > M) h0 = M - 8;  // M % 8 == 0 and M >= 8 here
+#pragma unroll
+        for (int bt = 0; bt < BT; ++bt) {
+          const int b = bt * 32 + l32;
+          hb[ks][bt] = load8(H + (int64_t)(b < B ? b : 0) * ldh + h0);
+        }
+      } else {
+#pragma unroll
+        for (int bt = 0; bt < BT; ++bt) {
+          const int b = bt * 32 + l32;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const int rid = __shfl(rid_cur, mk + j, kWave);
+            const int m = mb + mk + j;
+            hb[ks][bt][j] = (b < B && rid >= 0)
+                                ? H[(int64_t)b * ldh + (x_expanded ? (int64_t)rid : (int64_t)m)]
+                                : (half_t)0.f;
+          }
         }
       }
-      s_rid[tid] = (id >= 0 && id < Z) ? (int)id : -1;
     }
-    __syncthreads();
-    // wavefront w copies rows w, w+4, ..: one 1 KiB row segment per load instruction
-    half8_t stage[8];
-    const int col = col0 + lane * 8;
+  };
+  auto consume = [&]() {
 #pragma unroll
-    for (int r = 0; r < 8; ++r) {
-      const int rid = s_rid[wave + 4 * r];
-      stage[r] = (rid >= 0 && col < N) ? load8_stream(W + (int64_t)rid * ldw + col) : zero8();
-    }
-#pragma unroll
-    for (int r = 0; r < 8; ++r) store8(tile + (wave + 4 * r) * kMfmaColLdsRow + lane * 8, stage[r]);
-    __syncthreads();
-    // two K = 16 steps over the 32 staged rows
-#pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-      const int mk = ks * 16 + half_id * 8;  // first of this lane's 8 staged rows
-      half8_t hb[BT];
-      // the 8 staged rows of this lane are 8 consecutive entries of H[b, :] when the
-      // gather is compact (or one head block of the expanded layout): one 128-bit load
-      const int rid0 = s_rid[mk];
-      const int64_t h0 = x_expanded ? (int64_t)rid0 : (int64_t)(mb + mk);
-      const bool vec = h_vec_ok && rid0 >= 0 && s_rid[mk + 7] >= 0 && mb + mk + 8 <= m_end &&
-                       (!x_expanded || s_rid[mk + 7] == rid0 + 7);
-#pragma unroll
-      for (int bt = 0; bt < BT; ++bt) {
-        const int b = bt * 32 + l32;
-        if (vec) {
-          hb[bt] = b < B ? load8(H + (int64_t)b * ldh + h0) : zero8();
-          continue;
-        }
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int rid = s_rid[mk + j];
-          const int m = mb + mk + j;
-          hb[bt][j] = (b < B && rid >= 0) ? H[(int64_t)b * ldh + (x_expanded ? (int64_t)rid : (int64_t)m)]
-                                         : (half_t)0.f;
-        }
-      }
+    for (int ks = 0; ks < KS; ++ks) {
+      const int mk = ks * 16 + half_id * 8;
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
-        const int n_local = (wave * 4 + s) * 32 + l32;  // this lane's column inside the tile
+        const int n_local = s * 32 + l32;  // this lane's column inside the wavefront's tile
         half8_t a;
 #pragma unroll
         for (int j = 0; j < 8; ++j) a[j] = tile[(mk + j) * kMfmaColLdsRow + n_local];
 #pragma unroll
-        for (int bt = 0; bt < BT; ++bt) acc[s][bt] = mfma_32x32x16(a, hb[bt], acc[s][bt]);
+        for (int bt = 0; bt < BT; ++bt) acc[s][bt] = mfma_32x32x16(a, hb[ks][bt], acc[s][bt]);
       }
     }
+  };
+
+  if (any_rows) {
+    int rid_cur = to_row(m_begin, fetch_index(m_begin));
+    int rid_n1 = to_row(m_begin + kMfmaColRows, fetch_index(m_begin + kMfmaColRows));
+    load_stage(rid_cur);
+    int mb = m_begin;
+    for (; mb + kMfmaColRows < m_end; mb += kMfmaColRows) {
+      store_stage();
+      // H operands of this step and the index words of the step after next first, then the
+      // weight loads of the next step: the wait for the former leaves the latter in flight
+      load_h(mb, rid_cur);
+      const int64_t raw_n2 = fetch_index(mb + 2 * kMfmaColRows);
+      load_stage(rid_n1);
+      consume();
+      rid_cur = rid_n1;
+      rid_n1 = to_row(mb + 2 * kMfmaColRows, raw_n2);
+    }
+    store_stage();
+    load_h(mb, rid_cur);
+    consume();
   }
   // result rows are columns n of the tile, result columns are batch entries
 #pragma unroll
   for (int s = 0; s < 4; ++s)
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
-      const int n = col0 + (wave * 4 + s) * 32 + 8 * (v / 4) + 4 * half_id + (v % 4);
+      const int n = col0 + s * 32 + 8 * (v / 4) + 4 * half_id + (v % 4);
 #pragma unroll
       for (int bt = 0; bt < BT; ++bt) {
         const int b = bt * 32 + l32;
