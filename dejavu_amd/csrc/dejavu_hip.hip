@@ -361,11 +361,21 @@ int dv_predictor_logits_f16(const void* x, const void* Wa, int64_t ldwa, const v
                             void* logits, void* stream) {
   if (!x || !Wa || !Wb || !hidden || !logits || d <= 0 || r <= 0 || n_out <= 0)
     return DV_ERR_INVALID_ARG;
-  if (B < 1 || B > 8) return DV_ERR_UNSUPPORTED;
+  if (B < 1 || B > 64) return DV_ERR_UNSUPPORTED;
   if (d % 8 || r % 8 || ldwa % 8 || ldwb % 8 || ldwa < d || ldwb < r || !aligned16(x) ||
       !aligned16(Wa) || !aligned16(Wb) || !aligned16(hidden))
     return DV_ERR_ALIGNMENT;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (B > 8) {
+    // more rows than the fixed-order kernel keeps accumulators for: both products on the
+    // matrix cores (no gather, no bias), fp32 accumulation in the MFMA's own order
+    int rc = gather_rows_mfma(reinterpret_cast<const half_t*>(x), reinterpret_cast<const half_t*>(Wa), ldwa,
+                              nullptr, nullptr, 4, B, d, r, r, DV_ACT_ID, reinterpret_cast<half_t*>(hidden), s);
+    if (rc != DV_OK) return rc;
+    return gather_rows_mfma(reinterpret_cast<const half_t*>(hidden), reinterpret_cast<const half_t*>(Wb), ldwb,
+                            nullptr, nullptr, 4, B, r, n_out, n_out, DV_ACT_ID,
+                            reinterpret_cast<half_t*>(logits), s);
+  }
   int rc = canonical_gemv(reinterpret_cast<const half_t*>(x), reinterpret_cast<const half_t*>(Wa),
                           ldwa, B, r, d, reinterpret_cast<half_t*>(hidden), s);
   if (rc != DV_OK) return rc;

@@ -57,8 +57,9 @@ __global__ __launch_bounds__(kMfmaWaves * 64) void gather_rows_mfma_kernel(
     const int m_mine = t * kMfmaRows + l16;
     int64_t id = -1;
     if (m_mine < M)
-      id = IDX64 ? reinterpret_cast<const int64_t*>(idx)[m_mine]
-                 : (int64_t) reinterpret_cast<const int32_t*>(idx)[m_mine];
+      id = idx == nullptr ? (int64_t)m_mine  // no gather: row m of W itself
+           : IDX64        ? reinterpret_cast<const int64_t*>(idx)[m_mine]
+                          : (int64_t) reinterpret_cast<const int32_t*>(idx)[m_mine];
     const bool ok_mine = id >= 0 && id < Z;
     const int rid_mine = ok_mine ? (int)id : 0;
 

@@ -88,9 +88,10 @@ def predictor_logits(x: torch.Tensor, fc0_weight: torch.Tensor, fc1_weight: torc
     else:
         assert out.numel() == B * n_out and out.is_contiguous() and out.dtype == x.dtype
         logits = out.view(B, n_out)
-    # the kernel keeps one accumulator per batch row in registers: at most 8 rows per launch
-    for b0 in range(0, B, 8):
-        nb = min(8, B - b0)
+    # up to 8 rows: fixed summation order (bit-exact contract); 9..64 rows: one pass on the matrix cores
+    step = 8 if B <= 8 else 64
+    for b0 in range(0, B, step):
+        nb = min(step, B - b0)
         check(lib.dv_predictor_logits_f16(_ptr(x[b0:]), _ptr(fc0_weight), fc0_weight.stride(0), _ptr(fc1_weight),
                                           fc1_weight.stride(0), nb, d, r, n_out, _ptr(hidden[b0:]),
                                           _ptr(logits[b0:]), _stream()), "dv_predictor_logits_f16")

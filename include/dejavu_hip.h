@@ -54,7 +54,10 @@ DV_API int dv_canonical_lanes(int n);
  * Replaces ParallelSP.forward, Dejavu/src/ops/fused_dense_sparse_dejavu.py:73-76
  * (duplicate at Dejavu/src/models/modules/mha_dejavu.py:1118-1121).
  *   x (B, d); Wa (r, d) row stride ldwa; Wb (n_out, r) row stride ldwb;
- *   hidden (B, r) scratch/output; logits (B, n_out).  1 <= B <= 8.
+ *   hidden (B, r) scratch/output; logits (B, n_out).  1 <= B <= 64.
+ * Up to 8 rows the summation order is the fixed one (bit-reproducible on the
+ * host); 9..64 rows run as two MFMA products whose fp32 accumulation order is
+ * the matrix core's own (same values within fp16 rounding).
  */
 DV_API int dv_predictor_logits_f16(const void* x, const void* Wa, int64_t ldwa, const void* Wb,
                             int64_t ldwb, int B, int d, int r, int n_out, void* hidden,

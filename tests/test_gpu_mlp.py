@@ -68,6 +68,25 @@ def test_predictor_topk_indices_bit_exact(ops, cfg, batch, k):
     assert np.array_equal(np16(idx), want)
 
 
+@pytest.mark.parametrize("cfg,batch", [("opt-125m", 9), ("opt-6.7b", 16), ("opt-6.7b", 37), ("opt-125m", 64)])
+def test_predictor_more_than_eight_rows_runs_on_the_matrix_cores(ops, cfg, batch):
+    """9..64 rows: the logits come from MFMA products (the matrix core's own fp32 order), so they
+    are compared within tolerance; the union top-k is still the exact top-k of those logits."""
+    t = make(cfg, batch)
+    print(f"case predictor (MFMA) {cfg} B={batch}", flush=True)
+    hidden = torch.empty(batch, t["mlp_Wa"].shape[0], dtype=torch.float16, device="cuda")
+    got = ops.predictor_logits(dev(t["residual"]), dev(t["mlp_Wa"]), dev(t["mlp_Wb"]), hidden=hidden)
+    k = t["K"]
+    idx = ops.topk_indices(got, k)
+    torch.cuda.synchronize()
+    h_ref, l_ref = O.predictor_logits(np16(t["residual"]), np16(t["mlp_Wa"]), np16(t["mlp_Wb"]))
+    assert_close(np16(hidden), h_ref, "predictor hidden")
+    # the second product starts from the device's own fp16 hidden vector
+    want_logits = (np16(hidden).astype(np.float32) @ np16(t["mlp_Wb"]).astype(np.float32).T)
+    assert_close(np16(got), want_logits, "predictor logits")
+    assert np.array_equal(np16(idx), O.topk_lower_index(np16(got), k)), "union top-k of the device logits"
+
+
 # ---------------------------------------------------------------------- top-k
 @pytest.mark.parametrize("n", [12, 96, 97, 512, 3072, 16384, 20480, 36864, 49152, 65536])
 def test_topk_random_and_ties(ops, n):
