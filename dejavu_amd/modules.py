@@ -49,9 +49,8 @@ def side_stream(device=None) -> "torch.cuda.Stream":
 
 
 def join_side_stream() -> None:
-    """Makes the current stream wait for everything enqueued on the side stream so far.
-    Needed once at the end of a forward pass when predictor joins are deferred
-    (``ParallelFusedMLPDejavu.defer_predictor_join``), e.g. before a graph capture ends."""
+    """Makes the current stream wait for everything enqueued on the side stream so far
+    (e.g. before a graph capture that used the side stream ends)."""
     if USE_SIDE_STREAM and _side_streams:
         ev = torch.cuda.Event(enable_timing=False, blocking=False)
         st = side_stream()
@@ -138,12 +137,6 @@ class ParallelFusedMLPDejavu(nn.Module):
         self.sp_stream = None
         self.event_mlp = None
         self.event_mlp_sp = None
-        # When True, forward() returns while the predictor is still running on the side
-        # stream; the logits tensor carries its completion event (``_dv_ready``) and the
-        # next layer's attention module, which consumes it on the same side stream, needs
-        # no join.  Whoever reads the logits on another stream must wait for that event
-        # (or call join_side_stream()).  Off by default: forward() joins before returning.
-        self.defer_predictor_join = False
 
     def _streams(self):
         if self.sp_stream is None:
@@ -186,10 +179,7 @@ class ParallelFusedMLPDejavu(nn.Module):
             out = F.linear(h, self.fc2.weight, self.fc2.bias)
         # (tensor parallel all-reduce of `out` is the identity on one GPU)
         if side:
-            if self.defer_predictor_join:
-                mlp_logit._dv_ready = self.event_mlp_sp
-            else:
-                curr_stream.wait_event(self.event_mlp_sp)
+            curr_stream.wait_event(self.event_mlp_sp)
         return out, mlp_logit
 
 
@@ -284,11 +274,6 @@ class _MHABase(nn.Module):
         torch.cuda.current_stream().record_event(self.event_in)
         with torch.cuda.stream(self.sp_stream):
             self.sp_stream.wait_event(self.event_in)
-            # logits handed over with a deferred join were produced on this same side
-            # stream (in order); a foreign producer stream needs its event waited on
-            ready = getattr(mlp_sp_logit, "_dv_ready", None) if mlp_sp_logit is not None else None
-            if ready is not None:
-                self.sp_stream.wait_event(ready)
             if att_sp is not None:
                 att_idx = ops.topk_indices(att_sp(residual), att_k, dtype=torch.int32, out=att_idx_out)
             if mlp_sp_logit is not None:
