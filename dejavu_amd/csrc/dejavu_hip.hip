@@ -196,7 +196,10 @@ template <int BT, bool IDX64, bool RELU>
 int launch_rows_mfma(const half_t* x, const half_t* W, int64_t ldw, const half_t* bias, const void* idx,
                      int B, int N, int Z, int M, half_t* y, hipStream_t s) {
   auto kern = gather_rows_mfma_kernel<BT, IDX64, RELU>;
-  const size_t lds = (size_t)kMfmaWaves * 2 * kMfmaRows * kMfmaLdsRow * sizeof(half_t);
+  // one 16 x 256 staging tile per wavefront; the same memory later holds the partial result tiles
+  const size_t tile_bytes = (size_t)kMfmaWaves * kMfmaRows * kMfmaLdsRow * sizeof(half_t);
+  const size_t red_bytes = (size_t)kMfmaWaves * BT * 4 * 64 * sizeof(float);
+  const size_t lds = tile_bytes > red_bytes ? tile_bytes : red_bytes;
   static bool granted = false;
   if (!granted) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),

@@ -30,8 +30,13 @@ __device__ __forceinline__ float4_t mfma_16x16x32(half8_t a, half8_t b, float4_t
 // v_mfma_f32_16x16x32_f16 per batch tile of 16, rows as the A operand
 // (lane: row l % 16, k-group l / 16, 8 consecutive k) and X^T as the B operand
 // (lane: batch column l % 16, same k-group).  Result layout: value v of lane l
-// is row 4 * (l / 16) + v, column l % 16.  The 8 partial tiles are summed
-// through LDS in wavefront order.  N % 8 == 0, ldw % 8 == 0, B <= 16 * BT.
+// is row 4 * (l / 16) + v, column l % 16.  Per step a wavefront first stores the
+// tile it loaded during the previous step, then issues the X loads of this step
+// and the weight loads of the next one (all unconditional: addresses clamped,
+// results masked, so that the compiler can count them) and only then multiplies:
+// the weight stream stays in flight during the MFMAs.  The 8 partial tiles are
+// summed through LDS in wavefront order.  idx == nullptr means no gather (row m
+// of W).  N % 8 == 0, ldw % 8 == 0, B <= 16 * BT.
 // ---------------------------------------------------------------------------
 constexpr int kMfmaKC = 256;            // columns per staged chunk
 constexpr int kMfmaRowPad = 8;          // halfs of padding per LDS row (bank spread)
@@ -46,11 +51,14 @@ __global__ __launch_bounds__(kMfmaWaves * 64) void gather_rows_mfma_kernel(
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  half_t* tile = reinterpret_cast<half_t*>(smem_raw) + (size_t)wave * 2 * kMfmaRows * kMfmaLdsRow;
+  half_t* tile = reinterpret_cast<half_t*>(smem_raw) + (size_t)wave * kMfmaRows * kMfmaLdsRow;
   float* red = reinterpret_cast<float*>(smem_raw);  // reused after the main loop
   const int l16 = lane & 15, kg = lane >> 4;  // MFMA operand coordinates
   const int l32 = lane & 31, half_id = lane >> 5;  // staging coordinates
   const int nchunks = (N + kMfmaKC - 1) / kMfmaKC;
+  constexpr int KS = kMfmaKC / 32;  // MFMA k-steps per chunk
+  // batch tiles are multiplied in passes of at most two, to bound the X registers
+  constexpr int BP = BT < 2 ? BT : 2;
 
   for (int t = blockIdx.x; t * kMfmaRows < M; t += gridDim.x) {
     // row id of output row (t*16 + l16), replicated over the four 16-lane groups
@@ -62,53 +70,82 @@ __global__ __launch_bounds__(kMfmaWaves * 64) void gather_rows_mfma_kernel(
                           : (int64_t) reinterpret_cast<const int32_t*>(idx)[m_mine];
     const bool ok_mine = id >= 0 && id < Z;
     const int rid_mine = ok_mine ? (int)id : 0;
+    // the eight staging loads of a chunk: load q covers rows 2q and 2q+1
+    const half_t* wrow[8];
+    unsigned row_ok = 0;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const int row = 2 * q + half_id;
+      wrow[q] = W + (int64_t)__shfl(rid_mine, row, kWave) * ldw;
+      row_ok |= (unsigned)(__shfl((int)ok_mine, row, kWave) != 0) << q;
+    }
 
     float4_t acc[BT];
 #pragma unroll
     for (int bt = 0; bt < BT; ++bt) acc[bt] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    // two chunks (c and c + 8) are staged per iteration: 16 loads in flight per lane
-    for (int c = wave; c < nchunks; c += 2 * kMfmaWaves) {
-      half8_t stage[2][8];
+    half8_t stage[8];
+    auto load_stage = [&](int c) {
+      int col = c * kMfmaKC + l32 * 8;
+      if (col >= N) col = 0;  // masked when stored
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        const int col = (c + u * kMfmaWaves) * kMfmaKC + l32 * 8;
+      for (int q = 0; q < 8; ++q) stage[q] = load8_stream(wrow[q] + col);
+    };
+    auto store_stage = [&](int c) {
+      const bool col_ok = c * kMfmaKC + l32 * 8 < N;
+      __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");  // previous tile fully read
+      __builtin_amdgcn_wave_barrier();
 #pragma unroll
-        for (int r2 = 0; r2 < 8; ++r2) {
-          const int row = 2 * r2 + half_id;
-          const int rid = __shfl(rid_mine, row, kWave);
-          const bool ok = __shfl((int)ok_mine, row, kWave) != 0;
-          stage[u][r2] = (ok && col < N) ? load8_stream(W + (int64_t)rid * ldw + col) : zero8();
-        }
-      }
-#pragma unroll
-      for (int u = 0; u < 2; ++u)
-#pragma unroll
-        for (int r2 = 0; r2 < 8; ++r2)
-          store8(tile + (u * kMfmaRows + 2 * r2 + half_id) * kMfmaLdsRow + l32 * 8, stage[u][r2]);
-      // the tile is private to this wavefront, whose LDS accesses complete in order: a
-      // wavefront-scope fence (compiler ordering only) is all the synchronisation needed
+      for (int q = 0; q < 8; ++q)
+        store8(tile + (2 * q + half_id) * kMfmaLdsRow + l32 * 8,
+               (col_ok && ((row_ok >> q) & 1u)) ? stage[q] : zero8());
       __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
       __builtin_amdgcn_wave_barrier();
+    };
+    // X operands of chunk c for batch tiles [bt0, bt0 + BP): columns past N and batch rows
+    // past B read a valid address; the weights there are zero / the results are dropped
+    half8_t xb[KS][BP];
+    auto load_x = [&](int c, int bt0) {
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        const int k0 = (c + u * kMfmaWaves) * kMfmaKC;
-        if (k0 < N) {
+      for (int ks = 0; ks < KS; ++ks) {
+        int kk = c * kMfmaKC + ks * 32 + kg * 8;
+        if (kk >= N) kk = 0;
 #pragma unroll
-          for (int ks = 0; ks < kMfmaKC / 32; ++ks) {
-            const int kk = k0 + ks * 32 + kg * 8;
-            const half8_t a = load8(tile + (u * kMfmaRows + l16) * kMfmaLdsRow + ks * 32 + kg * 8);
-#pragma unroll
-            for (int bt = 0; bt < BT; ++bt) {
-              const int b = bt * 16 + l16;
-              const half8_t xb = (b < B && kk < N) ? load8(X + (int64_t)b * N + kk) : zero8();
-              acc[bt] = mfma_16x16x32(a, xb, acc[bt]);
-            }
-          }
+        for (int p = 0; p < BP; ++p) {
+          const int b = (bt0 + p) * 16 + l16;
+          xb[ks][p] = load8(X + (int64_t)(b < B ? b : 0) * N + kk);
         }
       }
-      __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");  // reads done before the tile is overwritten
-      __builtin_amdgcn_wave_barrier();
+    };
+    auto multiply = [&](int bt0) {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const half8_t a = load8(tile + l16 * kMfmaLdsRow + ks * 32 + kg * 8);
+#pragma unroll
+        for (int p = 0; p < BP; ++p) acc[bt0 + p] = mfma_16x16x32(a, xb[ks][p], acc[bt0 + p]);
+      }
+    };
+
+    int c = wave;
+    if (c < nchunks) {
+      load_stage(c);
+      for (; c + kMfmaWaves < nchunks; c += kMfmaWaves) {
+        store_stage(c);
+        load_x(c, 0);
+        load_stage(c + kMfmaWaves);
+        multiply(0);
+#pragma unroll
+        for (int bt0 = BP; bt0 < BT; bt0 += BP) {
+          load_x(c, bt0);
+          multiply(bt0);
+        }
+      }
+      store_stage(c);
+#pragma unroll
+      for (int bt0 = 0; bt0 < BT; bt0 += BP) {
+        load_x(c, bt0);
+        multiply(bt0);
+      }
     }
     // sum the 8 wavefronts' partial tiles (fixed order) and finish
     __syncthreads();  // every wavefront is done with its staging region
