@@ -191,6 +191,12 @@ int gather_cols(const half_t* x, int64_t ldx, int x_expanded, const half_t* W, i
   return launch_status();
 }
 
+// Largest batch the vector-ALU kernels take; above it the MFMA kernels are faster (measured at
+// the OPT-175B shape: fc1 19 us on MFMA against 24 / 39 us at batch 3 / 4, fc2 22-24 us on the
+// vector ALUs against 30 us on MFMA up to batch 4).
+constexpr int kRowsVecMaxBatch = 2;
+constexpr int kColsVecMaxBatch = 4;
+
 // ---- batched gathered GEMMs on the matrix cores (5 <= B <= 64) -------------------
 template <int BT, bool IDX64, bool RELU>
 int launch_rows_mfma(const half_t* x, const half_t* W, int64_t ldw, const half_t* bias, const void* idx,
@@ -321,15 +327,17 @@ int launch_qkv(const half_t* x, const half_t* W, const half_t* bias, const int* 
   return launch_status();
 }
 
-// More than eight window tokens: one pass on the matrix cores covers all 16 slots at a cost
-// that does not grow with the number of live ones (measured break-even at 6..8 tokens).
-inline bool qkv_use_mfma(int nb, int d) { return nb > 8 && d % 64 == 0; }
+// Window tokens from which one pass on the matrix cores (all 16 slots at a cost that hardly grows
+// with the number of live ones) beats the per-token dot products.
+// Measured at the OPT-175B shape: 47 us for one token on the vector path (49 us on MFMA), and
+// 47..49 us for 2..16 tokens on MFMA against 52..95 us on the vector path.
+inline bool qkv_use_mfma(int nb) { return nb >= 2; }
 
 int launch_qkv_mfma(const half_t* x, const half_t* W, const half_t* bias, const int* head_idx,
                     const int* batch_idx, int nb, int d, int H, int hd, int nnz, half_t* y,
                     half_t* k_cache, half_t* v_cache, const int* padding, int S, hipStream_t s) {
   const int ntasks = nnz * 3 * (hd / 16);
-  hipLaunchKernelGGL((qkv_window_mfma_kernel<kQkvMfmaWaves, kQkvMfmaUnroll>), dim3(ntasks), dim3(kQkvMfmaWaves * 64), 0, s,
+  hipLaunchKernelGGL((qkv_window_mfma_kernel<kQkvMfmaWaves>), dim3(ntasks), dim3(kQkvMfmaWaves * 64), 0, s,
                      x, W, bias, head_idx, batch_idx, nb, d, H, hd, nnz, y, k_cache, v_cache, padding, S);
   return launch_status();
 }
@@ -474,7 +482,7 @@ int dv_gather_gemv_f16(const void* x, const void* W, int64_t ldw, const void* bi
   const half_t* ww = reinterpret_cast<const half_t*>(W);
   const half_t* bb = reinterpret_cast<const half_t*>(bias);
   half_t* yy = reinterpret_cast<half_t*>(y);
-  if (B > 4) return gather_rows_mfma(xx, ww, ldw, bb, idx, idx_bytes, B, N, Z, M, act, yy, s);
+  if (B > kRowsVecMaxBatch) return gather_rows_mfma(xx, ww, ldw, bb, idx, idx_bytes, B, N, Z, M, act, yy, s);
   switch (B) {
     case 1: return gather_rows_b<1>(xx, ww, ldw, bb, idx, idx_bytes, N, Z, M, act, yy, s);
     case 2: return gather_rows_b<2>(xx, ww, ldw, bb, idx, idx_bytes, N, Z, M, act, yy, s);
@@ -485,7 +493,7 @@ int dv_gather_gemv_f16(const void* x, const void* W, int64_t ldw, const void* bi
 
 size_t dv_gather_transposed_gemv_workspace_bytes(int B, int N, int M) {
   if (B < 1 || N < 1 || M < 0) return 0;
-  return B > 4 ? cols_mfma_workspace_bytes(B, N, M) : cols_workspace_bytes(B, N, M);
+  return B > kColsVecMaxBatch ? cols_mfma_workspace_bytes(B, N, M) : cols_workspace_bytes(B, N, M);
 }
 
 int dv_gather_transposed_gemv_f16(const void* x, const void* W, int64_t ldw, const void* bias,
@@ -496,7 +504,7 @@ int dv_gather_transposed_gemv_f16(const void* x, const void* W, int64_t ldw, con
     return DV_ERR_INVALID_ARG;
   if (B < 1 || B > 64) return DV_ERR_UNSUPPORTED;
   if (N % 8 || ldw % 8 || ldw < N || !aligned16(W)) return DV_ERR_ALIGNMENT;
-  if (B > 4)
+  if (B > kColsVecMaxBatch)
     return gather_cols_mfma(reinterpret_cast<const half_t*>(x), M, 0, reinterpret_cast<const half_t*>(W),
                             ldw, reinterpret_cast<const half_t*>(bias), idx, idx_bytes, 1, B, N, Z, M,
                             reinterpret_cast<half_t*>(y), workspace, workspace_bytes,
@@ -527,15 +535,9 @@ int dv_qkv_proj_sparse_cache_f16(const void* x, const void* W, const void* bias,
   half_t* kc = reinterpret_cast<half_t*>(k_cache);
   half_t* vc = reinterpret_cast<half_t*>(v_cache);
   const int* pad = reinterpret_cast<const int*>(padding);
-  if (qkv_use_mfma(nb, d))
+  if (qkv_use_mfma(nb))
     return launch_qkv_mfma(xx, ww, bb, hi, bi, nb, d, H, hd, nnz, yy, kc, vc, pad, S, s);
-#define DV_QKV(NB) return launch_qkv<NB>(xx, ww, bb, hi, bi, nb, d, H, hd, nnz, yy, kc, vc, pad, S, s)
-  if (nb == 1) DV_QKV(1);
-  if (nb == 2) DV_QKV(2);
-  if (nb <= 4) DV_QKV(4);
-  if (nb <= 8) DV_QKV(8);
-  DV_QKV(16);
-#undef DV_QKV
+  return launch_qkv<1>(xx, ww, bb, hi, bi, nb, d, H, hd, nnz, yy, kc, vc, pad, S, s);
 }
 
 int dv_qkv_proj_sparse_f16(const void* x, const void* W, const void* bias, const void* head_idx,
@@ -899,7 +901,7 @@ int dv_sparse_layer_decode_f16(const dvSparseLayerArgs* args, void* stream) {
     QkvArgs q{x_cache, CH(a.Wqkv), CH(a.bqkv), head_idx, batch_idx, nb, a.d, a.H, a.hd, a.Hk, qkv,
               reinterpret_cast<half_t*>(a.k_cache), reinterpret_cast<half_t*>(a.v_cache),
               reinterpret_cast<const int*>(a.cache_offset), a.S};
-    const bool mfma = qkv_use_mfma(nb, a.d);
+    const bool mfma = qkv_use_mfma(nb);
     const int ntasks = a.Hk * 3 * (a.hd / 2);
     int nq = (ntasks + 3) / 4;
     if (nq > cus * 8) nq = cus * 8;
@@ -912,11 +914,7 @@ int dv_sparse_layer_decode_f16(const dvSparseLayerArgs* args, void* stream) {
   hipLaunchKernelGGL((layer_l2_kernel<NB>), grid, dim3(256), 0, s, q, nq, hp0, nh, CH(a.mlp_logit_in), \
                      a.ffn, topk_ws)
     if (mfma) DV_L2(0);
-    else if (nb == 1) DV_L2(1);
-    else if (nb == 2) DV_L2(2);
-    else if (nb <= 4) DV_L2(4);
-    else if (nb <= 8) DV_L2(8);
-    else DV_L2(16);
+    else DV_L2(1);
 #undef DV_L2
   }
   // L3: attention partials | head predictor fc1 | top-k threshold and counts

@@ -88,9 +88,9 @@ DV_API int dv_topk_search_f16(const void* logits, int B, int n, int k, void* idx
  * y = act(x . W[idx]^T + bias[idx]).  Replaces gather_gemv,
  * Dejavu/src/ops/triton/gather_gemv.py:198-254.
  *   x (B, N); W (Z, N) row stride ldw; bias (Z,) or NULL; idx (M,);
- *   y (B, M) fp16.  1 <= B <= 64: B <= 4 (the reference's own limit) runs as a
- *   bandwidth-bound GEMV on the vector ALUs; 5 <= B <= 64 stages the gathered
- *   rows through LDS into 32x32x16 fp16 MFMA tiles.
+ *   y (B, M) fp16.  1 <= B <= 64 (the reference stops at 4): B <= 2 runs as a
+ *   bandwidth-bound GEMV on the vector ALUs; 3 <= B <= 64 stages the gathered
+ *   rows through LDS into 16x16x32 fp16 MFMA tiles.
  */
 DV_API int dv_gather_gemv_f16(const void* x, const void* W, int64_t ldw, const void* bias,
                        const void* idx, int idx_bytes, int B, int N, int Z, int M, int act,

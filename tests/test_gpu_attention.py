@@ -38,7 +38,7 @@ def randh(g, *shape, std=1.0):
 # ------------------------------------------------------------------ QKV
 @pytest.mark.parametrize("H,hd,d,nb,nnz", [(12, 128, 12288, 16, 4), (12, 128, 1024, 1, 4), (6, 64, 768, 3, 2),
                                            (8, 128, 1152, 5, 8), (8, 32, 512, 8, 3), (12, 128, 2048, 2, 12),
-                                           # more than 8 rows: matrix-core kernel (d % 64 == 0) or its fallback
+                                           # two or more rows run on the matrix cores
                                            (8, 64, 1024, 12, 3), (5, 64, 384, 9, 5), (4, 32, 128, 16, 2),
                                            (6, 128, 640, 16, 3)])
 def test_qkv_proj_sparse(ops, H, hd, d, nb, nnz):
@@ -73,9 +73,9 @@ def test_qkv_proj_sparse(ops, H, hd, d, nb, nnz):
     assert np.array_equal(np16(out2) == 7.0, want == 7.0), "written / untouched pattern differs"
 
 
-def test_qkv_many_rows_with_hidden_size_not_a_multiple_of_64(ops):
+def test_qkv_many_rows_with_hidden_size_not_a_multiple_of_the_chunk(ops):
     """Straight through the C ABI (the Python operator keeps the reference's d % 128 == 0
-    precondition): 16 window rows with d % 64 != 0 take the per-row kernel."""
+    precondition): 16 window rows with d = 328, which ends in a partial 256-column chunk."""
     from dejavu_amd._lib import check, lib
 
     g = torch.Generator().manual_seed(3)
