@@ -840,7 +840,7 @@ int check_layer_args(const dvSparseLayerArgs& a) {
     return DV_ERR_INVALID_ARG;
   if (a.d <= 0 || a.ffn <= 0 || a.H <= 0 || a.Hk < 1 || a.Hk > a.H || a.att_k < 1 || a.att_k > a.H ||
       a.K < 1 || a.K > a.ffn || a.r_att <= 0 || a.r_mlp <= 0 || a.S <= 0 || a.n_len < 1 || a.n_len > a.S ||
-      a.counter < 0 || a.counter > 14)
+      a.counter < 0 || a.counter > 15 || (a.counter == 15 && a.Hk != a.H))
     return DV_ERR_INVALID_ARG;
   if ((a.hd != 64 && a.hd != 128) || a.H * a.hd != a.d || a.H > 1024 || a.ffn > 65536 || a.ffn <= 1024 ||
       a.d > 1024 * 8 * 4 || (size_t)a.d * 2 > 160 * 1024)
@@ -890,7 +890,8 @@ int dv_sparse_layer_decode_f16(const dvSparseLayerArgs* args, void* stream) {
 #define DV_L1(V)                                                                                      \
   hipLaunchKernelGGL((layer_l1_kernel<V>), dim3(1), dim3(kLnThreads), 0, s, CH(a.hidden), CH(a.residual), \
                      CH(a.ln1_w), CH(a.ln1_b), a.eps1, a.d, x, res1, x_cache + (size_t)a.counter * a.d, \
-                     reinterpret_cast<int*>(a.tracker), head_idx, a.Hk, a.H, a.counter, batch_idx)
+                     reinterpret_cast<int*>(a.tracker), head_idx, a.Hk, a.H, a.counter,        \
+                     a.counter == 15 ? 1 : 0, batch_idx)
     if (a.d <= kLnThreads * 8) DV_L1(1);
     else if (a.d <= kLnThreads * 16) DV_L1(2);
     else DV_L1(4);

@@ -34,9 +34,9 @@ __global__ __launch_bounds__(kLnThreads) void layer_l1_kernel(
     const half_t* __restrict__ gamma, const half_t* __restrict__ beta, float eps, int d,
     half_t* __restrict__ x, half_t* __restrict__ residual1, half_t* __restrict__ x_cache_row,
     int* __restrict__ tracker, const int* __restrict__ head_idx, int nnz, int H, int counter,
-    int* __restrict__ batch_idx) {
+    int flush, int* __restrict__ batch_idx) {
   add_layer_norm_body<kLnThreads, MAXV>(hidden, residual, gamma, beta, eps, d, x, residual1, x_cache_row, 0);
-  window_tracker_step(tracker, head_idx, nnz, H, counter, 0, batch_idx);
+  window_tracker_step(tracker, head_idx, nnz, H, counter, flush, batch_idx);
 }
 
 // ---- L2 -------------------------------------------------------------------

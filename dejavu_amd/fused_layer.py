@@ -1,7 +1,7 @@
 """Fast path for one decode step of a whole sparse block (``dv_sparse_layer_decode_f16``).
 
 ``BlockMlpAttSparse.forward`` takes it when the step is an ordinary head-sparse decode step
-(batch 1, one token, fp16, predictions available, not a window-flush step); everything else
+(batch 1, one token, fp16, predictions available), the window-flush step included; everything else
 goes through the modules' own forwards.  Same results either way: the fused entry point runs
 the same kernel bodies in nine launches instead of about twenty.
 """
@@ -77,7 +77,7 @@ def eligible(block, hidden_states, residual, head_idx, mlp_sp_logit, inference_p
         return False
     if not (hidden_states.is_cuda and hidden_states.dtype == torch.float16 and hidden_states.numel() == m.embed_dim):
         return False
-    if f.activation != "relu" or m.counter >= m.WINDOW - 1 or m.head_dim not in (64, 128):
+    if f.activation != "relu" or m.counter >= m.WINDOW or m.head_dim not in (64, 128):
         return False
     if mlp_sp_logit.dim() != 1 or f.fc1.out_features <= 1024 or f.fc1.out_features > 65536:
         return False
@@ -96,6 +96,11 @@ def sparse_layer_decode(block, hidden_states, residual, head_idx, mlp_sp_logit, 
         m.out_proj_weight_t = m.out_proj.weight.t().contiguous()
     if m.cache_offset is None:
         m._set_cache_offset(inference_params.sequence_len_offset - m.counter, dev)
+    flush = m.counter == m.WINDOW - 1
+    if flush:  # every 16th token all heads catch up on the whole window
+        if m._all_heads is None:
+            m._all_heads = torch.arange(H, dtype=torch.int32, device=dev)
+        head_idx = m._all_heads
     k_cache, v_cache = inference_params.key_value_memory_dict[m.layer_idx]
     b0 = inference_params.batch_size_offset
     kc, vc = k_cache[b0:b0 + 1], v_cache[b0:b0 + 1]
@@ -142,5 +147,8 @@ def sparse_layer_decode(block, hidden_states, residual, head_idx, mlp_sp_logit, 
     check(lib.dv_sparse_layer_decode_f16(ctypes.byref(a), torch.cuda.current_stream().cuda_stream),
           "dv_sparse_layer_decode_f16")
     m.counter += 1
+    if flush:  # window complete: start the next one
+        m.counter = 0
+        m.cache_offset += m.WINDOW
     block.last_mlp_idx = mlp_idx_out
     return hidden_out, residual_out, logit_out.view(-1), att_idx_out

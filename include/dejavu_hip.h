@@ -263,8 +263,9 @@ DV_API int dv_add_layer_norm_f16(const void* h, const void* residual, const void
  * Dejavu/src/models/modules/block_dejavu.py:555-663 (mixer:
  * Dejavu/src/models/modules/mha_dejavu.py:1283-1511, mlp:
  * Dejavu/src/ops/fused_dense_sparse_dejavu.py:889-951).
- * Steps that flush the window (every 16th token, all heads and all 16 tokens)
- * are not taken by this entry point: callers run them through the separate ones.
+ * The step that flushes the window (counter 15: every 16th token, all heads and
+ * all 16 tokens, mha_dejavu.py:1320-1326) is taken with head_idx = 0..H-1 and
+ * Hk = H.
  */
 typedef struct dvSparseLayerArgs {
   /* shapes */
@@ -272,7 +273,7 @@ typedef struct dvSparseLayerArgs {
   int r_att, r_mlp;       /* predictor ranks                                           */
   int K, Hk, att_k;       /* active neurons; heads computed now; heads predicted next  */
   int S;                  /* KV cache capacity                                         */
-  int counter;            /* window position of this token, 0..14                      */
+  int counter;            /* window position of this token, 0..15 (15: flush, Hk == H) */
   int n_len;              /* cached positions to attend, newest token included         */
   float eps1, eps2, softmax_scale;
   /* inputs (device, fp16 unless stated) */
