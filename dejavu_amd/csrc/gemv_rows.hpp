@@ -50,12 +50,23 @@ __device__ __forceinline__ void canonical_gemv_body(
           acc[b] = fma8_ordered(w[u], load8(xr + (int64_t)b * n + base + u * CH), acc[b]);
       }
     }
-    for (; base < n; base += CH) {
-      if (base + sub * 8 < n) {
-        half8_t w = load8_stream(wr + base);
+    if (base < n) {
+      // the remaining (fewer than U) chunks, the last one possibly partial: their loads are
+      // issued together like those of a full group; lanes past the row end take no part
+      half8_t w[U];
+      bool in[U];
 #pragma unroll
-        for (int b = 0; b < B; ++b)
-          acc[b] = fma8_ordered(w, load8(xr + (int64_t)b * n + base), acc[b]);
+      for (int u = 0; u < U; ++u) {
+        in[u] = base + u * CH + sub * 8 < n;
+        w[u] = in[u] ? load8_stream(wr + base + u * CH) : zero8();
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (in[u]) {
+#pragma unroll
+          for (int b = 0; b < B; ++b)
+            acc[b] = fma8_ordered(w[u], load8(xr + (int64_t)b * n + base + u * CH), acc[b]);
+        }
       }
     }
 #pragma unroll
