@@ -27,7 +27,8 @@ def ops():
     return _ops
 
 
-@pytest.mark.parametrize("cfg,B,K", [("opt-125m", 5, 1024), ("opt-125m", 16, 1024), ("opt-125m", 33, 1000),
+@pytest.mark.parametrize("cfg,B,K", [("opt-125m", 3, 1024), ("opt-6.7b", 4, 4096),  # fc1 on MFMA, fc2 on the vector ALUs
+                                     ("opt-125m", 5, 1024), ("opt-125m", 16, 1024), ("opt-125m", 33, 1000),
                                      ("opt-6.7b", 8, 2048), ("opt-6.7b", 16, 4096), ("opt-6.7b", 32, 2048),
                                      ("opt-6.7b", 64, 1024)])
 @pytest.mark.parametrize("idx_dtype", [torch.int64, torch.int32])
@@ -56,6 +57,11 @@ def test_batched_mlp_sparse_matches_oracle(ops, cfg, B, K, idx_dtype):
     torch.cuda.synchronize()
     assert_close(np16(h)[:1], np16(h1), "fc1 MFMA vs GEMV row 0")
     assert_close(np16(y)[:1], np16(y1), "fc2 MFMA vs GEMV row 0")
+
+
+def test_batched_mlp_sparse_at_the_headline_shape(ops):
+    """OPT-175B-shaped block, batch 32 (the matrix-core path at full size)."""
+    test_batched_mlp_sparse_matches_oracle(ops, "opt-175b", 32, 4096, torch.int64)
 
 
 def test_batched_edge_cases(ops):
