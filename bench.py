@@ -289,7 +289,7 @@ def decode_bench(args):
 
 def mlp_bench(args):
     """Sparse MLP block (predictor + union top-k + fc1 + fc2) at batch sizes 1..64: batches up to
-    4 stream the gathered rows through the vector ALUs, larger ones through LDS into MFMA tiles.
+    2 (fc1) / 4 (fc2) stream the gathered rows through the vector ALUs, larger ones run on MFMA tiles.
     Prints its own JSON line; a step is one block step at the given batch."""
     import torch
 
@@ -341,7 +341,7 @@ def mlp_bench(args):
             out["fc1_fc2"]["TFLOP/s"] = round(2.0 * B * (weight_bytes / 2) / out["fc1_fc2"]["us"] / 1e6, 2)
             out["tokens_per_s"] = round(B / (out["block"]["us"] * 1e-6), 1)
             out["path"] = ("vector ALU gather-GEMV" if B <= 2 else
-                           "fc1 on MFMA tiles, fc2 vector ALU" if B <= 4 else "LDS-staged MFMA tiles")
+                           "fc1 on MFMA tiles, fc2 vector ALU" if B <= 4 else "MFMA tiles (fc1 LDS-staged, fc2 register-transposed)")
             results[str(B)] = out
     print(json.dumps({
         "metric": f"us per sparse MLP block step, {args.config} shape, K={K}", "unit": "us/step", "n_gpus": 1,

@@ -243,9 +243,9 @@ ColsMfmaPlan plan_cols_mfma(int B, int N, int M) {
   ColsMfmaPlan p;
   p.col_tiles = (N + kMfmaColTile - 1) / kMfmaColTile;
   // Every row group writes a (B, N) fp32 partial that a second pass reads back, so few, long
-  // groups win: each wavefront (128 columns of one group) keeps 16 KiB of weights in flight
-  // and three to four of them per compute unit measured best for batch 8..64.
-  const int waves_per_cu = B <= 8 ? 4 : 3;
+  // groups win: each wavefront (256 columns of one group) keeps 16 KiB of weights in flight
+  // and three of them per compute unit measured best for batch 8..64.
+  const int waves_per_cu = 3;
   const int col_waves = (N + kMfmaColWave - 1) / kMfmaColWave;
   int groups = (compute_units() * waves_per_cu + col_waves - 1) / col_waves;
   const int max_groups = M > kMfmaColRows ? (M + kMfmaColRows - 1) / kMfmaColRows : 1;

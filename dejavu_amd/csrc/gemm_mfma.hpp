@@ -179,101 +179,85 @@ __global__ __launch_bounds__(kMfmaWaves * 64) void gather_rows_mfma_kernel(
 
 // ---------------------------------------------------------------------------
 // fc2 / out_proj over a transposed weight: Y[b, n] = sum_m H[b, m] * W[row(m), n].
-// The contraction index m runs over gathered ROWS, so the weight tile must be
-// transposed on its way to the MFMA.  Every wavefront works on its own: it owns
-// 128 of the workgroup's 512 columns and walks the workgroup's row group 64 rows
-// at a time.  Per step it copies 64 rows x 128 columns (sixteen loads of 4 rows x
-// 256 contiguous bytes) through registers into a private LDS tile, issues the
-// loads of the NEXT step, and only then consumes the tile: for each of its four
-// 32-column sub-tiles the A operand W^T (n x m) is gathered with 16-bit LDS
-// reads and multiplied by H^T (m x b), which comes straight from memory.  No
-// workgroup barrier is needed; the weight stream stays in flight during the
-// MFMAs.  Partial sums over the row groups (gridDim.y) go to `partial`
-// [(g * B + b) * N + n] and are reduced by cols_reduce_kernel; with one group
-// the result (+ bias) is written directly.
+// The contraction index m runs over gathered ROWS, while the MFMA wants 8
+// consecutive k per lane: the transposition happens inside each lane's registers,
+// no LDS involved.  A wavefront owns 256 columns.  Lanes 0..31 load 16 bytes
+// (8 columns) of row m, lanes 32..63 the same columns of row m + 8, eight rows
+// each per k-step of 16 (one load instruction reads 2 rows x 512 contiguous
+// bytes).  A lane then holds an 8 x 8 block (8 rows x its 8 columns); read
+// column-wise, column e of that block is exactly an operand of
+// v_mfma_f32_32x32x16_f16 for output column 8 * (lane % 32) + e and k-group
+// lane / 32, so eight MFMAs (e = 0..7) consume the 16 x 256 tile.  H^T (m x b) is
+// the other operand, straight from memory.  Two k-steps (32 rows) are in flight per
+// pipeline step; the next step's loads are issued before the MFMAs (all loads
+// unconditional so that the compiler can count them).  Partial sums over the
+// row groups (gridDim.y) go to `partial` [(g * B + b) * N + n] and are reduced by
+// cols_reduce_kernel; with one group the result (+ bias) is written directly.
 // Row mapping as gather_cols_kernel: BLOCKED ? idx[m / blk] * blk + m % blk : idx[m];
 // x_expanded: H is (B, Z) indexed by row(m) instead of (B, M) indexed by m.
 // HVEC: H is read with 128-bit loads; the host guarantees M % 8 == 0, ldh % 8 == 0, a
 // 16-byte aligned H and, for the expanded layout, blk % 8 == 0 (groups of 8 rows never
 // straddle a block).  Otherwise H is gathered element by element.
 // ---------------------------------------------------------------------------
-constexpr int kMfmaColTile = 512;               // columns per workgroup
-constexpr int kMfmaColWave = 128;               // columns per wavefront
-constexpr int kMfmaColLdsRow = kMfmaColWave + 8;  // halfs per LDS tile row (bank spread)
-constexpr int kMfmaColRows = 64;                // rows per step
+constexpr int kMfmaColWave = 256;                 // columns per wavefront
+constexpr int kMfmaColTile = 4 * kMfmaColWave;    // columns per workgroup
+constexpr int kMfmaColRows = 32;                  // rows per pipeline step (two k-steps of 16)
 
 template <int BT, bool IDX64, bool BLOCKED, bool HVEC>
 __global__ __launch_bounds__(256) void gather_cols_mfma_kernel(
     const half_t* __restrict__ H, int64_t ldh, int x_expanded, const half_t* __restrict__ W,
     int64_t ldw, const half_t* __restrict__ bias, const void* __restrict__ idx, int blk, int B, int N,
     int Z, int M, int rows_per_block, float* __restrict__ partial, half_t* __restrict__ Y) {
-  __shared__ __attribute__((aligned(16))) half_t tiles[4][kMfmaColRows * kMfmaColLdsRow];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  half_t* tile = tiles[wave];
   const int half_id = lane >> 5, l32 = lane & 31;
-  const int lrow = lane >> 4, lcol = (lane & 15) * 8;  // staging coordinates: 4 rows x 16 pieces of 8 columns
   const int ct = blockIdx.x, g = blockIdx.y, G = gridDim.y;
   const int col0 = ct * kMfmaColTile + wave * kMfmaColWave;
-  const bool col_ok = col0 + lcol < N;  // N % 8 == 0
+  // columns past N accumulate garbage that is never stored; their loads re-read column 0
+  const int wcol = col0 + l32 * 8 < N ? col0 + l32 * 8 : 0;
   const int m_begin = g * rows_per_block;
   int m_end = m_begin + rows_per_block;
   if (m_end > M) m_end = M;
   const bool any_rows = m_begin < m_end;
-  // Every load below is unconditional (addresses clamped to something valid, results
-  // masked afterwards): with a fixed number of loads per step the compiler can wait for
-  // the older H loads while the newer weight loads stay in flight.
-  // raw index word of row (mb + lane); rows past the group re-read its first row
+  // raw index word of row (mb + l32); rows past the group re-read its first row
   auto fetch_index = [&](int mb) -> int64_t {
     if (!any_rows) return -1;
-    int m = mb + lane;
+    int m = mb + l32;
     if (m >= m_end) m = m_begin;
     if (BLOCKED) m /= blk;
     return IDX64 ? reinterpret_cast<const int64_t*>(idx)[m]
                  : (int64_t) reinterpret_cast<const int32_t*>(idx)[m];
   };
-  // weight row of row (mb + lane), or -1
+  // weight row of row (mb + l32), or -1
   auto to_row = [&](int mb, int64_t raw) -> int {
-    const int m = mb + lane;
+    const int m = mb + l32;
     int64_t id = raw;
     if (BLOCKED) id = (raw >= 0 && raw < Z / blk) ? raw * blk + (m % blk) : -1;
     return (m < m_end && id >= 0 && id < Z) ? (int)id : -1;
   };
 
-  float16_t acc[4][BT];
+  float16_t acc[8][BT];
 #pragma unroll
-  for (int s = 0; s < 4; ++s)
+  for (int e = 0; e < 8; ++e)
 #pragma unroll
     for (int bt = 0; bt < BT; ++bt)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[s][bt][v] = 0.f;
+      for (int v = 0; v < 16; ++v) acc[e][bt][v] = 0.f;
 
-  constexpr int NQ = kMfmaColRows / 4;   // weight load instructions per step
-  constexpr int KS = kMfmaColRows / 16;  // MFMA k-steps per step
-  half8_t stage[NQ];
-  unsigned stage_ok = 0;  // bit q: stage[q] holds a real row
-  const int wcol = col_ok ? col0 + lcol : 0;
-
+  constexpr int KS = kMfmaColRows / 16;  // MFMA k-steps per pipeline step
+  constexpr int NQ = KS * 8;             // weight load instructions per step
+  half8_t next[NQ];                      // rows of the step being loaded
+  unsigned next_ok = 0;                  // bit q: next[q] holds a real row
+  // load q of a step fetches row (q / 8) * 16 + half_id * 8 + q % 8 of the step
   auto load_stage = [&](int rid_all) {
-    stage_ok = 0;
+    next_ok = 0;
 #pragma unroll
     for (int q = 0; q < NQ; ++q) {
-      const int rid = __shfl(rid_all, q * 4 + lrow, kWave);
-      stage[q] = load8_stream(W + (int64_t)(rid >= 0 ? rid : 0) * ldw + wcol);
-      stage_ok |= (unsigned)(rid >= 0 && col_ok) << q;
+      const int rid = __shfl(rid_all, (q / 8) * 16 + half_id * 8 + (q % 8), kWave);
+      next[q] = load8_stream(W + (int64_t)(rid >= 0 ? rid : 0) * ldw + wcol);
+      next_ok |= (unsigned)(rid >= 0) << q;
     }
-  };
-  auto store_stage = [&]() {
-    // reads of the previous step are done before the tile is overwritten (same wavefront:
-    // LDS operations complete in order, the fences only stop compiler reordering)
-    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-#pragma unroll
-    for (int q = 0; q < NQ; ++q)
-      store8(tile + (q * 4 + lrow) * kMfmaColLdsRow + lcol, ((stage_ok >> q) & 1u) ? stage[q] : zero8());
-    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
-    __builtin_amdgcn_wave_barrier();
   };
   half8_t hb[KS][BT];
   auto load_h = [&](int mb, int rid_cur) {
@@ -308,18 +292,22 @@ __global__ __launch_bounds__(256) void gather_cols_mfma_kernel(
       }
     }
   };
-  auto consume = [&]() {
+  half8_t cur[NQ];  // rows of the step being multiplied
+  auto consume = [&](unsigned cur_ok) {
+    if (__ballot(cur_ok != (1u << NQ) - 1u) != 0) {  // rare: rows without a valid id
+#pragma unroll
+      for (int q = 0; q < NQ; ++q)
+        if (!((cur_ok >> q) & 1u)) cur[q] = zero8();
+    }
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      const int mk = ks * 16 + half_id * 8;
 #pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        const int n_local = s * 32 + l32;  // this lane's column inside the wavefront's tile
-        half8_t a;
+      for (int e = 0; e < 8; ++e) {
+        half8_t a;  // column e of the lane's 8 x 8 block
 #pragma unroll
-        for (int j = 0; j < 8; ++j) a[j] = tile[(mk + j) * kMfmaColLdsRow + n_local];
+        for (int j = 0; j < 8; ++j) a[j] = cur[ks * 8 + j][e];
 #pragma unroll
-        for (int bt = 0; bt < BT; ++bt) acc[s][bt] = mfma_32x32x16(a, hb[ks][bt], acc[s][bt]);
+        for (int bt = 0; bt < BT; ++bt) acc[e][bt] = mfma_32x32x16(hb[ks][bt], a, acc[e][bt]);
       }
     }
   };
@@ -330,37 +318,50 @@ __global__ __launch_bounds__(256) void gather_cols_mfma_kernel(
     load_stage(rid_cur);
     int mb = m_begin;
     for (; mb + kMfmaColRows < m_end; mb += kMfmaColRows) {
-      store_stage();
+      const unsigned cur_ok = next_ok;
+#pragma unroll
+      for (int q = 0; q < NQ; ++q) cur[q] = next[q];
       // H operands of this step and the index words of the step after next first, then the
       // weight loads of the next step: the wait for the former leaves the latter in flight
       load_h(mb, rid_cur);
       const int64_t raw_n2 = fetch_index(mb + 2 * kMfmaColRows);
       load_stage(rid_n1);
-      consume();
+      consume(cur_ok);
       rid_cur = rid_n1;
       rid_n1 = to_row(mb + 2 * kMfmaColRows, raw_n2);
     }
-    store_stage();
+    const unsigned cur_ok = next_ok;
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) cur[q] = next[q];
     load_h(mb, rid_cur);
-    consume();
+    consume(cur_ok);
   }
-  // result rows are columns n of the tile, result columns are batch entries
+  // H^T is the first operand, so result rows are batch entries and result columns the lane's
+  // weight columns: value v of MFMA e is batch row 8 * (v / 4) + 4 * half_id + v % 4, column
+  // 8 * l32 + e.  For a fixed v the eight MFMAs hold eight consecutive columns: one vector store.
+  const int n0 = col0 + l32 * 8;
+  if (n0 < N) {  // N % 8 == 0: a lane's eight columns are all inside or all outside
 #pragma unroll
-  for (int s = 0; s < 4; ++s)
+    for (int bt = 0; bt < BT; ++bt)
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int n = col0 + s * 32 + 8 * (v / 4) + 4 * half_id + (v % 4);
+      for (int v = 0; v < 16; ++v) {
+        const int b = bt * 32 + 8 * (v / 4) + 4 * half_id + (v % 4);
+        if (b < B) {
+          if (G == 1) {
+            half8_t o;
 #pragma unroll
-      for (int bt = 0; bt < BT; ++bt) {
-        const int b = bt * 32 + l32;
-        if (n < N && b < B) {
-          if (G == 1)
-            Y[(int64_t)b * N + n] = (half_t)(acc[s][bt][v] + (bias ? (float)bias[n] : 0.f));
-          else
-            partial[((int64_t)g * B + b) * N + n] = acc[s][bt][v];
+            for (int e = 0; e < 8; ++e) o[e] = (half_t)(acc[e][bt][v] + (bias ? (float)bias[n0 + e] : 0.f));
+            store8(Y + (int64_t)b * N + n0, o);
+          } else {
+            float4_t lo{acc[0][bt][v], acc[1][bt][v], acc[2][bt][v], acc[3][bt][v]};
+            float4_t hi{acc[4][bt][v], acc[5][bt][v], acc[6][bt][v], acc[7][bt][v]};
+            float* dst = partial + ((int64_t)g * B + b) * N + n0;
+            *reinterpret_cast<float4_t*>(dst) = lo;
+            *reinterpret_cast<float4_t*>(dst + 4) = hi;
+          }
         }
       }
-    }
+  }
 }
 
 }  // namespace dv
