@@ -183,7 +183,7 @@ def kernel_table(torch, cfg, batch, layers):
     return table
 
 
-def cpu_baseline(torch, cfg, batch, L, timed=15, warm=3):
+def cpu_baseline(torch, cfg, batch, L, timed=40, warm=3):
     """PyTorch CPU index_select + matmul form of the same layer step on the host cores."""
     from oracle import cpu_baseline as C
     from dejavu_amd.workloads import pack_k_cache  # noqa: F401
