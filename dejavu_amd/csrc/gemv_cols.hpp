@@ -79,6 +79,17 @@ __device__ __forceinline__ void gather_cols_body(
       ok = id >= 0 && id < Z;
       rid = ok ? (int)id : 0;
     }
+    // the loop over full batches of U rows is software-pipelined: the next batch's weight
+    // loads are in flight during this batch's multiply-adds, and the first batch is issued
+    // before the activations (for ATTN: the merged attention partials) are known
+    const int cnt = (m_end - mb) < kWave ? (m_end - mb) : kWave;
+    const int nfull = cnt / U;
+    half8_t wn[U];
+    if (nfull > 0) {
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        wn[u] = load8_stream(wcol + (int64_t)__builtin_amdgcn_readlane(rid, u) * ldw);
+    }
     float xl[B];
     if (ATTN) {
       const int nheads = M / blk;
@@ -120,15 +131,7 @@ __device__ __forceinline__ void gather_cols_body(
         xl[b] = ok ? (float)X[(int64_t)b * ldx + (x_expanded ? (int64_t)rid : (int64_t)m)] : 0.f;
     }
 
-    const int cnt = (m_end - mb) < kWave ? (m_end - mb) : kWave;
-    int j = 0;
-    for (; j + U <= cnt; j += U) {
-      half8_t w[U];
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const int r = __builtin_amdgcn_readlane(rid, j + u);
-        w[u] = load8_stream(wcol + (int64_t)r * ldw);
-      }
+    auto consume = [&](const half8_t (&w)[U], int j) {
 #pragma unroll
       for (int u = 0; u < U; ++u) {
 #pragma unroll
@@ -139,6 +142,20 @@ __device__ __forceinline__ void gather_cols_body(
           for (int e = 0; e < 8; ++e) acc[b][e] = __builtin_fmaf((float)w[u][e], xs, acc[b][e]);
         }
       }
+    };
+    int j = 0;
+    for (int jb = 0; jb + 1 < nfull; ++jb, j += U) {
+      half8_t w[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) w[u] = wn[u];
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        wn[u] = load8_stream(wcol + (int64_t)__builtin_amdgcn_readlane(rid, j + U + u) * ldw);
+      consume(w, j);
+    }
+    if (nfull > 0) {
+      consume(wn, j);
+      j += U;
     }
     for (; j < cnt; ++j) {
       const int r = __builtin_amdgcn_readlane(rid, j);
