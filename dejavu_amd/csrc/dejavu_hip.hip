@@ -873,7 +873,6 @@ int dv_sparse_layer_decode_f16(const dvSparseLayerArgs* args, void* stream) {
   half_t* x = H16(p.off_x);
   half_t* res1 = H16(p.off_res1);
   half_t* attn_out = H16(p.off_attn_out);
-  half_t* x2 = H16(p.off_x2);
   half_t* qkv = H16(p.off_qkv);
   half_t* hp_hidden = H16(p.off_hp_hidden);
   half_t* mp_hidden = H16(p.off_mp_hidden);
@@ -946,40 +945,36 @@ int dv_sparse_layer_decode_f16(const dvSparseLayerArgs* args, void* stream) {
     hipLaunchKernelGGL(layer_l4_kernel, dim3(no + 1 + topk_blocks), dim3(256), 0, s, o, no, head_logits, a.H,
                        a.att_k, reinterpret_cast<int*>(a.att_idx_out), CH(a.mlp_logit_in), a.ffn, topk_ws,
                        reinterpret_cast<int64_t*>(a.mlp_idx_out), topk_blocks);
-    if (c.groups > 1)
-      hipLaunchKernelGGL(cols_reduce_kernel, dim3((unsigned)((a.d + 63) / 64)), dim3(256), 0, s, cols_part,
-                         CH(a.bout), c.groups, 1, a.d, attn_out);
-  }
-  // L6: add + LayerNorm 2
-  {
-    half_t* res2 = reinterpret_cast<half_t*>(a.residual_out);
-#define DV_L6(V)                                                                                    \
-  hipLaunchKernelGGL((add_layer_norm_kernel<kLnThreads, V>), dim3(1), dim3(kLnThreads), 0, s, attn_out, \
-                     res1, CH(a.ln2_w), CH(a.ln2_b), a.eps2, a.d, x2, res2)
-    if (a.d <= kLnThreads * 8) DV_L6(1);
-    else if (a.d <= kLnThreads * 16) DV_L6(2);
-    else DV_L6(4);
-#undef DV_L6
+    // L5: split reduction + bias, and the residual stream advanced by the attention output
+    hipLaunchKernelGGL(cols_reduce_kernel, dim3((unsigned)((a.d + 63) / 64)), dim3(256), 0, s,
+                       c.groups > 1 ? cols_part : nullptr, CH(a.bout), c.groups, 1, a.d, attn_out, res1,
+                       reinterpret_cast<half_t*>(a.residual_out));
   }
   const half_t* res2 = reinterpret_cast<const half_t*>(a.residual_out);
   const int64_t* mlp_idx = reinterpret_cast<const int64_t*>(a.mlp_idx_out);
-  // L7: fc1 gather | MLP predictor fc0
+  // L7: LayerNorm 2 + fc1 gather | MLP predictor fc0
   {
-    RowsArgs f{x2, CH(a.W1), CH(a.b1), mlp_idx, a.d, (int64_t)a.d, a.ffn, a.K, hbuf};
+    RowsArgs f{res2, CH(a.ln2_w), CH(a.ln2_b), a.eps2, CH(a.W1), CH(a.b1), mlp_idx, a.d, (int64_t)a.d, a.ffn,
+               a.K, hbuf};
     int nf = ((a.K + 1) / 2 + 3) / 4;
     if (nf > cus * 8) nf = cus * 8;
     CanonArgs mp0{res2, CH(a.mlp_Wa), (int64_t)a.d, a.r_mlp, a.d, mp_hidden};
     const int rw0 = a.d <= 1024 ? 4 : 1;
     const int nm = ((a.r_mlp + rw0 - 1) / rw0 + 3) / 4;
     const size_t lds = (size_t)a.d * sizeof(half_t);
-    static size_t lds_granted = 48 * 1024;
-    if (lds > lds_granted) {
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(layer_l7_kernel),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+    const int v = a.d <= 8192 ? 0 : (a.d <= 16384 ? 1 : 2);
+    const void* l7[3] = {reinterpret_cast<const void*>(layer_l7_kernel<1>),
+                         reinterpret_cast<const void*>(layer_l7_kernel<2>),
+                         reinterpret_cast<const void*>(layer_l7_kernel<4>)};
+    static size_t lds_granted[3] = {48 * 1024, 48 * 1024, 48 * 1024};
+    if (lds > lds_granted[v]) {
+      if (hipFuncSetAttribute(l7[v], hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
         return DV_ERR_UNSUPPORTED;
-      lds_granted = lds;
+      lds_granted[v] = lds;
     }
-    hipLaunchKernelGGL(layer_l7_kernel, dim3(nf + nm), dim3(256), lds, s, f, nf, mp0, nm);
+    if (v == 0) hipLaunchKernelGGL(layer_l7_kernel<1>, dim3(nf + nm), dim3(256), lds, s, f, nf, mp0, nm);
+    else if (v == 1) hipLaunchKernelGGL(layer_l7_kernel<2>, dim3(nf + nm), dim3(256), lds, s, f, nf, mp0, nm);
+    else hipLaunchKernelGGL(layer_l7_kernel<4>, dim3(nf + nm), dim3(256), lds, s, f, nf, mp0, nm);
   }
   // L8 + L9: fc2 gather | MLP predictor fc1, then the split reduction
   {

@@ -262,14 +262,23 @@ __global__ __launch_bounds__(256) void gather_cols_kernel(
 // Second pass of the non-fused path: Y[b, c] = fp16(sum_g partial[g, b, c] + bias[c]).
 // A workgroup owns 64 outputs; its four wavefronts each add every fourth group
 // (ascending), and the four slice sums are combined in a fixed order.
+// With R / Rout (optional) the residual stream is advanced in the same pass:
+// Rout[b, c] = fp16(Y[b, c] + R[b, c]), the rounded sum of the two fp16 values.
+// partial == nullptr: Y already holds the result, only the residual add is done.
 __global__ __launch_bounds__(256) void cols_reduce_kernel(const float* __restrict__ partial,
                                                           const half_t* __restrict__ bias, int G,
-                                                          int B, int N, half_t* __restrict__ Y) {
+                                                          int B, int N, half_t* __restrict__ Y,
+                                                          const half_t* __restrict__ R = nullptr,
+                                                          half_t* __restrict__ Rout = nullptr) {
   __shared__ float red[4][kWave];
   const int lane = threadIdx.x & 63;
   const int slice = threadIdx.x >> 6;
   const int64_t total = (int64_t)B * N;
   const int64_t o = (int64_t)blockIdx.x * kWave + lane;
+  if (partial == nullptr) {  // Y is complete already (single row group): only the residual add
+    if (slice == 0 && o < total && Rout != nullptr) Rout[o] = (half_t)((float)Y[o] + (float)R[o]);
+    return;
+  }
   float s = 0.f;
   if (o < total) {
     const float* p = partial + o;
@@ -287,7 +296,9 @@ __global__ __launch_bounds__(256) void cols_reduce_kernel(const float* __restric
   __syncthreads();
   if (slice == 0 && o < total) {
     const float r = (red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]);
-    Y[o] = (half_t)(r + (bias ? (float)bias[o % N] : 0.f));
+    const half_t y = (half_t)(r + (bias ? (float)bias[o % N] : 0.f));
+    Y[o] = y;
+    if (Rout != nullptr) Rout[o] = (half_t)((float)y + (float)R[o]);
   }
 }
 

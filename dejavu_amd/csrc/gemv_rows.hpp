@@ -91,13 +91,16 @@ __global__ __launch_bounds__(256) void canonical_gemv_kernel(
 // X is staged once per workgroup in LDS.  An index outside [0, Z) yields 0
 // instead of a wild read.  Requires n % 8 == 0 and ldw % 8 == 0.
 // ---------------------------------------------------------------------------
-template <int B, int R, int U, bool RELU>
+// STAGED: the caller has already put X into xs (and synchronised the workgroup).
+template <int B, int R, int U, bool RELU, bool STAGED = false>
 __device__ __forceinline__ void gather_rows_body(
     const half_t* __restrict__ X, const half_t* __restrict__ W, const half_t* __restrict__ bias,
     const void* __restrict__ idx, int idx_bytes, int n, int64_t ldw, int Z, int M,
     half_t* __restrict__ Y, half_t* xs, int block_id, int nblocks) {
-  for (int i = threadIdx.x * 8; i < B * n; i += blockDim.x * 8) store8(xs + i, load8(X + i));
-  __syncthreads();
+  if (!STAGED) {
+    for (int i = threadIdx.x * 8; i < B * n; i += blockDim.x * 8) store8(xs + i, load8(X + i));
+    __syncthreads();
+  }
 
   constexpr int CH = 8 * kWave;
   const int lane = threadIdx.x & 63;

@@ -1,4 +1,4 @@
-// One decode step of a whole sparse block in nine launches.  Kernels that are
+// One decode step of a whole sparse block in eight launches.  Kernels that are
 // independent of each other share a launch ("roles" picked by workgroup index),
 // so the small latency-bound pieces (LayerNorm, window step, predictors, top-k)
 // run beside the bandwidth-bound ones instead of each paying a launch of its own.
@@ -9,9 +9,10 @@
 //  L3  attention partials over the active heads        | head predictor fc1 | top-k threshold + counts
 //  L4  out_proj over W_out^T, merging the attention    | head top-k         | top-k emission
 //      partials on the fly
-//  L5  split reduction (+ bias)
-//  L6  add+LayerNorm 2
-//  L7  fc1 gather (+bias, ReLU)                         | MLP predictor fc0
+//  L5  split reduction (+ bias) + residual add
+//  L6  LayerNorm 2 of the residual stream, computed inside the fc1 workgroups while they
+//      stage their input row (same bits as the stand-alone kernel), then
+//      fc1 gather (+bias, ReLU)                         | MLP predictor fc0
 //  L8  fc2 gather                                       | MLP predictor fc1
 //  L9  split reduction (+ bias)
 #pragma once
@@ -157,7 +158,10 @@ __global__ __launch_bounds__(256) void layer_l4_kernel(OutProjArgs o, int nblk_o
 
 // ---- L7 / L8 --------------------------------------------------------------
 struct RowsArgs {
-  const half_t* X;
+  const half_t* X;  // residual stream after attention: normalised on the fly
+  const half_t* gamma;
+  const half_t* beta;
+  float eps;
   const half_t* W;
   const half_t* bias;
   const int64_t* idx;
@@ -167,12 +171,16 @@ struct RowsArgs {
   half_t* Y;
 };
 
+template <int MAXV>
 __global__ __launch_bounds__(256) void layer_l7_kernel(RowsArgs f, int nblk_fc1, CanonArgs mp0, int nblk_mp0) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   const int bid = blockIdx.x;
   if (bid < nblk_fc1) {
-    gather_rows_body<1, 2, 4, true>(f.X, f.W, f.bias, f.idx, 8, f.n, f.ldw, f.Z, f.M, f.Y,
-                                    reinterpret_cast<half_t*>(smem_raw), bid, nblk_fc1);
+    half_t* xs = reinterpret_cast<half_t*>(smem_raw);
+    add_layer_norm_body<256, MAXV>(f.X, nullptr, f.gamma, f.beta, f.eps, f.n, xs, nullptr, nullptr, 0);
+    __syncthreads();
+    gather_rows_body<1, 2, 4, true, true>(nullptr, f.W, f.bias, f.idx, 8, f.n, f.ldw, f.Z, f.M, f.Y, xs, bid,
+                                          nblk_fc1);
   } else {
     canonical_role(mp0, bid - nblk_fc1, nblk_mp0);
   }
