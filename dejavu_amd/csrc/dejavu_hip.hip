@@ -332,13 +332,23 @@ int launch_qkv(const half_t* x, const half_t* W, const half_t* bias, const int* 
 // Measured at the OPT-175B shape: 47 us for one token on the vector path (49 us on MFMA), and
 // 47..49 us for 2..16 tokens on MFMA against 52..95 us on the vector path.
 inline bool qkv_use_mfma(int nb) { return nb >= 2; }
+// Workgroups of 32 weight rows (half the x traffic, same bits) once there are enough of them
+// to fill the device: the flush step of a window (all heads).
+inline bool qkv_mfma_two_tiles(int nnz, int hd) {
+  return hd % 32 == 0 && nnz * 3 * (hd / 32) >= 3 * compute_units();
+}
 
 int launch_qkv_mfma(const half_t* x, const half_t* W, const half_t* bias, const int* head_idx,
                     const int* batch_idx, int nb, int d, int H, int hd, int nnz, half_t* y,
                     half_t* k_cache, half_t* v_cache, const int* padding, int S, hipStream_t s) {
-  const int ntasks = nnz * 3 * (hd / 16);
-  hipLaunchKernelGGL((qkv_window_mfma_kernel<kQkvMfmaWaves>), dim3(ntasks), dim3(kQkvMfmaWaves * 64), 0, s,
-                     x, W, bias, head_idx, batch_idx, nb, d, H, hd, nnz, y, k_cache, v_cache, padding, S);
+  if (qkv_mfma_two_tiles(nnz, hd))
+    hipLaunchKernelGGL((qkv_window_mfma_kernel<kQkvMfmaWaves, 2>), dim3(nnz * 3 * (hd / 32)),
+                       dim3(kQkvMfmaWaves * 64), 0, s, x, W, bias, head_idx, batch_idx, nb, d, H, hd, nnz, y,
+                       k_cache, v_cache, padding, S);
+  else
+    hipLaunchKernelGGL((qkv_window_mfma_kernel<kQkvMfmaWaves, 1>), dim3(nnz * 3 * (hd / 16)),
+                       dim3(kQkvMfmaWaves * 64), 0, s, x, W, bias, head_idx, batch_idx, nb, d, H, hd, nnz, y,
+                       k_cache, v_cache, padding, S);
   return launch_status();
 }
 
@@ -905,7 +915,8 @@ int dv_sparse_layer_decode_f16(const dvSparseLayerArgs* args, void* stream) {
     const int ntasks = a.Hk * 3 * (a.hd / 2);
     int nq = (ntasks + 3) / 4;
     if (nq > cus * 8) nq = cus * 8;
-    if (mfma) nq = a.Hk * 3 * (a.hd / 16);
+    const bool two = mfma && qkv_mfma_two_tiles(a.Hk, a.hd);
+    if (mfma) nq = a.Hk * 3 * (a.hd / (two ? 32 : 16));
     CanonArgs hp0{res1, CH(a.att_Wa), (int64_t)a.d, a.r_att, a.d, hp_hidden};
     const int rw0 = a.d <= 1024 ? 4 : 1;
     const int nh = ((a.r_att + rw0 - 1) / rw0 + 3) / 4;
@@ -913,7 +924,8 @@ int dv_sparse_layer_decode_f16(const dvSparseLayerArgs* args, void* stream) {
 #define DV_L2(NB)                                                                                 \
   hipLaunchKernelGGL((layer_l2_kernel<NB>), grid, dim3(256), 0, s, q, nq, hp0, nh, CH(a.mlp_logit_in), \
                      a.ffn, topk_ws)
-    if (mfma) DV_L2(0);
+    if (two) DV_L2(-1);
+    else if (mfma) DV_L2(0);
     else DV_L2(1);
 #undef DV_L2
   }

@@ -77,9 +77,10 @@ __global__ __launch_bounds__(256) void layer_l2_kernel(QkvArgs q, int nblk_qkv, 
                                                        unsigned* __restrict__ topk_ws) {
   const int bid = blockIdx.x;
   if (bid < nblk_qkv) {
-    if constexpr (NBMAX == 0)  // many live window tokens: matrix-core variant
-      qkv_window_mfma_body<kQkvMfmaWaves>(q.X, q.W, q.bias, q.head_idx, q.batch_idx, q.nb, q.d, q.H, q.hd,
-                                             q.nnz, q.Y, q.k_cache, q.v_cache, q.padding, q.S, bid, nblk_qkv);
+    if constexpr (NBMAX <= 0)  // several live window tokens: matrix-core variant (-1: 32-row workgroups)
+      qkv_window_mfma_body<kQkvMfmaWaves, NBMAX == 0 ? 1 : 2>(q.X, q.W, q.bias, q.head_idx, q.batch_idx, q.nb, q.d,
+                                                              q.H, q.hd, q.nnz, q.Y, q.k_cache, q.v_cache,
+                                                              q.padding, q.S, bid, nblk_qkv);
     else
       qkv_sparse_body<NBMAX, 2, 4>(q.X, q.W, q.bias, q.head_idx, q.batch_idx, q.nb, q.d, q.H, q.hd, q.nnz, q.Y,
                                    q.k_cache, q.v_cache, q.padding, q.S, bid, nblk_qkv);

@@ -17,6 +17,12 @@
 // loads stay in flight during the MFMAs.  The WAVES partial tiles are added
 // through LDS in wavefront order.  Requires d % 8 == 0 and hd % 16 == 0.  Same
 // outputs as qkv_sparse_body (the fp32 summation order differs).
+//
+// TILES = 2: a workgroup owns 32 consecutive weight rows (two MFMA row tiles,
+// hd % 32 == 0) and every x operand feeds two MFMAs, which halves the x traffic
+// from L2; that matters when all 16 slots are live (the flush step of a window,
+// where the x reads are as large as the weight reads).  Each accumulator sees
+// the same operands in the same order as with TILES = 1: identical bits.
 #pragma once
 #include "common.hpp"
 #include "gemm_mfma.hpp"
@@ -25,21 +31,23 @@ namespace dv {
 
 constexpr int kQkvMfmaWaves = 4;
 
-template <int WAVES>
+template <int WAVES, int TILES = 1>
 __device__ __forceinline__ void qkv_window_mfma_body(
     const half_t* __restrict__ X, const half_t* __restrict__ W, const half_t* __restrict__ bias,
     const int* __restrict__ head_idx, const int* __restrict__ batch_idx, int nb, int d, int H,
     int hd, int nnz, half_t* __restrict__ Y, half_t* __restrict__ k_cache,
     half_t* __restrict__ v_cache, const int* __restrict__ padding, int S, int block_id,
     int nblocks) {
-  __shared__ __attribute__((aligned(16))) half_t s_tiles[WAVES][kMfmaRows * kMfmaLdsRow];
-  static_assert(sizeof(half_t) * kMfmaRows * kMfmaLdsRow >= 256 * sizeof(float), "tile too small for the reduction");
+  constexpr int kTile = kMfmaRows * kMfmaLdsRow;  // halves per 16-row tile
+  __shared__ __attribute__((aligned(16))) half_t s_tiles[WAVES][TILES * kTile];
+  static_assert(sizeof(half_t) * TILES * kTile >= TILES * 256 * sizeof(float), "tile too small for the reduction");
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   half_t* tile = s_tiles[wave];
   const int l16 = lane & 15, kg = lane >> 4;       // MFMA operand coordinates
   const int l32 = lane & 31, half_id = lane >> 5;  // staging coordinates
-  const int groups_per_head = hd / 16;
+  constexpr int ROWS = 16 * TILES;
+  const int groups_per_head = hd / ROWS;
   const int ntasks = nnz * 3 * groups_per_head;
   const int nchunks = (d + kMfmaKC - 1) / kMfmaKC;
   constexpr int KS = kMfmaKC / 32;
@@ -48,7 +56,7 @@ __device__ __forceinline__ void qkv_window_mfma_body(
     const int i = task / (3 * groups_per_head);
     const int rem = task - i * 3 * groups_per_head;
     const int t = rem / groups_per_head;
-    const int j0 = (rem - t * groups_per_head) * 16;
+    const int j0 = (rem - t * groups_per_head) * ROWS;
     const int h = head_idx[i];
     if (h < 0 || h >= H) continue;  // uniform over the workgroup
     int slot = l16 < nb ? batch_idx[i * nb + l16] : -1;
@@ -59,20 +67,22 @@ __device__ __forceinline__ void qkv_window_mfma_body(
     const half_t* xrow = X + (slot >= 0 ? (int64_t)slot * d : 0);
     const bool live = slot >= 0;
 
-    float4_t acc = float4_t{0.f, 0.f, 0.f, 0.f};
-    half8_t stage[8];
+    float4_t acc[TILES];
+#pragma unroll
+    for (int r = 0; r < TILES; ++r) acc[r] = float4_t{0.f, 0.f, 0.f, 0.f};
+    half8_t stage[8 * TILES];
     auto load_stage = [&](int c) {
       int col = c * kMfmaKC + l32 * 8;
       if (col >= d) col = 0;  // masked when stored
 #pragma unroll
-      for (int q = 0; q < 8; ++q) stage[q] = load8_stream(W + (row0 + 2 * q + half_id) * d + col);
+      for (int q = 0; q < 8 * TILES; ++q) stage[q] = load8_stream(W + (row0 + 2 * q + half_id) * d + col);
     };
     auto store_stage = [&](int c) {
       const bool col_ok = c * kMfmaKC + l32 * 8 < d;
       __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");  // previous tile fully read
       __builtin_amdgcn_wave_barrier();
 #pragma unroll
-      for (int q = 0; q < 8; ++q)
+      for (int q = 0; q < 8 * TILES; ++q)  // row 2q + half_id of the 16 * TILES rows: tiles are contiguous
         store8(tile + (2 * q + half_id) * kMfmaLdsRow + l32 * 8, col_ok ? stage[q] : zero8());
       __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
       __builtin_amdgcn_wave_barrier();
@@ -89,8 +99,11 @@ __device__ __forceinline__ void qkv_window_mfma_body(
     auto multiply = [&]() {
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        const half8_t a = load8(tile + l16 * kMfmaLdsRow + ks * 32 + kg * 8);
-        acc = mfma_16x16x32(a, xb[ks], acc);
+#pragma unroll
+        for (int r = 0; r < TILES; ++r) {
+          const half8_t a = load8(tile + (r * 16 + l16) * kMfmaLdsRow + ks * 32 + kg * 8);
+          acc[r] = mfma_16x16x32(a, xb[ks], acc[r]);
+        }
       }
     };
 
@@ -110,9 +123,11 @@ __device__ __forceinline__ void qkv_window_mfma_body(
     __syncthreads();  // every wavefront is done with its tile: reuse it for the reduction
     float* red = reinterpret_cast<float*>(tile);
 #pragma unroll
-    for (int v = 0; v < 4; ++v) red[(4 * kg + v) * 16 + l16] = acc[v];
+    for (int r = 0; r < TILES; ++r)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) red[(r * 16 + 4 * kg + v) * 16 + l16] = acc[r][v];
     __syncthreads();
-    for (int o = threadIdx.x; o < 256; o += WAVES * kWave) {
+    for (int o = threadIdx.x; o < 256 * TILES; o += WAVES * kWave) {
       const int m = o >> 4, n = o & 15;
       int sl = n < nb ? batch_idx[i * nb + n] : -1;
       if (sl >= nb) sl = -1;
@@ -139,14 +154,14 @@ __device__ __forceinline__ void qkv_window_mfma_body(
   }
 }
 
-template <int WAVES>
+template <int WAVES, int TILES>
 __global__ __launch_bounds__(WAVES * 64) void qkv_window_mfma_kernel(
     const half_t* __restrict__ X, const half_t* __restrict__ W, const half_t* __restrict__ bias,
     const int* __restrict__ head_idx, const int* __restrict__ batch_idx, int nb, int d, int H,
     int hd, int nnz, half_t* __restrict__ Y, half_t* __restrict__ k_cache,
     half_t* __restrict__ v_cache, const int* __restrict__ padding, int S) {
-  qkv_window_mfma_body<WAVES>(X, W, bias, head_idx, batch_idx, nb, d, H, hd, nnz, Y, k_cache, v_cache,
-                              padding, S, blockIdx.x, gridDim.x);
+  qkv_window_mfma_body<WAVES, TILES>(X, W, bias, head_idx, batch_idx, nb, d, H, hd, nnz, Y, k_cache, v_cache,
+                                     padding, S, blockIdx.x, gridDim.x);
 }
 
 }  // namespace dv

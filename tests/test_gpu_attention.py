@@ -40,7 +40,9 @@ def randh(g, *shape, std=1.0):
                                            (8, 128, 1152, 5, 8), (8, 32, 512, 8, 3), (12, 128, 2048, 2, 12),
                                            # two or more rows run on the matrix cores
                                            (8, 64, 1024, 12, 3), (5, 64, 384, 9, 5), (4, 32, 128, 16, 2),
-                                           (6, 128, 640, 16, 3)])
+                                           (6, 128, 640, 16, 3),
+                                           # all 96 heads (the flush step of a window): 32-row workgroups
+                                           (96, 128, 1024, 16, 96), (100, 64, 384, 7, 100)])
 def test_qkv_proj_sparse(ops, H, hd, d, nb, nnz):
     """First case is the shape of the reference's own self-check
     (attention_proj_sparse.py:597-627): 12 heads, hidden 12288, 16 rows, 4 active heads,
