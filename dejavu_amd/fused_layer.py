@@ -3,7 +3,7 @@
 ``BlockMlpAttSparse.forward`` takes it when the step is an ordinary head-sparse decode step
 (batch 1, one token, fp16, predictions available), the window-flush step included; everything else
 goes through the modules' own forwards.  Same results either way: the fused entry point runs
-the same kernel bodies in nine launches instead of about twenty.
+the same kernel bodies in eight launches instead of about twenty.
 """
 from __future__ import annotations
 

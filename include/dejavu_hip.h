@@ -254,7 +254,7 @@ DV_API int dv_add_layer_norm_f16(const void* h, const void* residual, const void
                                  void* residual_out, void* stream);
 
 /*
- * One decode step (batch 1, one new token) of a whole sparse block in nine
+ * One decode step (batch 1, one new token) of a whole sparse block in eight
  * launches: add+LayerNorm 1, back-fill window step, QKV of the active heads with
  * cache scatter, attention, out_proj, add+LayerNorm 2, the sparse MLP, and beside
  * them the MLP top-k for this layer and both predictors (+ head top-k) for the

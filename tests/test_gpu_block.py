@@ -103,7 +103,7 @@ def test_sparse_block_decode_step_matches_oracle(d, ffn, H, r, K, Hk, S):
 
 @pytest.mark.parametrize("d,H,ffn,r", [(768, 12, 3072, 128), (1024, 8, 4096, 1000)])
 def test_fused_layer_equals_module_by_module_path(d, H, ffn, r):
-    """The nine-launch fused block step and the module-by-module path run the same kernel
+    """The eight-launch fused block step and the module-by-module path run the same kernel
     bodies: outputs, predictions, caches and window state must agree bit for bit over a
     whole back-fill window (the flush step falls back to the modules in both)."""
     import copy
