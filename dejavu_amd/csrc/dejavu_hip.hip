@@ -405,10 +405,19 @@ int dv_predictor_logits_f16(const void* x, const void* Wa, int64_t ldwa, const v
                         reinterpret_cast<half_t*>(logits), s);
 }
 
+}  // extern "C"
+namespace {
+// bytes of histograms, threshold and per-workgroup counts; the batch-maximum row follows
+size_t topk_max_row_offset(int n) {
+  const int blocks = (n + kTopkItemsPerBlock - 1) / kTopkItemsPerBlock;
+  return ((size_t)(kTopkCountsOff + 2 * blocks) * sizeof(unsigned) + 15) & ~(size_t)15;
+}
+}  // namespace
+extern "C" {
+
 size_t dv_topk_workspace_bytes(int n) {
   if (n <= 1024) return 0;
-  const int blocks = (n + kTopkItemsPerBlock - 1) / kTopkItemsPerBlock;
-  return (size_t)(kTopkCountsOff + 2 * blocks) * sizeof(unsigned);
+  return topk_max_row_offset(n) + (size_t)n * sizeof(half_t);
 }
 
 int dv_topk_f16(const void* logits, int B, int n, int k, void* idx_out, int idx_bytes,
@@ -429,6 +438,12 @@ int dv_topk_f16(const void* logits, int B, int n, int k, void* idx_out, int idx_
     return DV_ERR_WORKSPACE;
   unsigned* ws = reinterpret_cast<unsigned*>(workspace);
   const int blocks = (n + kTopkItemsPerBlock - 1) / kTopkItemsPerBlock;
+  if (B > 1 && B <= 64) {  // one wide pass reduces the batch to a row; the selection then reads that row
+    half_t* m = reinterpret_cast<half_t*>(reinterpret_cast<unsigned char*>(workspace) + topk_max_row_offset(n));
+    hipLaunchKernelGGL(topk_batch_max_kernel, dim3((n / 8 + 31) / 32), dim3(256), 0, s, lg, B, n, m);
+    lg = m;
+    B = 1;
+  }
   hipLaunchKernelGGL(topk_hist_kernel, dim3(blocks), dim3(256), 0, s, lg, B, n, ws);
   hipLaunchKernelGGL(topk_count_kernel, dim3(blocks), dim3(256), 0, s, lg, B, n, k, ws);
   hipLaunchKernelGGL(topk_emit_kernel, dim3(blocks), dim3(256), 0, s, lg, B, n, ws, idx_out, idx_bytes);

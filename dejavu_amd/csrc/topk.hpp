@@ -214,7 +214,8 @@ __global__ __launch_bounds__(256) void topk_small_kernel(const half_t* __restric
 //     it, emits its indices with key > T and those of the first `need` columns
 //     with key == T (ascending, exact positions), and clears its slice of the
 //     histograms for the next call.
-// Workspace layout (u32): fine[65536] coarse[256] meta[2] = {T, need} counts[2*WG].
+// Workspace layout (u32): fine[65536] coarse[256] meta[2] = {T, need} counts[2*WG], then (16-byte
+// aligned) n fp16 values: the column-wise maximum of a batch (topk_batch_max_kernel).
 // ---------------------------------------------------------------------------
 constexpr int kTopkItemsPerBlock = 256 * 8;
 constexpr int kTopkFine = 65536, kTopkCoarse = 256;
@@ -233,6 +234,53 @@ __device__ __forceinline__ void topk_load_keys(const half_t* __restrict__ logits
       const unsigned kk = topk_key(v[e]);
       key[e] = kk > key[e] ? kk : key[e];
     }
+  }
+}
+
+// Column-wise "maximum" of a (B, n) batch, as a row of fp16 values: m[j] = the logit of
+// column j with the largest key.  Top-k over m equals top-k over the batch with the
+// maximum-over-rows score, so a batch costs one wide pass (n / 256 workgroups, the rows of a
+// column spread over 8 threads, every thread's loads issued together) and the three
+// selection kernels then read one row instead of B.  Requires n % 8 == 0, B <= 64.
+__global__ __launch_bounds__(256) void topk_batch_max_kernel(const half_t* __restrict__ logits, int B,
+                                                             int n, half_t* __restrict__ m) {
+  __shared__ unsigned s_best[8][32][8];  // [row group][octet][element] = key << 16 | fp16 bits
+  const int oct_l = threadIdx.x & 31, rg = threadIdx.x >> 5;
+  const int i0 = (blockIdx.x * 32 + oct_l) * 8;
+  unsigned best[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) best[e] = 0u;
+  if (i0 < n) {
+    half8_t v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {  // rows rg, rg + 8, ...: past the batch the last own row repeats
+      int b = rg + 8 * u;
+      if (b >= B) b = rg < B ? rg : 0;
+      v[u] = load8(logits + (int64_t)b * n + i0);
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const half_t hv = v[u][e];  // a copy: bit-casting a vector element in place gave wrong lanes
+        const unsigned packed = (topk_key(hv) << 16) | (unsigned)__builtin_bit_cast(unsigned short, hv);
+        best[e] = packed > best[e] ? packed : best[e];
+      }
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) s_best[rg][oct_l][e] = best[e];
+  __syncthreads();
+  if (rg == 0 && i0 < n) {
+    half8_t o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      unsigned p = s_best[0][oct_l][e];
+#pragma unroll
+      for (int r = 1; r < 8; ++r) p = s_best[r][oct_l][e] > p ? s_best[r][oct_l][e] : p;
+      const unsigned short bits = (unsigned short)(p & 0xFFFFu);
+      o[e] = __builtin_bit_cast(half_t, bits);
+    }
+    store8(m + i0, o);
   }
 }
 
