@@ -217,7 +217,8 @@ int launch_rows_mfma(const half_t* x, const half_t* W, int64_t ldw, const half_t
   const int cap = compute_units() * 4;
   if (blocks > cap) blocks = cap;
   if (blocks < 1) blocks = 1;
-  hipLaunchKernelGGL(kern, dim3(blocks), dim3(kMfmaWaves * 64), lds, s, x, W, bias, idx, B, N, ldw, Z, M, y);
+  hipLaunchKernelGGL(kern, dim3(blocks), dim3(kMfmaWaves * 64), lds, s, x, W, bias, idx, B, N, ldw, Z, M, y, 0,
+                     static_cast<float*>(nullptr));
   return launch_status();
 }
 
@@ -233,6 +234,113 @@ int gather_rows_mfma(const half_t* x, const half_t* W, int64_t ldw, const half_t
   if (B <= 32) return DV_RM(2);
   return DV_RM(4);
 #undef DV_RM
+}
+
+// Few row tiles, long rows: split the chunks of a row over gridDim.y as well (see the kernel).
+// One chunk per wavefront at least; as many splits as it takes to have about two workgroups
+// per compute unit.
+struct RowsSplitPlan {
+  int nsplit, chunks_per_split;
+};
+
+RowsSplitPlan plan_rows_split(int N, int M) {
+  const int nchunks = (N + kMfmaKC - 1) / kMfmaKC;
+  const int ntiles = (M + kMfmaRows - 1) / kMfmaRows;
+  int want = ntiles > 0 ? 2 * compute_units() / ntiles : 1;
+  if (want < 1) want = 1;
+  int cps = (nchunks + want - 1) / want;
+  cps = (cps + kMfmaWaves - 1) / kMfmaWaves * kMfmaWaves;
+  RowsSplitPlan p;
+  p.chunks_per_split = cps;
+  p.nsplit = (nchunks + cps - 1) / cps;
+  return p;
+}
+
+size_t rows_split_workspace_bytes(int B, int N, int M) {
+  const RowsSplitPlan p = plan_rows_split(N, M);
+  // behind the completion counters other users of a shared workspace keep at its start
+  return p.nsplit > 1 ? kCounterBytes + (size_t)p.nsplit * B * M * sizeof(float) : 0;
+}
+
+// dense (no gather, bias or activation) product through the split kernel; falls back to the
+// unsplit kernel when one split is enough or no workspace was given
+int rows_mfma_dense(const half_t* x, const half_t* W, int64_t ldw, int B, int N, int M, half_t* y,
+                    void* workspace, size_t workspace_bytes, hipStream_t s) {
+  const RowsSplitPlan p = plan_rows_split(N, M);
+  if (p.nsplit <= 1 || workspace == nullptr || workspace_bytes < rows_split_workspace_bytes(B, N, M) ||
+      !aligned16(workspace))
+    return gather_rows_mfma(x, W, ldw, nullptr, nullptr, 4, B, N, M, M, DV_ACT_ID, y, s);
+  float* partial = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(workspace) + kCounterBytes);
+  const int ntiles = (M + kMfmaRows - 1) / kMfmaRows;
+  const dim3 grid(ntiles, p.nsplit);
+  const size_t tile_bytes = (size_t)kMfmaWaves * kMfmaRows * kMfmaLdsRow * sizeof(half_t);
+#define DV_RS(BT)                                                                                         \
+  do {                                                                                                    \
+    const size_t red_bytes = (size_t)kMfmaWaves * BT * 4 * 64 * sizeof(float);                            \
+    const size_t lds = tile_bytes > red_bytes ? tile_bytes : red_bytes;                                   \
+    static size_t granted = 48 * 1024;                                                                    \
+    if (lds > granted) {                                                                                  \
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(gather_rows_mfma_kernel<BT, false, false, true>), \
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)        \
+        return DV_ERR_UNSUPPORTED;                                                                        \
+      granted = lds;                                                                                      \
+    }                                                                                                     \
+    hipLaunchKernelGGL((gather_rows_mfma_kernel<BT, false, false, true>), grid, dim3(kMfmaWaves * 64), lds, s, x, \
+                       W, nullptr, nullptr, B, N, ldw, M, M, y, p.chunks_per_split, partial);             \
+  } while (0)
+  if (B <= 16) DV_RS(1);
+  else if (B <= 32) DV_RS(2);
+  else DV_RS(4);
+#undef DV_RS
+  const int64_t total = (int64_t)B * M;
+  hipLaunchKernelGGL(rows_split_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, partial,
+                     p.nsplit, total, y);
+  return launch_status();
+}
+
+// Dense short rows (N <= 1024, no gather, no bias): every wavefront owns whole 16-row tiles and
+// X sits in LDS.  The wavefront count per workgroup (one workgroup per compute unit) is the one
+// that spreads the tiles most evenly.  Returns DV_ERR_UNSUPPORTED when the shape does not fit
+// (the caller then takes the general kernel).
+template <int BT>
+int launch_rows_short(const half_t* x, const half_t* W, int64_t ldw, int B, int N, int M, half_t* y,
+                      hipStream_t s) {
+  const int ntiles = (M + kMfmaRows - 1) / kMfmaRows;
+  const int cus = compute_units();
+  int best_w = 0, best_cost = 0;
+  for (int w = 8; w >= 4; --w) {
+    const int cost = (ntiles + cus * w - 1) / (cus * w) * w;  // tiles the busiest compute unit walks
+    if (best_w == 0 || cost < best_cost) {
+      best_w = w;
+      best_cost = cost;
+    }
+  }
+  const int nchunks = (N + kMfmaKC - 1) / kMfmaKC;
+  const size_t lds = ((size_t)16 * BT * (nchunks * kMfmaKC + kMfmaRowPad) +
+                      (size_t)best_w * kMfmaRows * kMfmaLdsRow) * sizeof(half_t);
+  if (lds > 160 * 1024) return DV_ERR_UNSUPPORTED;
+  static size_t lds_granted = 48 * 1024;
+  if (lds > lds_granted) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(rows_short_mfma_kernel<BT>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return DV_ERR_UNSUPPORTED;
+    lds_granted = lds;
+  }
+  int grid = (ntiles + best_w - 1) / best_w;
+  if (grid > cus) grid = cus;
+  hipLaunchKernelGGL((rows_short_mfma_kernel<BT>), dim3(grid), dim3(best_w * 64), lds, s, x, W, ldw, B, N, M, y);
+  return launch_status();
+}
+
+// Shapes the short-row kernel is for: at most 32 batch rows (X in LDS), rows of at most 1024
+// elements, and enough 16-row tiles to give every compute unit several wavefronts.
+bool rows_short_fits(int B, int N, int M) {
+  return B <= 32 && N <= 1024 && (M + kMfmaRows - 1) / kMfmaRows >= 4 * compute_units();
+}
+
+int rows_short_mfma(const half_t* x, const half_t* W, int64_t ldw, int B, int N, int M, half_t* y,
+                    hipStream_t s) {
+  return B <= 16 ? launch_rows_short<1>(x, W, ldw, B, N, M, y, s) : launch_rows_short<2>(x, W, ldw, B, N, M, y, s);
 }
 
 struct ColsMfmaPlan {
@@ -377,9 +485,14 @@ const char* dv_error_string(int code) {
 
 int dv_canonical_lanes(int n) { return n <= 1024 ? 16 : 64; }
 
-int dv_predictor_logits_f16(const void* x, const void* Wa, int64_t ldwa, const void* Wb,
-                            int64_t ldwb, int B, int d, int r, int n_out, void* hidden,
-                            void* logits, void* stream) {
+size_t dv_predictor_workspace_bytes(int B, int d, int r) {
+  if (B <= 8 || B > 64 || d <= 0 || r <= 0) return 0;
+  return rows_split_workspace_bytes(B, d, r);
+}
+
+int dv_predictor_logits_ws_f16(const void* x, const void* Wa, int64_t ldwa, const void* Wb, int64_t ldwb,
+                               int B, int d, int r, int n_out, void* hidden, void* logits, void* workspace,
+                               size_t workspace_bytes, void* stream) {
   if (!x || !Wa || !Wb || !hidden || !logits || d <= 0 || r <= 0 || n_out <= 0)
     return DV_ERR_INVALID_ARG;
   if (B < 1 || B > 64) return DV_ERR_UNSUPPORTED;
@@ -389,10 +502,25 @@ int dv_predictor_logits_f16(const void* x, const void* Wa, int64_t ldwa, const v
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (B > 8) {
     // more rows than the fixed-order kernel keeps accumulators for: both products on the
-    // matrix cores (no gather, no bias), fp32 accumulation in the MFMA's own order
-    int rc = gather_rows_mfma(reinterpret_cast<const half_t*>(x), reinterpret_cast<const half_t*>(Wa), ldwa,
-                              nullptr, nullptr, 4, B, d, r, r, DV_ACT_ID, reinterpret_cast<half_t*>(hidden), s);
+    // matrix cores (no gather, no bias), fp32 accumulation in the MFMA's own order.  The
+    // first has few, long rows (split over the columns when a workspace is given), the
+    // second many short ones (whole tiles per wavefront, X in LDS, up to 32 batch rows).
+    int rc = rows_mfma_dense(reinterpret_cast<const half_t*>(x), reinterpret_cast<const half_t*>(Wa), ldwa, B, d, r,
+                             reinterpret_cast<half_t*>(hidden), workspace, workspace_bytes, s);
     if (rc != DV_OK) return rc;
+    // beyond 32 batch rows X no longer fits LDS next to the weight tiles: two passes of up to 32 rows
+    // (the weights stream twice, still faster than re-reading X from L2 for every 16-row tile)
+    const int pass_rows = B <= 32 ? B : 32;
+    if (rows_short_fits(pass_rows, r, n_out) && aligned16(logits) && ((int64_t)32 * n_out) % 8 == 0) {
+      rc = DV_OK;
+      for (int b0 = 0; b0 < B && rc == DV_OK; b0 += 32) {
+        const int nb = B - b0 < 32 ? B - b0 : 32;
+        rc = rows_short_mfma(reinterpret_cast<const half_t*>(hidden) + (int64_t)b0 * r,
+                             reinterpret_cast<const half_t*>(Wb), ldwb, nb, r, n_out,
+                             reinterpret_cast<half_t*>(logits) + (int64_t)b0 * n_out, s);
+      }
+      if (rc != DV_ERR_UNSUPPORTED) return rc;
+    }
     return gather_rows_mfma(reinterpret_cast<const half_t*>(hidden), reinterpret_cast<const half_t*>(Wb), ldwb,
                             nullptr, nullptr, 4, B, r, n_out, n_out, DV_ACT_ID,
                             reinterpret_cast<half_t*>(logits), s);
@@ -403,6 +531,12 @@ int dv_predictor_logits_f16(const void* x, const void* Wa, int64_t ldwa, const v
   return canonical_gemv(reinterpret_cast<const half_t*>(hidden),
                         reinterpret_cast<const half_t*>(Wb), ldwb, B, n_out, r,
                         reinterpret_cast<half_t*>(logits), s);
+}
+
+int dv_predictor_logits_f16(const void* x, const void* Wa, int64_t ldwa, const void* Wb,
+                            int64_t ldwb, int B, int d, int r, int n_out, void* hidden,
+                            void* logits, void* stream) {
+  return dv_predictor_logits_ws_f16(x, Wa, ldwa, Wb, ldwb, B, d, r, n_out, hidden, logits, nullptr, 0, stream);
 }
 
 }  // extern "C"

@@ -44,10 +44,16 @@ constexpr int kMfmaLdsRow = kMfmaKC + kMfmaRowPad;
 constexpr int kMfmaWaves = 8;
 constexpr int kMfmaRows = 16;
 
-template <int BT, bool IDX64, bool RELU>
+// SPLIT: few row tiles with long rows (the first product of a predictor: ~1000 rows of d
+// elements) would leave most compute units idle, so the chunks are also split over
+// gridDim.y: workgroup (t, y) takes chunks [y * chunks_per_split, (y + 1) * chunks_per_split)
+// and writes the raw fp32 sums to partial[(y * B + b) * M + m]; rows_split_reduce_kernel adds
+// the splits in ascending order.  No bias / activation in this mode.
+template <int BT, bool IDX64, bool RELU, bool SPLIT = false>
 __global__ __launch_bounds__(kMfmaWaves * 64) void gather_rows_mfma_kernel(
     const half_t* __restrict__ X, const half_t* __restrict__ W, const half_t* __restrict__ bias,
-    const void* __restrict__ idx, int B, int N, int64_t ldw, int Z, int M, half_t* __restrict__ Y) {
+    const void* __restrict__ idx, int B, int N, int64_t ldw, int Z, int M, half_t* __restrict__ Y,
+    int chunks_per_split = 0, float* __restrict__ partial = nullptr) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -56,6 +62,8 @@ __global__ __launch_bounds__(kMfmaWaves * 64) void gather_rows_mfma_kernel(
   const int l16 = lane & 15, kg = lane >> 4;  // MFMA operand coordinates
   const int l32 = lane & 31, half_id = lane >> 5;  // staging coordinates
   const int nchunks = (N + kMfmaKC - 1) / kMfmaKC;
+  const int c_begin = SPLIT ? (int)blockIdx.y * chunks_per_split : 0;
+  const int c_end = SPLIT ? (c_begin + chunks_per_split < nchunks ? c_begin + chunks_per_split : nchunks) : nchunks;
   constexpr int KS = kMfmaKC / 32;  // MFMA k-steps per chunk
   // batch tiles are multiplied in passes of at most two, to bound the X registers
   constexpr int BP = BT < 2 ? BT : 2;
@@ -126,10 +134,10 @@ __global__ __launch_bounds__(kMfmaWaves * 64) void gather_rows_mfma_kernel(
       }
     };
 
-    int c = wave;
-    if (c < nchunks) {
+    int c = c_begin + wave;
+    if (c < c_end) {
       load_stage(c);
-      for (; c + kMfmaWaves < nchunks; c += kMfmaWaves) {
+      for (; c + kMfmaWaves < c_end; c += kMfmaWaves) {
         store_stage(c);
         load_x(c, 0);
         load_stage(c + kMfmaWaves);
@@ -166,6 +174,11 @@ __global__ __launch_bounds__(kMfmaWaves * 64) void gather_rows_mfma_kernel(
           const int m = t * kMfmaRows + row;
           const int rid = __shfl(rid_mine, row, kWave);
           const bool ok = __shfl((int)ok_mine, row, kWave) != 0;
+          if (SPLIT) {
+            const int b = bt * 16 + l16;
+            if (m < M && b < B) partial[((int64_t)blockIdx.y * B + b) * M + m] = ok ? val : 0.f;
+            continue;
+          }
           val += (bias != nullptr && ok) ? (float)bias[rid] : 0.f;
           if (RELU) val = relu_f(val);
           if (!ok) val = 0.f;
@@ -174,6 +187,152 @@ __global__ __launch_bounds__(kMfmaWaves * 64) void gather_rows_mfma_kernel(
         }
     }
     __syncthreads();  // red is staging memory again
+  }
+}
+
+// Y[o] = fp16(sum_y partial[y * total + o]), splits added in ascending order.
+__global__ __launch_bounds__(256) void rows_split_reduce_kernel(const float* __restrict__ partial, int nsplit,
+                                                                int64_t total, half_t* __restrict__ Y) {
+  const int64_t o = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (o >= total) return;
+  float s = 0.f;
+  for (int y = 0; y < nsplit; ++y) s += partial[(int64_t)y * total + o];
+  Y[o] = (half_t)s;
+}
+
+// ---------------------------------------------------------------------------
+// Dense product with SHORT rows: Y[b, m] = sum_n X[b, n] * W[m, n], N <= 1024 (the second
+// product of a low-rank predictor: many rows of ~1000 elements).  Splitting such a row over
+// eight wavefronts leaves most of them idle and makes every 16-row tile re-read all of X, so
+// here every wavefront owns whole 16-row tiles (all N columns) and the workgroup stages X once
+// in LDS, zero-padded to 16 * BT rows of ceil(N / 256) * 256 columns, for all its wavefronts
+// and all the tiles they walk.  Weight tiles go through a wavefront-private LDS tile as in
+// gather_rows_mfma_kernel; two chunks of 256 columns are in flight per wavefront (registers
+// A / B), their loads unconditional and clamped so that the compiler can count them.  A lane
+// ends up with 4 consecutive m of one batch row per batch tile: one 8-byte store when M % 4 == 0.
+// blockDim.x = 64 * waves (the host picks the wavefront count that balances the tiles over the
+// compute units); dynamic LDS = 16 * BT * (NC * 256 + 8) halfs + waves * 16 * 264 halfs.
+// N % 8 == 0, ldw % 8 == 0, B <= 16 * BT.
+// ---------------------------------------------------------------------------
+template <int BT>
+__global__ __launch_bounds__(512) void rows_short_mfma_kernel(
+    const half_t* __restrict__ X, const half_t* __restrict__ W, int64_t ldw, int B, int N, int M,
+    half_t* __restrict__ Y) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int nwaves = blockDim.x >> 6;
+  const int nchunks = (N + kMfmaKC - 1) / kMfmaKC;
+  const int xs_row = nchunks * kMfmaKC + kMfmaRowPad;  // halfs per staged X row
+  half_t* xs = reinterpret_cast<half_t*>(smem_raw);
+  half_t* tile = xs + (size_t)16 * BT * xs_row + (size_t)wave * kMfmaRows * kMfmaLdsRow;
+  const int l16 = lane & 15, kg = lane >> 4;
+  const int l32 = lane & 31, half_id = lane >> 5;
+  constexpr int KS = kMfmaKC / 32;
+
+  // X, zero-padded, once per workgroup
+  const int vec_per_row = nchunks * kMfmaKC / 8;
+  for (int o = threadIdx.x; o < 16 * BT * vec_per_row; o += blockDim.x) {
+    const int b = o / vec_per_row, col = (o - b * vec_per_row) * 8;
+    store8(xs + (size_t)b * xs_row + col, (b < B && col < N) ? load8(X + (int64_t)b * N + col) : zero8());
+  }
+  __syncthreads();
+
+  const int ntiles = (M + kMfmaRows - 1) / kMfmaRows;
+  const int tstride = gridDim.x * nwaves;
+  const int t_first = blockIdx.x * nwaves + wave;
+  if (t_first >= ntiles) return;
+  const int my_tiles = (ntiles - t_first + tstride - 1) / tstride;
+  const int nsteps = my_tiles * nchunks;  // step s: tile t_first + (s / nchunks) * tstride, chunk s % nchunks
+
+  // weight tile of step s into 8 registers: rows 2q + half_id, 8 columns at l32 * 8 (rows past M
+  // and columns past N read a valid address and are zeroed when stored)
+  auto load_stage = [&](half8_t (&stage)[8], int sidx) {
+    const int t = t_first + (sidx / nchunks) * tstride, c = sidx % nchunks;
+    int col = c * kMfmaKC + l32 * 8;
+    if (col >= N) col = 0;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      int m = t * kMfmaRows + 2 * q + half_id;
+      if (m >= M) m = M - 1;
+      stage[q] = load8_stream(W + (int64_t)m * ldw + col);
+    }
+  };
+  auto store_stage = [&](const half8_t (&stage)[8], int sidx) {
+    const int t = t_first + (sidx / nchunks) * tstride, c = sidx % nchunks;
+    const bool col_ok = c * kMfmaKC + l32 * 8 < N;
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");  // previous tile fully read
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const bool ok = col_ok && t * kMfmaRows + 2 * q + half_id < M;
+      store8(tile + (2 * q + half_id) * kMfmaLdsRow + l32 * 8, ok ? stage[q] : zero8());
+    }
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  };
+  float4_t acc[BT];
+  auto multiply = [&](int sidx) {
+    const int c = sidx % nchunks;
+    if (c == 0) {
+#pragma unroll
+      for (int bt = 0; bt < BT; ++bt) acc[bt] = float4_t{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const half8_t a = load8(tile + l16 * kMfmaLdsRow + ks * 32 + kg * 8);
+#pragma unroll
+      for (int bt = 0; bt < BT; ++bt) {
+        const half8_t xv = load8(xs + (size_t)(bt * 16 + l16) * xs_row + c * kMfmaKC + ks * 32 + kg * 8);
+        acc[bt] = mfma_16x16x32(a, xv, acc[bt]);
+      }
+    }
+    if (c == nchunks - 1) {  // tile complete: value v of a lane is row 4 * kg + v, batch column l16
+      const int t = t_first + (sidx / nchunks) * tstride;
+      const int m0 = t * kMfmaRows + 4 * kg;
+#pragma unroll
+      for (int bt = 0; bt < BT; ++bt) {
+        const int b = bt * 16 + l16;
+        if (b < B) {
+          half_t* y = Y + (int64_t)b * M + m0;
+          if ((M & 3) == 0 && m0 < M) {
+            half4_t o;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) o[v] = (half_t)acc[bt][v];
+            *reinterpret_cast<half4_t*>(y) = o;
+          } else {
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+              if (m0 + v < M) y[v] = (half_t)acc[bt][v];
+          }
+        }
+      }
+    }
+  };
+
+  half8_t sa[8], sb[8];
+  load_stage(sa, 0);
+  if (nsteps > 1) load_stage(sb, 1);
+  int sidx = 0;
+  for (; sidx + 3 < nsteps; sidx += 2) {  // steps sidx, sidx + 1 with sidx + 2, sidx + 3 prefetched
+    store_stage(sa, sidx);
+    load_stage(sa, sidx + 2);
+    multiply(sidx);
+    store_stage(sb, sidx + 1);
+    load_stage(sb, sidx + 3);
+    multiply(sidx + 1);
+  }
+  // the last one to three steps: nothing, or one more tile, left to prefetch
+  store_stage(sa, sidx);
+  if (sidx + 2 < nsteps) load_stage(sa, sidx + 2);
+  multiply(sidx);
+  if (sidx + 1 < nsteps) {
+    store_stage(sb, sidx + 1);
+    multiply(sidx + 1);
+  }
+  if (sidx + 2 < nsteps) {
+    store_stage(sa, sidx + 2);
+    multiply(sidx + 2);
   }
 }
 

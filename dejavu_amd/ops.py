@@ -92,9 +92,12 @@ def predictor_logits(x: torch.Tensor, fc0_weight: torch.Tensor, fc1_weight: torc
     step = 8 if B <= 8 else 64
     for b0 in range(0, B, step):
         nb = min(step, B - b0)
-        check(lib.dv_predictor_logits_f16(_ptr(x[b0:]), _ptr(fc0_weight), fc0_weight.stride(0), _ptr(fc1_weight),
-                                          fc1_weight.stride(0), nb, d, r, n_out, _ptr(hidden[b0:]),
-                                          _ptr(logits[b0:]), _stream()), "dv_predictor_logits_f16")
+        nbytes = lib.dv_predictor_workspace_bytes(nb, d, r)
+        ws = _workspace(x.device, nbytes) if nbytes else None
+        check(lib.dv_predictor_logits_ws_f16(_ptr(x[b0:]), _ptr(fc0_weight), fc0_weight.stride(0), _ptr(fc1_weight),
+                                             fc1_weight.stride(0), nb, d, r, n_out, _ptr(hidden[b0:]),
+                                             _ptr(logits[b0:]), _ptr(ws), nbytes, _stream()),
+              "dv_predictor_logits_ws_f16")
     return logits
 
 

@@ -64,6 +64,20 @@ DV_API int dv_predictor_logits_f16(const void* x, const void* Wa, int64_t ldwa, 
                             void* logits, void* stream);
 
 /*
+ * The same with a workspace: for 9..64 rows the first product (r rows of d
+ * elements: few 16-row tiles) is also split over the columns, each split writing
+ * fp32 partial sums that a second launch adds in ascending order (deterministic).
+ * workspace: dv_predictor_workspace_bytes(B, d, r) bytes, 16-byte aligned; with
+ * NULL / 0 the call behaves like dv_predictor_logits_f16.  Up to 8 rows the
+ * workspace is not used.
+ */
+DV_API size_t dv_predictor_workspace_bytes(int B, int d, int r);
+DV_API int dv_predictor_logits_ws_f16(const void* x, const void* Wa, int64_t ldwa, const void* Wb,
+                                      int64_t ldwb, int B, int d, int r, int n_out, void* hidden,
+                                      void* logits, void* workspace, size_t workspace_bytes,
+                                      void* stream);
+
+/*
  * Index set of the k largest logits, ties to the lower index, written in
  * ascending index order.  For B > 1 a column's score is its maximum over the
  * B rows.  Replaces Tensor.topk(k, sorted=False) at

@@ -68,7 +68,8 @@ def test_predictor_topk_indices_bit_exact(ops, cfg, batch, k):
     assert np.array_equal(np16(idx), want)
 
 
-@pytest.mark.parametrize("cfg,batch", [("opt-125m", 9), ("opt-6.7b", 16), ("opt-6.7b", 37), ("opt-125m", 64)])
+@pytest.mark.parametrize("cfg,batch", [("opt-125m", 9), ("opt-6.7b", 16), ("opt-6.7b", 37), ("opt-125m", 64),
+                                       ("opt-6.7b", 9), ("opt-6.7b", 32)])
 def test_predictor_more_than_eight_rows_runs_on_the_matrix_cores(ops, cfg, batch):
     """9..64 rows: the logits come from MFMA products (the matrix core's own fp32 order), so they
     are compared within tolerance; the union top-k is still the exact top-k of those logits."""
@@ -85,6 +86,27 @@ def test_predictor_more_than_eight_rows_runs_on_the_matrix_cores(ops, cfg, batch
     want_logits = (np16(hidden).astype(np.float32) @ np16(t["mlp_Wb"]).astype(np.float32).T)
     assert_close(np16(got), want_logits, "predictor logits")
     assert np.array_equal(np16(idx), O.topk_lower_index(np16(got), k)), "union top-k of the device logits"
+
+
+@pytest.mark.parametrize("B,r,n_out", [(17, 520, 16390), (32, 1000, 20480), (12, 8, 16384), (32, 1024, 16386),
+                                       (9, 264, 49152), (40, 1000, 20480), (64, 512, 16384)])
+def test_predictor_second_product_with_short_rows(ops, B, r, n_out):
+    """Many short rows (second product of the predictor at 9..32 batch rows): whole 16-row tiles
+    per wavefront with X in LDS.  Ragged cases: a partial last 256-column chunk, a partial last
+    tile, an output width that is not a multiple of 4 (element-wise stores)."""
+    g = torch.Generator().manual_seed(B * 1000 + r)
+    d = 128
+    x = torch.randn(B, d, generator=g).half()
+    Wa = (torch.randn(r, d, generator=g) * 0.1).half()
+    Wb = (torch.randn(n_out, r, generator=g) * 0.1).half()
+    print(f"case predictor short rows B={B} r={r} n_out={n_out}", flush=True)
+    hidden = torch.empty(B, r, dtype=torch.float16, device="cuda")
+    got = ops.predictor_logits(x.cuda(), Wa.cuda(), Wb.cuda(), hidden=hidden)
+    torch.cuda.synchronize()
+    assert got.shape == (B, n_out)
+    assert_close(np16(hidden), x.float().numpy() @ Wa.float().numpy().T, "hidden")
+    want = np16(hidden).astype(np.float32) @ Wb.float().numpy().T
+    assert_close(np16(got), want, "logits from the device's hidden vector")
 
 
 # ---------------------------------------------------------------------- top-k
