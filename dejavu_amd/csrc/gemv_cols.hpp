@@ -157,15 +157,26 @@ __device__ __forceinline__ void gather_cols_body(
       consume(wn, j);
       j += U;
     }
-    for (; j < cnt; ++j) {
-      const int r = __builtin_amdgcn_readlane(rid, j);
-      const half8_t w = load8_stream(wcol + (int64_t)r * ldw);
+    if (j < cnt) {
+      // fewer than U rows left: their loads are issued together like those of a full batch
+      // (slots past the last row repeat it and take no part in the sums)
+      half8_t w[U];
 #pragma unroll
-      for (int b = 0; b < B; ++b) {
-        const float xs =
-            __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, xl[b]), j));
+      for (int u = 0; u < U; ++u) {
+        const int jj = j + u < cnt ? j + u : cnt - 1;
+        w[u] = load8_stream(wcol + (int64_t)__builtin_amdgcn_readlane(rid, jj) * ldw);
+      }
 #pragma unroll
-        for (int e = 0; e < 8; ++e) acc[b][e] = __builtin_fmaf((float)w[e], xs, acc[b][e]);
+      for (int u = 0; u < U; ++u) {
+        if (j + u < cnt) {
+#pragma unroll
+          for (int b = 0; b < B; ++b) {
+            const float xs = __builtin_bit_cast(
+                float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, xl[b]), j + u));
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[b][e] = __builtin_fmaf((float)w[u][e], xs, acc[b][e]);
+          }
+        }
       }
     }
   }
