@@ -180,6 +180,16 @@ def kernel_table(torch, cfg, batch, layers):
         table[name] = {"us": round(us, 2), "MB": round(nbytes[name] / 1e6, 2),
                        "GB/s": round(nbytes[name] / us / 1e3, 1),
                        "frac": round(nbytes[name] / us / 1e3 / HBM_PEAK_GBPS, 4)}
+    # latency-bound pieces (a few hundred KB at most): duration only
+    res = layers[0]["residual"].view(batch, d)
+    small = {
+        "mlp_topk": lambda L: ops.topk_indices(L["mlp_logit_in"], K),
+        "add_layer_norm": lambda L: ops.add_layer_norm(x, res, L["block"].norm1.weight, L["block"].norm1.bias,
+                                                       L["block"].norm1.eps),
+    }
+    for name, fn in small.items():
+        table[name] = {"us": round(time_kernel(torch, fn, layers), 2),
+                       "note": "eager call of the stand-alone operator: bounded by the host launch rate"}
     return table
 
 
@@ -443,6 +453,7 @@ def main():
         dv_modules.join_side_stream()
         torch.cuda.synchronize()
         whole = args.steps % period == 0 and args.warmup % period == 0 and not args.graph_per_step
+        spread = None
         if args.no_graph:
             us_per_layer = timed(step_fn, args.steps, args.warmup)
             graph_mode = "none"
@@ -451,6 +462,17 @@ def main():
             torch.cuda.synchronize()
             us_per_layer = timed(lambda i: g.replay() if i % period == 0 else None, args.steps, args.warmup)
             graph_mode = f"one graph of {period} steps"
+            # spread over single replays (outside the timed region): one event pair per replay
+            evs = [torch.cuda.Event(enable_timing=True) for _ in range(21)]
+            evs[0].record()
+            for e in evs[1:]:
+                g.replay()
+                e.record()
+            torch.cuda.synchronize()
+            per = sorted(a.elapsed_time(b) * 1e3 / period for a, b in zip(evs[:-1], evs[1:]))
+            spread = {"unit": f"us/layer over one replay of {period} steps", "replays": len(per),
+                      "median": round(per[len(per) // 2], 2), "p10": round(per[len(per) // 10], 2),
+                      "p90": round(per[(len(per) * 9) // 10], 2)}
         else:
             graphs = [capture(i, 1) for i in range(period)]
             torch.cuda.synchronize()
@@ -522,6 +544,7 @@ def main():
         "layer": {"algorithmic_MB": round(layer_bytes / 1e6, 1), "GB/s": round(layer_bytes / us_per_layer / 1e3, 1),
                   "frac_of_hbm_peak": round(layer_bytes / us_per_layer / 1e3 / HBM_PEAK_GBPS, 4),
                   "tokens_per_s_per_layer": round(batch / (us_per_layer * 1e-6), 1)},
+        "spread": spread,
         "kernels": table,
     }
     print(json.dumps(out))
