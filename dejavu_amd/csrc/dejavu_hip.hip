@@ -130,9 +130,8 @@ ColsPlan plan_cols(int N, int M) {
   return p;
 }
 
-// Workspace layout: completion counters first, at a fixed place, so that they
-// stay zero between launches of different shapes that share one workspace (the
-// kernels reset them; the partial sums behind them hold stale values).
+// Workspace layout: 4 KiB that no kernel writes (they stay zero; reserved for per-tile
+// counters at a place that does not depend on the shape), then the fp32 partial sums.
 constexpr size_t kCounterBytes = 4096;
 constexpr int kMaxColTiles = (int)(kCounterBytes / sizeof(unsigned));
 
@@ -146,14 +145,9 @@ void launch_cols(const ColsPlan& p, const half_t* x, int64_t ldx, int x_expanded
                  int64_t ldw, const half_t* bias, const void* idx, int blk, int N, int Z, int M,
                  float* partial, unsigned* counters, half_t* y, hipStream_t s) {
   dim3 grid(p.col_tiles, p.groups);
-  if (p.groups == 1) {
-    hipLaunchKernelGGL((gather_cols_kernel<B, 8, IDX64, BLOCKED, true>), grid, dim3(256), 0, s, x,
-                       ldx, x_expanded, W, ldw, bias, idx, blk, N, Z, M, p.rows_per_block, partial,
-                       counters, y);
-  } else {
-    hipLaunchKernelGGL((gather_cols_kernel<B, 8, IDX64, BLOCKED, false>), grid, dim3(256), 0, s, x,
-                       ldx, x_expanded, W, ldw, bias, idx, blk, N, Z, M, p.rows_per_block, partial,
-                       counters, y);
+  hipLaunchKernelGGL((gather_cols_kernel<B, 8, IDX64, BLOCKED>), grid, dim3(256), 0, s, x, ldx, x_expanded, W, ldw,
+                     bias, idx, blk, N, Z, M, p.rows_per_block, partial, counters, y);
+  if (p.groups > 1) {
     const int64_t total = (int64_t)B * N;
     hipLaunchKernelGGL(cols_reduce_kernel, dim3((unsigned)((total + 63) / 64)), dim3(256), 0, s,
                        partial, bias, p.groups, B, N, y);
@@ -861,7 +855,7 @@ int dv_attention_out_proj_f16(const void* q, int64_t ldq, const void* k_cache, c
   dim3 grid(p.col_tiles, p.groups);
   const int nsplit = attn_splits(n_len);
 #define DV_AO(BB)                                                                                 \
-  hipLaunchKernelGGL((gather_cols_kernel<BB, 8, false, true, false, true>), grid, dim3(256), 0, s, \
+  hipLaunchKernelGGL((gather_cols_kernel<BB, 8, false, true, true>), grid, dim3(256), 0, s, \
                      (const half_t*)nullptr, (int64_t)0, 1, ww, ldw, bb, head_idx, hd, N, H * hd, M, \
                      p.rows_per_block, partial, counters, yy, part, nsplit)
   switch (B) {

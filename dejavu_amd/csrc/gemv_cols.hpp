@@ -2,24 +2,16 @@
 // Lanes own 8 adjacent output columns each and stream the gathered rows with
 // 128-bit loads; no cross-lane reduction is needed.  The M rows are split over
 // gridDim.y row groups; each group writes an fp32 partial, and the partials are
-// summed in a fixed order (deterministic, no floating-point atomics) either by
-// the last group to finish a column tile (FUSED) or by cols_reduce_kernel.
+// summed in a fixed order (deterministic, no floating-point atomics) by
+// cols_reduce_kernel.  (Reducing inside this kernel -- the last group to finish a
+// column tile adds the partials -- measured slower than the second launch: 23.0 us
+// against 20.2 us for fc2 at the OPT-175B shape.)
 #pragma once
 #include "common.hpp"
 
 namespace dv {
 
 constexpr int kColTile = 8 * kWave;  // 512 columns per workgroup
-
-// Partials cross workgroups (and XCDs, whose L2s are not coherent with each
-// other): they are written and read with agent-scope accesses that go to the
-// device-wide coherence point, so no L2-wide write-back / invalidate is needed.
-__device__ __forceinline__ void store_agent(float* p, float v) {
-  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ float load_agent(const float* p) {
-  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
 
 // Row mapping: BLOCKED == false: row(m) = idx[m] (sparse-MLP fc2 over W2^T).
 // BLOCKED == true: row(m) = idx[m / blk] * blk + m % blk (out_proj over
@@ -29,7 +21,7 @@ __device__ __forceinline__ float load_agent(const float* p) {
 // fly from the un-normalised attention partials { max, sum, o[blk] } of
 // decode_attn_kernel (attn_nsplit splits per head), rounded to fp16 as a
 // stored context vector would be.
-template <int B, int U, bool IDX64, bool BLOCKED, bool FUSED, bool ATTN>
+template <int B, int U, bool IDX64, bool BLOCKED, bool ATTN>
 __device__ __forceinline__ void gather_cols_body(
     const half_t* __restrict__ X, int64_t ldx, int x_expanded, const half_t* __restrict__ W,
     int64_t ldw, const half_t* __restrict__ bias, const void* __restrict__ idx, int blk, int N,
@@ -37,7 +29,6 @@ __device__ __forceinline__ void gather_cols_body(
     half_t* __restrict__ Y, const float* __restrict__ attn_part, int attn_nsplit, int ct, int g,
     int G) {
   __shared__ float red[4][B][kColTile];
-  __shared__ int s_last;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -207,65 +198,21 @@ __device__ __forceinline__ void gather_cols_body(
     return;
   }
 
-  if (!FUSED) {
-#pragma unroll
-    for (int j = 0; j < PER_THREAD; ++j) {
-      const int o = j * 256 + tid;
-      const int b = o / kColTile, c = ct * kColTile + o % kColTile;
-      if (c < N) partial[((int64_t)g * B + b) * N + c] = sum[j];
-    }
-    return;
-  }
-
 #pragma unroll
   for (int j = 0; j < PER_THREAD; ++j) {
     const int o = j * 256 + tid;
     const int b = o / kColTile, c = ct * kColTile + o % kColTile;
-    if (c < N) store_agent(&partial[((int64_t)g * B + b) * N + c], sum[j]);
+    if (c < N) partial[((int64_t)g * B + b) * N + c] = sum[j];
   }
-  // every wavefront waits for its own partial stores to be acknowledged, then
-  // the workgroup meets, then one thread signals completion
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-  __builtin_amdgcn_s_waitcnt(0);
-  __syncthreads();
-  if (tid == 0) {
-    const unsigned old =
-        __hip_atomic_fetch_add(&counters[ct], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    s_last = (old == (unsigned)(G - 1));
-  }
-  __syncthreads();
-  if (!s_last) return;
-#pragma unroll
-  for (int j = 0; j < PER_THREAD; ++j) {
-    const int o = j * 256 + tid;
-    const int b = o / kColTile, c = ct * kColTile + o % kColTile;
-    if (c < N) {
-      const float* p = partial + (int64_t)b * N + c;
-      const int64_t gstride = (int64_t)B * N;
-      float s = 0.f;
-      int gg = 0;
-      for (; gg + 8 <= G; gg += 8) {
-        float v[8];
-#pragma unroll
-        for (int q = 0; q < 8; ++q) v[q] = load_agent(p + (gg + q) * gstride);
-#pragma unroll
-        for (int q = 0; q < 8; ++q) s += v[q];
-      }
-      for (; gg < G; ++gg) s += load_agent(p + gg * gstride);
-      Y[(int64_t)b * N + c] = (half_t)(s + (bias ? (float)bias[c] : 0.f));
-    }
-  }
-  if (tid == 0)
-    __hip_atomic_store(&counters[ct], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <int B, int U, bool IDX64, bool BLOCKED, bool FUSED, bool ATTN = false>
+template <int B, int U, bool IDX64, bool BLOCKED, bool ATTN = false>
 __global__ __launch_bounds__(256) void gather_cols_kernel(
     const half_t* __restrict__ X, int64_t ldx, int x_expanded, const half_t* __restrict__ W,
     int64_t ldw, const half_t* __restrict__ bias, const void* __restrict__ idx, int blk, int N,
     int Z, int M, int rows_per_block, float* __restrict__ partial, unsigned* __restrict__ counters,
     half_t* __restrict__ Y, const float* __restrict__ attn_part = nullptr, int attn_nsplit = 0) {
-  gather_cols_body<B, U, IDX64, BLOCKED, FUSED, ATTN>(X, ldx, x_expanded, W, ldw, bias, idx, blk, N, Z, M,
+  gather_cols_body<B, U, IDX64, BLOCKED, ATTN>(X, ldx, x_expanded, W, ldw, bias, idx, blk, N, Z, M,
                                                      rows_per_block, partial, counters, Y, attn_part,
                                                      attn_nsplit, blockIdx.x, blockIdx.y, gridDim.y);
 }

@@ -142,7 +142,7 @@ __global__ __launch_bounds__(256) void layer_l4_kernel(OutProjArgs o, int nblk_o
   const int bid = blockIdx.x;
   if (bid < nblk_out) {
     const int ct = bid % o.col_tiles, g = bid / o.col_tiles;
-    gather_cols_body<1, 8, false, true, false, true>(nullptr, 0, 1, o.W, o.ldw, o.bias, o.head_idx, o.hd, o.N,
+    gather_cols_body<1, 8, false, true, true>(nullptr, 0, 1, o.W, o.ldw, o.bias, o.head_idx, o.hd, o.N,
                                                      o.Z, o.M, o.rows_per_block, o.partial, nullptr, o.Y,
                                                      o.attn_part, o.nsplit, ct, g, o.groups);
   } else if (bid == nblk_out) {
@@ -202,7 +202,7 @@ __global__ __launch_bounds__(256) void layer_l8_kernel(ColsArgs c, int nblk_fc2,
   const int bid = blockIdx.x;
   if (bid < nblk_fc2) {
     const int ct = bid % c.col_tiles, g = bid / c.col_tiles;
-    gather_cols_body<1, 8, true, false, false, false>(c.X, c.M, 0, c.W, c.ldw, c.bias, c.idx, 1, c.N, c.Z, c.M,
+    gather_cols_body<1, 8, true, false, false>(c.X, c.M, 0, c.W, c.ldw, c.bias, c.idx, 1, c.N, c.Z, c.M,
                                                       c.rows_per_block, c.partial, nullptr, c.Y, nullptr, 0, ct,
                                                       g, c.groups);
   } else {

@@ -43,15 +43,14 @@ def _require_device(*tensors: Optional[torch.Tensor]) -> None:
 
 
 # ---------------------------------------------------------------------------
-# workspace (fp32 partial sums + completion counters of the split reductions)
+# workspace (fp32 partial sums of the split reductions behind 4 KiB kept at zero)
 # ---------------------------------------------------------------------------
 _workspaces: dict = {}
 
 
 def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
-    """Zero-initialised per-device scratch, grown on demand.  The kernels leave
-    their counters at zero, so it is only cleared when (re)allocated.  Ops that
-    share it must not run concurrently on different streams."""
+    """Zero-initialised per-device scratch, grown on demand; only cleared when
+    (re)allocated.  Ops that share it must not run concurrently on different streams."""
     key = (device.type, device.index)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
