@@ -85,6 +85,87 @@ __global__ __launch_bounds__(256) void canonical_gemv_kernel(
   canonical_gemv_body<LANES, B, U>(X, W, ldw, rows, n, Y, blockIdx.x, gridDim.x);
 }
 
+// Several batch rows (B >= 2) over short rows (B * n floats fit LDS): with one weight row per
+// lane group every 16 bytes of weights need B * 16 bytes of x from L1, which bounds the kernel
+// before memory does.  Here X is converted once per workgroup to fp32 in LDS and a lane group
+// owns R weight rows at a time that share each x read: row r of task t is
+// (t * R + r) * (64 / LANES) + group.  Same products in the same order per output as
+// canonical_gemv_body, so the same bits.  Dynamic LDS: B * n * 4 bytes.
+template <int LANES, int B, int U, int R>
+__global__ __launch_bounds__(256) void canonical_gemv_xlds_kernel(
+    const half_t* __restrict__ X, const half_t* __restrict__ W, int64_t ldw, int rows, int n,
+    half_t* __restrict__ Y) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  float* xf = reinterpret_cast<float*>(smem_raw);
+  for (int i = threadIdx.x * 8; i < B * n; i += blockDim.x * 8) {
+    const half8_t v = load8(X + i);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) xf[i + e] = (float)v[e];
+  }
+  __syncthreads();
+
+  constexpr int RW = kWave / LANES;
+  constexpr int CH = 8 * LANES;
+  const int lane = threadIdx.x & 63;
+  const int sub = lane % LANES;
+  const int grp = lane / LANES;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int ntasks = (rows + RW * R - 1) / (RW * R);
+  for (int t = blockIdx.x * 4 + wave; t < ntasks; t += gridDim.x * 4) {
+    const half_t* wr[R];
+    bool valid[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int row = (t * R + r) * RW + grp;
+      valid[r] = row < rows;
+      wr[r] = W + (int64_t)(valid[r] ? row : 0) * ldw + sub * 8;
+    }
+    float acc[R][B];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int b = 0; b < B; ++b) acc[r][b] = 0.f;
+    // groups of U chunks; the last group may be short and its last chunk partial: all loads are
+    // issued together, lanes past the row end take no part
+    for (int base = 0; base < n; base += U * CH) {
+      half8_t w[U][R];
+      bool in[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        in[u] = base + u * CH + sub * 8 < n;
+#pragma unroll
+        for (int r = 0; r < R; ++r) w[u][r] = in[u] ? load8_stream(wr[r] + base + u * CH) : zero8();
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (in[u]) {
+#pragma unroll
+          for (int b = 0; b < B; ++b) {
+            const float* xp = xf + b * n + base + u * CH + sub * 8;
+            const float4_t lo = *reinterpret_cast<const float4_t*>(xp);
+            const float4_t hi = *reinterpret_cast<const float4_t*>(xp + 4);
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) acc[r][b] = __builtin_fmaf((float)w[u][r][e], lo[e], acc[r][b]);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) acc[r][b] = __builtin_fmaf((float)w[u][r][4 + e], hi[e], acc[r][b]);
+            }
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int b = 0; b < B; ++b) {
+        const float v = butterfly_sum<LANES>(acc[r][b]);
+        const int row = (t * R + r) * RW + grp;
+        if (valid[r] && sub == 0) Y[(int64_t)b * rows + row] = (half_t)v;
+      }
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Y[b, m] = act( sum_i W[idx[m], i] * X[b, i] + bias[idx[m]] ), fp16 out.
 // One wavefront owns R gathered rows at a time (R independent load streams);
