@@ -48,12 +48,12 @@ int launch_canonical(const half_t* X, const half_t* W, int64_t ldw, int B, int r
   const int cap = compute_units() * 16;
   if (blocks > cap) blocks = cap;
   if (blocks < 1) blocks = 1;
-  // several batch rows over short rows (n <= 1024: X fits LDS as fp32): X in LDS; from five batch
-  // rows on, four weight rows per lane group share every x read (measured: batch 4 98 us per MLP
-  // block with one row per group against 102 us with four, batch 8 122 us against 121 us)
+  // short rows (n <= 1024: X fits LDS as fp32): X in LDS, R weight rows per lane group.  Measured at
+  // the OPT-175B predictor (49152 rows of 1000): batch 1, R = 2: 18 us against 22 us with one row per
+  // group; batch 4: 98 us per MLP block with R = 1 against 102 us with R = 4; batch 8: 122 against 121.
   const size_t xlds = (size_t)B * n * sizeof(float);
-  const bool use_xlds = LANES == 16 && B >= 2 && xlds <= 48 * 1024;
-  const int xr = B >= 5 ? 4 : 1;
+  const bool use_xlds = LANES == 16 && xlds <= 48 * 1024;
+  const int xr = B >= 5 ? 4 : (B == 1 ? 2 : 1);
   if (use_xlds) {
     blocks = ((rows + RW * xr - 1) / (RW * xr) + 3) / 4;
     if (blocks > cap) blocks = cap;
@@ -62,7 +62,7 @@ int launch_canonical(const half_t* X, const half_t* W, int64_t ldw, int B, int r
 #define DV_CASE(BB)                                                                                \
   case BB:                                                                                         \
     if (use_xlds)                                                                                  \
-      hipLaunchKernelGGL((canonical_gemv_xlds_kernel<LANES, BB, (BB >= 5 ? 4 : 8), (BB >= 5 ? 4 : 1)>), dim3(blocks), \
+      hipLaunchKernelGGL((canonical_gemv_xlds_kernel<LANES, BB, (BB >= 5 ? 4 : 8), (BB >= 5 ? 4 : (BB == 1 ? 2 : 1))>), dim3(blocks), \
                          dim3(256), xlds, s, X, W, ldw, rows, n, Y);                               \
     else                                                                                           \
       hipLaunchKernelGGL((canonical_gemv_kernel<LANES, BB, U>), dim3(blocks), dim3(256), 0, s, X, W, ldw, rows, n, \
@@ -1076,7 +1076,7 @@ int dv_sparse_layer_decode_f16(const dvSparseLayerArgs* args, void* stream) {
     const bool two = mfma && qkv_mfma_two_tiles(a.Hk, a.hd);
     if (mfma) nq = a.Hk * 3 * (a.hd / (two ? 32 : 16));
     CanonArgs hp0{res1, CH(a.att_Wa), (int64_t)a.d, a.r_att, a.d, hp_hidden};
-    const int rw0 = a.d <= 1024 ? 4 : 1;
+    const int rw0 = a.d <= 1024 ? 4 * kCanonShortRows : 1;
     const int nh = ((a.r_att + rw0 - 1) / rw0 + 3) / 4;
     const dim3 grid(nq + nh + topk_blocks);
 #define DV_L2(NB)                                                                                 \
@@ -1096,7 +1096,7 @@ int dv_sparse_layer_decode_f16(const dvSparseLayerArgs* args, void* stream) {
                 a.softmax_scale, attn_part};
     CanonArgs hp1{hp_hidden, CH(a.att_Wb), (int64_t)a.r_att, a.H, a.r_att, head_logits};
     const int na = nsplit * a.Hk;
-    const int rw1 = a.r_att <= 1024 ? 4 : 1;
+    const int rw1 = a.r_att <= 1024 ? 4 * kCanonShortRows : 1;
     const int nh1 = ((a.H + rw1 - 1) / rw1 + 3) / 4;
     const dim3 grid(na + nh1 + topk_blocks);
     if (a.hd == 128)
@@ -1129,7 +1129,7 @@ int dv_sparse_layer_decode_f16(const dvSparseLayerArgs* args, void* stream) {
     int nf = ((a.K + 1) / 2 + 3) / 4;
     if (nf > cus * 8) nf = cus * 8;
     CanonArgs mp0{res2, CH(a.mlp_Wa), (int64_t)a.d, a.r_mlp, a.d, mp_hidden};
-    const int rw0 = a.d <= 1024 ? 4 : 1;
+    const int rw0 = a.d <= 1024 ? 4 * kCanonShortRows : 1;
     const int nm = ((a.r_mlp + rw0 - 1) / rw0 + 3) / 4;
     const size_t lds = (size_t)a.d * sizeof(half_t);
     const int v = a.d <= 8192 ? 0 : (a.d <= 16384 ? 1 : 2);
@@ -1153,7 +1153,7 @@ int dv_sparse_layer_decode_f16(const dvSparseLayerArgs* args, void* stream) {
                 cols_part, reinterpret_cast<half_t*>(a.hidden_out), CH(a.b2)};
     CanonArgs mp1{mp_hidden, CH(a.mlp_Wb), (int64_t)a.r_mlp, a.ffn, a.r_mlp,
                   reinterpret_cast<half_t*>(a.mlp_logit_out)};
-    const int rw1 = a.r_mlp <= 1024 ? 4 : 1;
+    const int rw1 = a.r_mlp <= 1024 ? 4 * kCanonShortRows : 1;
     int nm = ((a.ffn + rw1 - 1) / rw1 + 3) / 4;
     if (nm > cus * 16) nm = cus * 16;
     const int nf = c.col_tiles * c.groups;

@@ -85,25 +85,27 @@ __global__ __launch_bounds__(256) void canonical_gemv_kernel(
   canonical_gemv_body<LANES, B, U>(X, W, ldw, rows, n, Y, blockIdx.x, gridDim.x);
 }
 
-// Several batch rows (B >= 2) over short rows (B * n floats fit LDS): with one weight row per
-// lane group every 16 bytes of weights need B * 16 bytes of x from L1, which bounds the kernel
-// before memory does.  Here X is converted once per workgroup to fp32 in LDS and a lane group
-// owns R weight rows at a time that share each x read: row r of task t is
+// Short rows (B * n floats fit LDS).  With one weight row per lane group a wavefront has only
+// one row's loads in flight per group, and for B >= 2 every 16 bytes of weights need B * 16
+// bytes of x from L1, which bounds the kernel before memory does.  Here X is converted once per
+// workgroup to fp32 in LDS and a lane group owns R weight rows at a time (R times the loads in
+// flight) that share each x read: row r of task t is
 // (t * R + r) * (64 / LANES) + group.  Same products in the same order per output as
 // canonical_gemv_body, so the same bits.  Dynamic LDS: B * n * 4 bytes.
-template <int LANES, int B, int U, int R>
-__global__ __launch_bounds__(256) void canonical_gemv_xlds_kernel(
-    const half_t* __restrict__ X, const half_t* __restrict__ W, int64_t ldw, int rows, int n,
-    half_t* __restrict__ Y) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  float* xf = reinterpret_cast<float*>(smem_raw);
-  for (int i = threadIdx.x * 8; i < B * n; i += blockDim.x * 8) {
+// count fp16 values (a multiple of 8) -> fp32 in LDS, by the whole workgroup (which then synchronises)
+__device__ __forceinline__ void stage_x_f32(const half_t* __restrict__ X, int count, float* xf) {
+  for (int i = threadIdx.x * 8; i < count; i += blockDim.x * 8) {
     const half8_t v = load8(X + i);
 #pragma unroll
     for (int e = 0; e < 8; ++e) xf[i + e] = (float)v[e];
   }
   __syncthreads();
+}
 
+template <int LANES, int B, int U, int R>
+__device__ __forceinline__ void canonical_gemv_lds_body(const float* xf, const half_t* __restrict__ W,
+                                                        int64_t ldw, int rows, int n,
+                                                        half_t* __restrict__ Y, int block_id, int nblocks) {
   constexpr int RW = kWave / LANES;
   constexpr int CH = 8 * LANES;
   const int lane = threadIdx.x & 63;
@@ -111,7 +113,8 @@ __global__ __launch_bounds__(256) void canonical_gemv_xlds_kernel(
   const int grp = lane / LANES;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int ntasks = (rows + RW * R - 1) / (RW * R);
-  for (int t = blockIdx.x * 4 + wave; t < ntasks; t += gridDim.x * 4) {
+  const int waves_per_block = blockDim.x >> 6;
+  for (int t = block_id * waves_per_block + wave; t < ntasks; t += nblocks * waves_per_block) {
     const half_t* wr[R];
     bool valid[R];
 #pragma unroll
@@ -164,6 +167,16 @@ __global__ __launch_bounds__(256) void canonical_gemv_xlds_kernel(
         if (valid[r] && sub == 0) Y[(int64_t)b * rows + row] = (half_t)v;
       }
   }
+}
+
+template <int LANES, int B, int U, int R>
+__global__ __launch_bounds__(256) void canonical_gemv_xlds_kernel(
+    const half_t* __restrict__ X, const half_t* __restrict__ W, int64_t ldw, int rows, int n,
+    half_t* __restrict__ Y) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  float* xf = reinterpret_cast<float*>(smem_raw);
+  stage_x_f32(X, B * n, xf);
+  canonical_gemv_lds_body<LANES, B, U, R>(xf, W, ldw, rows, n, Y, blockIdx.x, gridDim.x);
 }
 
 // ---------------------------------------------------------------------------

@@ -63,11 +63,16 @@ struct CanonArgs {
   half_t* Y;
 };
 
-// canonical GEMV role with the lane count the fixed summation order prescribes for n
+// canonical GEMV role with the lane count the fixed summation order prescribes for n; short rows
+// take the variant with x in LDS and two weight rows per lane group (more loads in flight)
+constexpr int kCanonShortRows = 2;
+
 __device__ __forceinline__ void canonical_role(const CanonArgs& c, int block_id, int nblocks) {
-  if (c.n <= 1024)
-    canonical_gemv_body<16, 1, 8>(c.X, c.W, c.ldw, c.rows, c.n, c.Y, block_id, nblocks);
-  else
+  if (c.n <= 1024) {
+    __shared__ __attribute__((aligned(16))) float s_xf[1024];
+    stage_x_f32(c.X, c.n, s_xf);
+    canonical_gemv_lds_body<16, 1, 8, kCanonShortRows>(s_xf, c.W, c.ldw, c.rows, c.n, c.Y, block_id, nblocks);
+  } else
     canonical_gemv_body<64, 1, 8>(c.X, c.W, c.ldw, c.rows, c.n, c.Y, block_id, nblocks);
 }
 
