@@ -70,17 +70,20 @@ __device__ __forceinline__ void gather_cols_body(
       ok = id >= 0 && id < Z;
       rid = ok ? (int)id : 0;
     }
-    // the loop over full batches of U rows is software-pipelined: the next batch's weight
-    // loads are in flight during this batch's multiply-adds, and the first batch is issued
-    // before the activations (for ATTN: the merged attention partials) are known
+    // the loop over full batches of U rows is software-pipelined two batches deep (registers
+    // wa / wb): two batches' weight loads are in flight during a batch's multiply-adds, and the
+    // first two are issued before the activations (for ATTN: the merged attention partials)
+    // are known
     const int cnt = (m_end - mb) < kWave ? (m_end - mb) : kWave;
     const int nfull = cnt / U;
-    half8_t wn[U];
-    if (nfull > 0) {
+    half8_t wa[U], wb[U];
+    auto load_batch = [&](half8_t (&w)[U], int jb) {
 #pragma unroll
       for (int u = 0; u < U; ++u)
-        wn[u] = load8_stream(wcol + (int64_t)__builtin_amdgcn_readlane(rid, u) * ldw);
-    }
+        w[u] = load8_stream(wcol + (int64_t)__builtin_amdgcn_readlane(rid, jb * U + u) * ldw);
+    };
+    if (nfull > 0) load_batch(wa, 0);
+    if (nfull > 1) load_batch(wb, 1);
     float xl[B];
     if (ATTN) {
       const int nheads = M / blk;
@@ -134,20 +137,28 @@ __device__ __forceinline__ void gather_cols_body(
         }
       }
     };
-    int j = 0;
-    for (int jb = 0; jb + 1 < nfull; ++jb, j += U) {
+    int jb = 0;
+    for (; jb + 3 < nfull; jb += 2) {  // batches jb, jb + 1 are in wa, wb; jb + 2, jb + 3 exist
       half8_t w[U];
 #pragma unroll
-      for (int u = 0; u < U; ++u) w[u] = wn[u];
+      for (int u = 0; u < U; ++u) w[u] = wa[u];
+      load_batch(wa, jb + 2);
+      consume(w, jb * U);
 #pragma unroll
-      for (int u = 0; u < U; ++u)
-        wn[u] = load8_stream(wcol + (int64_t)__builtin_amdgcn_readlane(rid, j + U + u) * ldw);
-      consume(w, j);
+      for (int u = 0; u < U; ++u) w[u] = wb[u];
+      load_batch(wb, jb + 3);
+      consume(w, (jb + 1) * U);
     }
-    if (nfull > 0) {
-      consume(wn, j);
-      j += U;
+    if (jb < nfull) {  // up to three batches left: jb in wa, jb + 1 in wb, jb + 2 not requested yet
+      half8_t w[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) w[u] = wa[u];
+      if (jb + 2 < nfull) load_batch(wa, jb + 2);
+      consume(w, jb * U);
+      if (jb + 1 < nfull) consume(wb, (jb + 1) * U);
+      if (jb + 2 < nfull) consume(wa, (jb + 2) * U);
     }
+    int j = nfull * U;
     if (j < cnt) {
       // fewer than U rows left: their loads are issued together like those of a full batch
       // (slots past the last row repeat it and take no part in the sums)
