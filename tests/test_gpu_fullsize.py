@@ -1,0 +1,132 @@
+"""The single ops at the OPT-175B sizes (d = 12288, ffn = 49152, 96 heads of 128, K = 4096, 32
+active heads), where the numpy oracle would take minutes: checked against PyTorch's own fp32
+library routines on the GPU (index_select + matmul / einsum, the closed forms the reference's
+docstrings give: gather_gemv.py:205-212, 578-584, attention_proj_sparse.py:118, 281) and
+through properties that do not depend on the size (linearity, invariance under a permutation
+of the index vector, exactness of the selected set)."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+D, FFN, H, HD, K, HK, R = 12288, 49152, 96, 128, 4096, 32, 1000
+MAX_ABS, REL_L2 = 2e-2, 1e-3
+
+
+def close(got, want, what, max_abs_tol=MAX_ABS, rel_tol=REL_L2):
+    got, want = got.double(), want.double()
+    max_abs = (got - want).abs().max().item()
+    rel = ((got - want).norm() / want.norm().clamp_min(1e-30)).item()
+    assert max_abs <= max_abs_tol and rel <= rel_tol, f"{what}: max_abs={max_abs:.3e} rel_l2={rel:.3e}"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from dejavu_amd import ops as _ops
+
+    return _ops
+
+
+@pytest.fixture(scope="module")
+def gen():
+    g = torch.Generator(device="cuda")
+    g.manual_seed(1234)
+    return g
+
+
+def randn(gen, *shape, std=1.0, mean=0.0):
+    return torch.empty(*shape, device="cuda", dtype=torch.float32).normal_(mean, std, generator=gen).half()
+
+
+def test_sparse_mlp_against_library_and_linearity(ops, gen):
+    W1, b1 = randn(gen, FFN, D, std=0.02), randn(gen, FFN, std=0.02, mean=-0.1)
+    W2t, b2 = randn(gen, FFN, D, std=0.02), randn(gen, D, std=0.02)
+    x = randn(gen, 1, D)
+    idx = torch.sort(torch.randperm(FFN, device="cuda", generator=gen)[:K]).values
+    print("case full-size sparse MLP", flush=True)
+    h = ops.gather_gemv(x, W1, idx, b1, "relu")
+    h_ref = torch.relu(x.float() @ W1.index_select(0, idx).float().t() + b1[idx].float())
+    close(h, h_ref, "fc1 against index_select + matmul")
+    y = ops.gather_transposed_gemv(h, W2t, idx, b2)
+    y_ref = h.float() @ W2t.index_select(0, idx).float() + b2.float()
+    close(y, y_ref, "fc2 against index_select + matmul")
+    close(ops.mlp_sparse(x, W1, W2t, idx, b1, b2), y_ref, "mlp_sparse")
+    # fc2 is linear in h (no bias): f(h1 + h2) = f(h1) + f(h2) up to fp16 rounding of the three results
+    h2 = randn(gen, 1, K).abs()
+    f = lambda v: ops.gather_transposed_gemv(v, W2t, idx, None).float()
+    close(f((h.float() + h2.float()).half()), f(h) + f(h2), "fc2 linearity", max_abs_tol=3e-2, rel_tol=3e-3)
+    # the same neurons in another order: the same sum up to fp32 re-association
+    perm = torch.randperm(K, device="cuda", generator=gen)
+    close(ops.gather_transposed_gemv(h[:, perm].contiguous(), W2t, idx[perm].contiguous(), b2), y_ref,
+          "fc2 under a permutation of the index vector")
+    close(ops.gather_gemv(x, W1, idx[perm].contiguous(), b1, "relu"), h_ref[:, perm], "fc1 under a permutation")
+
+
+def test_predictor_and_topk_properties(ops, gen):
+    Wa, Wb = randn(gen, R, D, std=0.05), randn(gen, FFN, R, std=0.05)
+    x = randn(gen, 1, D)
+    print("case full-size predictor + top-k", flush=True)
+    hidden = torch.empty(1, R, dtype=torch.float16, device="cuda")
+    logits = ops.predictor_logits(x, Wa, Wb, hidden=hidden)
+    close(hidden, x.float() @ Wa.float().t(), "predictor hidden against matmul")
+    close(logits, hidden.float() @ Wb.float().t(), "predictor logits against matmul")
+    idx = ops.topk_indices(logits, K)
+    assert idx.dtype == torch.int64 and idx.numel() == K
+    assert bool((idx[1:] > idx[:-1]).all()), "ascending, no duplicates"
+    sel = torch.zeros(FFN, dtype=torch.bool, device="cuda")
+    sel[idx] = True
+    lf = logits[0].float()
+    lo_in, hi_out = lf[sel].min().item(), lf[~sel].max().item()
+    assert hi_out <= lo_in, "an unselected logit beats a selected one"
+    # ties at the threshold go to the lower index
+    tied_out = (~sel & (lf == lo_in)).nonzero().flatten()
+    tied_in = (sel & (lf == lo_in)).nonzero().flatten()
+    if tied_out.numel():
+        assert tied_in.max().item() < tied_out.min().item()
+    # selecting again among the selected changes nothing (idempotence), and k = n selects everything
+    masked = torch.where(sel, logits[0], torch.full_like(logits[0], -65504.0)).unsqueeze(0).contiguous()
+    assert torch.equal(ops.topk_indices(masked, K), idx)
+    assert torch.equal(ops.topk_indices(logits, FFN), torch.arange(FFN, device="cuda"))
+
+
+def test_head_sparse_projections_against_library(ops, gen):
+    Wqkv, bqkv = randn(gen, 3, H, HD, D, std=0.02), randn(gen, 3, H, HD, std=0.02)
+    Wout_t, bout = randn(gen, H * HD, D, std=0.02), randn(gen, D, std=0.02)
+    x = randn(gen, 16, D)
+    head_idx = torch.sort(torch.randperm(H, device="cuda", generator=gen)[:HK]).values.int()
+    hi = head_idx.long()
+    print("case full-size QKV / out_proj", flush=True)
+    for nb in (1, 16):  # one token on the vector ALUs, a whole window on the matrix cores
+        batch_idx = torch.arange(nb, device="cuda", dtype=torch.int32).repeat(HK, 1).contiguous()
+        out = torch.zeros(nb, 3, H, HD, dtype=torch.float16, device="cuda")
+        ops.qkv_proj_sparse(x[:nb], Wqkv, head_idx, batch_idx, bqkv, out=out)
+        ref = torch.einsum("thjn,bn->bthj", Wqkv[:, hi].float(), x[:nb].float()) + bqkv[:, hi].float()
+        close(out[:, :, hi], ref, f"QKV of the active heads, {nb} row(s)")
+        others = torch.ones(H, dtype=torch.bool, device="cuda")
+        others[hi] = False
+        assert not out[:, :, others].any(), "inactive heads must not be written"
+    ctx = randn(gen, 1, H, HD)
+    y = ops.out_proj_sparse_t(ctx, Wout_t, head_idx, bout)
+    rows = (hi[:, None] * HD + torch.arange(HD, device="cuda")[None, :]).flatten()
+    ref = ctx.view(1, H * HD)[:, rows].float() @ Wout_t.index_select(0, rows).float() + bout.float()
+    close(y, ref, "out_proj over the active heads")
+    # the reference's (d, H, hd) weight layout gives the same result
+    close(ops.out_proj_sparse(ctx, Wout_t.t().contiguous().view(D, H, HD), head_idx, bout), ref, "out_proj, (d, H, hd)")
+
+
+def test_decode_attention_against_sdpa(ops, gen):
+    S, t = 2048, 2047
+    from dejavu_amd.workloads import pack_k_cache
+
+    k = randn(gen, 1, H, S, HD)
+    v = randn(gen, 1, H, S, HD)
+    q = randn(gen, 1, H, HD)
+    head_idx = torch.sort(torch.randperm(H, device="cuda", generator=gen)[:HK]).values.int()
+    hi = head_idx.long()
+    print("case full-size decode attention", flush=True)
+    k_cache, v_cache = pack_k_cache(k.cpu()).cuda(), v.clone()
+    ctx = ops.single_query_attention(q, None, None, k_cache, v_cache, None, t, head_idx=head_idx)
+    ref = torch.nn.functional.scaled_dot_product_attention(q[:, hi].float().unsqueeze(2), k[:, hi].float(),
+                                                           v[:, hi].float()).squeeze(2)
+    close(ctx[:, hi], ref, "attention over the active heads against SDPA")
