@@ -18,7 +18,10 @@ between consecutive tokens, the most back-fill work a window can have.
 Steps are replayed from HIP graphs (one graph of 3 layers x 16 positions when the
 step counts are multiples of 48, one graph per (layer, position) otherwise).
 
-Prints ONE JSON line (see README / DESIGN.md for the fields).
+Prints ONE JSON line: metric / value / unit (us per layer, whole-window average), the
+roofline of the dominant kernel (qkv_sparse_kernel, measured alone with HIP events), the CPU
+baseline (PyTorch index_select + matmul on the host cores, bounded sample), the first window
+position alone (window_start), the spread over single graph replays and a per-kernel table.
 """
 from __future__ import annotations
 
