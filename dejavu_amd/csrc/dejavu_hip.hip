@@ -1064,7 +1064,7 @@ int dv_sparse_layer_decode_f16(const dvSparseLayerArgs* args, void* stream) {
     else DV_L1(4);
 #undef DV_L1
   }
-  // L2: QKV + cache scatter | head predictor fc0 | key histogram of this layer's MLP logits
+  // L2: QKV + cache scatter | key histogram of this layer's MLP logits
   {
     QkvArgs q{x_cache, CH(a.Wqkv), CH(a.bqkv), head_idx, batch_idx, nb, a.d, a.H, a.hd, a.Hk, qkv,
               reinterpret_cast<half_t*>(a.k_cache), reinterpret_cast<half_t*>(a.v_cache),
@@ -1075,46 +1075,46 @@ int dv_sparse_layer_decode_f16(const dvSparseLayerArgs* args, void* stream) {
     if (nq > cus * 8) nq = cus * 8;
     const bool two = mfma && qkv_mfma_two_tiles(a.Hk, a.hd);
     if (mfma) nq = a.Hk * 3 * (a.hd / (two ? 32 : 16));
-    CanonArgs hp0{res1, CH(a.att_Wa), (int64_t)a.d, a.r_att, a.d, hp_hidden};
-    const int rw0 = a.d <= 1024 ? 4 * kCanonShortRows : 1;
-    const int nh = ((a.r_att + rw0 - 1) / rw0 + 3) / 4;
-    const dim3 grid(nq + nh + topk_blocks);
-#define DV_L2(NB)                                                                                 \
-  hipLaunchKernelGGL((layer_l2_kernel<NB>), grid, dim3(256), 0, s, q, nq, hp0, nh, CH(a.mlp_logit_in), \
-                     a.ffn, topk_ws)
+    const dim3 grid(nq + topk_blocks);
+#define DV_L2(NB) \
+  hipLaunchKernelGGL((layer_l2_kernel<NB>), grid, dim3(256), 0, s, q, nq, CH(a.mlp_logit_in), a.ffn, topk_ws)
     if (two) DV_L2(-1);
     else if (mfma) DV_L2(0);
     else DV_L2(1);
 #undef DV_L2
   }
-  // L3: attention partials | head predictor fc1 | top-k threshold and counts
+  // L3: attention partials | head predictor fc0 | top-k threshold and counts.  The head predictor
+  // (input: the residual stream after L1, output: only needed at the end of the step) runs one
+  // launch later than it could: the QKV launch is the fullest one, this one has bandwidth to spare.
   const int nsplit = a.seq_pos ? p.nsplit : attn_splits(a.n_len);
   {
     AttnArgs at{qkv + (size_t)a.counter * 3 * a.H * a.hd, (int64_t)3 * a.H * a.hd,
                 reinterpret_cast<const half_t*>(a.k_cache), reinterpret_cast<const half_t*>(a.v_cache),
                 head_idx, reinterpret_cast<const int*>(a.seq_pos), a.n_len, a.H, a.S, nsplit, a.Hk,
                 a.softmax_scale, attn_part};
-    CanonArgs hp1{hp_hidden, CH(a.att_Wb), (int64_t)a.r_att, a.H, a.r_att, head_logits};
+    CanonArgs hp0{res1, CH(a.att_Wa), (int64_t)a.d, a.r_att, a.d, hp_hidden};
     const int na = nsplit * a.Hk;
-    const int rw1 = a.r_att <= 1024 ? 4 * kCanonShortRows : 1;
-    const int nh1 = ((a.H + rw1 - 1) / rw1 + 3) / 4;
-    const dim3 grid(na + nh1 + topk_blocks);
+    const int rw0 = a.d <= 1024 ? 4 * kCanonShortRows : 1;
+    const int nh = ((a.r_att + rw0 - 1) / rw0 + 3) / 4;
+    const dim3 grid(na + nh + topk_blocks);
     if (a.hd == 128)
-      hipLaunchKernelGGL((layer_l3_kernel<128>), grid, dim3(256), 0, s, at, na, hp1, nh1, CH(a.mlp_logit_in),
+      hipLaunchKernelGGL((layer_l3_kernel<128>), grid, dim3(256), 0, s, at, na, hp0, nh, CH(a.mlp_logit_in),
                          a.ffn, a.K, topk_ws);
     else
-      hipLaunchKernelGGL((layer_l3_kernel<64>), grid, dim3(256), 0, s, at, na, hp1, nh1, CH(a.mlp_logit_in),
+      hipLaunchKernelGGL((layer_l3_kernel<64>), grid, dim3(256), 0, s, at, na, hp0, nh, CH(a.mlp_logit_in),
                          a.ffn, a.K, topk_ws);
   }
-  // L4 + L5: out_proj from the attention partials | head top-k | top-k emission; split reduction
+  // L4 + L5: out_proj from the attention partials | head predictor fc1 | top-k emission; split reduction
   {
     const ColsPlan& c = p.out_cols;
     OutProjArgs o{CH(a.Wout_t), (int64_t)a.d, CH(a.bout), head_idx, a.hd, a.d, a.H * a.hd, a.Hk * a.hd,
                   c.rows_per_block, c.col_tiles, c.groups, cols_part, attn_out, attn_part, nsplit};
+    CanonArgs hp1{hp_hidden, CH(a.att_Wb), (int64_t)a.r_att, a.H, a.r_att, head_logits};
+    const int rw1 = a.r_att <= 1024 ? 4 * kCanonShortRows : 1;
+    const int nh1 = ((a.H + rw1 - 1) / rw1 + 3) / 4;
     const int no = c.col_tiles * c.groups;
-    hipLaunchKernelGGL(layer_l4_kernel, dim3(no + 1 + topk_blocks), dim3(256), 0, s, o, no, head_logits, a.H,
-                       a.att_k, reinterpret_cast<int*>(a.att_idx_out), CH(a.mlp_logit_in), a.ffn, topk_ws,
-                       reinterpret_cast<int64_t*>(a.mlp_idx_out), topk_blocks);
+    hipLaunchKernelGGL(layer_l4_kernel, dim3(no + nh1 + topk_blocks), dim3(256), 0, s, o, no, hp1, nh1,
+                       CH(a.mlp_logit_in), a.ffn, topk_ws, reinterpret_cast<int64_t*>(a.mlp_idx_out), topk_blocks);
     // L5: split reduction + bias, and the residual stream advanced by the attention output
     hipLaunchKernelGGL(cols_reduce_kernel, dim3((unsigned)((a.d + 63) / 64)), dim3(256), 0, s,
                        c.groups > 1 ? cols_part : nullptr, CH(a.bout), c.groups, 1, a.d, attn_out, res1,
@@ -1122,7 +1122,7 @@ int dv_sparse_layer_decode_f16(const dvSparseLayerArgs* args, void* stream) {
   }
   const half_t* res2 = reinterpret_cast<const half_t*>(a.residual_out);
   const int64_t* mlp_idx = reinterpret_cast<const int64_t*>(a.mlp_idx_out);
-  // L7: LayerNorm 2 + fc1 gather | MLP predictor fc0
+  // L7: LayerNorm 2 + fc1 gather | MLP predictor fc0 | head top-k
   {
     RowsArgs f{res2, CH(a.ln2_w), CH(a.ln2_b), a.eps2, CH(a.W1), CH(a.b1), mlp_idx, a.d, (int64_t)a.d, a.ffn,
                a.K, hbuf};
@@ -1142,9 +1142,14 @@ int dv_sparse_layer_decode_f16(const dvSparseLayerArgs* args, void* stream) {
         return DV_ERR_UNSUPPORTED;
       lds_granted[v] = lds;
     }
-    if (v == 0) hipLaunchKernelGGL(layer_l7_kernel<1>, dim3(nf + nm), dim3(256), lds, s, f, nf, mp0, nm);
-    else if (v == 1) hipLaunchKernelGGL(layer_l7_kernel<2>, dim3(nf + nm), dim3(256), lds, s, f, nf, mp0, nm);
-    else hipLaunchKernelGGL(layer_l7_kernel<4>, dim3(nf + nm), dim3(256), lds, s, f, nf, mp0, nm);
+    int* att_out = reinterpret_cast<int*>(a.att_idx_out);
+    const dim3 grid(nf + nm + 1);  // + the head top-k
+    if (v == 0)
+      hipLaunchKernelGGL(layer_l7_kernel<1>, grid, dim3(256), lds, s, f, nf, mp0, nm, head_logits, a.H, a.att_k, att_out);
+    else if (v == 1)
+      hipLaunchKernelGGL(layer_l7_kernel<2>, grid, dim3(256), lds, s, f, nf, mp0, nm, head_logits, a.H, a.att_k, att_out);
+    else
+      hipLaunchKernelGGL(layer_l7_kernel<4>, grid, dim3(256), lds, s, f, nf, mp0, nm, head_logits, a.H, a.att_k, att_out);
   }
   // L8 + L9: fc2 gather | MLP predictor fc1, then the split reduction
   {

@@ -5,14 +5,14 @@
 // The role bodies are the very same device functions as the stand-alone kernels.
 //
 //  L1  add+LayerNorm 1 + back-fill window step
-//  L2  QKV (+ cache scatter) of the active heads       | head predictor fc0 | key histogram of the MLP logits
-//  L3  attention partials over the active heads        | head predictor fc1 | top-k threshold + counts
-//  L4  out_proj over W_out^T, merging the attention    | head top-k         | top-k emission
+//  L2  QKV (+ cache scatter) of the active heads       | key histogram of the MLP logits
+//  L3  attention partials over the active heads        | head predictor fc0 | top-k threshold + counts
+//  L4  out_proj over W_out^T, merging the attention    | head predictor fc1 | top-k emission
 //      partials on the fly
 //  L5  split reduction (+ bias) + residual add
 //  L6  LayerNorm 2 of the residual stream, computed inside the fc1 workgroups while they
 //      stage their input row (same bits as the stand-alone kernel), then
-//      fc1 gather (+bias, ReLU)                         | MLP predictor fc0
+//      fc1 gather (+bias, ReLU)                         | MLP predictor fc0  | head top-k
 //  L8  fc2 gather                                       | MLP predictor fc1
 //  L9  split reduction (+ bias)
 #pragma once
@@ -77,7 +77,7 @@ __device__ __forceinline__ void canonical_role(const CanonArgs& c, int block_id,
 }
 
 template <int NBMAX>
-__global__ __launch_bounds__(256) void layer_l2_kernel(QkvArgs q, int nblk_qkv, CanonArgs hp0, int nblk_hp0,
+__global__ __launch_bounds__(256) void layer_l2_kernel(QkvArgs q, int nblk_qkv,
                                                        const half_t* __restrict__ mlp_logits, int ffn,
                                                        unsigned* __restrict__ topk_ws) {
   const int bid = blockIdx.x;
@@ -89,10 +89,8 @@ __global__ __launch_bounds__(256) void layer_l2_kernel(QkvArgs q, int nblk_qkv, 
     else
       qkv_sparse_body<NBMAX, 2, 4>(q.X, q.W, q.bias, q.head_idx, q.batch_idx, q.nb, q.d, q.H, q.hd, q.nnz, q.Y,
                                    q.k_cache, q.v_cache, q.padding, q.S, bid, nblk_qkv);
-  } else if (bid < nblk_qkv + nblk_hp0) {
-    canonical_role(hp0, bid - nblk_qkv, nblk_hp0);
   } else {
-    topk_hist_body(mlp_logits, 1, ffn, topk_ws, bid - nblk_qkv - nblk_hp0);
+    topk_hist_body(mlp_logits, 1, ffn, topk_ws, bid - nblk_qkv);
   }
 }
 
@@ -110,7 +108,7 @@ struct AttnArgs {
 };
 
 template <int HD>
-__global__ __launch_bounds__(256) void layer_l3_kernel(AttnArgs a, int nblk_attn, CanonArgs hp1, int nblk_hp1,
+__global__ __launch_bounds__(256) void layer_l3_kernel(AttnArgs a, int nblk_attn, CanonArgs hp0, int nblk_hp0,
                                                        const half_t* __restrict__ mlp_logits, int ffn,
                                                        int K, unsigned* __restrict__ topk_ws) {
   const int bid = blockIdx.x;
@@ -118,10 +116,10 @@ __global__ __launch_bounds__(256) void layer_l3_kernel(AttnArgs a, int nblk_attn
     const int split = bid % a.nsplit, i = bid / a.nsplit;
     decode_attn_body<HD, 4>(a.Q, a.ldq, a.k_cache, a.v_cache, a.head_idx, a.seq_pos, a.n_len, a.H, a.S, a.scale,
                             a.nsplit, a.part, split, i, 0, a.nheads);
-  } else if (bid < nblk_attn + nblk_hp1) {
-    canonical_role(hp1, bid - nblk_attn, nblk_hp1);
+  } else if (bid < nblk_attn + nblk_hp0) {
+    canonical_role(hp0, bid - nblk_attn, nblk_hp0);
   } else {
-    topk_count_body(mlp_logits, 1, ffn, K, topk_ws, bid - nblk_attn - nblk_hp1);
+    topk_count_body(mlp_logits, 1, ffn, K, topk_ws, bid - nblk_attn - nblk_hp0);
   }
 }
 
@@ -138,9 +136,7 @@ struct OutProjArgs {
   int nsplit;
 };
 
-__global__ __launch_bounds__(256) void layer_l4_kernel(OutProjArgs o, int nblk_out,
-                                                       const half_t* __restrict__ head_logits, int H,
-                                                       int att_k, int* __restrict__ att_idx_out,
+__global__ __launch_bounds__(256) void layer_l4_kernel(OutProjArgs o, int nblk_out, CanonArgs hp1, int nblk_hp1,
                                                        const half_t* __restrict__ mlp_logits, int ffn,
                                                        unsigned* __restrict__ topk_ws,
                                                        int64_t* __restrict__ mlp_idx_out, int nblk_emit) {
@@ -148,17 +144,12 @@ __global__ __launch_bounds__(256) void layer_l4_kernel(OutProjArgs o, int nblk_o
   if (bid < nblk_out) {
     const int ct = bid % o.col_tiles, g = bid / o.col_tiles;
     gather_cols_body<1, 8, false, true, true>(nullptr, 0, 1, o.W, o.ldw, o.bias, o.head_idx, o.hd, o.N,
-                                                     o.Z, o.M, o.rows_per_block, o.partial, nullptr, o.Y,
-                                                     o.attn_part, o.nsplit, ct, g, o.groups);
-  } else if (bid == nblk_out) {
-    // head top-k for the next layer (rank selection, one workgroup)
-    __shared__ unsigned s_key[1024];
-    __shared__ unsigned s_sel[1024];
-    for (int j = threadIdx.x; j < H; j += blockDim.x) s_key[j] = topk_key(head_logits[j]);
-    __syncthreads();
-    rank_select_emit(s_key, s_sel, H, att_k, att_idx_out, 4);
+                                              o.Z, o.M, o.rows_per_block, o.partial, nullptr, o.Y,
+                                              o.attn_part, o.nsplit, ct, g, o.groups);
+  } else if (bid < nblk_out + nblk_hp1) {
+    canonical_role(hp1, bid - nblk_out, nblk_hp1);
   } else {
-    topk_emit_body(mlp_logits, 1, ffn, topk_ws, mlp_idx_out, 8, bid - nblk_out - 1, nblk_emit);
+    topk_emit_body(mlp_logits, 1, ffn, topk_ws, mlp_idx_out, 8, bid - nblk_out - nblk_hp1, nblk_emit);
   }
 }
 
@@ -178,7 +169,9 @@ struct RowsArgs {
 };
 
 template <int MAXV>
-__global__ __launch_bounds__(256) void layer_l7_kernel(RowsArgs f, int nblk_fc1, CanonArgs mp0, int nblk_mp0) {
+__global__ __launch_bounds__(256) void layer_l7_kernel(RowsArgs f, int nblk_fc1, CanonArgs mp0, int nblk_mp0,
+                                                       const half_t* __restrict__ head_logits, int H, int att_k,
+                                                       int* __restrict__ att_idx_out) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   const int bid = blockIdx.x;
   if (bid < nblk_fc1) {
@@ -187,8 +180,15 @@ __global__ __launch_bounds__(256) void layer_l7_kernel(RowsArgs f, int nblk_fc1,
     __syncthreads();
     gather_rows_body<1, 2, 4, true, true>(nullptr, f.W, f.bias, f.idx, 8, f.n, f.ldw, f.Z, f.M, f.Y, xs, bid,
                                           nblk_fc1);
-  } else {
+  } else if (bid < nblk_fc1 + nblk_mp0) {
     canonical_role(mp0, bid - nblk_fc1, nblk_mp0);
+  } else {
+    // head top-k for the next layer (rank selection, one workgroup)
+    __shared__ unsigned s_key[1024];
+    __shared__ unsigned s_sel[1024];
+    for (int j = threadIdx.x; j < H; j += blockDim.x) s_key[j] = topk_key(head_logits[j]);
+    __syncthreads();
+    rank_select_emit(s_key, s_sel, H, att_k, att_idx_out, 4);
   }
 }
 
