@@ -1052,19 +1052,20 @@ int dv_sparse_layer_decode_f16(const dvSparseLayerArgs* args, void* stream) {
   const int nb = a.counter + 1;
   const int topk_blocks = (a.ffn + kTopkItemsPerBlock - 1) / kTopkItemsPerBlock;
 
-  // L1: add + LayerNorm 1 + window step
+  // L1: add + LayerNorm 1 + window step | key histogram of this layer's MLP logits
   {
+    const int hist_blocks = topk_blocks;  // 256 * 8 columns each
 #define DV_L1(V)                                                                                      \
-  hipLaunchKernelGGL((layer_l1_kernel<V>), dim3(1), dim3(kLnThreads), 0, s, CH(a.hidden), CH(a.residual), \
-                     CH(a.ln1_w), CH(a.ln1_b), a.eps1, a.d, x, res1, x_cache + (size_t)a.counter * a.d, \
-                     reinterpret_cast<int*>(a.tracker), head_idx, a.Hk, a.H, a.counter,        \
-                     a.counter == 15 ? 1 : 0, batch_idx)
+  hipLaunchKernelGGL((layer_l1_kernel<V>), dim3(1 + hist_blocks), dim3(kLnThreads), 0, s, CH(a.hidden),   \
+                     CH(a.residual), CH(a.ln1_w), CH(a.ln1_b), a.eps1, a.d, x, res1,                     \
+                     x_cache + (size_t)a.counter * a.d, reinterpret_cast<int*>(a.tracker), head_idx, a.Hk, \
+                     a.H, a.counter, a.counter == 15 ? 1 : 0, batch_idx, CH(a.mlp_logit_in), a.ffn, topk_ws)
     if (a.d <= kLnThreads * 8) DV_L1(1);
     else if (a.d <= kLnThreads * 16) DV_L1(2);
     else DV_L1(4);
 #undef DV_L1
   }
-  // L2: QKV + cache scatter | key histogram of this layer's MLP logits
+  // L2: QKV + cache scatter
   {
     QkvArgs q{x_cache, CH(a.Wqkv), CH(a.bqkv), head_idx, batch_idx, nb, a.d, a.H, a.hd, a.Hk, qkv,
               reinterpret_cast<half_t*>(a.k_cache), reinterpret_cast<half_t*>(a.v_cache),
@@ -1075,9 +1076,8 @@ int dv_sparse_layer_decode_f16(const dvSparseLayerArgs* args, void* stream) {
     if (nq > cus * 8) nq = cus * 8;
     const bool two = mfma && qkv_mfma_two_tiles(a.Hk, a.hd);
     if (mfma) nq = a.Hk * 3 * (a.hd / (two ? 32 : 16));
-    const dim3 grid(nq + topk_blocks);
-#define DV_L2(NB) \
-  hipLaunchKernelGGL((layer_l2_kernel<NB>), grid, dim3(256), 0, s, q, nq, CH(a.mlp_logit_in), a.ffn, topk_ws)
+    const dim3 grid(nq);
+#define DV_L2(NB) hipLaunchKernelGGL((layer_l2_kernel<NB>), grid, dim3(256), 0, s, q)
     if (two) DV_L2(-1);
     else if (mfma) DV_L2(0);
     else DV_L2(1);

@@ -4,8 +4,8 @@
 // run beside the bandwidth-bound ones instead of each paying a launch of its own.
 // The role bodies are the very same device functions as the stand-alone kernels.
 //
-//  L1  add+LayerNorm 1 + back-fill window step
-//  L2  QKV (+ cache scatter) of the active heads       | key histogram of the MLP logits
+//  L1  add+LayerNorm 1 + back-fill window step          | key histogram of the MLP logits
+//  L2  QKV (+ cache scatter) of the active heads
 //  L3  attention partials over the active heads        | head predictor fc0 | top-k threshold + counts
 //  L4  out_proj over W_out^T, merging the attention    | head predictor fc1 | top-k emission
 //      partials on the fly
@@ -29,13 +29,21 @@ namespace dv {
 constexpr int kLnThreads = 1024;
 
 // ---- L1 -------------------------------------------------------------------
+// Workgroup 0: LayerNorm + window step; the others: key histogram of this layer's MLP logits (an
+// input of the step).  The histogram sits here because the QKV workgroups of the next launch fill
+// every slot of the device for its whole duration: a role behind them would only start at its end.
 template <int MAXV>
 __global__ __launch_bounds__(kLnThreads) void layer_l1_kernel(
     const half_t* __restrict__ hidden, const half_t* __restrict__ residual,
     const half_t* __restrict__ gamma, const half_t* __restrict__ beta, float eps, int d,
     half_t* __restrict__ x, half_t* __restrict__ residual1, half_t* __restrict__ x_cache_row,
     int* __restrict__ tracker, const int* __restrict__ head_idx, int nnz, int H, int counter,
-    int flush, int* __restrict__ batch_idx) {
+    int flush, int* __restrict__ batch_idx, const half_t* __restrict__ mlp_logits, int ffn,
+    unsigned* __restrict__ topk_ws) {
+  if (blockIdx.x != 0) {
+    topk_hist_body(mlp_logits, 1, ffn, topk_ws, (int)blockIdx.x - 1);
+    return;
+  }
   add_layer_norm_body<kLnThreads, MAXV>(hidden, residual, gamma, beta, eps, d, x, residual1, x_cache_row, 0);
   window_tracker_step(tracker, head_idx, nnz, H, counter, flush, batch_idx);
 }
@@ -77,21 +85,14 @@ __device__ __forceinline__ void canonical_role(const CanonArgs& c, int block_id,
 }
 
 template <int NBMAX>
-__global__ __launch_bounds__(256) void layer_l2_kernel(QkvArgs q, int nblk_qkv,
-                                                       const half_t* __restrict__ mlp_logits, int ffn,
-                                                       unsigned* __restrict__ topk_ws) {
-  const int bid = blockIdx.x;
-  if (bid < nblk_qkv) {
-    if constexpr (NBMAX <= 0)  // several live window tokens: matrix-core variant (-1: 32-row workgroups)
-      qkv_window_mfma_body<kQkvMfmaWaves, NBMAX == 0 ? 1 : 2>(q.X, q.W, q.bias, q.head_idx, q.batch_idx, q.nb, q.d,
-                                                              q.H, q.hd, q.nnz, q.Y, q.k_cache, q.v_cache,
-                                                              q.padding, q.S, bid, nblk_qkv);
-    else
-      qkv_sparse_body<NBMAX, 2, 4>(q.X, q.W, q.bias, q.head_idx, q.batch_idx, q.nb, q.d, q.H, q.hd, q.nnz, q.Y,
-                                   q.k_cache, q.v_cache, q.padding, q.S, bid, nblk_qkv);
-  } else {
-    topk_hist_body(mlp_logits, 1, ffn, topk_ws, bid - nblk_qkv);
-  }
+__global__ __launch_bounds__(256) void layer_l2_kernel(QkvArgs q) {
+  if constexpr (NBMAX <= 0)  // several live window tokens: matrix-core variant (-1: 32-row workgroups)
+    qkv_window_mfma_body<kQkvMfmaWaves, NBMAX == 0 ? 1 : 2>(q.X, q.W, q.bias, q.head_idx, q.batch_idx, q.nb, q.d,
+                                                            q.H, q.hd, q.nnz, q.Y, q.k_cache, q.v_cache,
+                                                            q.padding, q.S, blockIdx.x, gridDim.x);
+  else
+    qkv_sparse_body<NBMAX, 2, 4>(q.X, q.W, q.bias, q.head_idx, q.batch_idx, q.nb, q.d, q.H, q.hd, q.nnz, q.Y,
+                                 q.k_cache, q.v_cache, q.padding, q.S, blockIdx.x, gridDim.x);
 }
 
 // ---- L3 -------------------------------------------------------------------

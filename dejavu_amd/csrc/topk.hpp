@@ -284,15 +284,18 @@ __global__ __launch_bounds__(256) void topk_batch_max_kernel(const half_t* __res
   }
 }
 
+// A workgroup covers 256 * 8 columns with its first 256 threads (further threads, if the launch
+// has them, only take part in the barriers): spreading the atomics over many compute units
+// matters more than filling the workgroup.
 __device__ __forceinline__ void topk_hist_body(const half_t* __restrict__ logits, int B, int n,
                                                unsigned* __restrict__ ws, int block_id) {
   // the 256 coarse bins are hot (most logits share a few exponents): aggregate them in
   // LDS and add each non-empty bin to memory once per workgroup
   __shared__ unsigned s_coarse[kTopkCoarse];
-  s_coarse[threadIdx.x] = 0u;
+  if (threadIdx.x < kTopkCoarse) s_coarse[threadIdx.x] = 0u;
   __syncthreads();
   const int i0 = (block_id * 256 + threadIdx.x) * 8;
-  if (i0 < n) {
+  if (threadIdx.x < 256 && i0 < n) {
     unsigned key[8];
     topk_load_keys(logits, B, n, i0, key);
 #pragma unroll
@@ -302,8 +305,10 @@ __device__ __forceinline__ void topk_hist_body(const half_t* __restrict__ logits
     }
   }
   __syncthreads();
-  const unsigned c = s_coarse[threadIdx.x];
-  if (c != 0u) atomicAdd(&ws[kTopkFine + threadIdx.x], c);
+  if (threadIdx.x < kTopkCoarse) {
+    const unsigned c = s_coarse[threadIdx.x];
+    if (c != 0u) atomicAdd(&ws[kTopkFine + threadIdx.x], c);
+  }
 }
 
 __global__ __launch_bounds__(256) void topk_hist_kernel(const half_t* __restrict__ logits, int B, int n,
