@@ -644,8 +644,8 @@ int dv_topk_search_f16(const void* logits, int B, int n, int k, void* idx_out, i
 int dv_gather_gemv_f16(const void* x, const void* W, int64_t ldw, const void* bias,
                        const void* idx, int idx_bytes, int B, int N, int Z, int M, int act,
                        void* y, void* stream) {
-  if (!x || !W || N <= 0 || Z <= 0 || M < 0 || !idx_ok(idx_bytes) || (M > 0 && (!idx || !y)) ||
-      (act != DV_ACT_ID && act != DV_ACT_RELU))
+  if (!x || !W || N <= 0 || Z <= 0 || M < 0 || (idx && !idx_ok(idx_bytes)) || (M > 0 && !y) ||
+      (!idx && M > Z) || (act != DV_ACT_ID && act != DV_ACT_RELU))
     return DV_ERR_INVALID_ARG;
   if (B < 1 || B > 64) return DV_ERR_UNSUPPORTED;
   if (N % 8 || ldw % 8 || ldw < N || !aligned16(x) || !aligned16(W)) return DV_ERR_ALIGNMENT;

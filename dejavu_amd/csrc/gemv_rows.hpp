@@ -183,7 +183,7 @@ __global__ __launch_bounds__(256) void canonical_gemv_xlds_kernel(
 // Y[b, m] = act( sum_i W[idx[m], i] * X[b, i] + bias[idx[m]] ), fp16 out.
 // One wavefront owns R gathered rows at a time (R independent load streams);
 // X is staged once per workgroup in LDS.  An index outside [0, Z) yields 0
-// instead of a wild read.  Requires n % 8 == 0 and ldw % 8 == 0.
+// instead of a wild read; idx == nullptr means no gather (row m of W: a dense product).  Requires n % 8 == 0 and ldw % 8 == 0.
 // ---------------------------------------------------------------------------
 // STAGED: the caller has already put X into xs (and synchronised the workgroup).
 template <int B, int R, int U, bool RELU, bool STAGED = false>
@@ -208,7 +208,7 @@ __device__ __forceinline__ void gather_rows_body(
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const int m = t * R + r;
-      int64_t id = m < M ? load_index(idx, idx_bytes, m) : -1;
+      int64_t id = m < M ? (idx != nullptr ? load_index(idx, idx_bytes, m) : (int64_t)m) : -1;
       valid[r] = id >= 0 && id < Z;
       rid[r] = valid[r] ? id : 0;
       wr[r] = W + rid[r] * ldw + lane * 8;

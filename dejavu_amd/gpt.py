@@ -32,7 +32,8 @@ import torch.nn.functional as F
 from . import modules as dv_modules
 from . import ops
 from .block import BlockDejavu, BlockMlpAttSparse
-from .modules import InferenceParams, ParallelFusedMLPDejavu, ParallelMHADejavu, ParallelMHASparseAttMlp
+from .modules import (InferenceParams, ParallelFusedMLPDejavu, ParallelMHADejavu, ParallelMHASparseAttMlp,
+                      decode_linear)
 
 CausalLMOutput = namedtuple("CausalLMOutput", ["logits"])
 GreedySearchDecoderOnlyOutput = namedtuple("GreedySearchDecoderOnlyOutput", ["sequences", "scores"])
@@ -220,7 +221,7 @@ class GPTLMHeadModel(nn.Module):
         hidden_states = self.transformer(input_ids, position_ids=position_ids, inference_params=inference_params)
         if last_token_only:
             hidden_states = hidden_states[:, -1:]
-        return CausalLMOutput(logits=self.lm_head(hidden_states))
+        return CausalLMOutput(logits=decode_linear(self.lm_head, hidden_states.contiguous()))
 
     # ---- generation ---------------------------------------------------------------
     def _sparse_mixers(self):

@@ -174,13 +174,25 @@ class ParallelFusedMLPDejavu(nn.Module):
             out = ops.mlp_sparse(x.squeeze(1), self.fc1.weight, self.fc2_weight_t, idx, self.fc1.bias, self.fc2.bias)
             out = out.unsqueeze(1)
         else:
-            h = F.linear(x, self.fc1.weight, self.fc1.bias)
-            h = F.relu(h) if self.activation == "relu" else F.gelu(h, approximate="tanh")
-            out = F.linear(h, self.fc2.weight, self.fc2.bias)
+            if self.activation == "relu":
+                h = decode_linear(self.fc1, x, "relu")
+            else:
+                h = F.gelu(F.linear(x, self.fc1.weight, self.fc1.bias), approximate="tanh")
+            out = decode_linear(self.fc2, h)
         # (tensor parallel all-reduce of `out` is the identity on one GPU)
         if side:
             curr_stream.wait_event(self.event_mlp_sp)
         return out, mlp_logit
+
+
+def decode_linear(linear: nn.Linear, x: torch.Tensor, activation: str = "id") -> torch.Tensor:
+    """``linear(x)`` (+ ReLU).  The few rows of a decode step (x: (B, 1, d), fp16, on the GPU) are
+    streamed by the row GEMV kernels; anything else (the prompt phase) goes to the library GEMM."""
+    if x.is_cuda and x.dtype == torch.float16 and x.dim() == 3 and x.shape[1] == 1 and x.shape[0] <= 64 \
+            and linear.weight.dtype == torch.float16 and x.shape[-1] % 8 == 0:
+        return ops.dense_decode_linear(x, linear.weight, linear.bias, activation)
+    y = linear(x)
+    return F.relu(y) if activation == "relu" else y
 
 
 def _update_kv_cache(kv, inference_params, layer_idx):
@@ -301,10 +313,10 @@ class ParallelMHADejavu(_MHABase):
         assert seqlen is None, "sequence-parallel input layout is not used for generation"
         self._streams()
         mlp_idx, _ = self._side_work(mlp_sp_logit)
-        qkv = self.Wqkv(x)
+        qkv = decode_linear(self.Wqkv, x)
         qkv = qkv.view(x.shape[0], x.shape[1], 3, self.num_heads, self.head_dim)
         context = self._dense_context(qkv, inference_params)
-        out = self.out_proj(context)
+        out = decode_linear(self.out_proj, context)
         self._join_side()
         return out, mlp_idx
 
@@ -405,9 +417,9 @@ class ParallelMHASparseAttMlp(_MHABase):
                 self.counter = 0
                 self.cache_offset += self.WINDOW
         else:
-            qkv = self.Wqkv(x)
+            qkv = decode_linear(self.Wqkv, x)
             qkv = qkv.view(x.shape[0], x.shape[1], 3, self.num_heads, self.head_dim)
             context = self._dense_context(qkv, inference_params)
-            out = self.out_proj(context)
+            out = decode_linear(self.out_proj, context)
         self._join_side()
         return out, mlp_idx, att_idx

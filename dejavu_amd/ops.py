@@ -146,11 +146,12 @@ def topk_indices(logits: torch.Tensor, k: int, dtype: torch.dtype = torch.int64,
 # ---------------------------------------------------------------------------
 # sparse MLP
 # ---------------------------------------------------------------------------
-def gather_gemv(x: torch.Tensor, weight: torch.Tensor, idx: torch.Tensor,
+def gather_gemv(x: torch.Tensor, weight: torch.Tensor, idx: Optional[torch.Tensor],
                 bias: Optional[torch.Tensor] = None, activation: str = "id") -> torch.Tensor:
     """Compute y = activation(x @ weight[idx, :].T + bias[idx]).
 
     x: (batch, N); weight: (Z, N); idx: (M,); bias: (Z,) -> (batch, M).
+    idx=None: every row (a dense product, M = Z).
     """
     assert activation in ["id", "relu", "gelu", "gelu_approx", "squared_relu"]
     if activation not in _ACT:
@@ -160,7 +161,7 @@ def gather_gemv(x: torch.Tensor, weight: torch.Tensor, idx: torch.Tensor,
     batch, _ = x.shape
     assert x.shape == (batch, N)
     assert 1 <= batch <= 64  # the reference stops at 4; larger batches run on the matrix cores
-    (M,) = idx.shape
+    M = Z if idx is None else idx.shape[0]
     x = x.contiguous()
     if weight.stride(1) > 1:
         weight = weight.contiguous()
@@ -170,11 +171,22 @@ def gather_gemv(x: torch.Tensor, weight: torch.Tensor, idx: torch.Tensor,
         bias = bias.contiguous()
         assert bias.shape == (Z,), "Incompatible dimensions in between weight and bias"
         assert x.dtype == bias.dtype, f"Input and bias must have the same dtype, got {x.dtype} and {bias.dtype}"
-    idx = idx.contiguous()
+    idx = None if idx is None else idx.contiguous()
     output = torch.empty(batch, M, device=x.device, dtype=x.dtype)
-    check(lib.dv_gather_gemv_f16(_ptr(x), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(idx), _idx_bytes(idx),
+    check(lib.dv_gather_gemv_f16(_ptr(x), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(idx),
+                                 8 if idx is None else _idx_bytes(idx),
                                  batch, N, Z, M, _ACT[activation], _ptr(output), _stream()), "dv_gather_gemv_f16")
     return output
+
+
+def dense_decode_linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                        activation: str = "id") -> torch.Tensor:
+    """``activation(F.linear(x, weight, bias))`` for the few rows of a decode step (1..64), streamed
+    by the row kernels without a gather: the dense first block and the lm_head of a generation
+    step are as bandwidth-bound as the sparse blocks.  x: (..., N) -> (..., Z)."""
+    lead = x.shape[:-1]
+    y = gather_gemv(x.reshape(-1, x.shape[-1]), weight, None, bias, activation)
+    return y.view(*lead, weight.shape[0])
 
 
 def gather_transposed_gemv(x: torch.Tensor, weight: torch.Tensor, idx: torch.Tensor,

@@ -105,6 +105,8 @@ DV_API int dv_topk_search_f16(const void* logits, int B, int n, int k, void* idx
  *   y (B, M) fp16.  1 <= B <= 64 (the reference stops at 4): B <= 2 runs as a
  *   bandwidth-bound GEMV on the vector ALUs; 3 <= B <= 64 stages the gathered
  *   rows through LDS into 16x16x32 fp16 MFMA tiles.
+  * idx == NULL: no gather, row m of W (a dense product y = act(x W[:M]^T + bias), M <= Z),
+ * as the one-token decode step of a dense block or of the lm_head needs it.
  */
 DV_API int dv_gather_gemv_f16(const void* x, const void* W, int64_t ldw, const void* bias,
                        const void* idx, int idx_bytes, int B, int N, int Z, int M, int act,

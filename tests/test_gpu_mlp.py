@@ -109,6 +109,30 @@ def test_predictor_second_product_with_short_rows(ops, B, r, n_out):
     assert_close(np16(got), want, "logits from the device's hidden vector")
 
 
+@pytest.mark.parametrize("B,N,Z,act", [(1, 768, 2304, "id"), (1, 5120, 50272, "id"), (2, 1024, 4099, "relu"),
+                                       (5, 640, 1000, "relu"), (33, 512, 777, "id")])
+def test_gather_gemv_without_index_is_a_dense_linear(ops, B, N, Z, act):
+    """idx=None: every row of the weight, in order -- F.linear (+ ReLU) for the few rows of a decode
+    step (dense first block, lm_head); vector kernels up to batch 2, MFMA tiles above."""
+    g = torch.Generator().manual_seed(B * 7 + Z)
+    x = torch.randn(B, N, generator=g).half()
+    W = (torch.randn(Z, N, generator=g) * 0.05).half()
+    b = (torch.randn(Z, generator=g) * 0.1).half()
+    print(f"case dense rows B={B} N={N} Z={Z}", flush=True)
+    y = ops.gather_gemv(x.cuda(), W.cuda(), None, b.cuda(), act)
+    y3 = ops.dense_decode_linear(x.view(B, 1, N).cuda(), W.cuda(), None, act)
+    torch.cuda.synchronize()
+    ref = x.float() @ W.float().t()
+    want, want3 = ref + b.float(), ref
+    if act == "relu":
+        want, want3 = want.relu(), want3.relu()
+    assert y.shape == (B, Z) and y3.shape == (B, 1, Z)
+    assert_close(np16(y), want.numpy(), "dense rows + bias")
+    assert_close(np16(y3).reshape(B, Z), want3.numpy(), "dense rows, no bias")
+    same = ops.gather_gemv(x.cuda(), W.cuda(), torch.arange(Z, device="cuda"), b.cuda(), act)
+    assert torch.equal(same, y), "idx=None must equal idx=arange bit for bit"
+
+
 # ---------------------------------------------------------------------- top-k
 @pytest.mark.parametrize("n", [12, 96, 97, 512, 3072, 16384, 20480, 36864, 49152, 65536])
 def test_topk_random_and_ties(ops, n):
