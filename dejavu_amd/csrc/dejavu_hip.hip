@@ -598,6 +598,20 @@ int dv_topk_f16(const void* logits, int B, int n, int k, void* idx_out, int idx_
   return launch_status();
 }
 
+int dv_greedy_advance_f16(const void* logits, int vocab, void* token, void* position, void* seq_pos,
+                          void* sequences, void* out_index, void* scores, int64_t score_ld,
+                          void* score_index, void* stream) {
+  if (!logits || vocab < 1 || !token || !position || !seq_pos || !sequences || !out_index ||
+      (scores && (!score_index || score_ld < vocab)))
+    return DV_ERR_INVALID_ARG;
+  hipLaunchKernelGGL(greedy_advance_kernel, dim3(1), dim3(1024), 0, reinterpret_cast<hipStream_t>(stream),
+                     reinterpret_cast<const half_t*>(logits), vocab, reinterpret_cast<int64_t*>(token),
+                     reinterpret_cast<int64_t*>(position), reinterpret_cast<int*>(seq_pos),
+                     reinterpret_cast<int64_t*>(sequences), reinterpret_cast<int64_t*>(out_index),
+                     reinterpret_cast<half_t*>(scores), score_ld, reinterpret_cast<int64_t*>(score_index));
+  return launch_status();
+}
+
 // Single-launch variant without scratch memory (16-step bitwise search in one
 // workgroup); same result, slower for large n.
 int dv_topk_search_f16(const void* logits, int B, int n, int k, void* idx_out, int idx_bytes,

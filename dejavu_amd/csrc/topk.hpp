@@ -450,4 +450,59 @@ __global__ __launch_bounds__(256) void topk_emit_kernel(const half_t* __restrict
   topk_emit_body(logits, B, n, ws, idx_out, idx_bytes, blockIdx.x, gridDim.x);
 }
 
+// ---------------------------------------------------------------------------
+// Greedy step of a generation loop (batch 1), one workgroup: next token = argmax of the logits
+// (first index among equal values, NaN ranks highest -- as torch.argmax), then the device-side
+// bookkeeping that lets a captured step be replayed: token <- next, sequences[out_index++] <-
+// next, position++, seq_pos++; optionally the logits row is kept in scores[score_index++].
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(1024) void greedy_advance_kernel(
+    const half_t* __restrict__ logits, int vocab, int64_t* __restrict__ token, int64_t* __restrict__ position,
+    int* __restrict__ seq_pos, int64_t* __restrict__ sequences, int64_t* __restrict__ out_index,
+    half_t* __restrict__ scores, int64_t score_ld, int64_t* __restrict__ score_index) {
+  __shared__ unsigned s_key[16];
+  __shared__ int s_idx[16];
+  unsigned best = 0u;
+  int best_i = 0x7fffffff;
+  for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
+    const unsigned k = topk_key(logits[i]) + 1u;  // +1: any element beats the empty start value
+    if (k > best) {  // i ascends per thread: equal keys keep the lower index
+      best = k;
+      best_i = i;
+    }
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    const unsigned ok = (unsigned)__shfl_xor((int)best, off, kWave);
+    const int oi = __shfl_xor(best_i, off, kWave);
+    if (ok > best || (ok == best && oi < best_i)) {
+      best = ok;
+      best_i = oi;
+    }
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) {
+    s_key[wave] = best;
+    s_idx[wave] = best_i;
+  }
+  if (scores != nullptr) {
+    half_t* row = scores + score_index[0] * score_ld;
+    for (int i = threadIdx.x; i < vocab; i += blockDim.x) row[i] = logits[i];
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < (int)(blockDim.x >> 6); ++w)
+      if (s_key[w] > best || (s_key[w] == best && s_idx[w] < best_i)) {
+        best = s_key[w];
+        best_i = s_idx[w];
+      }
+    token[0] = best_i;
+    sequences[out_index[0]] = best_i;
+    out_index[0] += 1;
+    position[0] += 1;
+    seq_pos[0] += 1;
+    if (scores != nullptr) score_index[0] += 1;
+  }
+}
+
 }  // namespace dv

@@ -233,15 +233,8 @@ class GPTLMHeadModel(nn.Module):
         logits = self(cache.token, position_ids=cache.position, inference_params=cache.inference_params).logits[:, -1]
         if vocab_size is not None:
             logits = logits[..., :vocab_size]
-        if cache.scores is not None:
-            cache.scores.index_copy_(0, cache.score_index, logits)
-            cache.score_index.add_(1)
-        next_token = logits.argmax(dim=-1, keepdim=True)
-        cache.token.copy_(next_token)
-        cache.sequences.index_copy_(1, cache.out_index, next_token)
-        cache.position.add_(1)
-        cache.seq_pos.add_(1)
-        cache.out_index.add_(1)
+        ops.greedy_advance(logits[0].contiguous(), cache.token, cache.position, cache.seq_pos, cache.sequences,
+                           cache.out_index, cache.scores, cache.score_index)
 
     @torch.no_grad()
     def generate(self, input_ids, max_length, top_k=1, top_p=0.0, temperature=1.0, fused_ft_kernel=True, cg=False,

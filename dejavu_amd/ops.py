@@ -143,6 +143,25 @@ def topk_indices(logits: torch.Tensor, k: int, dtype: torch.dtype = torch.int64,
     return out
 
 
+def greedy_advance(logits: torch.Tensor, token: torch.Tensor, position: torch.Tensor, seq_pos: torch.Tensor,
+                   sequences: torch.Tensor, out_index: torch.Tensor, scores: Optional[torch.Tensor] = None,
+                   score_index: Optional[torch.Tensor] = None) -> None:
+    """Greedy step of a batch-1 generation loop, in one launch and entirely on the device:
+    ``token <- argmax(logits)`` (first index among equal values), ``sequences[0, out_index++] <-
+    token``, ``position++``, ``seq_pos++``, and with ``scores`` the logits row is kept at
+    ``scores[score_index++]``."""
+    _require_device(logits, token, position, seq_pos, sequences, out_index, scores, score_index)
+    assert logits.dtype == torch.float16 and logits.dim() == 1 and logits.is_contiguous()
+    assert token.dtype == position.dtype == out_index.dtype == sequences.dtype == torch.int64
+    assert seq_pos.dtype == torch.int32 and sequences.is_contiguous()
+    if scores is not None:
+        assert scores.dtype == torch.float16 and scores.stride(-1) == 1 and score_index.dtype == torch.int64
+    check(lib.dv_greedy_advance_f16(_ptr(logits), logits.numel(), _ptr(token), _ptr(position), _ptr(seq_pos),
+                                    _ptr(sequences), _ptr(out_index), _ptr(scores),
+                                    0 if scores is None else scores.stride(0), _ptr(score_index), _stream()),
+          "dv_greedy_advance_f16")
+
+
 # ---------------------------------------------------------------------------
 # sparse MLP
 # ---------------------------------------------------------------------------

@@ -270,6 +270,21 @@ DV_API int dv_add_layer_norm_f16(const void* h, const void* residual, const void
                                  void* residual_out, void* stream);
 
 /*
+ * Greedy step of the generation loop (batch 1): next = argmax(logits[0 .. vocab)), first index
+ * among equal values; then, all on the device so that a captured step can be replayed:
+ * token[0] = next, sequences[out_index[0]++] = next, position[0]++, seq_pos[0]++ and, with
+ * scores != NULL, scores[score_index[0]++, :vocab] = logits (rows of score_ld elements).
+ * Replaces the sampling step of the greedy loop the reference takes from flash-attention v0.2.8
+ * utils/generation.py (decode(): `sample(logits, top_k=1)` + sequence / length bookkeeping;
+ * call site Dejavu/benchmarks/benchmark_generation_opt_dejavu.py:187-196).
+ *   logits fp16; token, position, out_index, score_index int64[1]; seq_pos int32[1];
+ *   sequences int64 (row of the output); scores fp16 or NULL.
+ */
+DV_API int dv_greedy_advance_f16(const void* logits, int vocab, void* token, void* position,
+                                 void* seq_pos, void* sequences, void* out_index, void* scores,
+                                 int64_t score_ld, void* score_index, void* stream);
+
+/*
  * One decode step (batch 1, one new token) of a whole sparse block in eight
  * launches: add+LayerNorm 1, back-fill window step, QKV of the active heads with
  * cache scatter, attention, out_proj, add+LayerNorm 2, the sparse MLP, and beside

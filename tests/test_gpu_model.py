@@ -144,3 +144,46 @@ def test_graph_replayed_generation_equals_eager_bit_for_bit():
     e3 = model.generate(prompt3, max_length=5 + n_new, return_dict_in_generate=True, output_scores=True)
     torch.cuda.synchronize()
     assert torch.equal(g3.sequences, e3.sequences)
+
+
+@pytest.mark.parametrize("vocab", [7, 512, 50272])
+def test_greedy_advance_matches_torch_argmax_and_bookkeeping(vocab):
+    """The fused greedy step: first index among equal maxima (as torch.argmax), NaN on top, and the
+    device-side counters / sequence / score rows advanced exactly once."""
+    from dejavu_amd import ops
+
+    g = torch.Generator().manual_seed(vocab)
+    cases = {
+        "random": torch.randn(vocab, generator=g),
+        "ties": torch.randint(0, 3, (vocab,), generator=g).float(),
+        "all_equal": torch.full((vocab,), -2.5),
+        "signed_zero": torch.where(torch.rand(vocab, generator=g) < 0.5, torch.tensor(0.0), torch.tensor(-0.0)) - 0.0,
+    }
+    cases["nan"] = cases["random"].clone()
+    cases["nan"][vocab // 2] = float("nan")
+    max_len = 8
+    for name, lg in cases.items():
+        print(f"case greedy advance vocab={vocab} {name}", flush=True)
+        logits = lg.half().cuda()
+        token = torch.zeros(1, 1, dtype=torch.long, device="cuda")
+        position = torch.full((1, 1), 11, dtype=torch.long, device="cuda")
+        seq_pos = torch.full((1,), 11, dtype=torch.int32, device="cuda")
+        out_index = torch.full((1,), 3, dtype=torch.long, device="cuda")
+        score_index = torch.full((1,), 2, dtype=torch.long, device="cuda")
+        sequences = torch.full((1, max_len), -1, dtype=torch.long, device="cuda")
+        scores = torch.zeros(max_len, vocab, dtype=torch.float16, device="cuda")
+        ops.greedy_advance(logits, token, position, seq_pos, sequences, out_index, scores, score_index)
+        torch.cuda.synchronize()
+        if name == "nan":
+            want = vocab // 2
+        else:
+            want = int(torch.argmax(logits.float().cpu()))
+            assert float(logits[want]) == float(logits.float().max()) and not bool((logits[:want] == logits[want]).any())
+        assert int(token) == want and int(sequences[0, 3]) == want
+        assert sequences[0].tolist().count(-1) == max_len - 1
+        assert int(position) == 12 and int(seq_pos) == 12 and int(out_index) == 4 and int(score_index) == 3
+        assert torch.equal(scores[2].view(torch.int16), logits.view(torch.int16)) and not scores[3].any()
+        # without scores: the score arguments stay untouched
+        ops.greedy_advance(logits, token, position, seq_pos, sequences, out_index)
+        torch.cuda.synchronize()
+        assert int(out_index) == 5 and int(sequences[0, 4]) == want and int(score_index) == 3
