@@ -150,23 +150,20 @@ ColsPlan plan_cols(int N, int M) {
   return p;
 }
 
-// Workspace layout: 4 KiB that no kernel writes (they stay zero; reserved for per-tile
-// counters at a place that does not depend on the shape), then the fp32 partial sums.
-constexpr size_t kCounterBytes = 4096;
-constexpr int kMaxColTiles = (int)(kCounterBytes / sizeof(unsigned));
-
+// Workspace: the fp32 partial sums of the row groups, (groups, B, N).  Every word a call reads
+// it has written first, so the memory needs no initialisation.
 size_t cols_workspace_bytes(int B, int N, int M) {
   const ColsPlan p = plan_cols(N, M);
-  return kCounterBytes + (size_t)p.groups * B * N * sizeof(float);
+  return (size_t)p.groups * B * N * sizeof(float);
 }
 
 template <int B, bool IDX64, bool BLOCKED>
 void launch_cols(const ColsPlan& p, const half_t* x, int64_t ldx, int x_expanded, const half_t* W,
                  int64_t ldw, const half_t* bias, const void* idx, int blk, int N, int Z, int M,
-                 float* partial, unsigned* counters, half_t* y, hipStream_t s) {
+                 float* partial, half_t* y, hipStream_t s) {
   dim3 grid(p.col_tiles, p.groups);
   hipLaunchKernelGGL((gather_cols_kernel<B, 8, IDX64, BLOCKED>), grid, dim3(256), 0, s, x, ldx, x_expanded, W, ldw,
-                     bias, idx, blk, N, Z, M, p.rows_per_block, partial, counters, y);
+                     bias, idx, blk, N, Z, M, p.rows_per_block, partial, y);
   if (p.groups > 1) {
     const int64_t total = (int64_t)B * N;
     hipLaunchKernelGGL(cols_reduce_kernel, dim3((unsigned)((total + 63) / 64)), dim3(256), 0, s,
@@ -180,11 +177,8 @@ int gather_cols(const half_t* x, int64_t ldx, int x_expanded, const half_t* W, i
   const ColsPlan p = plan_cols(N, M);
   if (workspace == nullptr || workspace_bytes < cols_workspace_bytes(B, N, M))
     return DV_ERR_WORKSPACE;
-  if (p.col_tiles > kMaxColTiles) return DV_ERR_UNSUPPORTED;
-  unsigned* counters = reinterpret_cast<unsigned*>(workspace);
-  float* partial =
-      reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(workspace) + kCounterBytes);
-#define DV_ARGS p, x, ldx, x_expanded, W, ldw, bias, idx, blk, N, Z, M, partial, counters, y, s
+  float* partial = reinterpret_cast<float*>(workspace);
+#define DV_ARGS p, x, ldx, x_expanded, W, ldw, bias, idx, blk, N, Z, M, partial, y, s
 #define DV_CASE(BB)                                                   \
   case BB:                                                            \
     if (blk == 1) {                                                   \
@@ -272,8 +266,7 @@ RowsSplitPlan plan_rows_split(int N, int M) {
 
 size_t rows_split_workspace_bytes(int B, int N, int M) {
   const RowsSplitPlan p = plan_rows_split(N, M);
-  // behind the completion counters other users of a shared workspace keep at its start
-  return p.nsplit > 1 ? kCounterBytes + (size_t)p.nsplit * B * M * sizeof(float) : 0;
+  return p.nsplit > 1 ? (size_t)p.nsplit * B * M * sizeof(float) : 0;
 }
 
 // dense (no gather, bias or activation) product through the split kernel; falls back to the
@@ -284,7 +277,7 @@ int rows_mfma_dense(const half_t* x, const half_t* W, int64_t ldw, int B, int N,
   if (p.nsplit <= 1 || workspace == nullptr || workspace_bytes < rows_split_workspace_bytes(B, N, M) ||
       !aligned16(workspace))
     return gather_rows_mfma(x, W, ldw, nullptr, nullptr, 4, B, N, M, M, DV_ACT_ID, y, s);
-  float* partial = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(workspace) + kCounterBytes);
+  float* partial = reinterpret_cast<float*>(workspace);
   const int ntiles = (M + kMfmaRows - 1) / kMfmaRows;
   const dim3 grid(ntiles, p.nsplit);
   const size_t tile_bytes = (size_t)kMfmaWaves * kMfmaRows * kMfmaLdsRow * sizeof(half_t);
@@ -383,7 +376,7 @@ ColsMfmaPlan plan_cols_mfma(int B, int N, int M) {
 
 size_t cols_mfma_workspace_bytes(int B, int N, int M) {
   const ColsMfmaPlan p = plan_cols_mfma(B, N, M);
-  return kCounterBytes + (size_t)p.groups * B * N * sizeof(float);
+  return (size_t)p.groups * B * N * sizeof(float);
 }
 
 template <int BT, bool IDX64, bool BLOCKED, bool HVEC>
@@ -404,7 +397,7 @@ int gather_cols_mfma(const half_t* h, int64_t ldh, int x_expanded, const half_t*
                      half_t* y, void* workspace, size_t workspace_bytes, hipStream_t s) {
   const ColsMfmaPlan p = plan_cols_mfma(B, N, M);
   if (workspace == nullptr || workspace_bytes < cols_mfma_workspace_bytes(B, N, M)) return DV_ERR_WORKSPACE;
-  float* partial = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(workspace) + kCounterBytes);
+  float* partial = reinterpret_cast<float*>(workspace);
   const bool i64 = idx_bytes == 8, blocked = blk != 1;
   const bool hvec = M % 8 == 0 && ldh % 8 == 0 && aligned16(h) && (!x_expanded || blk % 8 == 0);
 #define DV_ARGS p, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M, partial, y, s
@@ -555,10 +548,9 @@ int dv_predictor_logits_f16(const void* x, const void* Wa, int64_t ldwa, const v
 
 }  // extern "C"
 namespace {
-// bytes of histograms, threshold and per-workgroup counts; the batch-maximum row follows
-size_t topk_max_row_offset(int n) {
-  const int blocks = (n + kTopkItemsPerBlock - 1) / kTopkItemsPerBlock;
-  return ((size_t)(kTopkCountsOff + 2 * blocks) * sizeof(unsigned) + 15) & ~(size_t)15;
+// bytes of the per-workgroup histograms and counts; the batch-maximum row follows
+size_t topk_max_row_offset(int) {
+  return ((size_t)kTopkWords * sizeof(unsigned) + 15) & ~(size_t)15;
 }
 }  // namespace
 extern "C" {
@@ -594,7 +586,7 @@ int dv_topk_f16(const void* logits, int B, int n, int k, void* idx_out, int idx_
   }
   hipLaunchKernelGGL(topk_hist_kernel, dim3(blocks), dim3(256), 0, s, lg, B, n, ws);
   hipLaunchKernelGGL(topk_count_kernel, dim3(blocks), dim3(256), 0, s, lg, B, n, k, ws);
-  hipLaunchKernelGGL(topk_emit_kernel, dim3(blocks), dim3(256), 0, s, lg, B, n, ws, idx_out, idx_bytes);
+  hipLaunchKernelGGL(topk_emit_kernel, dim3(blocks), dim3(256), 0, s, lg, B, n, k, ws, idx_out, idx_bytes);
   return launch_status();
 }
 
@@ -869,7 +861,7 @@ int dv_attention_out_proj_f16(const void* q, int64_t ldq, const void* k_cache, c
       workspace_bytes < dv_attention_out_proj_workspace_bytes(B, nheads, n_len, hd, N))
     return DV_ERR_WORKSPACE;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  // layout: [counters + out_proj partial sums][attention partials]
+  // layout: [out_proj partial sums][attention partials]
   const size_t cols_bytes = (cols_workspace_bytes(B, N, nheads * hd) + 255) & ~(size_t)255;
   unsigned char* base = reinterpret_cast<unsigned char*>(workspace);
   float* part = reinterpret_cast<float*>(base + cols_bytes);
@@ -880,9 +872,7 @@ int dv_attention_out_proj_f16(const void* q, int64_t ldq, const void* k_cache, c
   }
   const int M = nheads * hd;
   const ColsPlan p = plan_cols(N, M);
-  if (p.col_tiles > kMaxColTiles) return DV_ERR_UNSUPPORTED;
-  unsigned* counters = reinterpret_cast<unsigned*>(base);
-  float* partial = reinterpret_cast<float*>(base + kCounterBytes);
+  float* partial = reinterpret_cast<float*>(base);
   const half_t* ww = reinterpret_cast<const half_t*>(Wt);
   const half_t* bb = reinterpret_cast<const half_t*>(bias);
   half_t* yy = reinterpret_cast<half_t*>(y);
@@ -891,7 +881,7 @@ int dv_attention_out_proj_f16(const void* q, int64_t ldq, const void* k_cache, c
 #define DV_AO(BB)                                                                                 \
   hipLaunchKernelGGL((gather_cols_kernel<BB, 8, false, true, true>), grid, dim3(256), 0, s, \
                      (const half_t*)nullptr, (int64_t)0, 1, ww, ldw, bb, head_idx, hd, N, H * hd, M, \
-                     p.rows_per_block, partial, counters, yy, part, nsplit)
+                     p.rows_per_block, partial, yy, part, nsplit)
   switch (B) {
     case 1: DV_AO(1); break;
     case 2: DV_AO(2); break;
@@ -997,7 +987,7 @@ inline size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 LayerPlan plan_layer(const dvSparseLayerArgs& a) {
   LayerPlan p;
   size_t o = 0;
-  p.off_topk = o;  // zero-initialised region first
+  p.off_topk = o;
   o = align_up(o + dv_topk_workspace_bytes(a.ffn > 1024 ? a.ffn : 2048));
   p.off_x = o;            o = align_up(o + (size_t)a.d * 2);
   p.off_res1 = o;         o = align_up(o + (size_t)a.d * 2);
@@ -1133,7 +1123,8 @@ int dv_sparse_layer_decode_f16(const dvSparseLayerArgs* args, void* stream) {
     const int nh1 = ((a.H + rw1 - 1) / rw1 + 3) / 4;
     const int no = c.col_tiles * c.groups;
     hipLaunchKernelGGL(layer_l4_kernel, dim3(no + nh1 + topk_blocks), dim3(256), 0, s, o, no, hp1, nh1,
-                       CH(a.mlp_logit_in), a.ffn, topk_ws, reinterpret_cast<int64_t*>(a.mlp_idx_out), topk_blocks);
+                       CH(a.mlp_logit_in), a.ffn, a.K, topk_ws, reinterpret_cast<int64_t*>(a.mlp_idx_out),
+                       topk_blocks);
     // L5: split reduction + bias, and the residual stream advanced by the attention output
     hipLaunchKernelGGL(cols_reduce_kernel, dim3((unsigned)((a.d + 63) / 64)), dim3(256), 0, s,
                        c.groups > 1 ? cols_part : nullptr, CH(a.bout), c.groups, 1, a.d, attn_out, res1,

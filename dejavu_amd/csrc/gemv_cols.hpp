@@ -25,7 +25,7 @@ template <int B, int U, bool IDX64, bool BLOCKED, bool ATTN>
 __device__ __forceinline__ void gather_cols_body(
     const half_t* __restrict__ X, int64_t ldx, int x_expanded, const half_t* __restrict__ W,
     int64_t ldw, const half_t* __restrict__ bias, const void* __restrict__ idx, int blk, int N,
-    int Z, int M, int rows_per_block, float* __restrict__ partial, unsigned* __restrict__ counters,
+    int Z, int M, int rows_per_block, float* __restrict__ partial,
     half_t* __restrict__ Y, const float* __restrict__ attn_part, int attn_nsplit, int ct, int g,
     int G) {
   __shared__ float red[4][B][kColTile];
@@ -221,10 +221,10 @@ template <int B, int U, bool IDX64, bool BLOCKED, bool ATTN = false>
 __global__ __launch_bounds__(256) void gather_cols_kernel(
     const half_t* __restrict__ X, int64_t ldx, int x_expanded, const half_t* __restrict__ W,
     int64_t ldw, const half_t* __restrict__ bias, const void* __restrict__ idx, int blk, int N,
-    int Z, int M, int rows_per_block, float* __restrict__ partial, unsigned* __restrict__ counters,
+    int Z, int M, int rows_per_block, float* __restrict__ partial,
     half_t* __restrict__ Y, const float* __restrict__ attn_part = nullptr, int attn_nsplit = 0) {
   gather_cols_body<B, U, IDX64, BLOCKED, ATTN>(X, ldx, x_expanded, W, ldw, bias, idx, blk, N, Z, M,
-                                                     rows_per_block, partial, counters, Y, attn_part,
+                                                     rows_per_block, partial, Y, attn_part,
                                                      attn_nsplit, blockIdx.x, blockIdx.y, gridDim.y);
 }
 

@@ -112,16 +112,22 @@ template <int HD>
 __global__ __launch_bounds__(256) void layer_l3_kernel(AttnArgs a, int nblk_attn, CanonArgs hp0, int nblk_hp0,
                                                        const half_t* __restrict__ mlp_logits, int ffn,
                                                        int K, unsigned* __restrict__ topk_ws) {
-  const int bid = blockIdx.x;
-  if (bid < nblk_attn) {
-    const int split = bid % a.nsplit, i = bid / a.nsplit;
-    decode_attn_body<HD, 4>(a.Q, a.ldq, a.k_cache, a.v_cache, a.head_idx, a.seq_pos, a.n_len, a.H, a.S, a.scale,
-                            a.nsplit, a.part, split, i, 0, a.nheads);
-  } else if (bid < nblk_attn + nblk_hp0) {
-    canonical_role(hp0, bid - nblk_attn, nblk_hp0);
-  } else {
-    topk_count_body(mlp_logits, 1, ffn, K, topk_ws, bid - nblk_attn - nblk_hp0);
+  // the small roles with the longer dependency chains take the first block ids: they are dispatched first
+  const int nblk_count = (int)gridDim.x - nblk_attn - nblk_hp0;
+  int bid = blockIdx.x;
+  if (bid < nblk_count) {
+    topk_count_body(mlp_logits, 1, ffn, K, topk_ws, bid, nblk_count);
+    return;
   }
+  bid -= nblk_count;
+  if (bid < nblk_hp0) {
+    canonical_role(hp0, bid, nblk_hp0);
+    return;
+  }
+  bid -= nblk_hp0;
+  const int split = bid % a.nsplit, i = bid / a.nsplit;
+  decode_attn_body<HD, 4>(a.Q, a.ldq, a.k_cache, a.v_cache, a.head_idx, a.seq_pos, a.n_len, a.H, a.S, a.scale,
+                          a.nsplit, a.part, split, i, 0, a.nheads);
 }
 
 // ---- L4 -------------------------------------------------------------------
@@ -139,19 +145,23 @@ struct OutProjArgs {
 
 __global__ __launch_bounds__(256) void layer_l4_kernel(OutProjArgs o, int nblk_out, CanonArgs hp1, int nblk_hp1,
                                                        const half_t* __restrict__ mlp_logits, int ffn,
-                                                       unsigned* __restrict__ topk_ws,
+                                                       int K, const unsigned* __restrict__ topk_ws,
                                                        int64_t* __restrict__ mlp_idx_out, int nblk_emit) {
-  const int bid = blockIdx.x;
-  if (bid < nblk_out) {
-    const int ct = bid % o.col_tiles, g = bid / o.col_tiles;
-    gather_cols_body<1, 8, false, true, true>(nullptr, 0, 1, o.W, o.ldw, o.bias, o.head_idx, o.hd, o.N,
-                                              o.Z, o.M, o.rows_per_block, o.partial, nullptr, o.Y,
-                                              o.attn_part, o.nsplit, ct, g, o.groups);
-  } else if (bid < nblk_out + nblk_hp1) {
-    canonical_role(hp1, bid - nblk_out, nblk_hp1);
-  } else {
-    topk_emit_body(mlp_logits, 1, ffn, topk_ws, mlp_idx_out, 8, bid - nblk_out - nblk_hp1, nblk_emit);
+  int bid = blockIdx.x;
+  if (bid < nblk_emit) {
+    topk_emit_body(mlp_logits, 1, ffn, K, topk_ws, mlp_idx_out, 8, bid, nblk_emit);
+    return;
   }
+  bid -= nblk_emit;
+  if (bid < nblk_hp1) {
+    canonical_role(hp1, bid, nblk_hp1);
+    return;
+  }
+  bid -= nblk_hp1;
+  const int ct = bid % o.col_tiles, g = bid / o.col_tiles;
+  gather_cols_body<1, 8, false, true, true>(nullptr, 0, 1, o.W, o.ldw, o.bias, o.head_idx, o.hd, o.N,
+                                            o.Z, o.M, o.rows_per_block, o.partial, o.Y,
+                                            o.attn_part, o.nsplit, ct, g, o.groups);
 }
 
 // ---- L7 / L8 --------------------------------------------------------------
@@ -209,8 +219,8 @@ __global__ __launch_bounds__(256) void layer_l8_kernel(ColsArgs c, int nblk_fc2,
   if (bid < nblk_fc2) {
     const int ct = bid % c.col_tiles, g = bid / c.col_tiles;
     gather_cols_body<1, 8, true, false, false>(c.X, c.M, 0, c.W, c.ldw, c.bias, c.idx, 1, c.N, c.Z, c.M,
-                                                      c.rows_per_block, c.partial, nullptr, c.Y, nullptr, 0, ct,
-                                                      g, c.groups);
+                                               c.rows_per_block, c.partial, c.Y, nullptr, 0, ct, g,
+                                               c.groups);
   } else {
     canonical_role(mp1, bid - nblk_fc2, nblk_mp1);
   }

@@ -203,24 +203,30 @@ __global__ __launch_bounds__(256) void topk_small_kernel(const half_t* __restric
 }
 
 // ---------------------------------------------------------------------------
-// Large inputs: three launches, every one spread over many workgroups.
-//  1) topk_hist_kernel: fine[key] += 1 (65536 bins) and coarse[key >> 8] += 1
-//     (256 bins) for every column's key.  Integer atomics: order-independent.
-//  2) topk_count_kernel: every workgroup reads the threshold key T (largest T
-//     with count(key >= T) >= k) off the two histograms -- 256 coarse bins, then
-//     the 256 fine bins of the crossing coarse bin -- and counts its own columns
-//     above / at T.  Workgroup 0 also publishes T and the number of ties to take.
-//  3) topk_emit_kernel: every workgroup sums the counts of the workgroups before
-//     it, emits its indices with key > T and those of the first `need` columns
-//     with key == T (ascending, exact positions), and clears its slice of the
-//     histograms for the next call.
-// Workspace layout (u32): fine[65536] coarse[256] meta[2] = {T, need} counts[2*WG], then (16-byte
-// aligned) n fp16 values: the column-wise maximum of a batch (topk_batch_max_kernel).
+// Large inputs: three launches, every one spread over many workgroups (2048 columns each,
+// at most kTopkMaxBlocks of them).  No global atomics and no state between calls: every
+// workgroup publishes small per-workgroup histograms that the next launch adds up.
+//  1) topk_hist_kernel: coarse histogram (key >> 8, 256 bins) of the workgroup's columns,
+//     built in LDS, stored to wc[workgroup][256].
+//  2) topk_count_kernel: every workgroup adds the coarse histograms, finds the coarse bin c*
+//     in which the k-th largest key lies, and stores the fine histogram (key & 255) of ITS
+//     columns inside c* to wf[workgroup][256] plus the number of its columns in higher bins.
+//  3) topk_emit_kernel: every workgroup adds the fine histograms, which gives the threshold
+//     key T and the number of ties to take; from the per-workgroup histograms of the
+//     workgroups before it, it knows how many selected columns precede its own and emits its
+//     indices with key > T and those of the first `need` columns with key == T at their exact
+//     (ascending) positions.
+// Workspace layout (u32): wc[32][256], wf[32][256], above[32], meta[4] = {c*, columns above c*},
+// then (16-byte aligned) n fp16 values: the column-wise maximum of a batch
+// (topk_batch_max_kernel).
 // ---------------------------------------------------------------------------
 constexpr int kTopkItemsPerBlock = 256 * 8;
-constexpr int kTopkFine = 65536, kTopkCoarse = 256;
-constexpr int kTopkMetaOff = kTopkFine + kTopkCoarse;
-constexpr int kTopkCountsOff = kTopkMetaOff + 2;
+constexpr int kTopkBins = 256;
+constexpr int kTopkMaxBlocks = 32;  // n <= 65536
+constexpr int kTopkFineOff = kTopkMaxBlocks * kTopkBins;
+constexpr int kTopkAboveOff = 2 * kTopkMaxBlocks * kTopkBins;
+constexpr int kTopkMetaOff = kTopkAboveOff + kTopkMaxBlocks;
+constexpr int kTopkWords = kTopkMetaOff + 4;
 
 __device__ __forceinline__ void topk_load_keys(const half_t* __restrict__ logits, int B, int n, int i0,
                                                unsigned key[8]) {
@@ -285,30 +291,21 @@ __global__ __launch_bounds__(256) void topk_batch_max_kernel(const half_t* __res
 }
 
 // A workgroup covers 256 * 8 columns with its first 256 threads (further threads, if the launch
-// has them, only take part in the barriers): spreading the atomics over many compute units
-// matters more than filling the workgroup.
+// has them, only take part in the barriers).
 __device__ __forceinline__ void topk_hist_body(const half_t* __restrict__ logits, int B, int n,
                                                unsigned* __restrict__ ws, int block_id) {
-  // the 256 coarse bins are hot (most logits share a few exponents): aggregate them in
-  // LDS and add each non-empty bin to memory once per workgroup
-  __shared__ unsigned s_coarse[kTopkCoarse];
-  if (threadIdx.x < kTopkCoarse) s_coarse[threadIdx.x] = 0u;
+  __shared__ unsigned s_coarse[kTopkBins];
+  if (threadIdx.x < kTopkBins) s_coarse[threadIdx.x] = 0u;
   __syncthreads();
   const int i0 = (block_id * 256 + threadIdx.x) * 8;
   if (threadIdx.x < 256 && i0 < n) {
     unsigned key[8];
     topk_load_keys(logits, B, n, i0, key);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      atomicAdd(&ws[key[e]], 1u);
-      atomicAdd(&s_coarse[key[e] >> 8], 1u);
-    }
+    for (int e = 0; e < 8; ++e) atomicAdd(&s_coarse[key[e] >> 8], 1u);
   }
   __syncthreads();
-  if (threadIdx.x < kTopkCoarse) {
-    const unsigned c = s_coarse[threadIdx.x];
-    if (c != 0u) atomicAdd(&ws[kTopkFine + threadIdx.x], c);
-  }
+  if (threadIdx.x < kTopkBins) ws[block_id * kTopkBins + threadIdx.x] = s_coarse[threadIdx.x];
 }
 
 __global__ __launch_bounds__(256) void topk_hist_kernel(const half_t* __restrict__ logits, int B, int n,
@@ -331,91 +328,111 @@ __device__ __forceinline__ unsigned block256_inclusive_scan(unsigned v, unsigned
   return v;
 }
 
-// Threshold from the histograms; all 256 threads return the same (T, above).
-__device__ __forceinline__ void topk_find_threshold(const unsigned* __restrict__ ws, unsigned k,
-                                                    unsigned* s_w, unsigned* s_pair, unsigned& T,
-                                                    unsigned& above) {
-  const int t = threadIdx.x;
-  // coarse bins in descending key order: thread t owns bin 255 - t
-  const unsigned c = ws[kTopkFine + 255 - t];
-  const unsigned cinc = block256_inclusive_scan(c, s_w);
-  if (cinc - c < k && cinc >= k) {
-    s_pair[0] = 255u - t;  // crossing coarse bin
-    s_pair[1] = cinc - c;  // columns in higher coarse bins
+// In a 256-bin histogram given in DESCENDING bin order over the threads (thread t owns bin
+// 255 - t, count c): the bin in which the k-th largest element lies and the number of elements
+// in higher bins.  All threads return the same pair.
+__device__ __forceinline__ void topk_crossing_bin(unsigned c, unsigned k, unsigned* s_w, unsigned* s_pair,
+                                                  unsigned& bin, unsigned& above) {
+  const unsigned inc = block256_inclusive_scan(c, s_w);
+  if (inc - c < k && inc >= k) {
+    s_pair[0] = 255u - threadIdx.x;
+    s_pair[1] = inc - c;
   }
   __syncthreads();
-  const unsigned cstar = s_pair[0], above_c = s_pair[1];
-  const unsigned f = ws[cstar * 256 + 255 - t];
-  const unsigned finc = block256_inclusive_scan(f, s_w);
-  const unsigned k2 = k - above_c;
-  if (finc - f < k2 && finc >= k2) {
-    s_pair[2] = cstar * 256 + 255 - t;
-    s_pair[3] = above_c + finc - f;
-  }
-  __syncthreads();
-  T = s_pair[2];
-  above = s_pair[3];
+  bin = s_pair[0];
+  above = s_pair[1];
 }
 
+// 256 threads; nblocks = workgroups of the histogram launch = of this one.
 __device__ __forceinline__ void topk_count_body(const half_t* __restrict__ logits, int B, int n, int k,
-                                                unsigned* __restrict__ ws, int block_id) {
-  __shared__ unsigned s_w[4], s_pair[4], s_gt[4], s_eq[4];
+                                                unsigned* __restrict__ ws, int block_id, int nblocks) {
+  __shared__ unsigned s_w[4], s_pair[2], s_fine[kTopkBins], s_gt[4];
   unsigned key[8];
-  const int i0 = (block_id * 256 + threadIdx.x) * 8;
+  const int t = threadIdx.x;
+  const int i0 = (block_id * 256 + t) * 8;
   topk_load_keys(logits, B, n, i0, key);  // issued before the histogram reads
-  unsigned T, above;
-  topk_find_threshold(ws, (unsigned)k, s_w, s_pair, T, above);
-  unsigned gt = 0, eq = 0;
+  // all (at most 32) per-workgroup values of this thread's bin are requested at once: one round
+  // trip instead of one per group of workgroups (clamped addresses, masked sums)
+  unsigned c = 0;
+  {
+    unsigned v[kTopkMaxBlocks];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    gt += key[e] > T;
-    eq += key[e] == T;
+    for (int w = 0; w < kTopkMaxBlocks; ++w) v[w] = ws[(w < nblocks ? w : nblocks - 1) * kTopkBins + 255 - t];
+#pragma unroll
+    for (int w = 0; w < kTopkMaxBlocks; ++w) c += w < nblocks ? v[w] : 0u;
+  }
+  s_fine[t] = 0u;
+  unsigned cstar, above_c;
+  topk_crossing_bin(c, (unsigned)k, s_w, s_pair, cstar, above_c);  // (its barriers also cover s_fine)
+  unsigned gt = 0;
+  if (i0 < n) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const unsigned cb = key[e] >> 8;
+      gt += cb > cstar;
+      if (cb == cstar) atomicAdd(&s_fine[key[e] & 255u], 1u);
+    }
   }
 #pragma unroll
-  for (int off = kWave / 2; off >= 1; off >>= 1) {
-    gt += __shfl_xor(gt, off, kWave);
-    eq += __shfl_xor(eq, off, kWave);
-  }
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  if (lane == 0) {
-    s_gt[wave] = gt;
-    s_eq[wave] = eq;
-  }
+  for (int off = kWave / 2; off >= 1; off >>= 1) gt += __shfl_xor(gt, off, kWave);
+  if ((t & 63) == 0) s_gt[t >> 6] = gt;
   __syncthreads();
-  if (threadIdx.x == 0) {
-    ws[kTopkCountsOff + 2 * block_id] = s_gt[0] + s_gt[1] + s_gt[2] + s_gt[3];
-    ws[kTopkCountsOff + 2 * block_id + 1] = s_eq[0] + s_eq[1] + s_eq[2] + s_eq[3];
+  ws[kTopkFineOff + block_id * kTopkBins + t] = s_fine[t];
+  if (t == 0) {
+    ws[kTopkAboveOff + block_id] = s_gt[0] + s_gt[1] + s_gt[2] + s_gt[3];
     if (block_id == 0) {
-      ws[kTopkMetaOff] = T;
-      ws[kTopkMetaOff + 1] = (unsigned)k - above;  // ties to take, lowest index first
+      ws[kTopkMetaOff] = cstar;
+      ws[kTopkMetaOff + 1] = above_c;
     }
   }
 }
 
 __global__ __launch_bounds__(256) void topk_count_kernel(const half_t* __restrict__ logits, int B, int n,
                                                          int k, unsigned* __restrict__ ws) {
-  topk_count_body(logits, B, n, k, ws, blockIdx.x);
+  topk_count_body(logits, B, n, k, ws, blockIdx.x, gridDim.x);
 }
 
-__device__ __forceinline__ void topk_emit_body(const half_t* __restrict__ logits, int B, int n,
-                                               unsigned* __restrict__ ws, void* __restrict__ idx_out,
+__device__ __forceinline__ void topk_emit_body(const half_t* __restrict__ logits, int B, int n, int k,
+                                               const unsigned* __restrict__ ws, void* __restrict__ idx_out,
                                                int idx_bytes, int block_id, int nblocks) {
-  __shared__ unsigned s_w[4], s_base[2];
+  __shared__ unsigned s_w[4], s_pair[2], s_base[2];
   unsigned key[8];
-  const int i0 = (block_id * 256 + threadIdx.x) * 8;
+  const int t = threadIdx.x;
+  const int i0 = (block_id * 256 + t) * 8;
   topk_load_keys(logits, B, n, i0, key);
-  const unsigned T = ws[kTopkMetaOff], need = ws[kTopkMetaOff + 1];
-  // columns above / at T in the workgroups before this one
-  if (threadIdx.x < 2) {
-    unsigned acc = 0;
-    for (int w = 0; w < block_id; ++w) acc += ws[kTopkCountsOff + 2 * w + threadIdx.x];
-    s_base[threadIdx.x] = acc;
-  }
-  unsigned gt = 0, eq = 0;
+  const unsigned cstar = ws[kTopkMetaOff], above_c = ws[kTopkMetaOff + 1];
+  // fine bins of c* in descending order: thread t owns fine bin 255 - t; `mine` counts that bin in
+  // the workgroups before this one
+  unsigned f = 0, mine = 0;
+  {
+    unsigned v[kTopkMaxBlocks];  // one round trip, as in topk_count_body
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    gt += key[e] > T;
-    eq += key[e] == T;
+    for (int w = 0; w < kTopkMaxBlocks; ++w)
+      v[w] = ws[kTopkFineOff + (w < nblocks ? w : nblocks - 1) * kTopkBins + 255 - t];
+#pragma unroll
+    for (int w = 0; w < kTopkMaxBlocks; ++w) {
+      f += w < nblocks ? v[w] : 0u;
+      mine += w < block_id ? v[w] : 0u;
+    }
+  }
+  unsigned tlow, above_f;
+  topk_crossing_bin(f, (unsigned)k - above_c, s_w, s_pair, tlow, above_f);
+  const unsigned T = cstar * 256u + tlow;
+  const unsigned need = (unsigned)k - above_c - above_f;  // ties to take, lowest index first
+  // selected columns in the workgroups before this one: those in higher coarse bins, those in
+  // higher fine bins of c*, and the ties
+  unsigned gt_part = (255u - (unsigned)t > tlow) ? mine : 0u;
+  if (t < block_id) gt_part += ws[kTopkAboveOff + t];  // block_id <= 32 <= 256 threads
+  const unsigned gt_all = block256_inclusive_scan(gt_part, s_w);
+  if (t == 255) s_base[0] = gt_all;
+  if (255u - (unsigned)t == tlow) s_base[1] = mine;
+  unsigned gt = 0, eq = 0;
+  if (i0 < n) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      gt += key[e] > T;
+      eq += key[e] == T;
+    }
   }
   const unsigned gt_inc = block256_inclusive_scan(gt, s_w);
   const unsigned eq_inc = block256_inclusive_scan(eq, s_w);
@@ -424,30 +441,29 @@ __device__ __forceinline__ void topk_emit_body(const half_t* __restrict__ logits
   const unsigned eq_before = s_base[1] + eq_inc - eq;
   unsigned pos = gt_before + (eq_before < need ? eq_before : need);
   unsigned eq_rank = eq_before;
+  if (i0 < n) {
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    bool take = key[e] > T;
-    if (key[e] == T) {
-      take = eq_rank < need;
-      ++eq_rank;
-    }
-    if (take) {
-      if (idx_bytes == 8)
-        reinterpret_cast<int64_t*>(idx_out)[pos] = i0 + e;
-      else
-        reinterpret_cast<int32_t*>(idx_out)[pos] = i0 + e;
-      ++pos;
+    for (int e = 0; e < 8; ++e) {
+      bool take = key[e] > T;
+      if (key[e] == T) {
+        take = eq_rank < need;
+        ++eq_rank;
+      }
+      if (take) {
+        if (idx_bytes == 8)
+          reinterpret_cast<int64_t*>(idx_out)[pos] = i0 + e;
+        else
+          reinterpret_cast<int32_t*>(idx_out)[pos] = i0 + e;
+        ++pos;
+      }
     }
   }
-  // clear the histograms for the next call (nobody reads them in this kernel)
-  const int nthreads = nblocks * 256;
-  for (int j = block_id * 256 + threadIdx.x; j < kTopkFine + kTopkCoarse; j += nthreads) ws[j] = 0u;
 }
 
-__global__ __launch_bounds__(256) void topk_emit_kernel(const half_t* __restrict__ logits, int B, int n,
-                                                        unsigned* __restrict__ ws,
+__global__ __launch_bounds__(256) void topk_emit_kernel(const half_t* __restrict__ logits, int B, int n, int k,
+                                                        const unsigned* __restrict__ ws,
                                                         void* __restrict__ idx_out, int idx_bytes) {
-  topk_emit_body(logits, B, n, ws, idx_out, idx_bytes, blockIdx.x, gridDim.x);
+  topk_emit_body(logits, B, n, k, ws, idx_out, idx_bytes, blockIdx.x, gridDim.x);
 }
 
 // ---------------------------------------------------------------------------

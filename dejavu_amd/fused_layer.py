@@ -48,12 +48,11 @@ _workspaces: dict = {}
 
 
 def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
-    """Per-device scratch shared by all layers (they run one after the other); zero-filled
-    when (re)allocated, the kernels leave the parts that must be zero at zero."""
+    """Per-device scratch shared by all layers (they run one after the other)."""
     key = (device.type, device.index)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
-        ws = torch.zeros(nbytes, dtype=torch.uint8, device=device)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
 

@@ -43,18 +43,18 @@ def _require_device(*tensors: Optional[torch.Tensor]) -> None:
 
 
 # ---------------------------------------------------------------------------
-# workspace (fp32 partial sums of the split reductions behind 4 KiB kept at zero)
+# workspace (fp32 partial sums of the split reductions)
 # ---------------------------------------------------------------------------
 _workspaces: dict = {}
 
 
 def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
-    """Zero-initialised per-device scratch, grown on demand; only cleared when
-    (re)allocated.  Ops that share it must not run concurrently on different streams."""
+    """Per-device scratch, grown on demand (the kernels write every word before they read it).
+    Ops that share it must not run concurrently on different streams."""
     key = (device.type, device.index)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
-        ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
 
@@ -104,12 +104,11 @@ _topk_workspaces: dict = {}
 
 
 def _topk_workspace(device: torch.device) -> torch.Tensor:
-    """Zero-initialised histogram scratch per device; the kernels hand it back zeroed.
-    Top-k calls that share it must not overlap."""
+    """Histogram scratch per device.  Top-k calls that share it must not overlap."""
     key = (device.type, device.index)
     ws = _topk_workspaces.get(key)
     if ws is None:
-        ws = torch.zeros(lib.dv_topk_workspace_bytes(65536) // 4, dtype=torch.int32, device=device)
+        ws = torch.empty(lib.dv_topk_workspace_bytes(65536) // 4, dtype=torch.int32, device=device)
         _topk_workspaces[key] = ws
     return ws
 

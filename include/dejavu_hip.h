@@ -84,11 +84,12 @@ DV_API int dv_predictor_logits_ws_f16(const void* x, const void* Wa, int64_t ldw
  * Dejavu/src/models/modules/mha_dejavu.py:1069, 1369, 1506-1507.
  *   logits (B, n) fp16; idx_out (k,) int32/int64.  n <= 65536, 0 <= k <= n.
  * dv_topk_f16: n <= 1024 is ranked in one workgroup; larger n (n % 8 == 0)
- *   takes three launches spread over many workgroups: key histograms, the
- *   threshold read off them plus per-workgroup counts, then the ordered
- *   emission.  workspace: dv_topk_workspace_bytes(n) bytes, zero-filled before
- *   first use (the call leaves the histograms zeroed); calls sharing it must
- *   not overlap.
+ *   takes three launches spread over many workgroups: per-workgroup key
+ *   histograms, the threshold read off their sum plus per-workgroup counts,
+ *   then the ordered emission (no atomics on global memory: deterministic,
+ *   and no slower when many logits share a value).  workspace:
+ *   dv_topk_workspace_bytes(n) bytes, no initialisation needed; calls sharing
+ *   it must not overlap.
  * dv_topk_search_f16: same result in a single launch without scratch memory
  *   (16-step bitwise threshold search in one workgroup).
  */
@@ -118,8 +119,8 @@ DV_API int dv_gather_gemv_f16(const void* x, const void* W, int64_t ldw, const v
  * split over row groups instead of floating-point atomics).
  *   x (B, M); W (Z, N) row stride ldw; bias (N,) or NULL; idx (M,);
  *   y (B, N) fp16.  1 <= B <= 64 (vector ALUs up to 4, MFMA tiles above).
- *   workspace: dv_gather_transposed_gemv_workspace_bytes(B, N, M) bytes,
- *   zero-filled before its first use; calls sharing it must not overlap.
+ *   workspace: dv_gather_transposed_gemv_workspace_bytes(B, N, M) bytes, no
+ *   initialisation needed; calls sharing it must not overlap.
  */
 DV_API size_t dv_gather_transposed_gemv_workspace_bytes(int B, int N, int M);
 DV_API int dv_gather_transposed_gemv_f16(const void* x, const void* W, int64_t ldw, const void* bias,
@@ -246,8 +247,8 @@ DV_API int dv_out_proj_sparse_f16(const void* x, const void* W, const void* bias
  * ldw: the active heads become contiguous row blocks that stream like the fc2
  * gather (the reference does the same for fc2 with fc2_weight_t,
  * Dejavu/src/ops/fused_dense_sparse_dejavu.py:912-913).  Deterministic.
- *   workspace: dv_out_proj_sparse_t_workspace_bytes(...) bytes, zero-filled
- *   before first use (may be shared with dv_gather_transposed_gemv_f16).
+ *   workspace: dv_out_proj_sparse_t_workspace_bytes(...) bytes, no
+ *   initialisation needed (may be shared with dv_gather_transposed_gemv_f16).
  */
 DV_API size_t dv_out_proj_sparse_t_workspace_bytes(int B, int N, int nnz, int hd);
 DV_API int dv_out_proj_sparse_t_f16(const void* x, const void* Wt, int64_t ldw, const void* bias,
@@ -336,7 +337,7 @@ typedef struct dvSparseLayerArgs {
   void* mlp_logit_out;    /* (ffn,) logits for the NEXT layer's MLP                    */
   void* att_idx_out;      /* (att_k,) int32 heads for the NEXT layer                   */
   void* mlp_idx_out;      /* (K,) int64 neurons used by this layer                     */
-  /* scratch: dv_sparse_layer_workspace_bytes() bytes, zero-filled before first use */
+  /* scratch: dv_sparse_layer_workspace_bytes() bytes, no initialisation needed */
   void* workspace;
   size_t workspace_bytes;
 } dvSparseLayerArgs;

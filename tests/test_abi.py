@@ -54,7 +54,7 @@ def test_host_side_argument_checks_return_codes():
     assert L.dv_topk_f16(0x1000, 1, 1 << 20, 1, 0x1000, 8, None, 0, None) == -2  # n too large
     assert L.dv_topk_f16(0x1000, 1, 4096, 1, 0x1000, 8, None, 0, None) == -4  # histogram scratch missing
     assert L.dv_topk_search_f16(0x1000, 1, 8, 9, 0x1000, 8, None) == -1
-    assert L.dv_topk_workspace_bytes(96) == 0 and L.dv_topk_workspace_bytes(49152) > 65536 * 4
+    assert L.dv_topk_workspace_bytes(96) == 0 and L.dv_topk_workspace_bytes(49152) >= 2 * 32 * 256 * 4 + 49152 * 2
     assert L.dv_gather_gemv_f16(0x1000, 0x1000, 8, None, 0x1000, 8, 65, 8, 8, 1, 0, 0x1000, None) == -2  # B > 64
     assert L.dv_gather_gemv_f16(0x1000, 0x1000, 12, None, 0x1000, 8, 1, 12, 8, 1, 0, 0x1000, None) == -3  # N % 8
     assert L.dv_gather_transposed_gemv_f16(0x1000, 0x1000, 8, None, 0x1000, 8, 1, 8, 8, 4, 0x1000, None, 0, None) == -4

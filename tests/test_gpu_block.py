@@ -105,8 +105,12 @@ def test_sparse_block_decode_step_matches_oracle(d, ffn, H, r, K, Hk, S):
 def test_fused_layer_equals_module_by_module_path(d, H, ffn, r):
     """The eight-launch fused block step and the module-by-module path run the same kernel
     bodies: outputs, predictions, caches and window state must agree bit for bit over a
-    whole back-fill window (the flush step falls back to the modules in both)."""
+    whole back-fill window (the flush step falls back to the modules in both).  Every scratch
+    buffer is overwritten with 0xFF bytes (NaN as fp32) before each step: the kernels must not
+    depend on what a workspace holds when they start."""
     import copy
+
+    from dejavu_amd import fused_layer, ops
 
     from dejavu_amd.block import create_sparse_block, init_block_synthetic
     from dejavu_amd.modules import InferenceParams
@@ -139,6 +143,9 @@ def test_fused_layer_equals_module_by_module_path(d, H, ffn, r):
         head_idx = torch.sort(torch.randperm(H, generator=g)[:Hk]).values.int().cuda()
         logit = (torch.randn(ffn, generator=g) * 4).half().cuda()
         print(f"case fused vs modules d={d} step={step} counter={blk_a.mixer.counter}", flush=True)
+        for cache in (ops._workspaces, ops._topk_workspaces, ops._attn_workspaces, fused_layer._workspaces):
+            for ws in cache.values():
+                ws.view(torch.uint8).fill_(255)
         outs = []
         with torch.no_grad():
             for blk, ip in ((blk_a, ips[0]), (blk_b, ips[1])):
