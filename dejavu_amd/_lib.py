@@ -61,6 +61,10 @@ SIGNATURES = {
         _c_int,
         [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int,
          ctypes.c_float, _c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_size, _c_ptr]),
+    "dv_attention_out_proj_rows_f16": (
+        _c_int,
+        [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int,
+         ctypes.c_float, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_size, _c_ptr]),
     "dv_kv_cache_copy_sparse_f16": (
         _c_int,
         [_c_ptr, _c_ptr, _c_i64, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_int,

@@ -433,4 +433,159 @@ __global__ __launch_bounds__(256) void out_proj_rows_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------
+// out_proj in the (d, H, hd) layout straight from the un-normalised attention
+// partials { max, sum, o[HD] } of decode_attn_kernel (batch 1):
+//   ctx[i, :]  = fp16(merge over the splits of head_idx[i])     (arithmetic of decode_attn_combine_kernel)
+//   Y[n]       = fp16(sum_i ctx[i, :] . W[n, head_idx[i], :] + bias[n])  (lane order of out_proj_rows_kernel)
+//   Rout[n]    = fp16(Y[n] + Rin[n])                            (optional: the residual stream advanced)
+// Every output row is complete inside one wavefront, so there is no cross-workgroup reduction
+// and no second launch.  A workgroup first merges all partials into LDS (ctx: nnz * HD fp16,
+// then nnz segment offsets); the weight loads of its first head group are already in flight
+// by then.  A wavefront owns R rows: per head group (64 / (HD/8) heads) it issues R 16-byte
+// loads per lane, one group ahead of the multiply-adds.
+// Dynamic LDS: nnz * HD * 2 + nnz * 4 bytes.
+// ---------------------------------------------------------------------------
+template <int HD>
+__device__ __forceinline__ half8_t attn_merge8(const float* __restrict__ p, int nsplit, int j0) {
+  float m = -INFINITY, den = 0.f;
+  float num[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) num[e] = 0.f;
+  for (int s0 = 0; s0 < nsplit; s0 += 8) {  // online merge, 8 splits' loads in flight
+    float ms[8], ls[8];
+    float2 os[8][4];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const bool ok = s0 + q < nsplit;
+      const float* ps = p + (int64_t)(ok ? s0 + q : s0) * (HD + 2);
+      ms[q] = ok ? ps[0] : -INFINITY;
+      ls[q] = ps[1];
+#pragma unroll
+      for (int v = 0; v < 4; ++v) os[q][v] = *reinterpret_cast<const float2*>(ps + 2 + j0 + 2 * v);
+    }
+    float mc = m;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) mc = fmaxf(mc, ms[q]);
+    if (mc == -INFINITY) continue;
+    const float rescale = m == -INFINITY ? 0.f : __expf(m - mc);
+    den *= rescale;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) num[e] *= rescale;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const float w = ms[q] == -INFINITY ? 0.f : __expf(ms[q] - mc);
+      den += w * ls[q];
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        num[2 * v] += w * os[q][v].x;
+        num[2 * v + 1] += w * os[q][v].y;
+      }
+    }
+    m = mc;
+  }
+  half8_t out;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) out[e] = (half_t)(num[e] / den);
+  return out;
+}
+
+template <int R, int HD>
+__device__ __forceinline__ void out_proj_rows_attn_body(
+    const float* __restrict__ attn_part, int nsplit, const half_t* __restrict__ W,
+    const half_t* __restrict__ bias, const int* __restrict__ head_idx, int nnz, int H, int N,
+    half_t* __restrict__ Y, const half_t* __restrict__ Rin, half_t* __restrict__ Rout,
+    unsigned char* __restrict__ smem, int block_id, int nblocks) {
+  constexpr int PK = HD / 8;
+  constexpr int HPI = kWave / PK;  // heads per load instruction
+  half_t* ctx = reinterpret_cast<half_t*>(smem);
+  int* s_seg = reinterpret_cast<int*>(smem + (size_t)nnz * HD * sizeof(half_t));
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int grp = lane / PK, sub = lane % PK;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int waves = blockDim.x >> 6;
+  const int ntasks = (N + R - 1) / R;
+  const int niter = (nnz + HPI - 1) / HPI;
+  const int units = nnz * PK;
+  const int64_t ldw = (int64_t)H * HD;
+
+  // head ids this thread needs before LDS is filled: its merge unit and its first head group
+  const int hu = tid < units ? head_idx[tid / PK] : -1;
+  const int hg = grp < nnz ? head_idx[grp] : -1;
+  // seg < 0 (dead lane): the lane reads one cache-resident address and its activations are zero
+  auto load_group = [&](half8_t (&dst)[R], int n0, int seg) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int n = n0 + r < N ? n0 + r : N - 1;
+      dst[r] = load8_stream(W + (seg < 0 ? (int64_t)0 : (int64_t)n * ldw + seg) + sub * 8);
+    }
+  };
+  int task = block_id * waves + wave;
+  half8_t w[R];
+  if (task < ntasks) load_group(w, task * R, (hg >= 0 && hg < H) ? hg * HD : -1);  // in flight during the merge
+
+  // merge the attention partials into LDS
+  for (int u = tid; u < units; u += blockDim.x) {
+    const int i = u / PK, j0 = (u - i * PK) * 8;
+    const int h = u == tid ? hu : head_idx[i];
+    half8_t c = zero8();
+    if (h >= 0 && h < H) c = attn_merge8<HD>(attn_part + (int64_t)i * nsplit * (HD + 2), nsplit, j0);
+    *reinterpret_cast<half8_t*>(ctx + (size_t)i * HD + j0) = c;
+  }
+  for (int i = tid; i < nnz; i += blockDim.x) {
+    const int h = head_idx[i];
+    s_seg[i] = (h >= 0 && h < H) ? h * HD : -1;
+  }
+  __syncthreads();
+
+  for (; task < ntasks; task += nblocks * waves) {
+    const int n0 = task * R;
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = 0.f;
+    for (int it = 0; it < niter; ++it) {
+      // next head group (after the last one: the first group of this wavefront's next task)
+      half8_t wn[R];
+      int itn = it + 1, nn = n0;
+      if (itn == niter) {
+        itn = 0;
+        nn = (task + nblocks * waves) * R;
+      }
+      if (nn < N) {
+        const int in = itn * HPI + grp;
+        load_group(wn, nn, in < nnz ? s_seg[in] : -1);
+      }
+      const int i = it * HPI + grp;
+      const bool live = i < nnz && s_seg[i < nnz ? i : 0] >= 0;
+      half8_t x = zero8();
+      if (live) x = *reinterpret_cast<const half8_t*>(ctx + (size_t)i * HD + sub * 8);
+#pragma unroll
+      for (int r = 0; r < R; ++r) acc[r] = dot8_fast(w[r], x, acc[r]);
+#pragma unroll
+      for (int r = 0; r < R; ++r) w[r] = wn[r];
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const float v = butterfly_sum<kWave>(acc[r]);
+      const int n = n0 + r;
+      if (lane == r && n < N) {
+        const half_t y = (half_t)(v + (bias ? (float)bias[n] : 0.f));
+        Y[n] = y;
+        if (Rout != nullptr) Rout[n] = (half_t)((float)y + (float)Rin[n]);
+      }
+    }
+  }
+}
+
+template <int R, int HD>
+__global__ __launch_bounds__(512) void out_proj_rows_attn_kernel(
+    const float* __restrict__ attn_part, int nsplit, const half_t* __restrict__ W,
+    const half_t* __restrict__ bias, const int* __restrict__ head_idx, int nnz, int H, int N,
+    half_t* __restrict__ Y, const half_t* __restrict__ Rin, half_t* __restrict__ Rout) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  out_proj_rows_attn_body<R, HD>(attn_part, nsplit, W, bias, head_idx, nnz, H, N, Y, Rin, Rout, smem_raw,
+                                 blockIdx.x, gridDim.x);
+}
+
 }  // namespace dv

@@ -840,6 +840,70 @@ int dv_decode_attention_f16(const void* q, int64_t ldq, const void* k_cache, con
   return launch_status();
 }
 
+namespace {
+// out_proj over the (N, H, hd) weight from attention partials (batch 1); rin / rout optional
+constexpr int kOutRowsR = 4, kOutRowsWaves = 8;
+inline size_t out_rows_lds_bytes(int nnz, int hd) { return (size_t)nnz * hd * sizeof(half_t) + (size_t)nnz * 4; }
+inline int out_rows_blocks(int N) {
+  const int ntasks = (N + kOutRowsR - 1) / kOutRowsR;
+  int blocks = (ntasks + kOutRowsWaves - 1) / kOutRowsWaves;
+  const int cap = compute_units() * 2;
+  return blocks > cap ? cap : blocks;
+}
+int grant_out_rows_lds(int hd, size_t lds) {
+  static size_t granted[2] = {48 * 1024, 48 * 1024};
+  const int v = hd == 128 ? 1 : 0;
+  if (lds <= granted[v]) return DV_OK;
+  const void* fn = v ? reinterpret_cast<const void*>(out_proj_rows_attn_kernel<kOutRowsR, 128>)
+                     : reinterpret_cast<const void*>(out_proj_rows_attn_kernel<kOutRowsR, 64>);
+  if (lds > 160 * 1024 ||
+      hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+    return DV_ERR_UNSUPPORTED;
+  granted[v] = lds;
+  return DV_OK;
+}
+int launch_out_rows_attn(const float* part, int nsplit, const half_t* W, const half_t* bias, const int* head_idx,
+                         int nnz, int H, int hd, int N, half_t* y, const half_t* rin, half_t* rout,
+                         hipStream_t s) {
+  const size_t lds = out_rows_lds_bytes(nnz, hd);
+  const int rc = grant_out_rows_lds(hd, lds);
+  if (rc != DV_OK) return rc;
+  const dim3 grid(out_rows_blocks(N));
+  if (hd == 128)
+    hipLaunchKernelGGL((out_proj_rows_attn_kernel<kOutRowsR, 128>), grid, dim3(64 * kOutRowsWaves), lds, s, part,
+                       nsplit, W, bias, head_idx, nnz, H, N, y, rin, rout);
+  else
+    hipLaunchKernelGGL((out_proj_rows_attn_kernel<kOutRowsR, 64>), grid, dim3(64 * kOutRowsWaves), lds, s, part,
+                       nsplit, W, bias, head_idx, nnz, H, N, y, rin, rout);
+  return DV_OK;
+}
+}  // namespace
+
+int dv_attention_out_proj_rows_f16(const void* q, int64_t ldq, const void* k_cache, const void* v_cache,
+                                   const void* head_idx, int nheads, const void* lengths, int n_len, int H,
+                                   int hd, int S, float scale, const void* W, const void* bias, int N,
+                                   void* y, const void* residual_in, void* residual_out, void* workspace,
+                                   size_t workspace_bytes, void* stream) {
+  int rc = check_attn_args(q, ldq, k_cache, v_cache, nheads, n_len, 1, H, hd, S);
+  if (rc != DV_OK) return rc;
+  if (!head_idx || !W || !y || N <= 0 || nheads < 1 || (residual_out && !residual_in)) return DV_ERR_INVALID_ARG;
+  if (!aligned16(W)) return DV_ERR_ALIGNMENT;
+  if (!workspace || !aligned16(workspace) ||
+      workspace_bytes < dv_decode_attention_workspace_bytes(1, nheads, n_len, hd))
+    return DV_ERR_WORKSPACE;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  float* part = reinterpret_cast<float*>(workspace);
+  rc = launch_attn_partials(q, ldq, k_cache, v_cache, head_idx, nheads, lengths, n_len, 1, H, hd, S, scale,
+                            part, s);
+  if (rc != DV_OK) return rc;
+  rc = launch_out_rows_attn(part, attn_splits(n_len), reinterpret_cast<const half_t*>(W),
+                            reinterpret_cast<const half_t*>(bias), reinterpret_cast<const int*>(head_idx), nheads,
+                            H, hd, N, reinterpret_cast<half_t*>(y), reinterpret_cast<const half_t*>(residual_in),
+                            reinterpret_cast<half_t*>(residual_out), s);
+  if (rc != DV_OK) return rc;
+  return launch_status();
+}
+
 size_t dv_attention_out_proj_workspace_bytes(int B, int nheads, int n_len, int hd, int N) {
   if (B < 1 || nheads < 0 || n_len < 0 || hd <= 0 || N < 1) return 0;
   size_t a = dv_decode_attention_workspace_bytes(B, nheads, n_len, hd);

@@ -575,3 +575,49 @@ def attention_out_proj(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Te
                                         weight_t.stride(0), _ptr(bias), N, _ptr(out), _ptr(ws), ws.numel(),
                                         _stream()), "dv_attention_out_proj_f16")
     return out
+
+
+def attention_out_proj_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, head_idx: torch.Tensor,
+                            timestep: int, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                            lengths_per_sample: Optional[torch.Tensor] = None,
+                            softmax_scale: Optional[float] = None,
+                            residual: Optional[torch.Tensor] = None):
+    """``out_proj_sparse(single_query_attention(q, ...), weight, head_idx, bias)`` for one sequence in two
+    launches, weight in out_proj.weight's own layout (d, H, hd): the out_proj kernel merges the attention
+    splits itself and finishes every output row inside one wavefront (no split reduction).
+
+    q: (1, H, hd); caches already hold the newest token.  Returns y (1, d); with ``residual`` (1, d) or (d,)
+    returns (y, fp16(y + residual)), the residual stream advanced in the same launch.
+    """
+    _require_device(q, k_cache, v_cache, head_idx, weight, bias, lengths_per_sample, residual)
+    B, H, hd = q.shape
+    S = v_cache.shape[2]
+    N = weight.shape[0]
+    assert B == 1 and weight.numel() == N * H * hd and weight.is_contiguous()
+    assert head_idx.dtype == torch.int32 and head_idx.numel() >= 1
+    assert q.dtype == k_cache.dtype == v_cache.dtype == weight.dtype == torch.float16
+    assert v_cache.shape == (B, H, S, hd) and k_cache.shape == (B, H, hd // 8, S, 8)
+    assert k_cache.is_contiguous() and v_cache.is_contiguous() and q.stride(2) == 1 and q.stride(1) == hd
+    assert 0 <= timestep < S
+    head_idx = head_idx.contiguous()
+    nheads = head_idx.shape[0]
+    if bias is not None:
+        bias = bias.contiguous()
+        assert bias.shape == (N,)
+    if lengths_per_sample is not None:
+        assert lengths_per_sample.dtype == torch.int32 and lengths_per_sample.shape == (B,)
+    n_len = S if lengths_per_sample is not None else timestep + 1
+    scale = float(hd ** -0.5 if softmax_scale is None else softmax_scale)
+    out = torch.empty(B, N, device=q.device, dtype=q.dtype)
+    res_out = None
+    if residual is not None:
+        residual = residual.contiguous()
+        assert residual.numel() == N and residual.dtype == torch.float16
+        res_out = torch.empty_like(residual)
+    nbytes = lib.dv_decode_attention_workspace_bytes(1, nheads, n_len, hd)
+    ws = _attn_workspace(q.device, nbytes)
+    check(lib.dv_attention_out_proj_rows_f16(_ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(head_idx),
+                                             nheads, _ptr(lengths_per_sample), n_len, H, hd, S, scale, _ptr(weight),
+                                             _ptr(bias), N, _ptr(out), _ptr(residual), _ptr(res_out), _ptr(ws),
+                                             ws.numel(), _stream()), "dv_attention_out_proj_rows_f16")
+    return out if residual is None else (out, res_out)

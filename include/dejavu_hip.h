@@ -221,8 +221,16 @@ DV_API int dv_decode_attention_f16(const void* q, int64_t ldq, const void* k_cac
  * partials while it loads its activations.  Same arithmetic (the merged
  * context is rounded to fp16 as a stored one would be).
  *   head_idx (nheads,) int32, required; Wt (H*hd, N) row stride ldw; y (B, N);
- *   B <= 4; workspace: dv_attention_out_proj_workspace_bytes(...) bytes whose
- *   first 4 KiB are zero before first use.
+ *   B <= 4; workspace: dv_attention_out_proj_workspace_bytes(...) bytes, no
+ *   initialisation needed.
+ * dv_attention_out_proj_rows_f16 (batch 1): the same with the weight in
+ *   out_proj.weight's own (N, H, hd) layout, as dv_decode_attention_f16
+ *   followed by dv_out_proj_sparse_f16 (same bits).  Every output row is
+ *   complete inside one wavefront, so the attention partials + one launch
+ *   give y, and with residual_in / residual_out (optional, (N,)) also
+ *   residual_out = fp16(y + residual_in), the residual stream advanced as
+ *   Dejavu/src/models/modules/block_dejavu.py:625-631 does before norm2.
+ *   workspace: dv_decode_attention_workspace_bytes(1, nheads, n_len, hd).
  */
 DV_API size_t dv_attention_out_proj_workspace_bytes(int B, int nheads, int n_len, int hd, int N);
 DV_API int dv_attention_out_proj_f16(const void* q, int64_t ldq, const void* k_cache,
@@ -231,6 +239,12 @@ DV_API int dv_attention_out_proj_f16(const void* q, int64_t ldq, const void* k_c
                                      float scale, const void* Wt, int64_t ldw, const void* bias,
                                      int N, void* y, void* workspace, size_t workspace_bytes,
                                      void* stream);
+DV_API int dv_attention_out_proj_rows_f16(const void* q, int64_t ldq, const void* k_cache,
+                                          const void* v_cache, const void* head_idx, int nheads,
+                                          const void* lengths, int n_len, int H, int hd, int S,
+                                          float scale, const void* W, const void* bias, int N,
+                                          void* y, const void* residual_in, void* residual_out,
+                                          void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * y[b, n] = sum_{h in head_idx} x[b, h, :] . W[n, h, :] + bias[n], weight in

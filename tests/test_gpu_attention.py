@@ -275,3 +275,41 @@ def test_fused_qkv_cache_and_attention_out_proj_match_separate_ops(ops, nb):
                                         if False else np16(kc_a).copy(), np16(vc_a).copy(), S - 1, head_idx=head_idx.numpy())
     want = O.out_proj_sparse(want_ctx, np16(Wt).T.reshape(d, H, hd), head_idx.numpy(), np16(bo))
     assert_close(np16(out_b), want, "fused vs oracle")
+
+
+@pytest.mark.parametrize("H,hd,d,S,t,nnz", [(12, 128, 1536, 300, 299, 4), (8, 64, 512, 70, 40, 3),
+                                            (96, 128, 12288, 2048, 2047, 32), (12, 128, 1536, 520, 519, 12),
+                                            (72, 128, 9216, 1024, 1000, 24), (16, 64, 1024, 128, 5, 9)])
+def test_attention_out_proj_rows_matches_separate_ops(ops, H, hd, d, S, t, nnz):
+    """Attention partials + out_proj in the (d, H, hd) layout (two launches, no stored context, no split
+    reduction) give the bits of single_query_attention followed by out_proj_sparse, and the optional
+    residual output is the rounded sum of the fp16 result and the residual.  Also checked against the oracle."""
+    from dejavu_amd.workloads import pack_k_cache
+
+    g = torch.Generator().manual_seed(16)
+    q = randh(g, 1, H, hd).cuda()
+    kc = pack_k_cache(randh(g, 1, H, S, hd)).cuda()
+    vc = randh(g, 1, H, S, hd).cuda()
+    W = randh(g, d, H, hd, std=0.03).cuda()
+    bo = randh(g, d, std=0.1).cuda()
+    res = randh(g, d).cuda()
+    head_idx = torch.sort(torch.randperm(H, generator=g)[:nnz]).values.int().cuda()
+    print(f"case attention+out_proj rows H={H} hd={hd} d={d} S={S} t={t} nnz={nnz}", flush=True)
+    ctx = ops.single_query_attention(q, None, None, kc, vc, None, t, head_idx=head_idx)
+    want = ops.out_proj_sparse(ctx, W, head_idx, bo)
+    got = ops.attention_out_proj_rows(q, kc, vc, head_idx, t, W, bo)
+    got2, res_out = ops.attention_out_proj_rows(q, kc, vc, head_idx, t, W, bo, residual=res)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want), "must be bit-identical to the separate operators"
+    assert torch.equal(got2, want)
+    assert torch.equal(res_out, (want.float().view(-1) + res.float()).half())
+    # oracle: attention over the cached positions 0..t of the selected heads, then out_proj
+    kc_np = np16(kc).transpose(0, 1, 3, 2, 4).reshape(1, H, S, hd)
+    qn, vn, hi = np16(q)[0], np16(vc)[0], head_idx.cpu().numpy()
+    ctx_ref = np.zeros((1, H, hd), np.float32)
+    for h in hi:
+        sc = (kc_np[0, h, :t + 1] @ qn[h]) * hd ** -0.5
+        p = np.exp(sc - sc.max())
+        ctx_ref[0, h] = (p / p.sum()) @ vn[h, :t + 1]
+    ref = O.out_proj_sparse(ctx_ref.astype(np.float16).astype(np.float32), np16(W), hi, np16(bo))
+    assert_close(np16(got), ref, "attention+out_proj rows vs oracle")
