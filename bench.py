@@ -381,7 +381,8 @@ def main():
     ap.add_argument("--graph-per-step", action="store_true",
                     help="one HIP graph per step even when the step counts allow one graph per schedule period")
     ap.add_argument("--pmc-calibration", action="store_true",
-                    help="also run a plain 1 GiB device copy (known traffic) for counter calibration")
+                    help="for rocprofv3 --pmc runs: also run a plain 1 GiB device copy (known traffic) to calibrate the "
+                         "counters, and skip the replay-spread and window-start legs (thousands of dispatches)")
     ap.add_argument("--batches", type=int, nargs="+", default=[1, 4, 8, 16, 32],
                     help="batch sizes of --workload mlp")
     ap.add_argument("--workload", default="layer", choices=["layer", "decode", "mlp"],
@@ -466,7 +467,8 @@ def main():
             us_per_layer = timed(lambda i: g.replay() if i % period == 0 else None, args.steps, args.warmup)
             graph_mode = f"one graph of {period} steps"
             # spread over single replays (outside the timed region): one event pair per replay
-            evs = [torch.cuda.Event(enable_timing=True) for _ in range(21)]
+            # (a counter-collection run needs only one replay: every dispatch is serialised there)
+            evs = [torch.cuda.Event(enable_timing=True) for _ in range(2 if args.pmc_calibration else 21)]
             evs[0].record()
             for e in evs[1:]:
                 g.replay()
@@ -484,7 +486,7 @@ def main():
 
         # the same three layers at the first position of a window only (no back-fill work)
         window_start_us = None
-        if cycle and not args.no_graph:
+        if cycle and not args.no_graph and not args.pmc_calibration:
             cycle = False
             for L in layers:
                 L["block"].mixer.cache_offset.fill_(cfg["S"] - 1)
