@@ -139,8 +139,12 @@ __global__ __launch_bounds__(kMfmaWaves * 64) void gather_rows_mfma_kernel(
       load_stage(c);
       for (; c + kMfmaWaves < c_end; c += kMfmaWaves) {
         store_stage(c);
+        // x before the next chunk's weights, and the compiler must not swap them: the load counter
+        // retires in order, so the first multiplies wait for x alone while the weights stay in flight
         load_x(c, 0);
+        __builtin_amdgcn_sched_barrier(0);
         load_stage(c + kMfmaWaves);
+        __builtin_amdgcn_sched_barrier(0);
         multiply(0);
 #pragma unroll
         for (int bt0 = BP; bt0 < BT; bt0 += BP) {

@@ -112,8 +112,13 @@ __device__ __forceinline__ void qkv_window_mfma_body(
       load_stage(c);
       for (; c + WAVES < nchunks; c += WAVES) {
         store_stage(c);
+        // the x operands are requested BEFORE the next chunk's weights and the compiler must not
+        // swap them: the load counter retires in order, so the multiplies can then wait for x
+        // alone while the weight loads stay in flight
         load_x(c);
+        __builtin_amdgcn_sched_barrier(0);
         load_stage(c + WAVES);
+        __builtin_amdgcn_sched_barrier(0);
         multiply();
       }
       store_stage(c);
