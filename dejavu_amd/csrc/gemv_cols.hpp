@@ -248,6 +248,12 @@ __global__ __launch_bounds__(256) void cols_reduce_kernel(const float* __restric
     if (slice == 0 && o < total && Rout != nullptr) Rout[o] = (half_t)((float)Y[o] + (float)R[o]);
     return;
   }
+  // bias and residual are requested together with the partial sums, not after the barrier
+  float bv = 0.f, rv = 0.f;
+  if (slice == 0 && o < total) {
+    if (bias != nullptr) bv = (float)bias[o % N];
+    if (Rout != nullptr) rv = (float)R[o];
+  }
   float s = 0.f;
   if (o < total) {
     const float* p = partial + o;
@@ -265,9 +271,9 @@ __global__ __launch_bounds__(256) void cols_reduce_kernel(const float* __restric
   __syncthreads();
   if (slice == 0 && o < total) {
     const float r = (red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]);
-    const half_t y = (half_t)(r + (bias ? (float)bias[o % N] : 0.f));
+    const half_t y = (half_t)(r + bv);
     Y[o] = y;
-    if (Rout != nullptr) Rout[o] = (half_t)((float)y + (float)R[o]);
+    if (Rout != nullptr) Rout[o] = (half_t)((float)y + rv);
   }
 }
 
