@@ -101,8 +101,10 @@ def test_sparse_block_decode_step_matches_oracle(d, ffn, H, r, K, Hk, S):
     assert_close(np16(kcd)[:, :, :, t], kn[:, :, :, t], "key cache row of the new token")
 
 
-@pytest.mark.parametrize("d,H,ffn,r", [(768, 12, 3072, 128), (1024, 8, 4096, 1000)])
-def test_fused_layer_equals_module_by_module_path(d, H, ffn, r):
+@pytest.mark.parametrize("d,H,ffn,r,K,Hk", [(768, 12, 3072, 128, 512, 3), (1024, 8, 4096, 1000, 512, 3),
+                                            # OPT-13B- and OPT-66B-shaped layers: other launch plans
+                                            (5120, 40, 20480, 1000, 2048, 16), (9216, 72, 36864, 1000, 4096, 24)])
+def test_fused_layer_equals_module_by_module_path(d, H, ffn, r, K, Hk):
     """The eight-launch fused block step and the module-by-module path run the same kernel
     bodies: outputs, predictions, caches and window state must agree bit for bit over a
     whole back-fill window (the flush step falls back to the modules in both).  Every scratch
@@ -116,7 +118,7 @@ def test_fused_layer_equals_module_by_module_path(d, H, ffn, r):
     from dejavu_amd.modules import InferenceParams
     from dejavu_amd.workloads import pack_k_cache
 
-    K, Hk, S = 512, 3, 96
+    S = 96
     hd = d // H
     blk_a = create_sparse_block(d, ffn, H, r, K, r, Hk, layer_idx=0)
     init_block_synthetic(blk_a, seed=3)
