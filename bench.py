@@ -15,8 +15,8 @@ position 15 is the flush step that brings every head up to date.  The active
 heads are re-drawn at random for every (layer, position) -- no correlation
 between consecutive tokens, the most back-fill work a window can have.
 ``--window start`` times only the first position of a window (no back-fill).
-Steps are replayed from HIP graphs (one graph of 3 layers x 16 positions when the
-step counts are multiples of 48, one graph per (layer, position) otherwise).
+Steps are replayed from HIP graphs (one graph of up to four periods of 3 layers x 16 positions
+when the step counts are multiples of 48, one graph per (layer, position) otherwise).
 
 Prints ONE JSON line: metric / value / unit (us per layer, whole-window average), the
 roofline of the dominant kernel (qkv_sparse_kernel, measured alone with HIP events), the CPU
@@ -369,7 +369,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None, help="default 960 (20 windows of 3 layers x 16 positions)")
-    ap.add_argument("--warmup", type=int, default=None, help="default 96")
+    ap.add_argument("--warmup", type=int, default=None, help="default 192")
     ap.add_argument("--window", default="cycle", choices=["cycle", "start"],
                     help="cycle: steps walk through whole 16-token back-fill windows; "
                          "start: only the first position of a window (no back-fill)")
@@ -408,7 +408,7 @@ def main():
         args.steps = 300 if args.steps is None else args.steps
         return mlp_bench(args)
     args.steps = 960 if args.steps is None else args.steps
-    args.warmup = 96 if args.warmup is None else args.warmup
+    args.warmup = 192 if args.warmup is None else args.warmup
     dv_modules.USE_SIDE_STREAM = not args.single_stream
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
@@ -462,10 +462,17 @@ def main():
             us_per_layer = timed(step_fn, args.steps, args.warmup)
             graph_mode = "none"
         elif whole:
-            g = capture(0, period)
+            # one graph holds as many whole schedule periods as the step counts allow (up to 4):
+            # the gap between two graph launches is harness time, not part of a layer step
+            span = period
+            for reps in (4, 2):
+                if args.steps % (reps * period) == 0 and args.warmup % (reps * period) == 0:
+                    span = reps * period
+                    break
+            g = capture(0, span)
             torch.cuda.synchronize()
-            us_per_layer = timed(lambda i: g.replay() if i % period == 0 else None, args.steps, args.warmup)
-            graph_mode = f"one graph of {period} steps"
+            us_per_layer = timed(lambda i: g.replay() if i % span == 0 else None, args.steps, args.warmup)
+            graph_mode = f"one graph of {span} steps"
             # spread over single replays (outside the timed region): one event pair per replay
             # (a counter-collection run needs only one replay: every dispatch is serialised there)
             evs = [torch.cuda.Event(enable_timing=True) for _ in range(2 if args.pmc_calibration else 21)]
@@ -474,8 +481,8 @@ def main():
                 g.replay()
                 e.record()
             torch.cuda.synchronize()
-            per = sorted(a.elapsed_time(b) * 1e3 / period for a, b in zip(evs[:-1], evs[1:]))
-            spread = {"unit": f"us/layer over one replay of {period} steps", "replays": len(per),
+            per = sorted(a.elapsed_time(b) * 1e3 / span for a, b in zip(evs[:-1], evs[1:]))
+            spread = {"unit": f"us/layer over one replay of {span} steps", "replays": len(per),
                       "median": round(per[len(per) // 2], 2), "p10": round(per[len(per) // 10], 2),
                       "p90": round(per[(len(per) * 9) // 10], 2)}
         else:
@@ -492,9 +499,10 @@ def main():
                 L["block"].mixer.cache_offset.fill_(cfg["S"] - 1)
             for i in range(N_LAYERS):
                 step_fn(i)
-            g0 = capture(0, N_LAYERS)
+            span0 = 64 * N_LAYERS  # long graph: launch gaps between replays are harness time
+            g0 = capture(0, span0)
             torch.cuda.synchronize()
-            window_start_us = timed(lambda i: g0.replay() if i % N_LAYERS == 0 else None, 300, 30)
+            window_start_us = timed(lambda i: g0.replay() if i % span0 == 0 else None, 5 * span0, span0)
             cycle = True
 
         if args.pmc_calibration:
