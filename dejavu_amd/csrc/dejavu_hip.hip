@@ -1170,12 +1170,13 @@ int dv_sparse_layer_decode_f16(const dvSparseLayerArgs* args, void* stream) {
     const int rw0 = a.d <= 1024 ? 4 * kCanonShortRows : 1;
     const int nh = ((a.r_att + rw0 - 1) / rw0 + 3) / 4;
     const dim3 grid(na + nh + topk_blocks);
+    int* advance_ptr = (a.counter == 15 && a.advance_window) ? reinterpret_cast<int*>(a.cache_offset) : nullptr;
     if (a.hd == 128)
       hipLaunchKernelGGL((layer_l3_kernel<128>), grid, dim3(256), 0, s, at, na, hp0, nh, CH(a.mlp_logit_in),
-                         a.ffn, a.K, topk_ws);
+                         a.ffn, a.K, topk_ws, advance_ptr, 16);
     else
       hipLaunchKernelGGL((layer_l3_kernel<64>), grid, dim3(256), 0, s, at, na, hp0, nh, CH(a.mlp_logit_in),
-                         a.ffn, a.K, topk_ws);
+                         a.ffn, a.K, topk_ws, advance_ptr, 16);
   }
   // L4 + L5: out_proj from the attention partials | head predictor fc1 | top-k emission; split reduction
   {

@@ -111,7 +111,11 @@ struct AttnArgs {
 template <int HD>
 __global__ __launch_bounds__(256) void layer_l3_kernel(AttnArgs a, int nblk_attn, CanonArgs hp0, int nblk_hp0,
                                                        const half_t* __restrict__ mlp_logits, int ffn,
-                                                       int K, unsigned* __restrict__ topk_ws) {
+                                                       int K, unsigned* __restrict__ topk_ws,
+                                                       int* __restrict__ advance_ptr, int advance_by) {
+  // flush step: the window's K / V rows went into the caches in the launch before this one; the
+  // window now starts advance_by positions later (nothing in this launch or after it reads the value)
+  if (advance_ptr != nullptr && blockIdx.x == 0 && threadIdx.x == 0) *advance_ptr += advance_by;
   // the small roles with the longer dependency chains take the first block ids: they are dispatched first
   const int nblk_count = (int)gridDim.x - nblk_attn - nblk_hp0;
   int bid = blockIdx.x;

@@ -23,7 +23,7 @@ class SparseLayerArgs(ctypes.Structure):
         ("d", ctypes.c_int), ("ffn", ctypes.c_int), ("H", ctypes.c_int), ("hd", ctypes.c_int),
         ("r_att", ctypes.c_int), ("r_mlp", ctypes.c_int),
         ("K", ctypes.c_int), ("Hk", ctypes.c_int), ("att_k", ctypes.c_int),
-        ("S", ctypes.c_int), ("counter", ctypes.c_int), ("n_len", ctypes.c_int),
+        ("S", ctypes.c_int), ("counter", ctypes.c_int), ("n_len", ctypes.c_int), ("advance_window", ctypes.c_int),
         ("eps1", ctypes.c_float), ("eps2", ctypes.c_float), ("softmax_scale", ctypes.c_float),
         ("hidden", _p), ("residual", _p),
         ("ln1_w", _p), ("ln1_b", _p), ("ln2_w", _p), ("ln2_b", _p),
@@ -124,6 +124,7 @@ def sparse_layer_decode(block, hidden_states, residual, head_idx, mlp_sp_logit, 
     a.S = vc.shape[2]
     a.counter = m.counter
     a.n_len = inference_params.sequence_len_offset + 1
+    a.advance_window = int(flush and not m.hold_window)  # the kernels move cache_offset to the next window
     a.eps1, a.eps2 = block.norm1.eps, block.norm2.eps
     a.softmax_scale = float(hd ** -0.5 if m.softmax_scale is None else m.softmax_scale)
     a.hidden, a.residual = _ptr(hidden_states), _ptr(residual)
@@ -146,8 +147,7 @@ def sparse_layer_decode(block, hidden_states, residual, head_idx, mlp_sp_logit, 
     check(lib.dv_sparse_layer_decode_f16(ctypes.byref(a), torch.cuda.current_stream().cuda_stream),
           "dv_sparse_layer_decode_f16")
     m.counter += 1
-    if flush:  # window complete: start the next one
+    if flush:  # window complete: start the next one (cache_offset was advanced on the device)
         m.counter = 0
-        m.cache_offset += m.WINDOW
     block.last_mlp_idx = mlp_idx_out
     return hidden_out, residual_out, logit_out.view(-1), att_idx_out

@@ -344,6 +344,8 @@ class ParallelMHASparseAttMlp(_MHABase):
         self.tracker = torch.arange(self.WINDOW, dtype=torch.int32, device=device).repeat(num_heads, 1)
         self.counter = 0
         self.cache_offset = None  # device int32[1]: cache position of window token 0
+        # True keeps the window at its cache position after a flush (benchmarks that replay one window)
+        self.hold_window = False
         self.out_proj_weight_t = None
         self._all_heads = None
         # optional caller-owned buffer for the predicted heads (fixed address for graph capture)
@@ -415,7 +417,8 @@ class ParallelMHASparseAttMlp(_MHABase):
                                          inference_params.lengths_per_sample, self.softmax_scale).unsqueeze(1)
             if self.counter == self.WINDOW:  # window complete: start the next one
                 self.counter = 0
-                self.cache_offset += self.WINDOW
+                if not self.hold_window:
+                    self.cache_offset += self.WINDOW
         else:
             qkv = decode_linear(self.Wqkv, x)
             qkv = qkv.view(x.shape[0], x.shape[1], 3, self.num_heads, self.head_dim)

@@ -321,6 +321,8 @@ typedef struct dvSparseLayerArgs {
   int S;                  /* KV cache capacity                                         */
   int counter;            /* window position of this token, 0..15 (15: flush, Hk == H) */
   int n_len;              /* cached positions to attend, newest token included         */
+  int advance_window;     /* flush step only: != 0 adds 16 to cache_offset[0] once the  */
+                          /* window's K/V rows are in the caches (the next window)      */
   float eps1, eps2, softmax_scale;
   /* inputs (device, fp16 unless stated) */
   const void* hidden;     /* (d,) output of the previous block's MLP                   */
@@ -336,7 +338,7 @@ typedef struct dvSparseLayerArgs {
   const void *mlp_Wa, *mlp_Wb; /* (r_mlp, d), (ffn, r_mlp)                             */
   const void* head_idx;   /* (Hk,) int32 heads to compute                              */
   const void* mlp_logit_in; /* (ffn,) predictor logits for THIS layer's MLP            */
-  const void* cache_offset; /* int32[1]: cache position of window token 0             */
+  void* cache_offset;     /* int32[1]: cache position of window token 0 (see advance_window) */
   const void* seq_pos;    /* int32[1] cache position of the newest token, or NULL: when   */
                           /* given it replaces n_len - 1, so that a captured launch     */
                           /* sequence can be replayed as the sequence grows (the role of */

@@ -156,6 +156,7 @@ def test_fused_layer_equals_module_by_module_path(d, H, ffn, r, K, Hk):
         for name, xa, xb in zip(("hidden", "residual", "next_logit", "next_att_idx"), outs[0], outs[1]):
             assert torch.equal(xa.reshape(-1), xb.reshape(-1)), f"step {step}: {name} differs"
         assert blk_a.mixer.counter == blk_b.mixer.counter
+        assert torch.equal(blk_a.mixer.cache_offset, blk_b.mixer.cache_offset), f"step {step}: window offsets differ"
         assert torch.equal(blk_a.mixer.tracker, blk_b.mixer.tracker) and torch.equal(blk_a.mixer.x_cache[:max(1, blk_a.mixer.counter)],
                                                                                      blk_b.mixer.x_cache[:max(1, blk_b.mixer.counter)])
         for ca, cb in zip(ips[0].key_value_memory_dict[0], ips[1].key_value_memory_dict[0]):
