@@ -480,13 +480,35 @@ __global__ __launch_bounds__(1024) void greedy_advance_kernel(
   __shared__ int s_idx[16];
   unsigned best = 0u;
   int best_i = 0x7fffffff;
-  for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
-    const unsigned k = topk_key(logits[i]) + 1u;  // +1: any element beats the empty start value
+  auto take = [&](half_t v, int i) {
+    const unsigned k = topk_key(v) + 1u;  // +1: any element beats the empty start value
     if (k > best) {  // i ascends per thread: equal keys keep the lower index
       best = k;
       best_i = i;
     }
+  };
+  // 16-byte loads, eight of them in flight per thread (a thread's packets ascend in index)
+  const int npk = (reinterpret_cast<uintptr_t>(logits) & 15) == 0 ? vocab / 8 : 0;
+  for (int p0 = threadIdx.x; p0 < npk; p0 += 8 * blockDim.x) {
+    half8_t v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int p = p0 + u * blockDim.x;
+      v[u] = load8(logits + (int64_t)(p < npk ? p : p0) * 8);
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int p = p0 + u * blockDim.x;
+      if (p < npk) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const half_t hv = v[u][e];
+          take(hv, p * 8 + e);
+        }
+      }
+    }
   }
+  for (int i = npk * 8 + threadIdx.x; i < vocab; i += blockDim.x) take(logits[i], i);
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) {
     const unsigned ok = (unsigned)__shfl_xor((int)best, off, kWave);

@@ -146,7 +146,7 @@ def test_graph_replayed_generation_equals_eager_bit_for_bit():
     assert torch.equal(g3.sequences, e3.sequences)
 
 
-@pytest.mark.parametrize("vocab", [7, 512, 50272])
+@pytest.mark.parametrize("vocab", [7, 512, 8200, 50272, 50277, 70001])
 def test_greedy_advance_matches_torch_argmax_and_bookkeeping(vocab):
     """The fused greedy step: first index among equal maxima (as torch.argmax), NaN on top, and the
     device-side counters / sequence / score rows advanced exactly once."""
@@ -187,3 +187,9 @@ def test_greedy_advance_matches_torch_argmax_and_bookkeeping(vocab):
         ops.greedy_advance(logits, token, position, seq_pos, sequences, out_index)
         torch.cuda.synchronize()
         assert int(out_index) == 5 and int(sequences[0, 4]) == want and int(score_index) == 3
+        # a logits row that does not start on a 16-byte boundary (element-wise scan)
+        shifted = torch.cat([logits[:1], logits])[1:]
+        assert shifted.data_ptr() % 16 != 0
+        ops.greedy_advance(shifted, token, position, seq_pos, sequences, out_index)
+        torch.cuda.synchronize()
+        assert int(token) == want and int(out_index) == 6
