@@ -287,8 +287,9 @@ class GPTLMHeadModel(nn.Module):
         window = ParallelMHASparseAttMlp.WINDOW
         for step in range(n_new - 1):
             c = step % window  # position inside the back-fill window (== every sparse mixer's counter)
-            if cg and step >= window:
-                # each window position has run eagerly once: workspaces exist, capture is safe
+            if cg and (step >= window or c in cache.graphs):
+                # a window position is captured once it has run eagerly (workspaces exist then);
+                # later generations replay the graphs from their first decode step on
                 if c not in cache.graphs:
                     g = torch.cuda.CUDAGraph()
                     with torch.cuda.graph(g):
