@@ -37,11 +37,16 @@ __device__ __forceinline__ float block_sum_virtual(const float (&v)[kLnVirtual /
 // MAXV: 8-element vectors per virtual thread; requires d % 8 == 0 and d <= 8192 * MAXV.
 // Y may point to LDS (the row handed to a consumer in the same workgroup) or to memory;
 // Y2 (optional) receives a second copy of the normalised row (the back-fill window buffer).
-template <int REAL, int MAXV>
+struct LnNoHook {
+  __device__ __forceinline__ void operator()() const {}
+};
+// after_loads: called once the row's loads have been requested (a place to request memory the caller
+// needs later: requests queued before the row's loads would delay them, the load counter retires in order)
+template <int REAL, int MAXV, class AfterLoads = LnNoHook>
 __device__ __forceinline__ void add_layer_norm_body(
     const half_t* __restrict__ H, const half_t* __restrict__ R, const half_t* __restrict__ gamma,
     const half_t* __restrict__ beta, float eps, int d, half_t* __restrict__ Y,
-    half_t* __restrict__ Rout, half_t* __restrict__ Y2, int64_t row) {
+    half_t* __restrict__ Rout, half_t* __restrict__ Y2, int64_t row, AfterLoads after_loads = AfterLoads()) {
   constexpr int Q = kLnVirtual / REAL;
   constexpr bool EARLY = Q * MAXV <= 4;  // gamma / beta fetched up front while registers allow
   __shared__ float scratch[kLnVirtual / kWave];
@@ -66,6 +71,7 @@ __device__ __forceinline__ void add_layer_norm_body(
       v[q][j] = i < nvec ? load8(H + row * d + i * 8) : zero8();
       rr[q][j] = (R != nullptr && i < nvec) ? load8(R + row * d + i * 8) : zero8();
     }
+  after_loads();
   float s[Q];
 #pragma unroll
   for (int q = 0; q < Q; ++q) {
