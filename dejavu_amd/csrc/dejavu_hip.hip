@@ -356,19 +356,24 @@ struct ColsMfmaPlan {
 
 ColsMfmaPlan plan_cols_mfma(int B, int N, int M) {
   ColsMfmaPlan p;
-  p.col_tiles = (N + kMfmaColTile - 1) / kMfmaColTile;
   // Every row group writes a (B, N) fp32 partial that a second pass reads back, so few, long
-  // groups win: each wavefront (256 columns of one group) keeps 16 KiB of weights in flight
-  // and three of them per compute unit measured best for batch 8..64.
+  // groups win.  Each wavefront keeps 16 KiB of weights in flight and three of them per compute
+  // unit measured best for batch 8..64.  Up to batch 32 a workgroup's four wavefronts split the
+  // group's rows and add their sums through LDS (a quarter of the partials: fc2 at the OPT-175B
+  // shape 3 us faster at batch 16 and 32); above, they split the columns.
   const int waves_per_cu = 3;
-  const int col_waves = (N + kMfmaColWave - 1) / kMfmaColWave;
-  int groups = (compute_units() * waves_per_cu + col_waves - 1) / col_waves;
-  const int max_groups = M > kMfmaColRows ? (M + kMfmaColRows - 1) / kMfmaColRows : 1;
+  const bool split_rows = B <= 32;
+  const int col_tile = mfma_col_tile(split_rows ? 1 : 2);
+  p.col_tiles = (N + col_tile - 1) / col_tile;
+  const int blocks = (compute_units() * waves_per_cu + 3) / 4;
+  int groups = (blocks + p.col_tiles - 1) / p.col_tiles;
+  const int min_rows = split_rows ? kMfmaColSub * kMfmaColRows : kMfmaColRows;  // one pipeline step per wavefront
+  const int max_groups = M > min_rows ? (M + min_rows - 1) / min_rows : 1;
   if (groups > max_groups) groups = max_groups;
   if (groups < 1) groups = 1;
   int rpb = (M + groups - 1) / groups;
-  rpb = (rpb + kMfmaColRows - 1) / kMfmaColRows * kMfmaColRows;
-  if (rpb < kMfmaColRows) rpb = kMfmaColRows;
+  rpb = (rpb + min_rows - 1) / min_rows * min_rows;
+  if (rpb < min_rows) rpb = min_rows;
   p.rows_per_block = rpb;
   p.groups = M > 0 ? (M + rpb - 1) / rpb : 1;
   return p;

@@ -344,7 +344,8 @@ __global__ __launch_bounds__(512) void rows_short_mfma_kernel(
 // fc2 / out_proj over a transposed weight: Y[b, n] = sum_m H[b, m] * W[row(m), n].
 // The contraction index m runs over gathered ROWS, while the MFMA wants 8
 // consecutive k per lane: the transposition happens inside each lane's registers,
-// no LDS involved.  A wavefront owns 256 columns.  Lanes 0..31 load 16 bytes
+// no LDS involved.  A wavefront streams 256 columns; with one batch tile the four wavefronts of
+// a workgroup share their 256 columns and take a quarter of the group's rows each.  Lanes 0..31 load 16 bytes
 // (8 columns) of row m, lanes 32..63 the same columns of row m + 8, eight rows
 // each per k-step of 16 (one load instruction reads 2 rows x 512 contiguous
 // bytes).  A lane then holds an 8 x 8 block (8 rows x its 8 columns); read
@@ -363,8 +364,13 @@ __global__ __launch_bounds__(512) void rows_short_mfma_kernel(
 // straddle a block).  Otherwise H is gathered element by element.
 // ---------------------------------------------------------------------------
 constexpr int kMfmaColWave = 256;                 // columns per wavefront
-constexpr int kMfmaColTile = 4 * kMfmaColWave;    // columns per workgroup
+// Columns per workgroup.  One batch tile (B <= 32): the four wavefronts share 256 columns and split the
+// rows.  Two batch tiles: 256 accumulator registers per lane leave no room for the exchange (it
+// spilled: 110.6 us against 107.0 us for fc2 at batch 64), so there the wavefronts split the columns
+// and every wavefront writes its own partial.
+constexpr int mfma_col_tile(int bt) { return bt == 1 ? kMfmaColWave : 4 * kMfmaColWave; }
 constexpr int kMfmaColRows = 32;                  // rows per pipeline step (two k-steps of 16)
+constexpr int kMfmaColSub = 4;                    // row sub-ranges (wavefronts) per workgroup
 
 template <int BT, bool IDX64, bool BLOCKED, bool HVEC>
 __global__ __launch_bounds__(256) void gather_cols_mfma_kernel(
@@ -376,11 +382,15 @@ __global__ __launch_bounds__(256) void gather_cols_mfma_kernel(
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int half_id = lane >> 5, l32 = lane & 31;
   const int ct = blockIdx.x, g = blockIdx.y, G = gridDim.y;
-  const int col0 = ct * kMfmaColTile + wave * kMfmaColWave;
+  constexpr bool SPLIT_ROWS = BT == 1;
+  const int col0 = ct * mfma_col_tile(BT) + (SPLIT_ROWS ? 0 : wave * kMfmaColWave);
   // columns past N accumulate garbage that is never stored; their loads re-read column 0
   const int wcol = col0 + l32 * 8 < N ? col0 + l32 * 8 : 0;
-  const int m_begin = g * rows_per_block;
-  int m_end = m_begin + rows_per_block;
+  // the four wavefronts take consecutive quarters of the group's rows (whole pipeline steps)
+  const int rpw = ((rows_per_block + kMfmaColSub - 1) / kMfmaColSub + kMfmaColRows - 1) / kMfmaColRows * kMfmaColRows;
+  const int m_begin = g * rows_per_block + (SPLIT_ROWS ? wave * rpw : 0);
+  int m_end = m_begin + (SPLIT_ROWS ? rpw : rows_per_block);
+  if (m_end > (g + 1) * rows_per_block) m_end = (g + 1) * rows_per_block;
   if (m_end > M) m_end = M;
   const bool any_rows = m_begin < m_end;
   // raw index word of row (mb + l32); rows past the group re-read its first row
@@ -499,11 +509,46 @@ __global__ __launch_bounds__(256) void gather_cols_mfma_kernel(
     load_h(mb, rid_cur);
     consume(cur_ok);
   }
+  // The four wavefronts' sums are added through LDS in the fixed order (w0 + w2) + (w1 + w3), one
+  // batch tile at a time (2 x 32 KiB): a group then costs one (B, N) fp32 partial instead of four,
+  // and the partials are what the second pass has to write and read back.
+  __shared__ float red[SPLIT_ROWS ? 2 : 1][SPLIT_ROWS ? 8 * 16 : 1][kWave];
+#pragma unroll
+  for (int bt = 0; SPLIT_ROWS && bt < BT; ++bt) {
+    if (wave >= 2) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) red[wave - 2][e * 16 + v][lane] = acc[e][bt][v];
+    }
+    __syncthreads();
+    if (wave < 2) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[e][bt][v] += red[wave][e * 16 + v][lane];
+    }
+    __syncthreads();
+    if (wave == 1) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) red[0][e * 16 + v][lane] = acc[e][bt][v];
+    }
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[e][bt][v] += red[0][e * 16 + v][lane];
+    }
+    if (bt + 1 < BT) __syncthreads();
+  }
   // H^T is the first operand, so result rows are batch entries and result columns the lane's
   // weight columns: value v of MFMA e is batch row 8 * (v / 4) + 4 * half_id + v % 4, column
   // 8 * l32 + e.  For a fixed v the eight MFMAs hold eight consecutive columns: one vector store.
   const int n0 = col0 + l32 * 8;
-  if (n0 < N) {  // N % 8 == 0: a lane's eight columns are all inside or all outside
+  if ((wave == 0 || !SPLIT_ROWS) && n0 < N) {  // N % 8 == 0: a lane's eight columns are all inside or all outside
 #pragma unroll
     for (int bt = 0; bt < BT; ++bt)
 #pragma unroll
