@@ -206,12 +206,17 @@ constexpr int kRowsVecMaxBatch = 2;
 constexpr int kColsVecMaxBatch = 4;
 
 // ---- batched gathered GEMMs on the matrix cores (5 <= B <= 64) -------------------
+#ifndef DV_ROWS_XLDS
+#define DV_ROWS_XLDS 1
+#endif
 template <int BT, bool IDX64, bool RELU>
 int launch_rows_mfma(const half_t* x, const half_t* W, int64_t ldw, const half_t* bias, const void* idx,
                      int B, int N, int Z, int M, half_t* y, hipStream_t s) {
-  auto kern = gather_rows_mfma_kernel<BT, IDX64, RELU>;
-  // one 16 x 256 staging tile per wavefront; the same memory later holds the partial result tiles
-  const size_t tile_bytes = (size_t)kMfmaWaves * kMfmaRows * kMfmaLdsRow * sizeof(half_t);
+  constexpr bool XLDS = DV_ROWS_XLDS && BT <= 2;
+  auto kern = gather_rows_mfma_kernel<BT, IDX64, RELU, false, XLDS>;
+  // one 16 x 256 staging tile per wavefront (two with X staged as well); the same memory later
+  // holds the partial result tiles
+  const size_t tile_bytes = (size_t)kMfmaWaves * (XLDS ? 2 : 1) * kMfmaRows * kMfmaLdsRow * sizeof(half_t);
   const size_t red_bytes = (size_t)kMfmaWaves * BT * 4 * 64 * sizeof(float);
   const size_t lds = tile_bytes > red_bytes ? tile_bytes : red_bytes;
   static bool granted = false;

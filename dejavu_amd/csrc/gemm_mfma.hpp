@@ -49,7 +49,10 @@ constexpr int kMfmaRows = 16;
 // gridDim.y: workgroup (t, y) takes chunks [y * chunks_per_split, (y + 1) * chunks_per_split)
 // and writes the raw fp32 sums to partial[(y * B + b) * M + m]; rows_split_reduce_kernel adds
 // the splits in ascending order.  No bias / activation in this mode.
-template <int BT, bool IDX64, bool RELU, bool SPLIT = false>
+// XLDS (one batch tile only): the X operands take the same road as the weights -- coalesced loads
+// (2 batch rows x 512 contiguous bytes per instruction) one step ahead, a wavefront-private LDS tile,
+// read back in MFMA layout -- instead of 64-byte segments of 16 rows per load straight from memory.
+template <int BT, bool IDX64, bool RELU, bool SPLIT = false, bool XLDS = false>
 __global__ __launch_bounds__(kMfmaWaves * 64) void gather_rows_mfma_kernel(
     const half_t* __restrict__ X, const half_t* __restrict__ W, const half_t* __restrict__ bias,
     const void* __restrict__ idx, int B, int N, int64_t ldw, int Z, int M, half_t* __restrict__ Y,
@@ -57,7 +60,9 @@ __global__ __launch_bounds__(kMfmaWaves * 64) void gather_rows_mfma_kernel(
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  half_t* tile = reinterpret_cast<half_t*>(smem_raw) + (size_t)wave * kMfmaRows * kMfmaLdsRow;
+  static_assert(!XLDS || BT <= 2, "X through LDS: at most two batch tiles (passes through one LDS tile)");
+  half_t* tile = reinterpret_cast<half_t*>(smem_raw) + (size_t)wave * (XLDS ? 2 : 1) * kMfmaRows * kMfmaLdsRow;
+  half_t* xtile = tile + kMfmaRows * kMfmaLdsRow;
   float* red = reinterpret_cast<float*>(smem_raw);  // reused after the main loop
   const int l16 = lane & 15, kg = lane >> 4;  // MFMA operand coordinates
   const int l32 = lane & 31, half_id = lane >> 5;  // staging coordinates
@@ -66,7 +71,7 @@ __global__ __launch_bounds__(kMfmaWaves * 64) void gather_rows_mfma_kernel(
   const int c_end = SPLIT ? (c_begin + chunks_per_split < nchunks ? c_begin + chunks_per_split : nchunks) : nchunks;
   constexpr int KS = kMfmaKC / 32;  // MFMA k-steps per chunk
   // batch tiles are multiplied in passes of at most two, to bound the X registers
-  constexpr int BP = BT < 2 ? BT : 2;
+  constexpr int BP = (BT < 2 || XLDS) ? 1 : 2;
 
   for (int t = blockIdx.x; t * kMfmaRows < M; t += gridDim.x) {
     // row id of output row (t*16 + l16), replicated over the four 16-lane groups
@@ -93,9 +98,20 @@ __global__ __launch_bounds__(kMfmaWaves * 64) void gather_rows_mfma_kernel(
     for (int bt = 0; bt < BT; ++bt) acc[bt] = float4_t{0.f, 0.f, 0.f, 0.f};
 
     half8_t stage[8];
+    half8_t xstage[XLDS ? BT : 1][XLDS ? 8 : 1];
+    half8_t xhold[XLDS && BT > 1 ? 8 : 1];
     auto load_stage = [&](int c) {
       int col = c * kMfmaKC + l32 * 8;
       if (col >= N) col = 0;  // masked when stored
+      if (XLDS) {  // batch rows past B re-read row 0; their results are dropped
+#pragma unroll
+        for (int bt = 0; bt < BT; ++bt)
+#pragma unroll
+          for (int q = 0; q < 8; ++q) {
+            const int b = bt * 16 + 2 * q + half_id;
+            xstage[bt][q] = load8(X + (int64_t)(b < B ? b : 0) * N + col);
+          }
+      }
 #pragma unroll
       for (int q = 0; q < 8; ++q) stage[q] = load8_stream(wrow[q] + col);
     };
@@ -103,6 +119,14 @@ __global__ __launch_bounds__(kMfmaWaves * 64) void gather_rows_mfma_kernel(
       const bool col_ok = c * kMfmaKC + l32 * 8 < N;
       __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");  // previous tile fully read
       __builtin_amdgcn_wave_barrier();
+      if (XLDS) {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) store8(xtile + (2 * q + half_id) * kMfmaLdsRow + l32 * 8, xstage[0][q]);
+        if (BT > 1) {  // kept aside: the next chunk's loads are requested before the second pass
+#pragma unroll
+          for (int q = 0; q < 8; ++q) xhold[q] = xstage[BT - 1][q];
+        }
+      }
 #pragma unroll
       for (int q = 0; q < 8; ++q)
         store8(tile + (2 * q + half_id) * kMfmaLdsRow + l32 * 8,
@@ -114,6 +138,20 @@ __global__ __launch_bounds__(kMfmaWaves * 64) void gather_rows_mfma_kernel(
     // past B read a valid address; the weights there are zero / the results are dropped
     half8_t xb[KS][BP];
     auto load_x = [&](int c, int bt0) {
+      if (XLDS) {
+        if (bt0 > 0) {  // the second batch tile takes the first one's place in LDS
+          __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+#pragma unroll
+          for (int q = 0; q < 8; ++q)
+            store8(xtile + (2 * q + half_id) * kMfmaLdsRow + l32 * 8, xhold[q]);
+          __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+        }
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) xb[ks][0] = load8(xtile + l16 * kMfmaLdsRow + ks * 32 + kg * 8);
+        return;
+      }
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         int kk = c * kMfmaKC + ks * 32 + kg * 8;
