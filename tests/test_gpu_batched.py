@@ -29,6 +29,7 @@ def ops():
 
 @pytest.mark.parametrize("cfg,B,K", [("opt-125m", 3, 1024), ("opt-6.7b", 4, 4096),  # fc1 on MFMA, fc2 on the vector ALUs
                                      ("opt-125m", 5, 1024), ("opt-125m", 16, 1024), ("opt-125m", 33, 1000),
+                                     ("opt-125m", 27, 1000),  # two batch tiles, row groups of ragged length
                                      ("opt-6.7b", 8, 2048), ("opt-6.7b", 16, 4096), ("opt-6.7b", 32, 2048),
                                      ("opt-6.7b", 64, 1024)])
 @pytest.mark.parametrize("idx_dtype", [torch.int64, torch.int32])
@@ -64,14 +65,14 @@ def test_batched_mlp_sparse_at_the_headline_shape(ops):
     test_batched_mlp_sparse_matches_oracle(ops, "opt-175b", 32, 4096, torch.int64)
 
 
-def test_batched_edge_cases(ops):
+@pytest.mark.parametrize("B", [11, 27, 40])  # one / two batch tiles; fc2 split by rows / by columns
+def test_batched_edge_cases(ops, B):
     g = torch.Generator().manual_seed(3)
-    B = 11
     x = torch.randn(B, 776, generator=g).half()
     W = (torch.randn(300, 776, generator=g) * 0.05).half()
     bias = torch.randn(300, generator=g).half()
     idx = torch.tensor([299, 0, 0, 17, 5, 299, 123, 1000, -3] * 5 + [7, 8, 9], dtype=torch.int64)  # M = 48, ragged
-    print("case batched edge", flush=True)
+    print(f"case batched edge B={B}", flush=True)
     got = ops.gather_gemv(x.cuda(), W.cuda(), idx.cuda(), bias.cuda(), activation="id")
     torch.cuda.synchronize()
     valid = ((idx >= 0) & (idx < 300)).numpy()
