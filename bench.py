@@ -314,6 +314,11 @@ def mlp_bench(args):
 
     cfg = CONFIGS[args.config]
     d, ffn, r, K = cfg["d"], cfg["ffn"], cfg["r"], cfg["K"]
+    if args.K is not None:
+        if not 1 <= args.K <= ffn:
+            print(f"bench.py: --K must be in 1..{ffn}", file=sys.stderr)
+            sys.exit(2)
+        K = args.K
     torch.cuda.set_device(0)
     sets = [make_mlp(cfg, batch=64, device="cuda", seed=s) for s in range(N_LAYERS)]
     weight_bytes = 2 * K * d * 2
@@ -388,6 +393,8 @@ def main():
                          "counters, and skip the replay-spread and window-start legs (thousands of dispatches)")
     ap.add_argument("--batches", type=int, nargs="+", default=[1, 4, 8, 16, 32],
                     help="batch sizes of --workload mlp")
+    ap.add_argument("--K", type=int, default=None,
+                    help="--workload mlp: active neurons (default: the configuration's K; K = ffn is the dense block)")
     ap.add_argument("--workload", default="layer", choices=["layer", "decode", "mlp"],
                     help="layer: the headline sparse decode layer; decode: end-to-end greedy generation "
                          "(40-layer OPT-13B shape, --steps = new tokens, default 256)")
