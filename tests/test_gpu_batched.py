@@ -65,6 +65,11 @@ def test_batched_mlp_sparse_at_the_headline_shape(ops):
     test_batched_mlp_sparse_matches_oracle(ops, "opt-175b", 32, 4096, torch.int64)
 
 
+def test_batched_mlp_sparse_at_the_opt66b_shape(ops):
+    """OPT-66B-shaped block at batch 16: one full batch tile on the matrix cores."""
+    test_batched_mlp_sparse_matches_oracle(ops, "opt-66b", 16, 4096, torch.int64)
+
+
 @pytest.mark.parametrize("B", [11, 27, 40])  # one / two batch tiles; fc2 split by rows / by columns
 def test_batched_edge_cases(ops, B):
     g = torch.Generator().manual_seed(3)
