@@ -4,6 +4,8 @@
 #include "../../include/dejavu_hip.h"
 
 #include <hip/hip_runtime.h>
+
+#include <atomic>
 #include <stdlib.h>
 
 #include "attention.hpp"
@@ -25,18 +27,43 @@ inline bool idx_ok(int idx_bytes) { return idx_bytes == 4 || idx_bytes == 8; }
 
 inline int launch_status() { return hipGetLastError() == hipSuccess ? DV_OK : DV_ERR_LAUNCH; }
 
-int compute_units() {
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0, v = 0;
-    if (hipGetDevice(&dev) == hipSuccess &&
-        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
-      cus = v;
-    else
-      cus = 256;
-  }
-  return cus;
+constexpr int kMaxDevices = 64;
+
+int current_device() {
+  int dev = 0;
+  return (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < kMaxDevices) ? dev : -1;
 }
+
+// Compute units of the current device (remembered per device).
+int compute_units() {
+  static std::atomic<int> cus[kMaxDevices];
+  const int dev = current_device();
+  if (dev < 0) return 256;
+  int v = cus[dev].load(std::memory_order_relaxed);
+  if (v == 0) {
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
+    cus[dev].store(v, std::memory_order_relaxed);
+  }
+  return v;
+}
+
+// Dynamic LDS above 48 KiB has to be granted per kernel and per device.  One object per kernel
+// (static storage: starts at zero) remembers the largest size granted on each device, so a steady
+// stream of calls asks the runtime for nothing but the current device.
+struct LdsGrant {
+  std::atomic<size_t> granted[kMaxDevices];
+  int ensure(const void* fn, size_t bytes) {
+    if (bytes <= 48 * 1024) return DV_OK;
+    if (bytes > 160 * 1024) return DV_ERR_UNSUPPORTED;
+    const int dev = current_device();
+    if (dev < 0) return DV_ERR_UNSUPPORTED;
+    if (bytes <= granted[dev].load(std::memory_order_relaxed)) return DV_OK;
+    if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess)
+      return DV_ERR_UNSUPPORTED;
+    granted[dev].store(bytes, std::memory_order_relaxed);
+    return DV_OK;
+  }
+};
 
 // ---- canonical (predictor) GEMV -------------------------------------------
 template <int LANES, int U>
@@ -90,14 +117,8 @@ int launch_gather_rows(const half_t* x, const half_t* W, int64_t ldw, const half
                        hipStream_t s) {
   auto kern = gather_rows_kernel<B, R, U, RELU>;
   const size_t lds = (size_t)B * N * sizeof(half_t);
-  if (lds > 160 * 1024) return DV_ERR_UNSUPPORTED;
-  static size_t lds_granted = 48 * 1024;
-  if (lds > lds_granted) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-      return DV_ERR_UNSUPPORTED;
-    lds_granted = lds;
-  }
+  static LdsGrant grant;
+  if (int rc = grant.ensure(reinterpret_cast<const void*>(kern), lds); rc != DV_OK) return rc;
   const int ntasks = (M + R - 1) / R;
   int blocks = (ntasks + 3) / 4;
   const int cap = compute_units() * 8;
@@ -219,13 +240,8 @@ int launch_rows_mfma(const half_t* x, const half_t* W, int64_t ldw, const half_t
   const size_t tile_bytes = (size_t)kMfmaWaves * (XLDS ? 2 : 1) * kMfmaRows * kMfmaLdsRow * sizeof(half_t);
   const size_t red_bytes = (size_t)kMfmaWaves * BT * 4 * 64 * sizeof(float);
   const size_t lds = tile_bytes > red_bytes ? tile_bytes : red_bytes;
-  static bool granted = false;
-  if (!granted) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-      return DV_ERR_UNSUPPORTED;
-    granted = true;
-  }
+  static LdsGrant grant;
+  if (int rc = grant.ensure(reinterpret_cast<const void*>(kern), lds); rc != DV_OK) return rc;
   int blocks = (M + kMfmaRows - 1) / kMfmaRows;
   const int cap = compute_units() * 4;
   if (blocks > cap) blocks = cap;
@@ -290,13 +306,10 @@ int rows_mfma_dense(const half_t* x, const half_t* W, int64_t ldw, int B, int N,
   do {                                                                                                    \
     const size_t red_bytes = (size_t)kMfmaWaves * BT * 4 * 64 * sizeof(float);                            \
     const size_t lds = tile_bytes > red_bytes ? tile_bytes : red_bytes;                                   \
-    static size_t granted = 48 * 1024;                                                                    \
-    if (lds > granted) {                                                                                  \
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(gather_rows_mfma_kernel<BT, false, false, true>), \
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)        \
-        return DV_ERR_UNSUPPORTED;                                                                        \
-      granted = lds;                                                                                      \
-    }                                                                                                     \
+    static LdsGrant grant;                                                                                \
+    if (int rc = grant.ensure(reinterpret_cast<const void*>(gather_rows_mfma_kernel<BT, false, false, true>), lds); \
+        rc != DV_OK)                                                                                      \
+      return rc;                                                                                          \
     hipLaunchKernelGGL((gather_rows_mfma_kernel<BT, false, false, true>), grid, dim3(kMfmaWaves * 64), lds, s, x, \
                        W, nullptr, nullptr, B, N, ldw, M, M, y, p.chunks_per_split, partial);             \
   } while (0)
@@ -330,14 +343,8 @@ int launch_rows_short(const half_t* x, const half_t* W, int64_t ldw, int B, int 
   const int nchunks = (N + kMfmaKC - 1) / kMfmaKC;
   const size_t lds = ((size_t)16 * BT * (nchunks * kMfmaKC + kMfmaRowPad) +
                       (size_t)best_w * kMfmaRows * kMfmaLdsRow) * sizeof(half_t);
-  if (lds > 160 * 1024) return DV_ERR_UNSUPPORTED;
-  static size_t lds_granted = 48 * 1024;
-  if (lds > lds_granted) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(rows_short_mfma_kernel<BT>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-      return DV_ERR_UNSUPPORTED;
-    lds_granted = lds;
-  }
+  static LdsGrant grant;
+  if (int rc = grant.ensure(reinterpret_cast<const void*>(rows_short_mfma_kernel<BT>), lds); rc != DV_OK) return rc;
   int grid = (ntiles + best_w - 1) / best_w;
   if (grid > cus) grid = cus;
   hipLaunchKernelGGL((rows_short_mfma_kernel<BT>), dim3(grid), dim3(best_w * 64), lds, s, x, W, ldw, B, N, M, y);
@@ -861,16 +868,11 @@ inline int out_rows_blocks(int N) {
   return blocks > cap ? cap : blocks;
 }
 int grant_out_rows_lds(int hd, size_t lds) {
-  static size_t granted[2] = {48 * 1024, 48 * 1024};
+  static LdsGrant grant[2];
   const int v = hd == 128 ? 1 : 0;
-  if (lds <= granted[v]) return DV_OK;
   const void* fn = v ? reinterpret_cast<const void*>(out_proj_rows_attn_kernel<kOutRowsR, 128>)
                      : reinterpret_cast<const void*>(out_proj_rows_attn_kernel<kOutRowsR, 64>);
-  if (lds > 160 * 1024 ||
-      hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-    return DV_ERR_UNSUPPORTED;
-  granted[v] = lds;
-  return DV_OK;
+  return grant[v].ensure(fn, lds);
 }
 int launch_out_rows_attn(const float* part, int nsplit, const half_t* W, const half_t* bias, const int* head_idx,
                          int nnz, int H, int hd, int N, half_t* y, const half_t* rin, half_t* rout,
@@ -1221,12 +1223,8 @@ int dv_sparse_layer_decode_f16(const dvSparseLayerArgs* args, void* stream) {
     const void* l7[3] = {reinterpret_cast<const void*>(layer_l7_kernel<1>),
                          reinterpret_cast<const void*>(layer_l7_kernel<2>),
                          reinterpret_cast<const void*>(layer_l7_kernel<4>)};
-    static size_t lds_granted[3] = {48 * 1024, 48 * 1024, 48 * 1024};
-    if (lds > lds_granted[v]) {
-      if (hipFuncSetAttribute(l7[v], hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-        return DV_ERR_UNSUPPORTED;
-      lds_granted[v] = lds;
-    }
+    static LdsGrant grant[3];
+    if (int rc = grant[v].ensure(l7[v], lds); rc != DV_OK) return rc;
     int* att_out = reinterpret_cast<int*>(a.att_idx_out);
     const dim3 grid(nf + nm + 1);  // + the head top-k
     if (v == 0)
