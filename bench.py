@@ -292,7 +292,7 @@ def decode_bench(args):
         "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": "opt-13b-shaped greedy decode", "layers": layers, "d": d, "ffn": ffn, "heads": H,
                    "K": K, "active_heads": Hk, "vocab": vocab, "prompt": prompt_len, "new_tokens": new_tokens,
-                   "hip_graphs": 16},
+                   "hip_graphs": "one graph per 16-token back-fill window"},
         "prompt_ms": round(t_prompt * 1e3, 2), "total_ms": round(t_total * 1e3, 2),
         "eager_total_ms": round(t_eager * 1e3, 2), "graph_equals_eager": same,
         "us_per_layer": round(decode_s / steps / layers * 1e6, 2),
@@ -385,7 +385,8 @@ def main():
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying HIP graphs")
-    ap.add_argument("--single-stream", action="store_true", help="no side stream for predictors / top-k")
+    ap.add_argument("--side-stream", action="store_true",
+                    help="module path: predictors / top-k on a side stream, as the reference's sp_stream (slower here)")
     ap.add_argument("--graph-per-step", action="store_true",
                     help="one HIP graph per step even when the step counts allow one graph per schedule period")
     ap.add_argument("--pmc-calibration", action="store_true",
@@ -410,6 +411,7 @@ def main():
     import dejavu_amd.modules as dv_modules
     from dejavu_amd.workloads import CONFIGS
 
+    dv_modules.USE_SIDE_STREAM = args.side_stream
     if args.workload == "decode":
         args.steps = 256 if args.steps is None else args.steps
         args.warmup = 1 if args.warmup is None else args.warmup
@@ -419,7 +421,6 @@ def main():
         return mlp_bench(args)
     args.steps = 960 if args.steps is None else args.steps
     args.warmup = 192 if args.warmup is None else args.warmup
-    dv_modules.USE_SIDE_STREAM = not args.single_stream
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(1)

@@ -15,7 +15,9 @@ call site Dejavu/benchmarks/benchmark_generation_opt_dejavu.py:187-196).  With
 token / position / sequence length) is replayed from HIP graphs: the values that
 change from token to token live in device buffers, and the one host-side
 quantity a step depends on, the position inside the 16-token back-fill window,
-selects one of 16 graphs.
+selects the graph: one graph holds a whole window (16 tokens per launch), and 16
+single-position graphs serve the tokens before the first and after the last whole
+window.
 """
 from __future__ import annotations
 
@@ -285,8 +287,32 @@ class GPTLMHeadModel(nn.Module):
 
         mixers = self._sparse_mixers()
         window = ParallelMHASparseAttMlp.WINDOW
-        for step in range(n_new - 1):
+        total = n_new - 1
+        step = 0
+        while step < total:
             c = step % window  # position inside the back-fill window (== every sparse mixer's counter)
+            if cg and c == 0 and total - step >= window and (step >= window or "window" in cache.graphs):
+                # A whole back-fill window (16 tokens) is one graph: the gap between two graph
+                # launches is paid once per window instead of once per token.  Captured once every
+                # position has run eagerly (workspaces exist then); nothing in it depends on the
+                # host: token, position and sequence length live on the device.
+                if "window" not in cache.graphs:
+                    offset = ip.sequence_len_offset
+                    g = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(g):
+                        for _ in range(window):
+                            self._decode_step(cache, vocab_size)
+                            dv_modules.join_side_stream()
+                            ip.sequence_len_offset += 1
+                    ip.sequence_len_offset = offset
+                    cache.graphs["window"] = g
+                    cache.counters_after["window"] = [m.counter for m in mixers]
+                cache.graphs["window"].replay()
+                for m, v in zip(mixers, cache.counters_after["window"]):
+                    m.counter = v
+                ip.sequence_len_offset += window
+                step += window
+                continue
             if cg and (step >= window or c in cache.graphs):
                 # a window position is captured once it has run eagerly (workspaces exist then);
                 # later generations replay the graphs from their first decode step on
@@ -303,6 +329,7 @@ class GPTLMHeadModel(nn.Module):
             else:
                 self._decode_step(cache, vocab_size)
             ip.sequence_len_offset += 1
+            step += 1
         sequences = cache.sequences.clone()
         if return_dict_in_generate:
             return GreedySearchDecoderOnlyOutput(sequences=sequences,

@@ -27,9 +27,13 @@ from . import ops
 from ._lib import check, lib
 
 
-# Side-stream overlap of predictor / top-k work with the main kernels.  Off = everything
-# is enqueued on the current stream in program order.
-USE_SIDE_STREAM = True
+# Side-stream overlap of predictor / top-k work with the main kernels (the reference's
+# sp_stream).  Off = everything is enqueued on the current stream in program order.  Off by
+# default: on one GPU there is no all-reduce to hide the predictors behind, the kernels are
+# bandwidth-bound either way, and a fork / join inside a captured decode step slows the whole
+# graph down (greedy decode of the 40-layer OPT-13B shape, only the dense first block on the
+# module path: 322 tokens/s with the side stream, 357 without; eager 792 -> 765 ms).
+USE_SIDE_STREAM = False
 
 _side_streams: dict = {}
 

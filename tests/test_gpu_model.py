@@ -117,7 +117,7 @@ def test_graph_replayed_generation_equals_eager_bit_for_bit():
     L, d, H, ffn, r, V, P = 4, 256, 4, 2048, 64, 512, 128
     model, _ = build(L, d, H, ffn, r, V, P, 512, (2, 3), seed=23)
     prompt = torch.tensor([[9, 100, 31, 77, 2]], device="cuda")
-    n_new = 70  # 16 eager steps, then every window position replayed at least three times
+    n_new = 70  # 16 eager steps, three replays of the whole-window graph, five single-position graphs
     print("case generate eager (reference for graphs)", flush=True)
     eager = model.generate(prompt, max_length=5 + n_new, return_dict_in_generate=True, output_scores=True)
     torch.cuda.synchronize()
@@ -126,7 +126,7 @@ def test_graph_replayed_generation_equals_eager_bit_for_bit():
     torch.cuda.synchronize()
     assert torch.equal(g1.sequences, eager.sequences)
     assert torch.equal(g1.scores, eager.scores)
-    assert len(model._decoding_cache.graphs) == 16
+    assert set(model._decoding_cache.graphs) == {"window", 0, 1, 2, 3, 4}
     # second call: all graphs exist; a different prompt of the same length must not see stale state
     prompt2 = torch.tensor([[1, 2, 3, 4, 5]], device="cuda")
     print("case generate cg=True, second call (replays only)", flush=True)
@@ -144,6 +144,34 @@ def test_graph_replayed_generation_equals_eager_bit_for_bit():
     e3 = model.generate(prompt3, max_length=5 + n_new, return_dict_in_generate=True, output_scores=True)
     torch.cuda.synchronize()
     assert torch.equal(g3.sequences, e3.sequences)
+
+
+def test_side_stream_generation_equals_single_stream_bit_for_bit():
+    """The reference's sp_stream overlap (predictors and top-ks on a side stream) is optional
+    here and off by default: same tokens and scores either way, eager and from graphs."""
+    import dejavu_amd.modules as dv_modules
+
+    L, d, H, ffn, r, V, P = 3, 256, 4, 2048, 64, 512, 128
+    model, _ = build(L, d, H, ffn, r, V, P, 512, (2, 3), seed=29)
+    prompt = torch.tensor([[3, 14, 15, 92, 65, 35]], device="cuda")
+    assert dv_modules.USE_SIDE_STREAM is False
+    print("case generate single stream", flush=True)
+    single = model.generate(prompt, max_length=6 + 40, return_dict_in_generate=True, output_scores=True)
+    torch.cuda.synchronize()
+    try:
+        dv_modules.USE_SIDE_STREAM = True
+        model._decoding_cache = None
+        print("case generate side stream, eager", flush=True)
+        side = model.generate(prompt, max_length=6 + 40, return_dict_in_generate=True, output_scores=True)
+        torch.cuda.synchronize()
+        print("case generate side stream, graphs", flush=True)
+        side_cg = model.generate(prompt, max_length=6 + 40, cg=True, return_dict_in_generate=True, output_scores=True)
+        torch.cuda.synchronize()
+    finally:
+        dv_modules.USE_SIDE_STREAM = False
+        model._decoding_cache = None
+    assert torch.equal(side.sequences, single.sequences) and torch.equal(side.scores, single.scores)
+    assert torch.equal(side_cg.sequences, single.sequences) and torch.equal(side_cg.scores, single.scores)
 
 
 @pytest.mark.parametrize("vocab", [7, 512, 8200, 50272, 50277, 70001])
