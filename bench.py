@@ -274,7 +274,7 @@ def decode_bench(args):
             return time.perf_counter() - t0, out
 
         for _ in range(max(1, args.warmup)):
-            run(True)  # first call captures the 16 graphs
+            run(True)  # first call captures the graphs
         t_total, seq_cg = min((run(True) for _ in range(3)), key=lambda r: r[0])
         t_prompt, _ = min((run(True, prompt_len + 1) for _ in range(3)), key=lambda r: r[0])
         t_eager, seq_eager = run(False)
