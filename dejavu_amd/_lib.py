@@ -50,6 +50,10 @@ SIGNATURES = {
         [_c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_size,
          _c_ptr],
     ),
+    "dv_gather_transposed_gemv_static_f16": (
+        _c_int,
+        [_c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr],
+    ),
     "dv_qkv_proj_sparse_f16": (
         _c_int, [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr]),
     "dv_qkv_proj_sparse_cache_f16": (

@@ -711,6 +711,46 @@ int dv_gather_transposed_gemv_f16(const void* x, const void* W, int64_t ldw, con
                      reinterpret_cast<hipStream_t>(stream));
 }
 
+}  // extern "C"
+namespace {
+// Scratch of dv_gather_transposed_gemv_static_f16: one array per device, resident until the
+// process ends.  In host code the array's name is only a handle: the device address comes from
+// hipGetSymbolAddress, once per device, and is what the kernels are given.
+__device__ __align__(256) unsigned char scratch[DV_STATIC_SCRATCH_BYTES];
+std::atomic<void*> scratch_ptr[kMaxDevices];
+
+int static_scratch(void** out) {
+  const int dev = current_device();
+  if (dev < 0) return DV_ERR_UNSUPPORTED;
+  void* p = scratch_ptr[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) {
+      (void)hipGetLastError();
+      return DV_ERR_LAUNCH;
+    }
+    scratch_ptr[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return DV_OK;
+}
+}  // namespace
+extern "C" {
+
+int dv_gather_transposed_gemv_static_f16(const void* x, const void* W, int64_t ldw, const void* bias,
+                                         const void* idx, int idx_bytes, int B, int N, int Z, int M,
+                                         void* y, void* stream) {
+  if (B < 1 || N < 1 || M < 0) return DV_ERR_INVALID_ARG;
+  if (B > 64) return DV_ERR_UNSUPPORTED;
+  // the partial sums of this shape must fit the fixed array; nothing is allocated here
+  const size_t need = dv_gather_transposed_gemv_workspace_bytes(B, N, M);
+  if (need > (size_t)DV_STATIC_SCRATCH_BYTES) return DV_ERR_WORKSPACE;
+  void* ws = nullptr;
+  if (int rc = static_scratch(&ws); rc != DV_OK) return rc;
+  // every word of the partial sums is written before it is read: nothing to clear between calls
+  return dv_gather_transposed_gemv_f16(x, W, ldw, bias, idx, idx_bytes, B, N, Z, M, y, ws,
+                                       (size_t)DV_STATIC_SCRATCH_BYTES, stream);
+}
+
 int dv_qkv_proj_sparse_cache_f16(const void* x, const void* W, const void* bias,
                                  const void* head_idx, const void* batch_idx, int nb, int d, int H,
                                  int hd, int nnz, void* y, void* k_cache, void* v_cache,

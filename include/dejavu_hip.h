@@ -129,6 +129,23 @@ DV_API int dv_gather_transposed_gemv_f16(const void* x, const void* W, int64_t l
                                   void* stream);
 
 /*
+ * dv_gather_transposed_gemv_f16 without a workspace argument and without any allocation: the
+ * fp32 partial sums of the split go to a fixed DV_STATIC_SCRATCH_BYTES array in device memory
+ * that belongs to the library (one per GPU, held until the process ends).  It has no
+ * counterpart in the reference; it is for callers that cannot allocate or size scratch memory:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * Same kernels and same bits as dv_gather_transposed_gemv_f16.  Shapes whose partial sums
+ * exceed the array (dv_gather_transposed_gemv_workspace_bytes(B, N, M) >
+ * DV_STATIC_SCRATCH_BYTES: at the OPT shapes, batches above 32) return DV_ERR_WORKSPACE.
+ * All calls on one GPU share the array: calls that overlap in time on different streams of one
+ * GPU race.  The array needs no clearing between calls (every word is written before it is read).
+ */
+#define DV_STATIC_SCRATCH_BYTES (8u << 20)
+DV_API int dv_gather_transposed_gemv_static_f16(const void* x, const void* W, int64_t ldw,
+                                                const void* bias, const void* idx, int idx_bytes,
+                                                int B, int N, int Z, int M, void* y, void* stream);
+
+/*
  * QKV projection restricted to the active heads and the live window tokens:
  *   y[b, t, h, :] = x[b, :] . W[t, h, :, :]^T + bias[t, h, :]
  * for h = head_idx[i] and every b = batch_idx[i, s] >= 0.  Nothing is written
