@@ -35,6 +35,16 @@ How each function is pinned (see tests/test_oracle.py):
   predictions feed layer l+1, the first layer runs dense).  The greedy loop
   itself restates flash-attention v0.2.8 ``flash_attn/utils/generation.py``
   (``decode``), a dependency the reference does not vendor.
+* ``sparse_attention_step_dense_kv``: against a float64 dense QKV projection,
+  torch SDPA and the head-masked dense out_proj of the accuracy simulator, and
+  against a pure-Python brute force on a tiny shape.
+* ``batched_sparse_attention_step`` / ``block_decode_step_batched`` (batch
+  extension, not in the reference, which asserts batch 1): row b against the
+  single-sequence functions run on sequence b alone with the shared selections
+  (bit-equal), against per-sequence float64 attention + head-masked out_proj,
+  and B = 1 against ``block_decode_step`` (bit-equal).
+* ``WindowTracker``: against a literal index-by-index replay of the reference's
+  ParallelTracker calls over several windows.
 * top-k tie order: the reference (``torch.topk(sorted=False)`` on CUDA) leaves
   it unspecified and holds no vectors; the rule "ties go to the lower index" is
   this build's definition: parity unpinned against the reference's CUDA tie
@@ -563,6 +573,64 @@ def block_decode_step(p, hidden_states, residual, head_idx, mlp_sp_logit, k_cach
     r2_pred = r2 if residual2_override is None else np.asarray(residual2_override, F16)
     _, next_mlp_logit = predictor_logits(r2_pred, p["mlp_Wa"], p["mlp_Wb"])
     return dict(hidden=hidden, residual=r2, next_mlp_logit=next_mlp_logit[0], next_att_idx=next_att_idx,
+                mlp_idx=mlp_idx, residual1=r1, attn_out=attn_out)
+
+
+def batched_sparse_attention_step(x, Wqkv, bqkv, Wout, bout, head_idx, k_cache, v_cache, lengths,
+                                  softmax_scale=None):
+    """Head-sparse attention for B sequences that each decode one token, with ONE
+    head set shared by the batch and one KV cache per sequence.
+
+    The reference's sparse attention is single-sequence
+    (Dejavu/src/models/modules/mha_dejavu.py:1469 asserts batch 1); this is the
+    batch extension the benchmark configurations ask for, built from the same
+    three steps in the same order (mha_dejavu.py:1333-1352 QKV of the selected
+    heads, :1439-1446 one-query attention that appends k, v at the sequence's
+    own position, :1472-1482 out_proj over the selected heads), each applied to
+    every row of the batch.
+    x: (B, d) LayerNorm-1 outputs; Wqkv (3, H, hd, d); bqkv (3, H, hd) or None;
+    Wout (d, H, hd); bout (d,) or None; head_idx (Hk,) int32;
+    k_cache (B, H, hd/8, S, 8), v_cache (B, H, S, hd): complete for the
+    selected heads up to lengths[b] - 1, updated in place at lengths[b].
+    Returns (out (B, d) fp16, ctx (B, H, hd) fp16, zero outside head_idx).
+    """
+    x = np.asarray(x, F16)
+    B = x.shape[0]
+    hi = np.asarray(head_idx, dtype=np.int32)
+    rows = np.tile(np.arange(B, dtype=np.int32), (len(hi), 1))
+    qkv = qkv_proj_sparse(x, Wqkv, hi, rows, bqkv)
+    ctx = single_query_attention(qkv[:, 0], qkv[:, 1], qkv[:, 2], k_cache, v_cache, 0, softmax_scale=softmax_scale,
+                                 head_idx=hi, lengths_per_sample=np.asarray(lengths).astype(np.int64))
+    out = out_proj_sparse(ctx, Wout, hi, bout)
+    return out, ctx
+
+
+def block_decode_step_batched(p, hidden_states, residual, head_idx, mlp_sp_logit, k_cache, v_cache, lengths):
+    """``block_decode_step`` for B sequences decoding one token each.
+
+    Same algebra per row (Dejavu/src/models/modules/block_dejavu.py:555-663).
+    The selections are shared by the batch: the MLP neurons are the top-K of the
+    column-wise maximum of the (B, ffn) predictor logits ("union of the
+    per-token top-K, capped at K", see ``batch_scores``), and the heads predicted
+    for the next block are the top-att_K of the column-wise maximum of the
+    (B, H) head logits, by the same rule.  hidden_states, residual: (B, d);
+    head_idx (Hk,) int32; mlp_sp_logit (B, ffn); caches per sequence, see
+    ``batched_sparse_attention_step``.  For B = 1 this is ``block_decode_step``.
+    Returns dict(hidden, residual, next_mlp_logit (B, ffn), next_att_idx, mlp_idx, residual1, attn_out).
+    """
+    r1 = _add_f16(hidden_states, residual) if residual is not None else np.asarray(hidden_states, F16)
+    x = layer_norm(r1, p["ln1_w"], p["ln1_b"])
+    hi = np.asarray(head_idx, dtype=np.int32)
+    attn_out, _ = batched_sparse_attention_step(x, p["Wqkv"], p["bqkv"], p["Wout"], p["bout"], hi, k_cache, v_cache,
+                                                lengths)
+    mlp_idx = topk_lower_index(mlp_sp_logit, p["mlp_K"])
+    _, att_logit = predictor_logits(r1, p["att_Wa"], p["att_Wb"])
+    next_att_idx = topk_lower_index(att_logit, p["att_K"]).astype(np.int32)
+    r2 = _add_f16(attn_out, r1)
+    x2 = layer_norm(r2, p["ln2_w"], p["ln2_b"])
+    hidden = mlp_sparse(x2, p["W1"], p["W2t"], mlp_idx, p["b1"], p["b2"])
+    _, next_mlp_logit = predictor_logits(r2, p["mlp_Wa"], p["mlp_Wb"])
+    return dict(hidden=hidden, residual=r2, next_mlp_logit=next_mlp_logit, next_att_idx=next_att_idx,
                 mlp_idx=mlp_idx, residual1=r1, attn_out=attn_out)
 
 

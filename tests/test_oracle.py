@@ -353,3 +353,259 @@ def test_layer_norm_matches_torch():
     ref = torch.nn.functional.layer_norm(torch.from_numpy(x.astype(np.float32)), (256,),
                                          torch.from_numpy(w.astype(np.float32)), torch.from_numpy(b.astype(np.float32))).numpy()
     assert np.allclose(O.layer_norm(x, w, b).astype(np.float32), ref, rtol=2e-3, atol=2e-3)
+
+
+# ------------------------------------------------- attention step, dense K/V
+def _attention_case(g, T=9, H=5, hd=16, d=80):
+    x_hist = randn16(g, T, d)
+    Wqkv = randn16(g, 3, H, hd, d, std=0.08)
+    bqkv = randn16(g, 3, H, hd, std=0.1)
+    Wout = randn16(g, d, H, hd, std=0.08)
+    bout = randn16(g, d, std=0.1)
+    return x_hist, Wqkv, bqkv, Wout, bout
+
+
+def test_sparse_attention_step_dense_kv_matches_float64_sdpa_and_masked_out_proj():
+    """float64 dense QKV projection of every token -> torch SDPA for the newest query -> heads outside
+    the selection zeroed -> dense out_proj (hf_opt_sparse_mlp_attention.py:365-373)."""
+    g = rng(21)
+    x_hist, Wqkv, bqkv, Wout, bout = _attention_case(g, T=33, H=6, hd=32, d=192)
+    T, d = x_hist.shape
+    H, hd = Wqkv.shape[1:3]
+    head_idx = np.array([4, 0, 3], dtype=np.int32)
+    out, ctx = O.sparse_attention_step_dense_kv(x_hist, Wqkv, bqkv, Wout, bout, head_idx)
+    qkv = (x_hist.astype(np.float64) @ Wqkv.astype(np.float64).reshape(3 * H * hd, d).T
+           + bqkv.astype(np.float64).reshape(-1)).reshape(T, 3, H, hd)
+    q = torch.from_numpy(qkv[-1:, 0]).permute(1, 0, 2).unsqueeze(0)  # (1, H, 1, hd)
+    k = torch.from_numpy(qkv[:, 1]).permute(1, 0, 2).unsqueeze(0)    # (1, H, T, hd)
+    v = torch.from_numpy(qkv[:, 2]).permute(1, 0, 2).unsqueeze(0)
+    ref_ctx = torch.nn.functional.scaled_dot_product_attention(q, k, v)[0, :, 0].numpy()  # (H, hd)
+    mask = np.zeros(H)
+    mask[head_idx] = 1
+    ref_out = (ref_ctx * mask[:, None]).reshape(-1) @ Wout.astype(np.float64).reshape(d, H * hd).T + bout.astype(np.float64)
+    assert np.all(ctx[[1, 2, 5]] == 0)
+    assert np.abs(ctx[head_idx].astype(np.float64) - ref_ctx[head_idx]).max() <= 4e-3
+    err = out.astype(np.float64) - ref_out
+    assert np.abs(err).max() <= 1e-2 and np.linalg.norm(err) / np.linalg.norm(ref_out) <= 2e-3
+    # a different selection must change the answer (the mask is not a no-op)
+    out2, _ = O.sparse_attention_step_dense_kv(x_hist, Wqkv, bqkv, Wout, bout, np.array([4, 0], dtype=np.int32))
+    assert np.abs(out2.astype(np.float64) - ref_out).max() > 2e-2
+
+
+def test_sparse_attention_step_dense_kv_tiny_bruteforce():
+    """Scalar loops over a tiny case: softmax(q.k/sqrt(hd)) v per selected head, then the out_proj sum over
+    the selected heads only."""
+    import math
+
+    g = rng(22)
+    x_hist, Wqkv, bqkv, Wout, bout = _attention_case(g, T=4, H=3, hd=8, d=24)
+    T, d = x_hist.shape
+    H, hd = Wqkv.shape[1:3]
+    head_idx = [2, 0]
+    out, _ = O.sparse_attention_step_dense_kv(x_hist, Wqkv, bqkv, Wout, bout, np.array(head_idx, dtype=np.int32))
+    xf, Wf, bf = x_hist.astype(float), Wqkv.astype(float), bqkv.astype(float)
+    want = [float(bout[n]) for n in range(d)]
+    for h in head_idx:
+        proj = lambda t, s: [sum(Wf[t, h, j, c] * xf[s, c] for c in range(d)) + bf[t, h, j] for j in range(hd)]
+        q = proj(0, T - 1)
+        scores = [sum(a * b for a, b in zip(q, proj(1, s))) / math.sqrt(hd) for s in range(T)]
+        m = max(scores)
+        w = [math.exp(v - m) for v in scores]
+        z = sum(w)
+        ctx = [sum(w[s] / z * proj(2, s)[j] for s in range(T)) for j in range(hd)]
+        for n in range(d):
+            want[n] += sum(float(Wout[n, h, j]) * ctx[j] for j in range(hd))
+    assert np.abs(out.astype(np.float64) - np.array(want)).max() <= 6e-3
+
+
+def test_sparse_attention_step_equals_cached_single_query_path():
+    """The dense-K/V closed form and the cache-based ops (qkv_proj_sparse of every token into the caches,
+    then single_query_attention + out_proj_sparse for the newest) are the same arithmetic: equal bits."""
+    g = rng(23)
+    x_hist, Wqkv, bqkv, Wout, bout = _attention_case(g, T=7, H=4, hd=16, d=64)
+    T, d = x_hist.shape
+    H, hd = Wqkv.shape[1:3]
+    head_idx = np.array([1, 3], dtype=np.int32)
+    out, ctx = O.sparse_attention_step_dense_kv(x_hist, Wqkv, bqkv, Wout, bout, head_idx)
+    every = np.tile(np.arange(T, dtype=np.int32), (len(head_idx), 1))
+    qkv = O.qkv_proj_sparse(x_hist, Wqkv, head_idx, every, bqkv)
+    k_cache = np.zeros((1, H, hd // 8, T, 8), F16)
+    v_cache = np.zeros((1, H, T, hd), F16)
+    O.k_cache_copy_sparse(qkv[:, 1], k_cache, head_idx, every[:, : T - 1])
+    O.v_cache_copy_sparse(qkv[:, 2], v_cache, head_idx, every[:, : T - 1])
+    ctx2 = O.single_query_attention(qkv[-1:, 0], qkv[-1:, 1], qkv[-1:, 2], k_cache, v_cache, T - 1, head_idx=head_idx)
+    assert np.array_equal(ctx2[0].view(np.uint16), ctx.view(np.uint16))
+    out2 = O.out_proj_sparse(ctx2, Wout, head_idx, bout)[0]
+    assert np.array_equal(out2.view(np.uint16), out.view(np.uint16))
+
+
+# ------------------------------------------- tracker against the reference's calls
+class _LiteralTracker:
+    """ParallelTracker (mha_dejavu.py:1124-1149) replayed entry by entry: a table of token ids per
+    head; get_batch_idx returns the first n entries of the listed heads' rows, update overwrites with
+    -1 exactly the entries whose returned value was not -1, reset re-arms rows to 0..15."""
+
+    def __init__(self, H):
+        self.H = H
+        self.reset()
+
+    def reset(self):
+        self.table = [[s for s in range(16)] for _ in range(self.H)]
+
+    def get_batch_idx(self, head_idx, n):
+        return [[self.table[h][s] for s in range(n)] for h in head_idx]
+
+    def update(self, head_idx, seq_idx, compute_idx):
+        for i, h in enumerate(head_idx):
+            for s in range(seq_idx + 1):
+                if compute_idx[i][s] != -1:
+                    self.table[h][s] = -1
+
+
+def test_window_tracker_matches_literal_replay_of_reference_calls():
+    """Drives the oracle's WindowTracker and the call sequence of ParallelMHASparseAttMlp.forward
+    (mha_dejavu.py:1318-1329 reset + all heads at counter 15, get_batch_idx(head_idx, counter + 1);
+    :1355-1359 update unless counter == 15, counter += 1; :1485-1492 counter wraps at 16) side by side
+    over three and a half windows with random head selections, including repeated and empty ones."""
+    g = rng(24)
+    H = 7
+    lit = _LiteralTracker(H)
+    counter = 0
+    tr = O.WindowTracker(H)
+    for step in range(56):
+        n_sel = int(g.integers(0, 4))
+        sel = np.sort(g.permutation(H)[:n_sel]).astype(np.int32)
+        # reference sequence
+        ref_heads = [int(h) for h in sel]
+        if counter == 15:
+            lit.reset()
+            ref_heads = list(range(H))
+        ref_idx = lit.get_batch_idx(ref_heads, counter + 1)
+        if counter != 15:
+            lit.update(ref_heads, counter, ref_idx)
+        counter += 1
+        wrapped_ref = counter == 16
+        if wrapped_ref:
+            counter = 0
+        # oracle
+        assert tr.counter == (counter - 1) % 16
+        heads, batch_idx = tr.begin_step(sel)
+        wrapped = tr.end_step(heads, batch_idx)
+        assert [int(h) for h in heads] == ref_heads
+        assert batch_idx.tolist() == ref_idx or (len(ref_heads) == 0 and batch_idx.size == 0)
+        assert wrapped == wrapped_ref
+        assert tr.tracker.tolist() == lit.table
+        assert tr.counter == counter
+
+
+# ------------------------------------------------------- batch extension
+def _block_params(g, d=64, H=4, hd=16, ffn=256, r=24, mlp_K=96, att_K=2):
+    return dict(ln1_w=randn16(g, d, std=0.1, mean=1.0), ln1_b=randn16(g, d, std=0.1),
+                ln2_w=randn16(g, d, std=0.1, mean=1.0), ln2_b=randn16(g, d, std=0.1),
+                Wqkv=randn16(g, 3, H, hd, d, std=0.08), bqkv=randn16(g, 3, H, hd, std=0.05),
+                Wout=randn16(g, d, H, hd, std=0.08), bout=randn16(g, d, std=0.05),
+                W1=randn16(g, ffn, d, std=0.08), b1=randn16(g, ffn, std=0.05, mean=-0.1),
+                W2t=randn16(g, ffn, d, std=0.08), b2=randn16(g, d, std=0.05),
+                mlp_Wa=randn16(g, r, d, std=0.1), mlp_Wb=randn16(g, ffn, r, std=0.1),
+                att_Wa=randn16(g, r, d, std=0.1), att_Wb=randn16(g, H, r, std=0.1), mlp_K=mlp_K, att_K=att_K)
+
+
+def _batch_caches(g, B, H, hd, S):
+    kc = randn16(g, B, S, H, hd)
+    return O.pack_k_cache(kc), randn16(g, B, H, S, hd)
+
+
+def test_batched_attention_step_rows_equal_single_sequence_runs():
+    """Row b of the batched step == the single-sequence ops on sequence b alone with the shared head set
+    (bit-equal), and == float64 attention + head-masked dense out_proj on that sequence (tolerance)."""
+    g = rng(25)
+    B, H, hd, d, S = 3, 5, 16, 80, 24
+    x = randn16(g, B, d)
+    _, Wqkv, bqkv, Wout, bout = _attention_case(g, T=1, H=H, hd=hd, d=d)
+    k_cache, v_cache = _batch_caches(g, B, H, hd, S)
+    lengths = np.array([5, 23, 0], dtype=np.int32)
+    head_idx = np.array([3, 1], dtype=np.int32)
+    k0, v0 = k_cache.copy(), v_cache.copy()
+    out, ctx = O.batched_sparse_attention_step(x, Wqkv, bqkv, Wout, bout, head_idx, k_cache, v_cache, lengths)
+    assert out.shape == (B, d) and ctx.shape == (B, H, hd)
+    for b in range(B):
+        t = int(lengths[b])
+        kb, vb = k0[b:b + 1].copy(), v0[b:b + 1].copy()
+        qkv = O.qkv_proj_sparse(x[b:b + 1], Wqkv, head_idx, np.zeros((2, 1), np.int32), bqkv)
+        c1 = O.single_query_attention(qkv[:, 0], qkv[:, 1], qkv[:, 2], kb, vb, t, head_idx=head_idx)
+        o1 = O.out_proj_sparse(c1, Wout, head_idx, bout)
+        assert np.array_equal(out[b].view(np.uint16), o1[0].view(np.uint16))
+        assert np.array_equal(ctx[b].view(np.uint16), c1[0].view(np.uint16))
+        # the batched call wrote this sequence's cache exactly as the single-sequence call did
+        assert np.array_equal(k_cache[b], kb[0]) and np.array_equal(v_cache[b], vb[0])
+        # float64: K/V of positions < t from the original cache, position t from the projection
+        K = O.unpack_k_cache(k0)[b].astype(np.float64)[:, : t + 1]  # (H, t+1, hd)
+        V = v0[b].astype(np.float64)[:, : t + 1]
+        proj = (Wqkv.astype(np.float64).reshape(3 * H * hd, d) @ x[b].astype(np.float64)
+                + bqkv.astype(np.float64).reshape(-1)).reshape(3, H, hd)
+        K[:, t], V[:, t] = proj[1], proj[2]
+        sc = np.einsum("hd,hsd->hs", proj[0], K) / np.sqrt(hd)
+        pr = np.exp(sc - sc.max(-1, keepdims=True))
+        pr /= pr.sum(-1, keepdims=True)
+        c64 = np.einsum("hs,hsd->hd", pr, V)
+        want = O.out_proj_head_masked(c64[None].astype(np.float32).astype(F16), Wout, head_idx, bout)[0]
+        err = out[b].astype(np.float64) - want
+        assert np.abs(err).max() <= 2e-2 and np.linalg.norm(err) / np.linalg.norm(want) <= 4e-3
+    # untouched: every cache entry outside (selected head, position lengths[b])
+    km, vm = np.ones_like(k0, bool), np.ones_like(v0, bool)
+    for b in range(B):
+        km[b, head_idx, :, lengths[b], :] = False
+        vm[b, head_idx, lengths[b], :] = False
+    assert np.array_equal(k_cache[km], k0[km]) and np.array_equal(v_cache[vm], v0[vm])
+
+
+def test_block_decode_step_batched_reduces_to_single_sequence_block():
+    g = rng(26)
+    p = _block_params(g)
+    d, H, hd, ffn = 64, 4, 16, 256
+    S = 20
+    k_cache, v_cache = _batch_caches(g, 1, H, hd, S)
+    hidden, residual = randn16(g, 1, d), randn16(g, 1, d)
+    logit = randn16(g, ffn)
+    head_idx = np.array([0, 2], dtype=np.int32)
+    ka, va = k_cache.copy(), v_cache.copy()
+    one = O.block_decode_step(p, hidden, residual, head_idx, logit, ka, va, 11)
+    kb, vb = k_cache.copy(), v_cache.copy()
+    bat = O.block_decode_step_batched(p, hidden, residual, head_idx, logit[None], kb, vb, np.array([11]))
+    for key in ("hidden", "residual", "residual1", "attn_out"):
+        assert np.array_equal(one[key].view(np.uint16), bat[key].view(np.uint16)), key
+    assert np.array_equal(one["next_mlp_logit"].view(np.uint16), bat["next_mlp_logit"][0].view(np.uint16))
+    assert np.array_equal(one["mlp_idx"], bat["mlp_idx"]) and np.array_equal(one["next_att_idx"], bat["next_att_idx"])
+    assert np.array_equal(ka, kb) and np.array_equal(va, vb)
+
+
+def test_block_decode_step_batched_shares_selections_and_keeps_rows_independent():
+    """Selections are the top-k of the column-wise maximum over the batch (a subset of the union of the
+    per-row top-k sets); given the selections, row b of every output depends on row b alone: it equals the
+    single-sequence block run with the shared index sets forced."""
+    g = rng(27)
+    B, d, H, hd, ffn, S = 4, 64, 4, 16, 256, 20
+    p = _block_params(g)
+    k_cache, v_cache = _batch_caches(g, B, H, hd, S)
+    hidden, residual = randn16(g, B, d), randn16(g, B, d)
+    logit = randn16(g, B, ffn)
+    lengths = np.array([3, 19, 7, 7], dtype=np.int32)
+    head_idx = np.array([1, 3], dtype=np.int32)
+    k0, v0 = k_cache.copy(), v_cache.copy()
+    bat = O.block_decode_step_batched(p, hidden, residual, head_idx, logit, k_cache, v_cache, lengths)
+    per_row = [set(O.topk_lower_index(logit[b], p["mlp_K"]).tolist()) for b in range(B)]
+    assert set(bat["mlp_idx"].tolist()) <= set().union(*per_row) and len(bat["mlp_idx"]) == p["mlp_K"]
+    colmax = logit.astype(np.float32).max(axis=0)
+    assert np.array_equal(bat["mlp_idx"], O.topk_bruteforce(colmax, p["mlp_K"]))
+    _, head_logit = O.predictor_logits(bat["residual1"], p["att_Wa"], p["att_Wb"])
+    assert np.array_equal(bat["next_att_idx"], O.topk_bruteforce(head_logit.astype(np.float32).max(axis=0), p["att_K"]))
+    for b in range(B):
+        # single-sequence block with the batch's neuron set forced: a logit row that is 1 on the set, 0 elsewhere
+        forced = np.zeros(ffn, F16)
+        forced[bat["mlp_idx"]] = 1
+        kb, vb = k0[b:b + 1].copy(), v0[b:b + 1].copy()
+        one = O.block_decode_step(p, hidden[b:b + 1], residual[b:b + 1], head_idx, forced, kb, vb, int(lengths[b]))
+        for key in ("hidden", "residual", "residual1", "attn_out"):
+            assert np.array_equal(one[key][0].view(np.uint16), bat[key][b].view(np.uint16)), (key, b)
+        assert np.array_equal(one["next_mlp_logit"].view(np.uint16), bat["next_mlp_logit"][b].view(np.uint16))
+        assert np.array_equal(k_cache[b], kb[0]) and np.array_equal(v_cache[b], vb[0])
