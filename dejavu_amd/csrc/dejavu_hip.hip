@@ -783,6 +783,32 @@ int dv_qkv_proj_sparse_f16(const void* x, const void* W, const void* bias, const
                                       nullptr, nullptr, 0, stream);
 }
 
+int dv_qkv_proj_batch_f16(const void* x, int64_t ldx, const void* W, const void* bias, const void* head_idx,
+                          const void* live, int live_stride, int nnz, int B, int d, int H, int hd, void* y,
+                          void* k_cache, void* v_cache, const void* positions, int per_sample, int pos_add,
+                          int S, void* stream) {
+  if (!x || !W || !y || B < 1 || d <= 0 || H <= 0 || nnz < 0 || (nnz > 0 && !head_idx) ||
+      ((k_cache == nullptr) != (v_cache == nullptr)) || (k_cache && S <= 0) || (live && live_stride < 1))
+    return DV_ERR_INVALID_ARG;
+  if (B > 32 || (hd != 32 && hd != 64 && hd != 128)) return DV_ERR_UNSUPPORTED;
+  if (d % 8 || ldx % 8 || ldx < d || !aligned16(x) || !aligned16(W)) return DV_ERR_ALIGNMENT;
+  if (nnz == 0) return DV_OK;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const dim3 grid(nnz * 3 * (hd / 16));
+#define DV_QB(XT)                                                                                          \
+  hipLaunchKernelGGL((qkv_batch_mfma_kernel<kQkvMfmaWaves, XT>), grid, dim3(kQkvMfmaWaves * 64), 0, s,      \
+                     reinterpret_cast<const half_t*>(x), ldx, reinterpret_cast<const half_t*>(W),          \
+                     reinterpret_cast<const half_t*>(bias), reinterpret_cast<const int*>(head_idx),        \
+                     reinterpret_cast<const int*>(live), live_stride, B, d, H, hd, nnz,                    \
+                     reinterpret_cast<half_t*>(y), reinterpret_cast<half_t*>(k_cache),                     \
+                     reinterpret_cast<half_t*>(v_cache), reinterpret_cast<const int*>(positions), per_sample, \
+                     pos_add, S)
+  if (B <= 16) DV_QB(1);
+  else DV_QB(2);
+#undef DV_QB
+  return launch_status();
+}
+
 int dv_kv_cache_copy_sparse_f16(const void* k, const void* v, int64_t ld_src, int nsrc,
                                 void* k_cache, void* v_cache, const void* head_idx,
                                 const void* seq_idx, int nnz, int nslots, const void* padding,

@@ -169,4 +169,151 @@ __global__ __launch_bounds__(WAVES * 64) void qkv_window_mfma_kernel(
                                      padding, S, blockIdx.x, gridDim.x);
 }
 
+// ---------------------------------------------------------------------------
+// QKV projection of the active heads for ONE token of each of B sequences
+// (B <= 16 * XT rows of X, all live), K / V rows appended to per-sequence caches.
+// Same tile scheme as qkv_window_mfma_body with one 16-row weight tile per
+// workgroup; XT batch tiles share every weight operand.  `live` (nnz, or null)
+// lets a pass skip heads: head i is computed when live[i * live_stride] >= 0
+// (a back-fill pass over one window token touches only the heads that miss it).
+// Cache position of row b: positions[per_sample ? b : 0] + pos_add (positions
+// null = 0); rows whose position falls outside [0, S) are projected but not
+// cached.  Caches: k_cache (B, H, hd/8, S, 8), v_cache (B, H, S, hd).
+// ---------------------------------------------------------------------------
+template <int WAVES, int XT>
+__device__ __forceinline__ void qkv_batch_mfma_body(
+    const half_t* __restrict__ X, int64_t ldx, const half_t* __restrict__ W, const half_t* __restrict__ bias,
+    const int* __restrict__ head_idx, const int* __restrict__ live, int live_stride, int B, int d, int H,
+    int hd, int nnz, half_t* __restrict__ Y, half_t* __restrict__ k_cache, half_t* __restrict__ v_cache,
+    const int* __restrict__ positions, int per_sample, int pos_add, int S, int block_id, int nblocks) {
+  constexpr int kTile = kMfmaRows * kMfmaLdsRow;
+  __shared__ __attribute__((aligned(16))) half_t s_tiles[WAVES][kTile];
+  static_assert(sizeof(half_t) * kTile >= XT * 256 * sizeof(float), "tile too small for the reduction");
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  half_t* tile = s_tiles[wave];
+  const int l16 = lane & 15, kg = lane >> 4;
+  const int l32 = lane & 31, half_id = lane >> 5;
+  const int groups_per_head = hd / 16;
+  const int ntasks = nnz * 3 * groups_per_head;
+  const int nchunks = (d + kMfmaKC - 1) / kMfmaKC;
+  constexpr int KS = kMfmaKC / 32;
+
+  const half_t* xrow[XT];
+  bool row_live[XT];
+#pragma unroll
+  for (int xt = 0; xt < XT; ++xt) {
+    const int n = xt * 16 + l16;
+    row_live[xt] = n < B;
+    xrow[xt] = X + (row_live[xt] ? (int64_t)n * ldx : 0);  // dead rows: one shared address
+  }
+
+  for (int task = block_id; task < ntasks; task += nblocks) {
+    const int i = task / (3 * groups_per_head);
+    const int rem = task - i * 3 * groups_per_head;
+    const int t = rem / groups_per_head;
+    const int j0 = (rem - t * groups_per_head) * 16;
+    const int h = head_idx[i];
+    if (h < 0 || h >= H) continue;  // uniform over the workgroup
+    if (live != nullptr && live[(int64_t)i * live_stride] < 0) continue;
+    const int64_t row0 = ((int64_t)t * H + h) * hd + j0;
+
+    float4_t acc[XT];
+#pragma unroll
+    for (int xt = 0; xt < XT; ++xt) acc[xt] = float4_t{0.f, 0.f, 0.f, 0.f};
+    half8_t stage[8];
+    auto load_stage = [&](int c) {
+      int col = c * kMfmaKC + l32 * 8;
+      if (col >= d) col = 0;  // masked when stored
+#pragma unroll
+      for (int q = 0; q < 8; ++q) stage[q] = load8_stream(W + (row0 + 2 * q + half_id) * d + col);
+    };
+    auto store_stage = [&](int c) {
+      const bool col_ok = c * kMfmaKC + l32 * 8 < d;
+      __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");  // previous tile fully read
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int q = 0; q < 8; ++q)
+        store8(tile + (2 * q + half_id) * kMfmaLdsRow + l32 * 8, col_ok ? stage[q] : zero8());
+      __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+    };
+    half8_t xb[XT][KS];
+    auto load_x = [&](int c) {
+#pragma unroll
+      for (int xt = 0; xt < XT; ++xt)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          int kk = c * kMfmaKC + ks * 32 + kg * 8;
+          if (kk >= d || !row_live[xt]) kk = 0;
+          xb[xt][ks] = load8(xrow[xt] + kk);
+        }
+    };
+    // columns beyond d meet zeros in the weight tile; the accumulator columns of dead rows are never stored
+    auto multiply = [&]() {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const half8_t a = load8(tile + l16 * kMfmaLdsRow + ks * 32 + kg * 8);
+#pragma unroll
+        for (int xt = 0; xt < XT; ++xt) acc[xt] = mfma_16x16x32(a, xb[xt][ks], acc[xt]);
+      }
+    };
+
+    int c = wave;
+    if (c < nchunks) {
+      load_stage(c);
+      for (; c + WAVES < nchunks; c += WAVES) {
+        store_stage(c);
+        load_x(c);  // x first, then the next weights: the load counter retires in order
+        __builtin_amdgcn_sched_barrier(0);
+        load_stage(c + WAVES);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply();
+      }
+      store_stage(c);
+      load_x(c);
+      multiply();
+    }
+    __syncthreads();  // every wavefront is done with its tile: reuse it for the reduction
+    float* red = reinterpret_cast<float*>(tile);
+#pragma unroll
+    for (int xt = 0; xt < XT; ++xt)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) red[(xt * 16 + l16) * 16 + 4 * kg + v] = acc[xt][v];  // [x row][weight row]
+    __syncthreads();
+    for (int o = threadIdx.x; o < 256 * XT; o += WAVES * kWave) {
+      const int m = o & 15, n = o >> 4;  // weight row fastest: 32-byte runs in Y and the value cache
+      if (n < B) {
+        float val = 0.f;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) val += reinterpret_cast<const float*>(s_tiles[w])[o];
+        if (bias != nullptr) val += (float)bias[row0 + m];
+        const half_t hv = (half_t)val;
+        Y[(int64_t)n * 3 * H * hd + row0 + m] = hv;
+        if (t != 0 && k_cache != nullptr) {
+          const int dst = (positions ? positions[per_sample ? n : 0] : 0) + pos_add;
+          const int j = j0 + m;
+          if (dst >= 0 && dst < S) {
+            if (t == 1)
+              k_cache[((((int64_t)n * H + h) * (hd / 8) + j / 8) * S + dst) * 8 + (j & 7)] = hv;
+            else
+              v_cache[(((int64_t)n * H + h) * S + dst) * hd + j] = hv;
+          }
+        }
+      }
+    }
+    __syncthreads();  // the tiles are staging memory again
+  }
+}
+
+template <int WAVES, int XT>
+__global__ __launch_bounds__(WAVES * 64) void qkv_batch_mfma_kernel(
+    const half_t* __restrict__ X, int64_t ldx, const half_t* __restrict__ W, const half_t* __restrict__ bias,
+    const int* __restrict__ head_idx, const int* __restrict__ live, int live_stride, int B, int d, int H,
+    int hd, int nnz, half_t* __restrict__ Y, half_t* __restrict__ k_cache, half_t* __restrict__ v_cache,
+    const int* __restrict__ positions, int per_sample, int pos_add, int S) {
+  qkv_batch_mfma_body<WAVES, XT>(X, ldx, W, bias, head_idx, live, live_stride, B, d, H, hd, nnz, Y, k_cache,
+                                 v_cache, positions, per_sample, pos_add, S, blockIdx.x, gridDim.x);
+}
+
 }  // namespace dv

@@ -344,6 +344,7 @@ class ParallelMHASparseAttMlp(_MHABase):
         self.att_k = self.sp.K
         # LayerNorm outputs of the current 16-token window, to recompute K/V of skipped heads
         self.x_cache = torch.zeros((self.WINDOW, embed_dim), dtype=torch.float16, device=device)
+        self.x_cache_batch = None  # (16, B * embed_dim): the same for B > 1 sequences, made on first use
         # tracker[h, s] == s while window token s has no K/V for head h, else -1
         self.tracker = torch.arange(self.WINDOW, dtype=torch.int32, device=device).repeat(num_heads, 1)
         self.counter = 0
@@ -396,6 +397,49 @@ class ParallelMHASparseAttMlp(_MHABase):
         self.counter += 1
         return qkv, head_idx, kc, vc
 
+    def _sparse_decode_batched(self, x, head_idx, inference_params):
+        """x: (B, 1, d), B > 1 sequences that decode in lockstep and share the head set and the
+        back-fill window (the reference's sparse attention is single-sequence, mha_dejavu.py:1469;
+        this is its batch extension).  The window buffer holds the B LayerNorm rows of each of
+        the 16 window tokens; the tracker is the one of the single-sequence path.  The newest
+        token's QKV is one pass over the active heads' weights for all B rows; each earlier
+        window token that some active head still misses costs one more pass restricted to
+        those heads (the flush step: 16 passes over every head)."""
+        dev = x.device
+        assert x.dtype == torch.float16 and x.is_contiguous()
+        B, d, H, hd = x.shape[0], self.embed_dim, self.num_heads, self.head_dim
+        if self.x_cache_batch is None or self.x_cache_batch.shape[1] != B * d:
+            assert self.counter == 0, "the batch size cannot change inside a back-fill window"
+            self.x_cache_batch = torch.zeros((self.WINDOW, B * d), dtype=torch.float16, device=dev)
+        flush = self.counter == self.WINDOW - 1
+        if flush:
+            if self._all_heads is None:
+                self._all_heads = torch.arange(H, dtype=torch.int32, device=dev)
+            head_idx = self._all_heads
+        nnz = head_idx.shape[0]
+        nb = self.counter + 1
+        batch_idx = torch.empty(nnz, nb, dtype=torch.int32, device=dev)
+        check(lib.dv_window_step_f16(x.data_ptr(), self.x_cache_batch.data_ptr(), B * d, self.tracker.data_ptr(),
+                                     head_idx.data_ptr(), nnz, H, self.counter, int(flush), batch_idx.data_ptr(),
+                                     torch.cuda.current_stream().cuda_stream), "dv_window_step_f16")
+        k_cache, v_cache = inference_params.key_value_memory_dict[self.layer_idx]
+        b0 = inference_params.batch_size_offset
+        kc, vc = k_cache[b0:b0 + B], v_cache[b0:b0 + B]
+        if self.cache_offset is None:
+            self._set_cache_offset(inference_params.sequence_len_offset - self.counter, dev)
+        lengths = inference_params.lengths_per_sample
+        weight = self.Wqkv.weight.view(3, H, hd, d)
+        bias = None if self.Wqkv.bias is None else self.Wqkv.bias.view(3, H, hd)
+        qkv = torch.empty(B, 3, H, hd, dtype=torch.float16, device=dev)
+        scratch = qkv if nb == 1 else torch.empty_like(qkv)
+        for s in range(nb):  # window token s: position cache_offset + s, or lengths[b] - (counter - s)
+            ops.qkv_proj_batch(self.x_cache_batch[s].view(B, d), weight, head_idx, bias,
+                               out=qkv if s == nb - 1 else scratch, k_cache=kc, v_cache=vc,
+                               positions=self.cache_offset if lengths is None else lengths,
+                               pos_add=s if lengths is None else s - self.counter, live=batch_idx[:, s])
+        self.counter += 1
+        return qkv, head_idx, kc, vc
+
     def forward(self, x, residual, head_idx=None, mlp_sp_logit=None, seqlen=None, inference_params=None, **kwargs):
         """x, residual: (B, s, d).  head_idx: (Hk,) int32 heads to compute, or None
         for dense attention.  mlp_sp_logit: predictor logits for this layer's MLP.
@@ -411,14 +455,20 @@ class ParallelMHASparseAttMlp(_MHABase):
                                            self.att_k, self.att_idx_out)
         if sparse:
             assert x.size(1) == 1
-            assert x.size(0) == 1, "head-sparse decode keeps one back-fill window: batch size 1"
-            qkv, head_idx, kc, vc = self._sparse_decode(x, head_idx, inference_params)
-            # the caches now hold the newest token for the active heads
             if self.out_proj_weight_t is None:
                 self.out_proj_weight_t = self.out_proj.weight.t().contiguous()
-            out = ops.attention_out_proj(qkv[-1:, 0], kc, vc, head_idx, inference_params.sequence_len_offset,
-                                         self.out_proj_weight_t, self.out_proj.bias,
-                                         inference_params.lengths_per_sample, self.softmax_scale).unsqueeze(1)
+            if x.size(0) == 1:
+                qkv, head_idx, kc, vc = self._sparse_decode(x, head_idx, inference_params)
+                # the caches now hold the newest token for the active heads
+                out = ops.attention_out_proj(qkv[-1:, 0], kc, vc, head_idx, inference_params.sequence_len_offset,
+                                             self.out_proj_weight_t, self.out_proj.bias,
+                                             inference_params.lengths_per_sample, self.softmax_scale).unsqueeze(1)
+            else:
+                qkv, head_idx, kc, vc = self._sparse_decode_batched(x, head_idx, inference_params)
+                ctx = ops.single_query_attention(qkv[:, 0], None, None, kc, vc, inference_params.lengths_per_sample,
+                                                 inference_params.sequence_len_offset, self.rotary_emb_dim,
+                                                 head_idx=head_idx, softmax_scale=self.softmax_scale)
+                out = ops.out_proj_sparse_t(ctx, self.out_proj_weight_t, head_idx, self.out_proj.bias).unsqueeze(1)
             if self.counter == self.WINDOW:  # window complete: start the next one
                 self.counter = 0
                 if not self.hold_window:

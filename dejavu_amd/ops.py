@@ -317,6 +317,58 @@ def qkv_proj_sparse(x: torch.Tensor, weight: torch.Tensor, head_idx: torch.Tenso
     return out
 
 
+def qkv_proj_batch(x: torch.Tensor, weight: torch.Tensor, head_idx: torch.Tensor,
+                   bias: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+                   k_cache: Optional[torch.Tensor] = None, v_cache: Optional[torch.Tensor] = None,
+                   positions: Optional[torch.Tensor] = None, pos_add: int = 0,
+                   live: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """QKV of the active heads for one token of each of B sequences (one shared head set), on the
+    matrix cores, the weights streamed once for the whole batch; with caches the K / V rows are
+    appended to sequence b's cache at ``positions[b] + pos_add`` (``positions``: int32, (B,) per
+    sequence or (1,) for all; None = 0).
+
+    :param x: (B, hidden_dim), B <= 32 (rows may be strided)
+    :param weight: (3, nheads, head_dim, hidden_dim)
+    :param head_idx: int32, (nnz,)
+    :param live: optional int32 vector or strided column, one entry per active head: heads with a
+        negative entry are skipped (back-fill passes)
+    :param k_cache, v_cache: (B, nheads, head_dim / 8, S, 8), (B, nheads, S, head_dim)
+    :return: (B, 3, nheads, head_dim); rows of inactive / skipped heads keep the content of ``out``
+    """
+    _require_device(x, weight, head_idx, bias, k_cache, v_cache, positions, live)
+    three, nheads, head_dim, hidden_dim = weight.shape
+    assert three == 3 and head_dim in [32, 64, 128] and hidden_dim % 8 == 0
+    B = x.shape[0]
+    assert x.shape == (B, hidden_dim) and 1 <= B <= 32 and x.stride(1) == 1
+    assert x.dtype == weight.dtype == torch.float16 and weight.is_contiguous()
+    n_active = head_idx.shape[0]
+    assert head_idx.dtype == torch.int32 and head_idx.is_contiguous() and n_active <= nheads
+    if bias is not None:
+        assert bias.shape == (3, nheads, head_dim) and bias.is_contiguous() and bias.dtype == x.dtype
+    if out is None:
+        out = torch.empty(B, 3, nheads, head_dim, device=x.device, dtype=x.dtype)
+    else:
+        assert out.shape == (B, 3, nheads, head_dim) and out.is_contiguous() and out.dtype == x.dtype
+    S, per_sample = 0, 0
+    if k_cache is not None:
+        assert v_cache is not None
+        S = v_cache.shape[2]
+        assert v_cache.shape == (B, nheads, S, head_dim) and k_cache.shape == (B, nheads, head_dim // 8, S, 8)
+        assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dtype == v_cache.dtype == x.dtype
+    if positions is not None:
+        assert positions.dtype == torch.int32 and positions.is_contiguous() and positions.numel() in (1, B)
+        per_sample = int(positions.numel() == B and B > 1)
+    live_stride = 1
+    if live is not None:
+        assert live.dtype == torch.int32 and live.dim() == 1 and live.shape[0] == n_active
+        live_stride = live.stride(0)
+    check(lib.dv_qkv_proj_batch_f16(_ptr(x), x.stride(0), _ptr(weight), _ptr(bias), _ptr(head_idx), _ptr(live),
+                                    live_stride, n_active, B, hidden_dim, nheads, head_dim, _ptr(out), _ptr(k_cache),
+                                    _ptr(v_cache), _ptr(positions), per_sample, int(pos_add), S, _stream()),
+          "dv_qkv_proj_batch_f16")
+    return out
+
+
 def out_proj_sparse(x: torch.Tensor, weight: torch.Tensor, head_idx: torch.Tensor,
                     bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """

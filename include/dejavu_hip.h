@@ -173,6 +173,27 @@ DV_API int dv_qkv_proj_sparse_cache_f16(const void* x, const void* W, const void
                                         void* v_cache, const void* padding, int S, void* stream);
 
 /*
+ * QKV projection of the active heads for one token of each of B sequences that share the head
+ * set, with the K / V rows appended to per-sequence caches:
+ *   y[b, t, h, :] = x[b, :] . W[t, h, :, :]^T + bias[t, h, :]   for h = head_idx[i], every b < B
+ *   k_cache[b, h, :, p_b, :], v_cache[b, h, p_b, :] <- the K / V rows, p_b = positions[per_sample ? b : 0] + pos_add
+ * Batch extension of qkv_proj_sparse + k/v_cache_copy_sparse
+ * (Dejavu/src/models/modules/mha_dejavu.py:1333-1352, 1425-1438; the reference's sparse
+ * attention is single-sequence, mha_dejavu.py:1469): all B rows are multiplied against each
+ * weight tile on the matrix cores, the weights stream once.
+ *   x (B, d) row stride ldx, B <= 32; W (3, H, hd, d); bias (3, H, hd) or NULL; head_idx (nnz,)
+ *   int32; live: int32 or NULL, head i is skipped when live[i * live_stride] < 0 (a back-fill
+ *   pass over one window token computes only the heads that miss it); y (B, 3, H, hd);
+ *   k_cache (B, H, hd/8, S, 8), v_cache (B, H, S, hd): both or neither NULL; positions: device
+ *   int32, (B,) when per_sample != 0, else (1,), or NULL (= 0); rows whose position is outside
+ *   [0, S) are projected but not cached.  hd in {32, 64, 128}.
+ */
+DV_API int dv_qkv_proj_batch_f16(const void* x, int64_t ldx, const void* W, const void* bias,
+                                 const void* head_idx, const void* live, int live_stride, int nnz, int B,
+                                 int d, int H, int hd, void* y, void* k_cache, void* v_cache,
+                                 const void* positions, int per_sample, int pos_add, int S, void* stream);
+
+/*
  * Scatter of (re)computed keys / values into the caches:
  *   k_cache[0, h, dp, s + pad, p] = k[s, h, dp*8 + p];  v_cache[0, h, s + pad, :] = v[s, h, :]
  * for h = head_idx[i], s = seq_idx[i, slot] >= 0.  Either cache may be NULL.

@@ -605,7 +605,8 @@ def batched_sparse_attention_step(x, Wqkv, bqkv, Wout, bout, head_idx, k_cache, 
     return out, ctx
 
 
-def block_decode_step_batched(p, hidden_states, residual, head_idx, mlp_sp_logit, k_cache, v_cache, lengths):
+def block_decode_step_batched(p, hidden_states, residual, head_idx, mlp_sp_logit, k_cache, v_cache, lengths,
+                              residual2_override=None):
     """``block_decode_step`` for B sequences decoding one token each.
 
     Same algebra per row (Dejavu/src/models/modules/block_dejavu.py:555-663).
@@ -616,7 +617,9 @@ def block_decode_step_batched(p, hidden_states, residual, head_idx, mlp_sp_logit
     (B, H) head logits, by the same rule.  hidden_states, residual: (B, d);
     head_idx (Hk,) int32; mlp_sp_logit (B, ffn); caches per sequence, see
     ``batched_sparse_attention_step``.  For B = 1 this is ``block_decode_step``.
-    Returns dict(hidden, residual, next_mlp_logit (B, ffn), next_att_idx, mlp_idx, residual1, attn_out).
+    ``residual2_override``: as in ``block_decode_step``.
+    Returns dict(hidden, residual, next_mlp_logit (B, ffn), next_att_idx, att_logit (B, H), mlp_idx,
+    residual1, attn_out).
     """
     r1 = _add_f16(hidden_states, residual) if residual is not None else np.asarray(hidden_states, F16)
     x = layer_norm(r1, p["ln1_w"], p["ln1_b"])
@@ -629,9 +632,10 @@ def block_decode_step_batched(p, hidden_states, residual, head_idx, mlp_sp_logit
     r2 = _add_f16(attn_out, r1)
     x2 = layer_norm(r2, p["ln2_w"], p["ln2_b"])
     hidden = mlp_sparse(x2, p["W1"], p["W2t"], mlp_idx, p["b1"], p["b2"])
-    _, next_mlp_logit = predictor_logits(r2, p["mlp_Wa"], p["mlp_Wb"])
+    r2_pred = r2 if residual2_override is None else np.asarray(residual2_override, F16)
+    _, next_mlp_logit = predictor_logits(r2_pred, p["mlp_Wa"], p["mlp_Wb"])
     return dict(hidden=hidden, residual=r2, next_mlp_logit=next_mlp_logit, next_att_idx=next_att_idx,
-                mlp_idx=mlp_idx, residual1=r1, attn_out=attn_out)
+                att_logit=att_logit, mlp_idx=mlp_idx, residual1=r1, attn_out=attn_out)
 
 
 # --------------------------------------------------------------------------

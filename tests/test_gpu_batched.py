@@ -65,6 +65,11 @@ def test_batched_mlp_sparse_at_the_headline_shape(ops):
     test_batched_mlp_sparse_matches_oracle(ops, "opt-175b", 32, 4096, torch.int64)
 
 
+def test_batched_mlp_sparse_at_the_headline_shape_batch_8(ops):
+    """OPT-175B-shaped block at batch 8: fc1 and fc2 on the matrix cores, half a batch tile."""
+    test_batched_mlp_sparse_matches_oracle(ops, "opt-175b", 8, 4096, torch.int64)
+
+
 def test_batched_mlp_sparse_at_the_opt66b_shape(ops):
     """OPT-66B-shaped block at batch 16: one full batch tile on the matrix cores."""
     test_batched_mlp_sparse_matches_oracle(ops, "opt-66b", 16, 4096, torch.int64)

@@ -1,0 +1,247 @@
+"""GPU parity of the batch extension of the head-sparse layer: B sequences decode one token
+each with one shared head set and per-sequence KV caches (the reference's sparse attention is
+single-sequence, mha_dejavu.py:1469).  The oracle side is block_decode_step_batched /
+batched_sparse_attention_step, pinned on the CPU against the single-sequence functions."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import dejavu_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def assert_close(got, want, what="", max_abs_tol=2e-2, rel_tol=1e-3):
+    got = np.asarray(got, dtype=np.float64)
+    want = np.asarray(want, dtype=np.float64)
+    max_abs = np.max(np.abs(got - want)) if got.size else 0.0
+    rel = np.linalg.norm(got - want) / max(np.linalg.norm(want), 1e-30)
+    assert max_abs <= max_abs_tol and rel <= rel_tol, f"{what}: max_abs={max_abs:.3e} rel_l2={rel:.3e}"
+
+
+def np16(t):
+    return t.detach().cpu().numpy()
+
+
+def randh(g, *shape, std=1.0, mean=0.0):
+    return (torch.randn(*shape, generator=g) * std + mean).half()
+
+
+@pytest.mark.parametrize("B,H,hd,d,S", [(2, 6, 64, 512, 40), (5, 4, 128, 776, 24), (16, 6, 64, 512, 40),
+                                        (17, 3, 32, 264, 20), (32, 5, 128, 1024, 33)])
+def test_qkv_proj_batch_matches_oracle(B, H, hd, d, S):
+    """All B rows against each selected head's weights, K / V appended at per-sequence positions;
+    heads masked out by `live` and unselected heads leave outputs and caches untouched; a ragged
+    last 256-column chunk (d = 776, 264) and a second batch tile (B > 16) are covered."""
+    from dejavu_amd import ops
+    from dejavu_amd.workloads import pack_k_cache
+
+    g = torch.Generator().manual_seed(B * 100 + H)
+    xbig = randh(g, B, d + 24)
+    x = xbig[:, :d]  # strided rows
+    W = randh(g, 3, H, hd, d, std=0.05)
+    bias = randh(g, 3, H, hd, std=0.1)
+    head_idx = torch.sort(torch.randperm(H, generator=g)[: max(2, H // 2 + 1)]).values.int()
+    nnz = head_idx.numel()
+    live = torch.arange(nnz, dtype=torch.int32) * 3
+    live[1] = -1  # this head is skipped by the pass
+    positions = torch.randint(0, S, (B,), generator=g).int()
+    positions[0] = S - 1
+    kc0, vc0 = randh(g, B, H, S, hd), randh(g, B, H, S, hd)
+    k_cache, v_cache = pack_k_cache(kc0).cuda(), vc0.clone().cuda()
+    out = torch.full((B, 3, H, hd), 7.0, dtype=torch.float16, device="cuda")
+    print(f"case qkv batch B={B} H={H} hd={hd} d={d}", flush=True)
+    ops.qkv_proj_batch(xbig.cuda()[:, :d], W.cuda(), head_idx.cuda(), bias.cuda(), out=out, k_cache=k_cache,
+                       v_cache=v_cache, positions=positions.cuda(), pos_add=0, live=live.cuda())
+    torch.cuda.synchronize()
+    used = [int(h) for i, h in enumerate(head_idx) if live[i] >= 0]
+    rows = np.tile(np.arange(B, dtype=np.int32), (len(used), 1))
+    want = O.qkv_proj_sparse(x.numpy(), W.numpy(), np.array(used, np.int32), rows, bias.numpy())
+    got = np16(out)
+    assert_close(got[:, :, used], want[:, :, used], "qkv rows")
+    others = [h for h in range(H) if h not in used]
+    assert np.all(got[:, :, others] == 7.0), "skipped / unselected heads must not be written"
+    kn, vn = np16(k_cache), np16(v_cache)
+    k_unpacked = O.unpack_k_cache(kn)  # (B, H, S, hd)
+    for b in range(B):
+        p = int(positions[b])
+        for h in range(H):
+            if h in used:
+                assert np.array_equal(k_unpacked[b, h, p], got[b, 1, h]) and np.array_equal(vn[b, h, p], got[b, 2, h])
+                keep = np.arange(S) != p
+                assert np.array_equal(k_unpacked[b, h, keep], kc0[b, h].numpy()[keep])
+                assert np.array_equal(vn[b, h, keep], vc0[b, h].numpy()[keep])
+            else:
+                assert np.array_equal(k_unpacked[b, h], kc0[b, h].numpy()) and np.array_equal(vn[b, h], vc0[b, h].numpy())
+    # one shared position (+ offset) and no mask; a position outside the cache is projected but not stored
+    out2 = torch.zeros_like(out)
+    k2, v2 = pack_k_cache(kc0).cuda(), vc0.clone().cuda()
+    base = torch.tensor([S - 3], dtype=torch.int32, device="cuda")
+    ops.qkv_proj_batch(x.cuda().contiguous(), W.cuda(), head_idx.cuda(), None, out=out2, k_cache=k2, v_cache=v2,
+                       positions=base, pos_add=2)
+    ops.qkv_proj_batch(x.cuda().contiguous(), W.cuda(), head_idx.cuda(), None, out=out2, k_cache=k2, v_cache=v2,
+                       positions=base, pos_add=3)
+    torch.cuda.synchronize()
+    hs = [int(h) for h in head_idx]
+    want2 = O.qkv_proj_sparse(x.numpy(), W.numpy(), head_idx.numpy(), np.tile(np.arange(B, dtype=np.int32), (nnz, 1)))
+    assert_close(np16(out2)[:, :, hs], want2[:, :, hs], "qkv rows, no bias")
+    assert np.array_equal(np16(v2)[:, hs, S - 1], np16(out2)[:, 2, hs])
+    keep = np.arange(S) != S - 1
+    assert np.array_equal(np16(v2)[:, :, keep], vc0.numpy()[:, :, keep])
+
+
+def build_attention(g, d, H, r, Hk, mlp_k, layer_idx=1):
+    from dejavu_amd.modules import ParallelMHASparseAttMlp
+
+    sp_kwargs = {"embed_dim": d, "low_rank_dim": r, "out_dim": H, "K": Hk}
+    att = ParallelMHASparseAttMlp(d, H, None, sp_kwargs, layer_idx=layer_idx, sequence_parallel=False,
+                                  softmax_scale=(d // H) ** -0.5, causal=True, device="cuda", dtype=torch.float16)
+    att.mlp_k = mlp_k
+    with torch.no_grad():
+        att.Wqkv.weight.copy_(randh(g, 3 * d, d, std=0.05))
+        att.Wqkv.bias.copy_(randh(g, 3 * d, std=0.1))
+        att.out_proj.weight.copy_(randh(g, d, d, std=0.05))
+        att.out_proj.bias.copy_(randh(g, d, std=0.1))
+        att.sp.fc0.weight.copy_(randh(g, r, d, std=0.05))
+        att.sp.fc1.weight.copy_(randh(g, H, r, std=0.05))
+    return att
+
+
+@pytest.mark.parametrize("B,d,H,Hk,prompt,steps", [(3, 256, 4, 2, 5, 36), (18, 512, 8, 3, 3, 20)])
+def test_batched_sparse_attention_module_backfills_skipped_heads(B, d, H, Hk, prompt, steps):
+    """B sequences, dense prompt, then decode steps with a different random shared head subset each
+    step: every row of every step must equal attention over dense K/V of that sequence's whole past,
+    which only holds if the K/V a head skipped are recomputed, for all B sequences, when it returns.
+    The predicted heads / neurons are the top-k of the column-wise maxima over the batch."""
+    from dejavu_amd.modules import InferenceParams
+
+    g = torch.Generator().manual_seed(40 + B)
+    hd, r, ffn, mlp_k = d // H, 64, 512, 100
+    att = build_attention(g, d, H, r, Hk, mlp_k)
+    Wqkv = np16(att.Wqkv.weight).reshape(3, H, hd, d)
+    bqkv = np16(att.Wqkv.bias).reshape(3, H, hd)
+    Wout = np16(att.out_proj.weight).reshape(d, H, hd)
+    bout = np16(att.out_proj.bias)
+    S = prompt + steps + 4
+    ip = InferenceParams(max_sequence_len=S, max_batch_size=B)
+    xs = randh(g, B, prompt + steps, d)
+    with torch.no_grad():
+        xp = xs[:, :prompt].cuda()
+        out_p, _, _ = att(xp, xp, inference_params=ip)
+    torch.cuda.synchronize()
+    assert out_p.shape == (B, prompt, d)
+    ip.sequence_len_offset = prompt
+    for step in range(steps):
+        t = prompt + step
+        head_idx = torch.sort(torch.randperm(H, generator=g)[:Hk]).values.int()
+        x = xs[:, t].contiguous().cuda().view(B, 1, d)
+        residual = randh(g, B, 1, d).cuda()
+        mlp_sp_logit = randh(g, B, ffn, std=3.0).cuda()
+        print(f"case batched attention module B={B} step={step} heads={head_idx.tolist()} counter={att.counter}", flush=True)
+        with torch.no_grad():
+            out, mlp_idx, att_idx = att(x, residual, head_idx=head_idx.cuda(), mlp_sp_logit=mlp_sp_logit,
+                                        inference_params=ip)
+        torch.cuda.synchronize()
+        used = np.arange(H) if step % 16 == 15 else head_idx.numpy()
+        for b in range(B):
+            want, _ = O.sparse_attention_step_dense_kv(xs[b, : t + 1].numpy(), Wqkv, bqkv, Wout, bout, used, hd ** -0.5)
+            assert_close(np16(out)[b, 0], want, f"step {step} row {b}", max_abs_tol=3e-2, rel_tol=3e-3)
+        assert np.array_equal(np16(mlp_idx), O.topk_lower_index(np16(mlp_sp_logit), mlp_k))
+        dev_logits = att.sp(residual)  # (B, H) as the module computed them
+        assert np.array_equal(np16(att_idx).astype(np.int64), O.topk_lower_index(np16(dev_logits), Hk))
+        _, l_ref = O.predictor_logits(np16(residual)[:, 0], np16(att.sp.fc0.weight), np16(att.sp.fc1.weight))
+        if B <= 8:
+            assert np.array_equal(np16(dev_logits).view(np.uint16), l_ref.view(np.uint16))
+        else:
+            assert_close(np16(dev_logits), l_ref, "head logits (matrix-core order)")
+        ip.sequence_len_offset += 1
+
+
+def _block_params(block, H, hd, d, K, Hk):
+    m, f = block.mixer, block.mlp
+    return dict(ln1_w=np16(block.norm1.weight), ln1_b=np16(block.norm1.bias), ln2_w=np16(block.norm2.weight),
+                ln2_b=np16(block.norm2.bias), Wqkv=np16(m.Wqkv.weight).reshape(3, H, hd, d),
+                bqkv=np16(m.Wqkv.bias).reshape(3, H, hd), Wout=np16(m.out_proj.weight).reshape(d, H, hd),
+                bout=np16(m.out_proj.bias), W1=np16(f.fc1.weight), b1=np16(f.fc1.bias),
+                W2t=np.ascontiguousarray(np16(f.fc2.weight).T), b2=np16(f.fc2.bias), mlp_Wa=np16(f.sp.fc0.weight),
+                mlp_Wb=np16(f.sp.fc1.weight), att_Wa=np16(m.sp.fc0.weight), att_Wb=np16(m.sp.fc1.weight),
+                mlp_K=K, att_K=Hk)
+
+
+@pytest.mark.parametrize("cfg,B", [("opt-125m", 3), ("opt-125m", 16), ("opt-66b", 16), ("opt-175b", 8),
+                                   ("opt-175b", 32)])
+def test_batched_sparse_block_decode_step_matches_oracle(cfg, B):
+    """One decode step of a whole block for B sequences (OPT-66B shape at batch 16, OPT-175B shape at
+    batch 8 and 32, full-size weights and caches) against block_decode_step_batched.  Up to 8 rows
+    the predictors are bit-exact; above, their logits come from the matrix cores and are compared
+    within tolerance, the selections being checked as the exact top-k of the device's own logits."""
+    from dejavu_amd.block import create_sparse_block, init_block_synthetic
+    from dejavu_amd.modules import InferenceParams
+    from dejavu_amd.workloads import CONFIGS, pack_k_cache
+
+    c = CONFIGS[cfg]
+    d, ffn, H, hd, r, K, Hk, S = (c[k] for k in ("d", "ffn", "H", "hd", "r", "K", "Hk", "S"))
+    block = create_sparse_block(d, ffn, H, r, K, r, Hk, layer_idx=2)
+    init_block_synthetic(block, seed=0)
+    with torch.no_grad():
+        g = torch.Generator().manual_seed(9)
+        for n in (block.norm1, block.norm2):
+            n.weight.copy_((1 + 0.1 * torch.randn(d, generator=g)).half())
+            n.bias.copy_((0.1 * torch.randn(d, generator=g)).half())
+        block.mixer.Wqkv.bias.copy_((0.1 * torch.randn(3 * d, generator=g)).half())
+        block.mixer.out_proj.bias.copy_((0.1 * torch.randn(d, generator=g)).half())
+    g = torch.Generator().manual_seed(10 + B)
+    gd = torch.Generator(device="cuda").manual_seed(10 + B)
+    kc = torch.randn(B, H, S, hd, generator=gd, device="cuda", dtype=torch.float16)
+    vc = torch.randn(B, H, S, hd, generator=gd, device="cuda", dtype=torch.float16)
+    lengths = torch.randint(S // 2, S, (B,), generator=g).int()
+    lengths[0] = S - 1
+    ip = InferenceParams(max_sequence_len=S, max_batch_size=B, sequence_len_offset=int(lengths.max()))
+    ip.lengths_per_sample = lengths.cuda()
+    k_packed = pack_k_cache(kc)
+    del kc
+    k0, v0 = k_packed.clone(), vc.clone()
+    ip.key_value_memory_dict[2] = (k_packed, vc)
+    hs = torch.randn(B, 1, d, generator=g).half()
+    res = torch.randn(B, 1, d, generator=g).half()
+    head_idx = torch.sort(torch.randperm(H, generator=g)[:Hk]).values.int()
+    mlp_sp_logit = (torch.randn(B, ffn, generator=g) * 4).half()
+    print(f"case batched sparse block decode step {cfg} B={B}", flush=True)
+    with torch.no_grad():
+        hidden, residual, next_logit, next_att = block(hs.cuda(), res.cuda(), mixer_kwargs={"inference_params": ip},
+                                                       head_idx=head_idx.cuda(), mlp_sp_logit=mlp_sp_logit.cuda())
+        r1 = (hs.cuda().float() + res.cuda().float()).half()
+        dev_head_logits = block.mixer.sp(r1)
+    torch.cuda.synchronize()
+    assert hidden.shape == (B, 1, d) and residual.shape == (B, 1, d) and next_logit.shape == (B, ffn)
+    p = _block_params(block, H, hd, d, K, Hk)
+    kn, vn = np16(k0), np16(v0)  # the oracle appends its own rows to these copies
+    want = O.block_decode_step_batched(p, hs.numpy()[:, 0], res.numpy()[:, 0], head_idx.numpy(), mlp_sp_logit.numpy(),
+                                       kn, vn, lengths.numpy(), residual2_override=np16(residual)[:, 0])
+    assert_close(np16(residual)[:, 0], want["residual"], "residual stream after attention")
+    assert_close(np16(hidden)[:, 0], want["hidden"], "block output", max_abs_tol=3e-2, rel_tol=3e-3)
+    assert np.array_equal(np16(next_att).astype(np.int64), O.topk_lower_index(np16(dev_head_logits), Hk)), \
+        "next heads are not the top-k of the batch maxima of the device's head logits"
+    if B <= 8:
+        assert np.array_equal(np16(next_att).astype(np.int64), want["next_att_idx"].astype(np.int64))
+        assert np.array_equal(np16(next_logit).view(np.uint16), want["next_mlp_logit"].view(np.uint16)), \
+            "next-layer MLP logits not bit-exact"
+    else:
+        # logits reach +-60 here: the absolute bound is 2e-2 or two fp16 steps of the largest logit
+        # (the hidden vector they start from is itself rounded in a different summation order)
+        for got_l, want_l, what in ((dev_head_logits, want["att_logit"], "head logits"),
+                                    (next_logit, want["next_mlp_logit"], "next-layer MLP logits")):
+            top = float(np.abs(want_l.astype(np.float32)).max())
+            two_steps = 2.0 * 2.0 ** (np.floor(np.log2(max(top, 1e-3))) - 10)
+            assert_close(np16(got_l), want_l, what + " (matrix-core order)", max_abs_tol=max(2e-2, two_steps))
+    # the appended K / V rows are projections (within tolerance of the oracle's); every other cache
+    # entry is untouched bit for bit
+    kcd, vcd = ip.key_value_memory_dict[2]
+    sel = head_idx.long().cuda()
+    for b in range(B):
+        t = int(lengths[b])
+        assert_close(np16(vcd[b, sel, t]), vn[b, head_idx.numpy(), t], f"value cache row of the new token, sequence {b}")
+        assert_close(np16(kcd[b, sel, :, t]), kn[b, head_idx.numpy(), :, t], f"key cache row of the new token, sequence {b}")
+        vcd[b, sel, t] = v0[b, sel, t]
+        kcd[b, sel, :, t] = k0[b, sel, :, t]
+    assert torch.equal(vcd, v0) and torch.equal(kcd, k0), "cache entries other than the appended rows changed"

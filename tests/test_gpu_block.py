@@ -107,7 +107,8 @@ def test_sparse_block_decode_step_matches_oracle(d, ffn, H, r, K, Hk, S):
 def test_fused_layer_equals_module_by_module_path(d, H, ffn, r, K, Hk):
     """The eight-launch fused block step and the module-by-module path run the same kernel
     bodies: outputs, predictions, caches and window state must agree bit for bit over a
-    whole back-fill window (the flush step falls back to the modules in both).  Every scratch
+    whole back-fill window and into the next one (the flush step is a fused step too, with every
+    head active).  Every scratch
     buffer is overwritten with 0xFF bytes (NaN as fp32) before each step: the kernels must not
     depend on what a workspace holds when they start."""
     import copy

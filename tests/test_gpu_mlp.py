@@ -254,3 +254,40 @@ def test_workspace_shared_across_shapes(ops):
         got = ops.gather_transposed_gemv(h.cuda(), W, idx.cuda(), None)
         torch.cuda.synchronize()
         assert_close(np16(got), O.gather_transposed_gemv(h.numpy(), W.cpu().numpy(), idx.numpy(), None), f"M={M} B={B}")
+
+
+# ------------------------------------------- OPT-6.7B block: the whole batch x K grid
+_GRID_CACHE = {}
+
+
+def _grid_case(batch):
+    """OPT-6.7B-shaped block at one batch size: host tensors, device tensors, oracle logits (made once)."""
+    if batch not in _GRID_CACHE:
+        _GRID_CACHE.clear()  # one batch size resident at a time
+        t = make("opt-6.7b", batch, seed=100 + batch)
+        g = {k: dev(v) for k, v in t.items()}
+        _, l_ref = O.predictor_logits(np16(t["residual"]), np16(t["mlp_Wa"]), np16(t["mlp_Wb"]))
+        _GRID_CACHE[batch] = (t, g, l_ref)
+    return _GRID_CACHE[batch]
+
+
+@pytest.mark.parametrize("K", [1024, 2048, 4096, 16384])
+@pytest.mark.parametrize("batch", [1, 4, 8])
+def test_opt67b_block_batch_by_k_grid(ops, batch, K):
+    """Predictor -> union top-K (capped at K) -> fc1 -> fc2 for every batch in {1, 4, 8} and every
+    K in {1024, 2048, 4096, 16384 (dense)}: logits and index set bit-exact, outputs within tolerance."""
+    t, g, l_ref = _grid_case(batch)
+    print(f"case opt-6.7b grid B={batch} K={K}", flush=True)
+    logits = ops.predictor_logits(g["residual"], g["mlp_Wa"], g["mlp_Wb"])
+    idx_t = ops.topk_indices(logits, K)
+    y = ops.mlp_sparse(g["x2"], g["W1"], g["W2t"], idx_t, g["b1"], g["b2"])
+    torch.cuda.synchronize()
+    assert np.array_equal(np16(logits).view(np.uint16), l_ref.view(np.uint16)), "predictor logits"
+    idx = O.topk_lower_index(l_ref, K)
+    assert np.array_equal(np16(idx_t), idx), "union top-K"
+    if K == 16384:
+        assert np.array_equal(idx, np.arange(16384))
+    assert_close(np16(y), O.mlp_sparse(np16(t["x2"]), np16(t["W1"]), np16(t["W2t"]), idx, np16(t["b1"]), np16(t["b2"])),
+                 "mlp_sparse")
+    if batch == 8 and K == 16384:
+        _GRID_CACHE.clear()
