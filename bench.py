@@ -15,13 +15,21 @@ position 15 is the flush step that brings every head up to date.  The active
 heads are re-drawn at random for every (layer, position) -- no correlation
 between consecutive tokens, the most back-fill work a window can have.
 ``--window start`` times only the first position of a window (no back-fill).
-Steps are replayed from HIP graphs (one graph of up to four periods of 3 layers x 16 positions
-when the step counts are multiples of 48, one graph per (layer, position) otherwise).
 
-Prints ONE JSON line: metric / value / unit (us per layer, whole-window average), the
-roofline of the dominant kernel (qkv_sparse_kernel, measured alone with HIP events), the CPU
-baseline (PyTorch index_select + matmul on the host cores, bounded sample), the first window
-position alone (window_start), the spread over single graph replays and a per-kernel table.
+Timing: the W warm-up steps and the K timed steps are steps 0..W-1 and W..W+K-1 of that
+schedule (period: 3 layers x 16 positions = 48 steps), captured in HIP graphs of up to 192
+consecutive steps, so exactly K steps run between the two synchronisations and no host launch
+gap falls between two steps of a graph.  ``positions`` in the JSON says which window positions
+the K steps covered; the byte count they are priced with is the sum over exactly those steps.
+Whatever K is, ``window_average`` (whole periods) and ``window_start`` (first position only)
+are measured as well.  ``--batch B`` (B > 1): B sequences decode in lockstep with one shared
+head / neuron set and per-sequence KV caches, every step at the first position of a window.
+
+Prints ONE JSON line: metric / value / unit (us per layer), ``roofline`` for the QKV projection
+as the timed schedule runs it (time-weighted over its three kernels, each timed alone from a
+HIP graph between two HIP events), ``mlp_pair`` (fc1 + fc2 + split reduction against 4 K d
+bytes), the CPU baseline (PyTorch index_select + matmul on the host cores, bounded sample)
+and a per-kernel table.
 """
 from __future__ import annotations
 
@@ -38,10 +46,81 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0
 N_LAYERS = 3
 WINDOW = 16
-# HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (scaled by a 1 GiB copy; see profiles/layer_opt175b_pmc_traffic.md).  Not measurable from inside
-# this script, so only reported for the shape it was taken on.
-MEASURED_TRAFFIC_BYTES = {("opt-175b", 1, "qkv_sparse"): 302.45e6 + 0.05e6}
+MAX_GRAPH_STEPS = 192  # steps per HIP graph (four schedule periods)
+TRAFFIC_JSON = os.path.join(ROOT, "profiles", "traffic.json")
+CSRC_DIR = os.path.join(ROOT, "dejavu_amd", "csrc")
+
+
+def csrc_digest():
+    """SHA-256 over the kernel sources: ties a counter measurement to the code it was taken on."""
+    import hashlib
+
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(CSRC_DIR)):
+        if name.endswith((".hip", ".hpp")):
+            with open(os.path.join(CSRC_DIR, name), "rb") as f:
+                h.update(name.encode() + b"\0" + f.read())
+    return h.hexdigest()
+
+
+def measured_traffic(config, batch, kernel):
+    """HBM bytes per launch from the last rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+    (profiles/traffic.json, written by ``bench.py --traffic-from``), or None when there is no
+    entry for this shape or the kernel sources changed since the counters were read."""
+    try:
+        with open(TRAFFIC_JSON) as f:
+            t = json.load(f)
+    except (OSError, ValueError):
+        return None
+    if t.get("csrc_sha256") != csrc_digest():
+        return None
+    return t.get("bytes_per_launch", {}).get(f"{config}/batch{batch}/{kernel}")
+
+
+def write_traffic(fetch_csv, write_csv):
+    """Reads the two rocprofv3 counter CSVs of ``bench.py --pmc-calibration`` runs (one with
+    --pmc FETCH_SIZE, one with --pmc WRITE_SIZE), scales each counter by what it reads for the
+    1 GiB device copy of the same run, and writes profiles/traffic.json."""
+    import csv
+    import subprocess
+
+    def per_kernel(path, counter):
+        acc = {}
+        with open(path, newline="") as f:
+            for row in csv.DictReader(f):
+                if row.get("Counter_Name") != counter:
+                    continue
+                acc.setdefault(row["Kernel_Name"], []).append(float(row["Counter_Value"]))
+        return {k: sum(v) / len(v) for k, v in acc.items()}
+
+    def find(table, needle):
+        hits = [v for k, v in table.items() if needle in k]
+        return hits[0] if hits else None
+
+    fetch, write = per_kernel(fetch_csv, "FETCH_SIZE"), per_kernel(write_csv, "WRITE_SIZE")
+    copy_kib = float(1 << 20)
+    f_scale = copy_kib / find(fetch, "copyBuffer")
+    w_scale = copy_kib / find(write, "copyBuffer")
+    names = {"qkv_sparse_kernel": "qkv_sparse", "layer_l2_kernel<1>": "qkv_l2_one_token",
+             "layer_l2_kernel<0>": "qkv_l2_mfma", "layer_l2_kernel<-1>": "qkv_l2_flush"}
+    out = {}
+    for needle, key in names.items():
+        fr, wr = find(fetch, needle), find(write, needle)
+        if fr is not None and wr is not None:
+            out[f"opt-175b/batch1/{key}"] = round((fr * f_scale + wr * w_scale) * 1024)
+    try:
+        commit = subprocess.run(["git", "-C", ROOT, "rev-parse", "--short", "HEAD"], capture_output=True,
+                                text=True).stdout.strip()
+    except OSError:
+        commit = ""
+    doc = {"csrc_sha256": csrc_digest(), "commit": commit, "unit": "HBM bytes per launch (read + written)",
+           "scale": {"FETCH_SIZE": round(f_scale, 4), "WRITE_SIZE": round(w_scale, 4),
+                     "calibration": "1 GiB device-to-device copy in the same run"},
+           "bytes_per_launch": out}
+    with open(TRAFFIC_JSON, "w") as f:
+        json.dump(doc, f, indent=1, sort_keys=True)
+        f.write("\n")
+    print(json.dumps(doc))
 
 
 def algorithmic_bytes(cfg, batch):
@@ -95,7 +174,7 @@ def build_layers(cfg, batch, device):
     # predictions travel from layer l to layer l+1 through fixed buffers
     for l, L in enumerate(layers):
         L["att_idx_in"] = torch.sort(torch.randperm(H, generator=gen, device=device)[:Hk]).values.int()
-        L["mlp_logit_in"] = randn((ffn,), 4.0)
+        L["mlp_logit_in"] = randn((ffn,) if batch == 1 else (batch, ffn), 4.0)
         # active heads per window position, independent draws
         L["heads"] = [torch.sort(torch.randperm(H, generator=gen, device=device)[:Hk]).values.int()
                       for _ in range(WINDOW)]
@@ -133,23 +212,30 @@ def window_step(L, c):
                       head_idx=L["heads"][c], mlp_sp_logit=L["mlp_logit_in"])
 
 
-def time_kernel(torch, fn, layers, iters=60):
-    """Average duration (us) of back-to-back launches bracketed by two HIP events
-    on the launch stream."""
+def time_kernel(torch, fn, layers, launches=30, replays=5):
+    """Average duration (us) of one launch of ``fn``: ``launches`` calls (cycling over the layers)
+    captured in one HIP graph, replayed back to back between two HIP events on the launch stream.
+    Eager launches would be bounded by the host's launch rate for the short kernels."""
     for L in layers:
         fn(L)
     torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for i in range(launches):
+            fn(layers[i % len(layers)])
+    g.replay()
+    torch.cuda.synchronize()
     a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     a.record()
-    for i in range(iters):
-        fn(layers[i % len(layers)])
+    for _ in range(replays):
+        g.replay()
     b.record()
     torch.cuda.synchronize()
-    return a.elapsed_time(b) * 1e3 / iters
+    return a.elapsed_time(b) * 1e3 / (launches * replays)
 
 
 def kernel_table(torch, cfg, batch, layers):
-    """Per-kernel durations and achieved bandwidth, each launched alone."""
+    """Per-operator durations and achieved bandwidth, each operator alone (graph-replayed)."""
     from dejavu_amd import ops
 
     d, ffn, H, hd, K, Hk, S = (cfg[k] for k in ("d", "ffn", "H", "hd", "K", "Hk", "S"))
@@ -157,11 +243,13 @@ def kernel_table(torch, cfg, batch, layers):
     dev = layers[0]["hidden"].device
     x = layers[0]["hidden"].view(batch, d)
     head_idx = layers[0]["att_idx_in"]
+    all_heads = torch.arange(H, dtype=torch.int32, device=dev)
     batch_idx = torch.zeros(Hk, 1, dtype=torch.int32, device=dev)
     idx = ops.topk_indices(layers[0]["mlp_logit_in"], K)
     h = ops.gather_gemv(x, layers[0]["block"].mlp.fc1.weight, idx, layers[0]["block"].mlp.fc1.bias, "relu")
-    qkv = torch.zeros(1, 3, H, hd, dtype=torch.float16, device=dev)
+    qkv = torch.zeros(max(batch, 16), 3, H, hd, dtype=torch.float16, device=dev)
     ctx = torch.zeros(batch, H, hd, dtype=torch.float16, device=dev)
+    lengths = torch.full((batch,), S - 1, dtype=torch.int32, device=dev)
 
     def m(L):
         return L["block"].mixer
@@ -169,33 +257,61 @@ def kernel_table(torch, cfg, batch, layers):
     def f(L):
         return L["block"].mlp
 
+    def W(L):
+        return m(L).Wqkv.weight.view(3, H, hd, d)
+
+    def bq(L):
+        return m(L).Wqkv.bias.view(3, H, hd)
+
+    def caches(L):
+        return L["ip"].key_value_memory_dict[m(L).layer_idx]
+
     fns = {
-        "qkv_sparse": lambda L: ops.qkv_proj_sparse(x[:1], m(L).Wqkv.weight.view(3, H, hd, d), head_idx, batch_idx,
-                                                    m(L).Wqkv.bias.view(3, H, hd), out=qkv),
-        "decode_attn": lambda L: ops.single_query_attention(qkv[:, 0], None, None, *L["ip"].key_value_memory_dict[
-            L["block"].mixer.layer_idx], None, S - 1, head_idx=head_idx, out=ctx),
+        "decode_attn": lambda L: ops.single_query_attention(qkv[:batch, 0], None, None, *caches(L), lengths, S - 1,
+                                                            head_idx=head_idx, out=ctx),
         "out_proj_sparse": lambda L: ops.out_proj_sparse_t(ctx, m(L).out_proj_weight_t, head_idx, m(L).out_proj.bias),
         "fc1_gather": lambda L: ops.gather_gemv(x, f(L).fc1.weight, idx, f(L).fc1.bias, "relu"),
         "fc2_gather": lambda L: ops.gather_transposed_gemv(h, f(L).fc2_weight_t, idx, f(L).fc2.bias),
         "mlp_predictor": lambda L: ops.predictor_logits(x, f(L).sp.fc0.weight, f(L).sp.fc1.weight),
         "head_predictor": lambda L: ops.predictor_logits(x, m(L).sp.fc0.weight, m(L).sp.fc1.weight),
     }
+    if batch == 1:
+        # the three QKV kernels of a back-fill window: position 0 (one window token, vector ALUs),
+        # positions 1..14 (2..15 window slots on the matrix cores; timed with 8 slots, all live),
+        # position 15 (flush: every head, all 16 slots)
+        xw = layers[0]["block"].mixer.x_cache
+        bi8 = torch.arange(8, dtype=torch.int32, device=dev).repeat(Hk, 1)
+        bi16 = torch.arange(16, dtype=torch.int32, device=dev).repeat(H, 1)
+        fns["qkv_sparse"] = lambda L: ops.qkv_proj_sparse(x[:1], W(L), head_idx, batch_idx, bq(L), out=qkv[:1])
+        fns["qkv_window_mfma"] = lambda L: ops.qkv_proj_sparse(xw[:8], W(L), head_idx, bi8, bq(L), out=qkv[:8])
+        fns["qkv_flush_mfma"] = lambda L: ops.qkv_proj_sparse(xw, W(L), all_heads, bi16, bq(L), out=qkv[:16])
+        nbytes["qkv_window_mfma"] = nbytes["qkv_sparse"]
+        nbytes["qkv_flush_mfma"] = 3 * H * hd * d * 2
+    else:
+        fns["qkv_batch"] = lambda L: ops.qkv_proj_batch(x, W(L), head_idx, bq(L), out=qkv[:batch])
+        nbytes["qkv_batch"] = nbytes["qkv_sparse"]
     table = {}
     for name, fn in fns.items():
         us = time_kernel(torch, fn, layers)
         table[name] = {"us": round(us, 2), "MB": round(nbytes[name] / 1e6, 2),
                        "GB/s": round(nbytes[name] / us / 1e3, 1),
                        "frac": round(nbytes[name] / us / 1e3 / HBM_PEAK_GBPS, 4)}
+    # fc1 -> fc2 -> split reduction, back to back as in a layer step: 4 K d bytes
+    us = time_kernel(torch, lambda L: ops.mlp_sparse(x, f(L).fc1.weight, f(L).fc2_weight_t, idx, f(L).fc1.bias,
+                                                     f(L).fc2.bias), layers)
+    pair_bytes = nbytes["fc1_gather"] + nbytes["fc2_gather"]
+    table["mlp_pair"] = {"us": round(us, 2), "MB": round(pair_bytes / 1e6, 2), "GB/s": round(pair_bytes / us / 1e3, 1),
+                         "frac": round(pair_bytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
     # latency-bound pieces (a few hundred KB at most): duration only
     res = layers[0]["residual"].view(batch, d)
+    logit_rows = layers[0]["mlp_logit_in"].view(-1, ffn)
     small = {
-        "mlp_topk": lambda L: ops.topk_indices(L["mlp_logit_in"], K),
+        "mlp_topk": lambda L: ops.topk_indices(logit_rows, K),
         "add_layer_norm": lambda L: ops.add_layer_norm(x, res, L["block"].norm1.weight, L["block"].norm1.bias,
                                                        L["block"].norm1.eps),
     }
     for name, fn in small.items():
-        table[name] = {"us": round(time_kernel(torch, fn, layers), 2),
-                       "note": "eager call of the stand-alone operator: bounded by the host launch rate"}
+        table[name] = {"us": round(time_kernel(torch, fn, layers), 2)}
     return table
 
 
@@ -278,6 +394,21 @@ def decode_bench(args):
         t_total, seq_cg = min((run(True) for _ in range(3)), key=lambda r: r[0])
         t_prompt, _ = min((run(True, prompt_len + 1) for _ in range(3)), key=lambda r: r[0])
         t_eager, seq_eager = run(False)
+        # roofline of the kernel that carries the largest share of a token's bytes (the QKV projection of
+        # a sparse block, one launch per block and token), alone, graph-replayed between two HIP events
+        from dejavu_amd import ops
+
+        d_, H_, hd_, Hk_ = cfg["d"], cfg["H"], cfg["hd"], cfg["Hk"]
+        blocks = list(model.transformer.layers[1:4]) if layers >= 4 else list(model.transformer.layers)
+        xq = torch.randn(1, d_, device="cuda", dtype=torch.float16, generator=gen)
+        hq = torch.sort(torch.randperm(H_, device="cuda", generator=gen)[:Hk_]).values.int()
+        bq = torch.zeros(Hk_, 1, dtype=torch.int32, device="cuda")
+        yq = torch.zeros(1, 3, H_, hd_, dtype=torch.float16, device="cuda")
+        qkv_us = time_kernel(torch, lambda b: ops.qkv_proj_sparse(xq, b.mixer.Wqkv.weight.view(3, H_, hd_, d_), hq, bq,
+                                                                  b.mixer.Wqkv.bias.view(3, H_, hd_), out=yq), blocks)
+        cpu = None
+        if not args.no_cpu_baseline:
+            cpu = decode_cpu_baseline(torch, cfg, model, layers, vocab)
     same = bool(torch.equal(seq_cg, seq_eager))
     decode_s = t_total - t_prompt
     steps = new_tokens - 1
@@ -299,8 +430,52 @@ def decode_bench(args):
         "weight_MB_per_token": round(token_bytes / 1e6, 1),
         "GB/s": round(token_bytes * steps / decode_s / 1e9, 1),
         "frac_of_hbm_peak": round(token_bytes * steps / decode_s / 1e9 / HBM_PEAK_GBPS, 4),
+        "roofline": {"bound": "hbm", "kernel": "qkv_sparse_kernel (one launch per sparse block and token)",
+                     "achieved": round(3 * Hk * hd * d * 2 / qkv_us / 1e3, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(3 * Hk * hd * d * 2 / qkv_us / 1e3 / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "bytes_per_launch": 3 * Hk * hd * d * 2, "us_per_launch": round(qkv_us, 2)},
+        "cpu_baseline": cpu,
     }
     print(json.dumps(out))
+
+
+def decode_cpu_baseline(torch, cfg, model, layers, vocab, timed=12, warm=2):
+    """tokens/s of the PyTorch-CPU index_select + matmul form: one sparse block step timed on the host
+    cores, scaled to the model's layer count, plus the lm_head product."""
+    from oracle import cpu_baseline as C
+
+    H, hd, d, S = cfg["H"], cfg["hd"], cfg["d"], cfg["S"]
+    blk = model.transformer.layers[1]
+    m, f = blk.mixer, blk.mlp
+    g = torch.Generator().manual_seed(3)
+    t = {
+        "x": torch.randn(1, d, generator=g).half(), "x2": torch.randn(1, d, generator=g).half(),
+        "residual": torch.randn(1, d, generator=g).half(),
+        "Wqkv": m.Wqkv.weight.view(3, H, hd, d).cpu(), "bqkv": m.Wqkv.bias.view(3, H, hd).cpu(),
+        "Wout_t": m.out_proj.weight.t().contiguous().cpu(), "bout": m.out_proj.bias.cpu(),
+        "k_cache_bhsd": torch.randn(1, H, S, hd, generator=g).half(), "v_cache": torch.randn(1, H, S, hd, generator=g).half(),
+        "W1": f.fc1.weight.cpu(), "b1": f.fc1.bias.cpu(), "W2t": f.fc2.weight.t().contiguous().cpu(),
+        "b2": f.fc2.bias.cpu(), "mlp_Wa": f.sp.fc0.weight.cpu(), "mlp_Wb": f.sp.fc1.weight.cpu(),
+        "att_Wa": m.sp.fc0.weight.cpu(), "att_Wb": m.sp.fc1.weight.cpu(), "K": cfg["K"], "Hk": cfg["Hk"], "S": S,
+    }
+    head = model.lm_head.weight[:vocab].cpu()
+    ts, th = [], []
+    with torch.no_grad():
+        for i in range(warm + timed):
+            t0 = time.perf_counter()
+            C.layer_step(t)
+            t1 = time.perf_counter()
+            (t["x"].float() @ head.float().t()).argmax()
+            t2 = time.perf_counter()
+            if i >= warm:
+                ts.append(t1 - t0)
+                th.append(t2 - t1)
+    ts.sort()
+    th.sort()
+    per_token = ts[len(ts) // 2] * layers + th[len(th) // 2]
+    return {"value": round(1.0 / per_token, 3), "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"median of {timed} steps of one sparse block (x {layers} layers) + the lm_head product, torch "
+                      f"{torch.__version__} CPU index_select+matmul, fp32 compute from the same fp16 weights"}
 
 
 def mlp_bench(args):
@@ -364,7 +539,35 @@ def mlp_bench(args):
             out["path"] = ("vector ALU gather-GEMV" if B <= 2 else
                            "fc1 on MFMA tiles, fc2 vector ALU" if B <= 4 else "MFMA tiles (fc1 LDS-staged, fc2 register-transposed)")
             results[str(B)] = out
+    # roofline: the fc1 gather alone at the largest batch of the sweep; CPU baseline: the same block at batch 1
+    Bmax = max(args.batches)
+    with torch.no_grad():
+        fc1_us = time_kernel(torch, lambda t: ops.gather_gemv(t["x2"][:Bmax], t["W1"], t["idx"], t["b1"], "relu"), sets)
+    cpu = None
+    if not args.no_cpu_baseline:
+        from oracle import cpu_baseline as C
+
+        t = {k: (v.cpu() if isinstance(v, torch.Tensor) else v) for k, v in sets[0].items()}
+        ts = []
+        with torch.no_grad():
+            for i in range(2 + 15):
+                t0 = time.perf_counter()
+                ci, _ = C.predictor_topk(t["residual"][:1], t["mlp_Wa"], t["mlp_Wb"], K)
+                C.mlp_sparse(t["x2"][:1], t["W1"], t["W2t"], ci, t["b1"], t["b2"])
+                if i >= 2:
+                    ts.append(time.perf_counter() - t0)
+        ts.sort()
+        cpu = {"value": round(ts[len(ts) // 2] * 1e6, 1), "unit": "us/step", "cores": torch.get_num_threads(),
+               "kind": "port", "sample": "median of 15 block steps at batch 1 (predictor + top-k + index_select + "
+                                         f"matmul), torch {torch.__version__} CPU, fp32 compute from the same fp16 tensors"}
     print(json.dumps({
+        "value": results[str(args.batches[0])]["block"]["us"], "warmup": 5, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": round(results[str(args.batches[0])]["block"]["us"] / 1e3, 5),
+        "roofline": {"bound": "hbm", "kernel": f"fc1 gather at batch {Bmax} (gather_rows kernels)",
+                     "achieved": round(K * d * 2 / fc1_us / 1e3, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(K * d * 2 / fc1_us / 1e3 / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "bytes_per_launch": K * d * 2, "us_per_launch": round(fc1_us, 2)},
+        "cpu_baseline": cpu,
         "metric": f"us per sparse MLP block step, {args.config} shape, K={K}", "unit": "us/step", "n_gpus": 1,
         "steps": args.steps, "dtype": "f16", "data": "synthetic", "higher_is_better": False,
         "config": {"workload": f"{args.config} sparse MLP block, batch sweep", "d": d, "ffn": ffn, "K": K,
@@ -387,8 +590,6 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying HIP graphs")
     ap.add_argument("--side-stream", action="store_true",
                     help="module path: predictors / top-k on a side stream, as the reference's sp_stream (slower here)")
-    ap.add_argument("--graph-per-step", action="store_true",
-                    help="one HIP graph per step even when the step counts allow one graph per schedule period")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="for rocprofv3 --pmc runs: also run a plain 1 GiB device copy (known traffic) to calibrate the "
                          "counters, and skip the replay-spread and window-start legs (thousands of dispatches)")
@@ -400,11 +601,16 @@ def main():
                     help="layer: the headline sparse decode layer; decode: end-to-end greedy generation "
                          "(40-layer OPT-13B shape, --steps = new tokens, default 256)")
     ap.add_argument("--decode-layers", type=int, default=40)
+    ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"), default=None,
+                    help="no GPU work: read the counter CSVs of two `rocprofv3 --pmc` runs of `bench.py "
+                         "--pmc-calibration` (FETCH_SIZE, then WRITE_SIZE) and write profiles/traffic.json")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs the sparse decode layer on ONE GPU (no sharding); "
               "use --gpus 1", file=sys.stderr)
         sys.exit(2)
+    if args.traffic_from:
+        return write_traffic(*args.traffic_from)
 
     import torch
 
@@ -424,10 +630,17 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(1)
+    if args.steps < 1 or args.warmup < 0:
+        print("bench.py: --steps must be >= 1 and --warmup >= 0", file=sys.stderr)
+        sys.exit(2)
     torch.cuda.set_device(0)
     cfg = CONFIGS[args.config]
     batch = args.batch
-    assert batch == 1, "the head-sparse decode layer keeps one back-fill window (batch 1)"
+    if not 1 <= batch <= 32:
+        print("bench.py: --batch must be in 1..32", file=sys.stderr)
+        sys.exit(2)
+    if batch > 1:
+        args.window = "start"  # B sequences in lockstep: every step at the first position of a window
     device = torch.device("cuda:0")
     layers = build_layers(cfg, batch, device)
     cycle = args.window == "cycle"
@@ -440,23 +653,61 @@ def main():
             return window_step(layers[l], c)
         return layer_step(layers[i % N_LAYERS])
 
-    def capture(first, count):
-        g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g):
-            for i in range(first, first + count):
-                step_fn(i)
-            dv_modules.join_side_stream()
-        return g
+    graphs = {}
 
-    def timed(run, steps, warmup):
-        for i in range(warmup):
-            run(i)
+    def graph_for(first, count):
+        """HIP graph of steps first .. first+count-1; the schedule repeats with `period`, so graphs
+        are shared by (phase, length).  Capturing runs the host side of every step in order."""
+        key = (first % period, count)
+        if key not in graphs:
+            # bring the host-side window state to the phase the graph starts at
+            c0 = (first % period) // N_LAYERS if cycle else 0
+            if cycle:
+                for l, L in enumerate(layers):
+                    L["block"].mixer.counter = c0 + (1 if l < (first % period) % N_LAYERS else 0)
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                for i in range(first, first + count):
+                    step_fn(i)
+                dv_modules.join_side_stream()
+            graphs[key] = g
+        return graphs[key]
+
+    def plan(first, count):
+        """Graphs that cover steps first .. first+count-1 in chunks of at most MAX_GRAPH_STEPS."""
+        out = []
+        while count > 0:
+            n = min(count, MAX_GRAPH_STEPS)
+            out.append(graph_for(first, n))
+            first += n
+            count -= n
+        return out
+
+    def run_timed(first_warm, n_warm, n_timed):
+        """Replays the warm-up steps, synchronises, then times exactly n_timed steps."""
+        warm = plan(first_warm, n_warm) if n_warm > 0 else []
+        timed = plan(first_warm + n_warm, n_timed)
+        for g in warm:
+            g.replay()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for i in range(steps):
-            run(i)
+        for g in timed:
+            g.replay()
         torch.cuda.synchronize()
-        return (time.perf_counter() - t0) / steps * 1e6
+        return (time.perf_counter() - t0) / n_timed * 1e6
+
+    nbytes = algorithmic_bytes(cfg, batch)
+    start_bytes = sum(nbytes.values())
+    flush_bytes = flush_step_bytes(cfg, batch)
+
+    def schedule_bytes(first, count):
+        """Algorithmic bytes and window positions of steps first .. first+count-1."""
+        total, hist = 0, [0] * WINDOW
+        for i in range(first, first + count):
+            c = (i % period) // N_LAYERS if cycle else 0
+            hist[c] += 1
+            total += flush_bytes if (cycle and c == WINDOW - 1) else start_bytes
+        return total, hist
 
     with torch.no_grad():
         if not cycle:
@@ -468,55 +719,56 @@ def main():
             step_fn(i)
         dv_modules.join_side_stream()
         torch.cuda.synchronize()
-        whole = args.steps % period == 0 and args.warmup % period == 0 and not args.graph_per_step
         spread = None
         if args.no_graph:
-            us_per_layer = timed(step_fn, args.steps, args.warmup)
-            graph_mode = "none"
-        elif whole:
-            # one graph holds as many whole schedule periods as the step counts allow (up to 4):
-            # the gap between two graph launches is harness time, not part of a layer step
-            span = period
-            for reps in (4, 2):
-                if args.steps % (reps * period) == 0 and args.warmup % (reps * period) == 0:
-                    span = reps * period
-                    break
-            g = capture(0, span)
+            for i in range(args.warmup):
+                step_fn(i)
             torch.cuda.synchronize()
-            us_per_layer = timed(lambda i: g.replay() if i % span == 0 else None, args.steps, args.warmup)
-            graph_mode = f"one graph of {span} steps"
-            # spread over single replays (outside the timed region): one event pair per replay
-            # (a counter-collection run needs only one replay: every dispatch is serialised there)
-            evs = [torch.cuda.Event(enable_timing=True) for _ in range(2 if args.pmc_calibration else 21)]
+            t0 = time.perf_counter()
+            for i in range(args.warmup, args.warmup + args.steps):
+                step_fn(i)
+            torch.cuda.synchronize()
+            us_per_layer = (time.perf_counter() - t0) / args.steps * 1e6
+            graph_mode = "none"
+        else:
+            us_per_layer = run_timed(0, args.warmup, args.steps)
+            graph_mode = f"graphs of up to {MAX_GRAPH_STEPS} consecutive steps"
+        timed_bytes, positions = schedule_bytes(args.warmup, args.steps)
+        layer_bytes = timed_bytes / args.steps
+
+        # whole windows (every position equally often) and the first position alone, whatever --steps is
+        window_average_us = window_start_us = None
+        if cycle and not args.no_graph and not args.pmc_calibration:
+            if args.steps % period == 0:
+                window_average_us = us_per_layer
+            else:
+                window_average_us = run_timed(0, period, 4 * period)
+            # spread over single replays of one four-period graph: one event pair per replay
+            g = graph_for(0, 4 * period)
+            evs = [torch.cuda.Event(enable_timing=True) for _ in range(21)]
+            g.replay()
             evs[0].record()
             for e in evs[1:]:
                 g.replay()
                 e.record()
             torch.cuda.synchronize()
-            per = sorted(a.elapsed_time(b) * 1e3 / span for a, b in zip(evs[:-1], evs[1:]))
-            spread = {"unit": f"us/layer over one replay of {span} steps", "replays": len(per),
+            per = sorted(a.elapsed_time(b) * 1e3 / (4 * period) for a, b in zip(evs[:-1], evs[1:]))
+            spread = {"unit": f"us/layer over one replay of {4 * period} steps", "replays": len(per),
                       "median": round(per[len(per) // 2], 2), "p10": round(per[len(per) // 10], 2),
                       "p90": round(per[(len(per) * 9) // 10], 2)}
-        else:
-            graphs = [capture(i, 1) for i in range(period)]
-            torch.cuda.synchronize()
-            us_per_layer = timed(lambda i: graphs[i % period].replay(), args.steps, args.warmup)
-            graph_mode = "one graph per step"
-
-        # the same three layers at the first position of a window only (no back-fill work)
-        window_start_us = None
-        if cycle and not args.no_graph and not args.pmc_calibration:
-            cycle = False
+            cycle, period_saved = False, period
+            period = N_LAYERS
+            graphs_saved, graphs = graphs, {}
             for L in layers:
                 L["block"].mixer.cache_offset.fill_(cfg["S"] - 1)
                 L["offset_mode"] = "start"
             for i in range(N_LAYERS):
                 step_fn(i)
-            span0 = 64 * N_LAYERS  # long graph: launch gaps between replays are harness time
-            g0 = capture(0, span0)
             torch.cuda.synchronize()
-            window_start_us = timed(lambda i: g0.replay() if i % span0 == 0 else None, 5 * span0, span0)
-            cycle = True
+            window_start_us = run_timed(0, MAX_GRAPH_STEPS, 5 * MAX_GRAPH_STEPS)
+            cycle, period, graphs = True, period_saved, graphs_saved
+        elif not cycle and not args.no_graph:
+            window_start_us = us_per_layer
 
         if args.pmc_calibration:
             src = torch.empty(1 << 30, dtype=torch.uint8, device=device)
@@ -526,21 +778,53 @@ def main():
             torch.cuda.synchronize()
             del src, dst
 
-        nbytes = algorithmic_bytes(cfg, batch)
-        start_bytes = sum(nbytes.values())
-        # a window = 15 steps with the predicted heads + 1 flush step with all heads
-        layer_bytes = (15 * start_bytes + flush_step_bytes(cfg, batch)) / 16 if args.window == "cycle" \
-            else start_bytes
         table = kernel_table(torch, cfg, batch, layers)
-        dom = "qkv_sparse"  # largest share of the layer's bytes
-        roofline = {"bound": "hbm", "kernel": "qkv_sparse_kernel", "achieved": table[dom]["GB/s"],
-                    "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": table[dom]["frac"],
-                    "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, batch, dom)),
-                    "bytes_per_launch": nbytes[dom], "us_per_launch": table[dom]["us"]}
+        if batch == 1:
+            # the QKV projection as the schedule runs it: position 0 on the vector ALUs, positions
+            # 1..14 on the matrix cores, position 15 the flush over all heads; weighted by how often
+            # the timed steps visit each
+            n0 = positions[0] if cycle else args.steps
+            n1 = sum(positions[1:WINDOW - 1]) if cycle else 0
+            n2 = positions[WINDOW - 1] if cycle else 0
+            mix = (("qkv_sparse", n0), ("qkv_window_mfma", n1), ("qkv_flush_mfma", n2))
+            mix_bytes = sum(table[k]["MB"] * 1e6 * n for k, n in mix)
+            mix_us = sum(table[k]["us"] * n for k, n in mix)
+            launches = n0 + n1 + n2
+            roofline = {"bound": "hbm", "kernel": "QKV projection of the timed schedule: qkv_sparse_kernel (window "
+                        "position 0), qkv_window_mfma_kernel<4,1> (positions 1-14), qkv_window_mfma_kernel<4,2> "
+                        "(flush); the fused layer runs the same bodies as layer_l2_kernel<1>, <0>, <-1>",
+                        "achieved": round(mix_bytes / mix_us / 1e3, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                        "frac": round(mix_bytes / mix_us / 1e3 / HBM_PEAK_GBPS, 4),
+                        "traffic": measured_traffic(args.config, batch, "qkv_sparse"),
+                        "traffic_kernel": "qkv_sparse_kernel",
+                        "bytes_per_launch": round(mix_bytes / launches), "us_per_launch": round(mix_us / launches, 2),
+                        "launch_mix": {k: n for k, n in mix},
+                        "standalone": {k: table[k] for k, _ in mix}}
+        else:
+            dom = "decode_attn" if nbytes["decode_attn"] >= nbytes["qkv_sparse"] else "qkv_batch"
+            roofline = {"bound": "hbm", "kernel": {"decode_attn": "decode_attn_kernel", "qkv_batch":
+                                                   "qkv_batch_mfma_kernel"}[dom],
+                        "achieved": table[dom]["GB/s"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                        "frac": table[dom]["frac"], "traffic": None,
+                        "bytes_per_launch": round(table[dom]["MB"] * 1e6), "us_per_launch": table[dom]["us"]}
         cpu = None
         if not args.no_cpu_baseline:
-            cpu = cpu_baseline(torch, cfg, batch, layers[0])
+            cpu = cpu_baseline(torch, cfg, batch, layers[0], timed=40 if batch == 1 else 12)
 
+    def leg(us, nb):
+        return None if us is None else {"us_per_layer": round(us, 2), "algorithmic_MB": round(nb / 1e6, 1),
+                                        "GB/s": round(nb / us / 1e3, 1),
+                                        "frac_of_hbm_peak": round(nb / us / 1e3 / HBM_PEAK_GBPS, 4)}
+
+    covered = [c for c in range(WINDOW) if positions[c]]
+    if not cycle:
+        what = "every step at the first position of a back-fill window (no back-fill work)"
+    elif args.steps % period == 0:
+        what = "steps walk whole 16-token back-fill windows (heads re-drawn every token, flush step included)"
+    else:
+        what = (f"steps {args.warmup}..{args.warmup + args.steps - 1} of the window-walking schedule: window positions "
+                f"{covered[0]}..{covered[-1]}" + (", flush step included" if positions[WINDOW - 1] else ", no flush step")
+                + "; see window_average for whole windows")
     out = {
         "metric": "us_per_layer, sparse MLP+attn decode, OPT-175B layer K=4096" if args.config == "opt-175b"
         else f"us_per_layer, sparse MLP+attn decode, {args.config}",
@@ -555,21 +839,17 @@ def main():
         "vs_baseline": None,
         "dtype": "f16",
         "data": "synthetic",
-        "config": {"workload": f"{args.config} sparse decode layer, batch 1, " + (
-            "steps walk 16-token back-fill windows (heads re-drawn every token, flush step included)"
-            if args.window == "cycle" else "first position of a back-fill window"), "d": cfg["d"], "ffn": cfg["ffn"],
-                   "heads": cfg["H"], "head_dim": cfg["hd"], "K": cfg["K"], "active_heads": cfg["Hk"],
-                   "predictor_rank": cfg["r"], "kv_len": cfg["S"], "batch": batch,
+        "config": {"workload": f"{args.config} sparse decode layer, batch {batch}, " + what, "d": cfg["d"],
+                   "ffn": cfg["ffn"], "heads": cfg["H"], "head_dim": cfg["hd"], "K": cfg["K"],
+                   "active_heads": cfg["Hk"], "predictor_rank": cfg["r"], "kv_len": cfg["S"], "batch": batch,
                    "layers_cycled": N_LAYERS, "window": args.window, "hip_graph": graph_mode},
+        "positions": {"steps_per_window_position": positions, "schedule_period": period},
         "roofline": roofline,
+        "mlp_pair": table["mlp_pair"],
         "cpu_baseline": cpu,
-        "window_start": None if window_start_us is None else {
-            "us_per_layer": round(window_start_us, 2), "algorithmic_MB": round(start_bytes / 1e6, 1),
-            "GB/s": round(start_bytes / window_start_us / 1e3, 1),
-            "frac_of_hbm_peak": round(start_bytes / window_start_us / 1e3 / HBM_PEAK_GBPS, 4)},
-        "layer": {"algorithmic_MB": round(layer_bytes / 1e6, 1), "GB/s": round(layer_bytes / us_per_layer / 1e3, 1),
-                  "frac_of_hbm_peak": round(layer_bytes / us_per_layer / 1e3 / HBM_PEAK_GBPS, 4),
-                  "tokens_per_s_per_layer": round(batch / (us_per_layer * 1e-6), 1)},
+        "layer": dict(leg(us_per_layer, layer_bytes), tokens_per_s_per_layer=round(batch / (us_per_layer * 1e-6), 1)),
+        "window_start": leg(window_start_us, start_bytes),
+        "window_average": leg(window_average_us, (15 * start_bytes + flush_bytes) / 16) if cycle else None,
         "spread": spread,
         "kernels": table,
     }

@@ -35,8 +35,8 @@ SIGNATURES = {
     "dv_predictor_workspace_bytes": (_c_size, [_c_int, _c_int, _c_int]),
     "dv_predictor_logits_ws_f16": (_c_int, [_c_ptr, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int,
                                             _c_ptr, _c_ptr, _c_ptr, _c_size, _c_ptr]),
-    "dv_greedy_advance_f16": (_c_int, [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64,
-                                       _c_ptr, _c_ptr]),
+    "dv_greedy_advance_f16": (_c_int, [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_i64,
+                                       _c_i64, _c_ptr, _c_ptr]),
     "dv_topk_workspace_bytes": (_c_size, [_c_int]),
     "dv_topk_f16": (_c_int, [_c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_ptr, _c_size, _c_ptr]),
     "dv_topk_search_f16": (_c_int, [_c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_int, _c_ptr]),

@@ -608,16 +608,17 @@ int dv_topk_f16(const void* logits, int B, int n, int k, void* idx_out, int idx_
 }
 
 int dv_greedy_advance_f16(const void* logits, int vocab, void* token, void* position, void* seq_pos,
-                          void* sequences, void* out_index, void* scores, int64_t score_ld,
-                          void* score_index, void* stream) {
-  if (!logits || vocab < 1 || !token || !position || !seq_pos || !sequences || !out_index ||
-      (scores && (!score_index || score_ld < vocab)))
+                          void* sequences, int64_t seq_capacity, void* out_index, void* scores,
+                          int64_t score_ld, int64_t score_rows, void* score_index, void* stream) {
+  if (!logits || vocab < 1 || !token || !position || !seq_pos || !sequences || !out_index || seq_capacity < 0 ||
+      (scores && (!score_index || score_ld < vocab || score_rows < 0)))
     return DV_ERR_INVALID_ARG;
   hipLaunchKernelGGL(greedy_advance_kernel, dim3(1), dim3(1024), 0, reinterpret_cast<hipStream_t>(stream),
                      reinterpret_cast<const half_t*>(logits), vocab, reinterpret_cast<int64_t*>(token),
                      reinterpret_cast<int64_t*>(position), reinterpret_cast<int*>(seq_pos),
                      reinterpret_cast<int64_t*>(sequences), reinterpret_cast<int64_t*>(out_index),
-                     reinterpret_cast<half_t*>(scores), score_ld, reinterpret_cast<int64_t*>(score_index));
+                     reinterpret_cast<half_t*>(scores), score_ld, reinterpret_cast<int64_t*>(score_index),
+                     seq_capacity, score_rows);
   return launch_status();
 }
 
@@ -1043,7 +1044,7 @@ int dv_out_proj_sparse_f16(const void* x, const void* W, const void* bias, const
                            int nnz, int B, int H, int hd, int N, void* y, void* stream) {
   if (!x || !W || !y || nnz < 0 || B < 1 || H <= 0 || N <= 0 || (nnz > 0 && !head_idx))
     return DV_ERR_INVALID_ARG;
-  if (B > 4 || (hd != 64 && hd != 128)) return DV_ERR_UNSUPPORTED;
+  if (B > 16 || (hd != 32 && hd != 64 && hd != 128)) return DV_ERR_UNSUPPORTED;
   if (!aligned16(x) || !aligned16(W)) return DV_ERR_ALIGNMENT;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   constexpr int R = 4;
@@ -1051,17 +1052,28 @@ int dv_out_proj_sparse_f16(const void* x, const void* W, const void* bias, const
   int blocks = (ntasks + 3) / 4;
   const int cap = compute_units() * 8;
   if (blocks > cap) blocks = cap;
+  // up to four batch rows share one pass over the weights; larger batches (the reference takes up
+  // to 16) run as passes of four: this layout is kept for compatibility, the transposed weight
+  // (dv_out_proj_sparse_t_f16) is the one that streams a batch in a single pass
+  for (int b0 = 0; b0 < B; b0 += 4) {
+    const int nb = B - b0 < 4 ? B - b0 : 4;
+    const half_t* xx = reinterpret_cast<const half_t*>(x) + (int64_t)b0 * H * hd;
+    half_t* yy = reinterpret_cast<half_t*>(y) + (int64_t)b0 * N;
 #define DV_OP(BB, HH)                                                                          \
-  hipLaunchKernelGGL((out_proj_rows_kernel<BB, R, HH>), dim3(blocks), dim3(256), 0, s,          \
-                     reinterpret_cast<const half_t*>(x), reinterpret_cast<const half_t*>(W),   \
-                     reinterpret_cast<const half_t*>(bias), reinterpret_cast<const int*>(head_idx), \
-                     nnz, H, N, reinterpret_cast<half_t*>(y))
-  if (hd == 128) {
-    switch (B) { case 1: DV_OP(1, 128); break; case 2: DV_OP(2, 128); break; case 3: DV_OP(3, 128); break; default: DV_OP(4, 128); }
-  } else {
-    switch (B) { case 1: DV_OP(1, 64); break; case 2: DV_OP(2, 64); break; case 3: DV_OP(3, 64); break; default: DV_OP(4, 64); }
+  hipLaunchKernelGGL((out_proj_rows_kernel<BB, R, HH>), dim3(blocks), dim3(256), 0, s, xx,      \
+                     reinterpret_cast<const half_t*>(W), reinterpret_cast<const half_t*>(bias), \
+                     reinterpret_cast<const int*>(head_idx), nnz, H, N, yy)
+#define DV_OPB(HH)                                                                   \
+  switch (nb) {                                                                      \
+    case 1: DV_OP(1, HH); break;                                                     \
+    case 2: DV_OP(2, HH); break;                                                     \
+    case 3: DV_OP(3, HH); break;                                                     \
+    default: DV_OP(4, HH);                                                           \
   }
+    if (hd == 128) { DV_OPB(128) } else if (hd == 64) { DV_OPB(64) } else { DV_OPB(32) }
+#undef DV_OPB
 #undef DV_OP
+  }
   return launch_status();
 }
 

@@ -475,7 +475,8 @@ __global__ __launch_bounds__(256) void topk_emit_kernel(const half_t* __restrict
 __global__ __launch_bounds__(1024) void greedy_advance_kernel(
     const half_t* __restrict__ logits, int vocab, int64_t* __restrict__ token, int64_t* __restrict__ position,
     int* __restrict__ seq_pos, int64_t* __restrict__ sequences, int64_t* __restrict__ out_index,
-    half_t* __restrict__ scores, int64_t score_ld, int64_t* __restrict__ score_index) {
+    half_t* __restrict__ scores, int64_t score_ld, int64_t* __restrict__ score_index, int64_t seq_capacity,
+    int64_t score_rows) {
   __shared__ unsigned s_key[16];
   __shared__ int s_idx[16];
   unsigned best = 0u;
@@ -523,7 +524,8 @@ __global__ __launch_bounds__(1024) void greedy_advance_kernel(
     s_key[wave] = best;
     s_idx[wave] = best_i;
   }
-  if (scores != nullptr) {
+  // a replay past the end of the output buffers (the host loop normally stops first) stores nothing
+  if (scores != nullptr && score_index[0] >= 0 && score_index[0] < score_rows) {
     half_t* row = scores + score_index[0] * score_ld;
     for (int i = threadIdx.x; i < vocab; i += blockDim.x) row[i] = logits[i];
   }
@@ -535,7 +537,7 @@ __global__ __launch_bounds__(1024) void greedy_advance_kernel(
         best_i = s_idx[w];
       }
     token[0] = best_i;
-    sequences[out_index[0]] = best_i;
+    if (out_index[0] >= 0 && out_index[0] < seq_capacity) sequences[out_index[0]] = best_i;
     out_index[0] += 1;
     position[0] += 1;
     seq_pos[0] += 1;

@@ -48,13 +48,11 @@ _workspaces: dict = {}
 
 
 def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
-    """Per-device scratch shared by all layers (they run one after the other)."""
-    key = (device.type, device.index)
-    ws = _workspaces.get(key)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
-        _workspaces[key] = ws
-    return ws
+    """Per-device scratch shared by all layers (they run one after the other).  A buffer that is
+    outgrown stays allocated (captured HIP graphs may hold its address)."""
+    from . import ops
+
+    return ops._grown(_workspaces, device, nbytes, 16 << 20)
 
 
 def _ptr(t):
@@ -89,10 +87,8 @@ def sparse_layer_decode(block, hidden_states, residual, head_idx, mlp_sp_logit, 
     dev = hidden_states.device
     d, H, hd = m.embed_dim, m.num_heads, m.head_dim
     ffn = f.fc1.out_features
-    if f.fc2_weight_t is None:
-        f.fc2_weight_t = f.fc2.weight.t().contiguous()
-    if m.out_proj_weight_t is None:
-        m.out_proj_weight_t = m.out_proj.weight.t().contiguous()
+    f.transposed_fc2()
+    m.transposed_out_proj()
     if m.cache_offset is None:
         m._set_cache_offset(inference_params.sequence_len_offset - m.counter, dev)
     flush = m.counter == m.WINDOW - 1

@@ -264,6 +264,9 @@ class GPTLMHeadModel(nn.Module):
         elif not output_scores and cache.scores is not None:
             cache.scores = None
             cache.graphs.clear()
+        if getattr(cache, "graph_key", None) != (vocab_size, bool(output_scores)):
+            cache.graphs.clear()  # captured steps hold the logits slice and the score buffer of their run
+            cache.graph_key = (vocab_size, bool(output_scores))
         ip = cache.inference_params
 
         # prompt: dense, fills the caches

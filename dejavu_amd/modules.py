@@ -62,6 +62,20 @@ def join_side_stream() -> None:
         torch.cuda.current_stream().wait_event(ev)
 
 
+def _transposed_copy(module, attr: str, weight: torch.Tensor) -> torch.Tensor:
+    """``weight.t().contiguous()`` kept in ``module.<attr>`` and rebuilt when the weight has been
+    written since (load_state_dict, an in-place update) or replaced.  A tensor the caller put
+    there itself is taken as matching the weight at that moment."""
+    stamp = (weight.data_ptr(), weight._version, tuple(weight.shape))
+    cur = getattr(module, attr)
+    if cur is None or (getattr(module, attr + "_stamp", None) not in (None, stamp)) or \
+            cur.shape != (weight.shape[1], weight.shape[0]):
+        cur = weight.t().contiguous()
+        setattr(module, attr, cur)
+    setattr(module, attr + "_stamp", stamp)
+    return cur
+
+
 def _world_size(process_group) -> int:
     if process_group is None:
         return 1
@@ -148,6 +162,10 @@ class ParallelFusedMLPDejavu(nn.Module):
             self.event_mlp = torch.cuda.Event(enable_timing=False, blocking=False)
             self.event_mlp_sp = torch.cuda.Event(enable_timing=False, blocking=False)
 
+    def transposed_fc2(self) -> torch.Tensor:
+        """fc2.weight as (hidden, out), contiguous; follows updates of fc2.weight."""
+        return _transposed_copy(self, "fc2_weight_t", self.fc2.weight)
+
     def forward(self, x, residual, idx=None):
         """x, residual: (B, 1, d) at decode (or (B, s, d) for the prompt).
         idx: (K,) active neurons or None for the dense MLP.
@@ -173,9 +191,8 @@ class ParallelFusedMLPDejavu(nn.Module):
             assert x.size(1) == 1
             if self.activation != "relu":
                 raise NotImplementedError("the sparse MLP kernels fuse ReLU (OPT); gelu_approx runs dense only")
-            if self.fc2_weight_t is None:
-                self.fc2_weight_t = self.fc2.weight.t().contiguous()
-            out = ops.mlp_sparse(x.squeeze(1), self.fc1.weight, self.fc2_weight_t, idx, self.fc1.bias, self.fc2.bias)
+            out = ops.mlp_sparse(x.squeeze(1), self.fc1.weight, self.transposed_fc2(), idx, self.fc1.bias,
+                                 self.fc2.bias)
             out = out.unsqueeze(1)
         else:
             if self.activation == "relu":
@@ -356,6 +373,10 @@ class ParallelMHASparseAttMlp(_MHABase):
         # optional caller-owned buffer for the predicted heads (fixed address for graph capture)
         self.att_idx_out = None
 
+    def transposed_out_proj(self) -> torch.Tensor:
+        """out_proj.weight as (H * hd, d), contiguous; follows updates of out_proj.weight."""
+        return _transposed_copy(self, "out_proj_weight_t", self.out_proj.weight)
+
     def _set_cache_offset(self, value: int, device) -> None:
         """Updated in place once it exists: captured launch sequences hold its address."""
         if self.cache_offset is None:
@@ -455,8 +476,7 @@ class ParallelMHASparseAttMlp(_MHABase):
                                            self.att_k, self.att_idx_out)
         if sparse:
             assert x.size(1) == 1
-            if self.out_proj_weight_t is None:
-                self.out_proj_weight_t = self.out_proj.weight.t().contiguous()
+            self.transposed_out_proj()
             if x.size(0) == 1:
                 qkv, head_idx, kc, vc = self._sparse_decode(x, head_idx, inference_params)
                 # the caches now hold the newest token for the active heads

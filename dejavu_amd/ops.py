@@ -46,17 +46,27 @@ def _require_device(*tensors: Optional[torch.Tensor]) -> None:
 # workspace (fp32 partial sums of the split reductions)
 # ---------------------------------------------------------------------------
 _workspaces: dict = {}
+# Scratch buffers that were replaced by larger ones.  They are kept for the life of the process:
+# a captured HIP graph holds the raw address of the buffer that was current when it was captured,
+# so that memory must never go back to the allocator while such a graph may still be replayed.
+_retired_workspaces: list = []
+
+
+def _grown(cache: dict, device: torch.device, nbytes: int, floor: int) -> torch.Tensor:
+    key = (device.type, device.index)
+    ws = cache.get(key)
+    if ws is None or ws.numel() < nbytes:
+        if ws is not None:
+            _retired_workspaces.append(ws)
+        ws = torch.empty(max(nbytes, floor), dtype=torch.uint8, device=device)
+        cache[key] = ws
+    return ws
 
 
 def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
     """Per-device scratch, grown on demand (the kernels write every word before they read it).
     Ops that share it must not run concurrently on different streams."""
-    key = (device.type, device.index)
-    ws = _workspaces.get(key)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
-        _workspaces[key] = ws
-    return ws
+    return _grown(_workspaces, device, nbytes, 8 << 20)
 
 
 # ---------------------------------------------------------------------------
@@ -156,8 +166,9 @@ def greedy_advance(logits: torch.Tensor, token: torch.Tensor, position: torch.Te
     if scores is not None:
         assert scores.dtype == torch.float16 and scores.stride(-1) == 1 and score_index.dtype == torch.int64
     check(lib.dv_greedy_advance_f16(_ptr(logits), logits.numel(), _ptr(token), _ptr(position), _ptr(seq_pos),
-                                    _ptr(sequences), _ptr(out_index), _ptr(scores),
-                                    0 if scores is None else scores.stride(0), _ptr(score_index), _stream()),
+                                    _ptr(sequences), sequences.numel(), _ptr(out_index), _ptr(scores),
+                                    0 if scores is None else scores.stride(0),
+                                    0 if scores is None else scores.shape[0], _ptr(score_index), _stream()),
           "dv_greedy_advance_f16")
 
 
@@ -389,8 +400,6 @@ def out_proj_sparse(x: torch.Tensor, weight: torch.Tensor, head_idx: torch.Tenso
     assert head_idx.shape == (n_active,)
     assert head_idx.dtype == torch.int32
     assert batch <= 16
-    if batch > 4 or head_dim == 32:
-        raise NotImplementedError("out_proj_sparse kernels cover batch <= 4 and head_dim in {64, 128}")
     x = x.contiguous()
     weight = weight.contiguous()
     assert x.dtype == weight.dtype, f"Input and weight must have the same dtype, got {x.dtype} and {weight.dtype}"
@@ -521,6 +530,7 @@ def single_query_attention(q: torch.Tensor, k: Optional[torch.Tensor], v: Option
     assert rotary_emb_dim == 0, "OPT has no rotary embedding"
     B, H, hd = q.shape
     S = v_cache.shape[2]
+    assert hd in [64, 128], "the decode attention kernels are built for head_dim 64 and 128"
     assert q.dtype == torch.float16 and k_cache.dtype == torch.float16 and v_cache.dtype == torch.float16
     assert v_cache.shape == (B, H, S, hd) and k_cache.shape == (B, H, hd // 8, S, 8)
     assert k_cache.is_contiguous() and v_cache.is_contiguous()
@@ -557,12 +567,7 @@ _attn_workspaces: dict = {}
 
 
 def _attn_workspace(device: torch.device, nbytes: int) -> torch.Tensor:
-    key = (device.type, device.index)
-    ws = _attn_workspaces.get(key)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
-        _attn_workspaces[key] = ws
-    return ws
+    return _grown(_attn_workspaces, device, nbytes, 4 << 20)
 
 
 # ---------------------------------------------------------------------------

@@ -288,7 +288,8 @@ DV_API int dv_attention_out_proj_rows_f16(const void* q, int64_t ldq, const void
  * y[b, n] = sum_{h in head_idx} x[b, h, :] . W[n, h, :] + bias[n], weight in
  * out_proj.weight's own (d, H, hd) layout.  Replaces out_proj_sparse,
  * Dejavu/src/ops/triton/attention_proj_sparse.py:274-338.
- *   x (B, H, hd) contiguous, B <= 4; W (N, H, hd) contiguous; head_idx int32.
+ *   x (B, H, hd) contiguous, B <= 16 (passes of four rows over the weights); W (N, H, hd)
+ *   contiguous; head_idx int32; hd in {32, 64, 128}.
  */
 DV_API int dv_out_proj_sparse_f16(const void* x, const void* W, const void* bias,
                                   const void* head_idx, int nnz, int B, int H, int hd, int N,
@@ -327,6 +328,8 @@ DV_API int dv_add_layer_norm_f16(const void* h, const void* residual, const void
  * among equal values; then, all on the device so that a captured step can be replayed:
  * token[0] = next, sequences[out_index[0]++] = next, position[0]++, seq_pos[0]++ and, with
  * scores != NULL, scores[score_index[0]++, :vocab] = logits (rows of score_ld elements).
+ * The two stores are skipped (the counters still advance) once out_index[0] reaches seq_capacity
+ * or score_index[0] reaches score_rows: a replayed step cannot write past the buffers.
  * Replaces the sampling step of the greedy loop the reference takes from flash-attention v0.2.8
  * utils/generation.py (decode(): `sample(logits, top_k=1)` + sequence / length bookkeeping;
  * call site Dejavu/benchmarks/benchmark_generation_opt_dejavu.py:187-196).
@@ -334,8 +337,9 @@ DV_API int dv_add_layer_norm_f16(const void* h, const void* residual, const void
  *   sequences int64 (row of the output); scores fp16 or NULL.
  */
 DV_API int dv_greedy_advance_f16(const void* logits, int vocab, void* token, void* position,
-                                 void* seq_pos, void* sequences, void* out_index, void* scores,
-                                 int64_t score_ld, void* score_index, void* stream);
+                                 void* seq_pos, void* sequences, int64_t seq_capacity, void* out_index,
+                                 void* scores, int64_t score_ld, int64_t score_rows, void* score_index,
+                                 void* stream);
 
 /*
  * One decode step (batch 1, one new token) of a whole sparse block in eight

@@ -116,7 +116,10 @@ def test_qkv_proj_sparse_no_bias_and_empty(ops):
 
 # ------------------------------------------------------------- out_proj
 @pytest.mark.parametrize("H,hd,d,B,nnz", [(12, 128, 12288, 2, 4), (12, 64, 768, 1, 4), (72, 128, 1152, 1, 24),
-                                          (8, 128, 520, 4, 3), (16, 128, 1024, 3, 16)])
+                                          (8, 128, 520, 4, 3), (16, 128, 1024, 3, 16),
+                                          # up to 16 rows as the reference op takes (passes of four), head_dim 32
+                                          (8, 128, 1024, 5, 3), (12, 64, 768, 16, 5), (16, 32, 512, 2, 6),
+                                          (16, 32, 512, 13, 6)])
 def test_out_proj_sparse_both_layouts(ops, H, hd, d, B, nnz):
     g = torch.Generator().manual_seed(2)
     if d % 128:
