@@ -44,6 +44,18 @@ SIGNATURES = {
         _c_int,
         [_c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr],
     ),
+    "dv_gather_gemv_workspace_bytes": (_c_size, [_c_int, _c_int, _c_int]),
+    "dv_gather_gemv_ws_f16": (
+        _c_int,
+        [_c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr,
+         _c_size, _c_ptr],
+    ),
+    "dv_dense_linear_workspace_bytes": (_c_size, [_c_int, _c_int, _c_int]),
+    "dv_dense_linear_f16": (
+        _c_int,
+        [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_i64, _c_ptr, _c_size,
+         _c_ptr],
+    ),
     "dv_gather_transposed_gemv_workspace_bytes": (_c_size, [_c_int, _c_int, _c_int]),
     "dv_gather_transposed_gemv_f16": (
         _c_int,
@@ -64,6 +76,9 @@ SIGNATURES = {
         _c_int,
         [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr,
          _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr]),
+    "dv_prefill_attention_f16": (
+        _c_int,
+        [_c_ptr, _c_int, _c_int, _c_int, _c_int, ctypes.c_float, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr]),
     "dv_attention_out_proj_workspace_bytes": (_c_size, [_c_int, _c_int, _c_int, _c_int, _c_int]),
     "dv_attention_out_proj_f16": (
         _c_int,

@@ -11,10 +11,12 @@
 #include "attention.hpp"
 #include "common.hpp"
 #include "gemm_mfma.hpp"
+#include "gemm_tiled.hpp"
 #include "gemv_cols.hpp"
 #include "gemv_rows.hpp"
 #include "layer_fused.hpp"
 #include "norm.hpp"
+#include "prefill.hpp"
 #include "qkv_mfma.hpp"
 #include "topk.hpp"
 
@@ -362,6 +364,95 @@ int rows_short_mfma(const half_t* x, const half_t* W, int64_t ldw, int B, int N,
   return B <= 16 ? launch_rows_short<1>(x, W, ldw, B, N, M, y, s) : launch_rows_short<2>(x, W, ldw, B, N, M, y, s);
 }
 
+// ---- X-shared split-K products (gemm_tiled.hpp) ---------------------------------
+struct TiledPlan {
+  int bt, wt, kc, xblocks, row_groups, nsplit, chunks_per_split;
+};
+
+TiledPlan plan_tiled(int B, int N, int M) {
+  TiledPlan p;
+  p.bt = B <= 16 ? 1 : (B <= 32 ? 2 : (B <= 64 ? 4 : 8));
+  p.kc = p.bt == 8 ? 128 : 256;
+  p.xblocks = (B + 16 * p.bt - 1) / (16 * p.bt);
+  const int cus = compute_units();
+  // 32 rows per wavefront halve the LDS reads of X per weight byte; worth it when the matrix still
+  // gives every compute unit a workgroup
+  // (LDS holds 32-row wavefront tiles next to one or eight batch tiles of X, not next to two or four)
+  p.wt = (p.bt == 8 || (p.bt == 1 && (int64_t)M * p.xblocks >= (int64_t)256 * cus)) ? 2 : 1;
+  p.row_groups = (M + kTgWaves * 16 * p.wt - 1) / (kTgWaves * 16 * p.wt);
+  const int nchunks = (N + p.kc - 1) / p.kc;
+  // one workgroup per compute unit is resident: pick the split count whose workgroups fill whole
+  // rounds of the device best, charging each split for the partial sums it writes and reads back
+  const int64_t base = (int64_t)p.row_groups * p.xblocks;
+  int best = 1;
+  double best_score = -1.0;
+  const int max_split = nchunks / 4 > 1 ? (nchunks / 4 < 16 ? nchunks / 4 : 16) : 1;
+  for (int ns = 1; ns <= max_split; ++ns) {
+    const int cps = (nchunks + ns - 1) / ns;
+    if ((nchunks + cps - 1) / cps != ns) continue;  // this count cannot be realised with whole chunks
+    const int64_t wgs = base * ns;
+    const int64_t rounds = (wgs + cus - 1) / cus;
+    const double fill = (double)wgs / (double)(rounds * cus);
+    const double extra = ns > 1 ? 8.0 * ns * (16.0 * p.bt * p.xblocks) / (2.0 * N) : 0.0;  // partial bytes / weight bytes
+    const double score = fill / (1.0 + extra);
+    if (score > best_score + 1e-9) {
+      best_score = score;
+      best = ns;
+    }
+  }
+  p.nsplit = best;
+  p.chunks_per_split = (nchunks + best - 1) / best;
+  return p;
+}
+
+size_t tiled_workspace_bytes(int B, int N, int M) {
+  const TiledPlan p = plan_tiled(B, N, M);
+  return p.nsplit > 1 ? (size_t)p.nsplit * B * M * sizeof(float) : 0;
+}
+
+template <int BT, int WT, int KC>
+int launch_tiled(const TiledPlan& p, const half_t* X, int64_t ldx, const half_t* W, int64_t ldw, const half_t* bias,
+                 const void* idx, int idx_bytes, int B, int N, int Z, int M, half_t* Y, int64_t ldy, int relu,
+                 float* partial, hipStream_t s) {
+  auto kern = gemm_tiled_mfma_kernel<BT, WT, KC>;
+  constexpr size_t lds = tiled_lds_bytes<BT, WT, KC>();
+  static LdsGrant grant;
+  if (int rc = grant.ensure(reinterpret_cast<const void*>(kern), lds); rc != DV_OK) return rc;
+  const dim3 grid(p.xblocks, p.row_groups, p.nsplit);
+  hipLaunchKernelGGL(kern, grid, dim3(kTgWaves * 64), lds, s, X, ldx, W, ldw, bias, idx, idx_bytes, B, N, Z, M, Y,
+                     ldy, relu, p.nsplit > 1 ? p.chunks_per_split : 0, partial);
+  return DV_OK;
+}
+
+// Y (B, M) row stride ldy = act(X (B, N) . W[idx]^T + bias[idx]); idx == nullptr: rows 0..M-1 of W.
+int gemm_tiled(const half_t* X, int64_t ldx, const half_t* W, int64_t ldw, const half_t* bias, const void* idx,
+               int idx_bytes, int B, int N, int Z, int M, int act, half_t* Y, int64_t ldy, void* workspace,
+               size_t workspace_bytes, hipStream_t s) {
+  const TiledPlan p = plan_tiled(B, N, M);
+  float* partial = nullptr;
+  if (p.nsplit > 1) {
+    if (workspace == nullptr || !aligned16(workspace) || workspace_bytes < tiled_workspace_bytes(B, N, M))
+      return DV_ERR_WORKSPACE;
+    partial = reinterpret_cast<float*>(workspace);
+  }
+  const int relu = act == DV_ACT_RELU;
+  int rc;
+#define DV_TG(BT, WT, KC) \
+  rc = launch_tiled<BT, WT, KC>(p, X, ldx, W, ldw, bias, idx, idx_bytes, B, N, Z, M, Y, ldy, relu, partial, s)
+  if (p.bt == 1) { if (p.wt == 2) DV_TG(1, 2, 256); else DV_TG(1, 1, 256); }
+  else if (p.bt == 2) DV_TG(2, 1, 256);
+  else if (p.bt == 4) DV_TG(4, 1, 256);
+  else DV_TG(8, 2, 128);
+#undef DV_TG
+  if (rc != DV_OK) return rc;
+  if (p.nsplit > 1) {
+    const int64_t total = (int64_t)B * M;
+    hipLaunchKernelGGL(gemm_split_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, partial,
+                       p.nsplit, B, M, bias, idx, idx_bytes, Z, relu, Y, ldy);
+  }
+  return launch_status();
+}
+
 struct ColsMfmaPlan {
   int col_tiles, groups, rows_per_block;
 };
@@ -688,6 +779,49 @@ int dv_gather_gemv_f16(const void* x, const void* W, int64_t ldw, const void* bi
   }
 }
 
+// Batches from which the X-shared split-K kernel takes over from the 16-row-tile kernel (measured at
+// the OPT-175B fc1: see the kernel table of the batched benchmark).
+constexpr int kTiledMinBatch = 17;
+
+size_t dv_gather_gemv_workspace_bytes(int B, int N, int M) {
+  if (B < kTiledMinBatch || B > 64 || N <= 0 || M <= 0) return 0;
+  return tiled_workspace_bytes(B, N, M);
+}
+
+int dv_gather_gemv_ws_f16(const void* x, const void* W, int64_t ldw, const void* bias, const void* idx,
+                          int idx_bytes, int B, int N, int Z, int M, int act, void* y, void* workspace,
+                          size_t workspace_bytes, void* stream) {
+  if (B < kTiledMinBatch || B > 64 || M <= 0 || workspace == nullptr ||
+      workspace_bytes < dv_gather_gemv_workspace_bytes(B, N, M) || !aligned16(workspace))
+    return dv_gather_gemv_f16(x, W, ldw, bias, idx, idx_bytes, B, N, Z, M, act, y, stream);
+  if (!x || !W || N <= 0 || Z <= 0 || (idx && !idx_ok(idx_bytes)) || !y || (!idx && M > Z) ||
+      (act != DV_ACT_ID && act != DV_ACT_RELU))
+    return DV_ERR_INVALID_ARG;
+  if (N % 8 || ldw % 8 || ldw < N || !aligned16(x) || !aligned16(W)) return DV_ERR_ALIGNMENT;
+  return gemm_tiled(reinterpret_cast<const half_t*>(x), N, reinterpret_cast<const half_t*>(W), ldw,
+                    reinterpret_cast<const half_t*>(bias), idx, idx_bytes, B, N, Z, M, act,
+                    reinterpret_cast<half_t*>(y), M, workspace, workspace_bytes, reinterpret_cast<hipStream_t>(stream));
+}
+
+size_t dv_dense_linear_workspace_bytes(int rows, int N, int M) {
+  if (rows < 1 || N <= 0 || M <= 0) return 0;
+  return tiled_workspace_bytes(rows, N, M);
+}
+
+int dv_dense_linear_f16(const void* x, int64_t ldx, const void* W, int64_t ldw, const void* bias, int rows, int N,
+                        int M, int act, void* y, int64_t ldy, void* workspace, size_t workspace_bytes,
+                        void* stream) {
+  if (!x || !W || !y || rows < 0 || N <= 0 || M <= 0 || (act != DV_ACT_ID && act != DV_ACT_RELU))
+    return DV_ERR_INVALID_ARG;
+  if (N % 8 || ldx % 8 || ldw % 8 || ldx < N || ldw < N || ldy < M || !aligned16(x) || !aligned16(W))
+    return DV_ERR_ALIGNMENT;
+  if (rows == 0) return DV_OK;
+  return gemm_tiled(reinterpret_cast<const half_t*>(x), ldx, reinterpret_cast<const half_t*>(W), ldw,
+                    reinterpret_cast<const half_t*>(bias), nullptr, 4, rows, N, M, M, act,
+                    reinterpret_cast<half_t*>(y), ldy, workspace, workspace_bytes,
+                    reinterpret_cast<hipStream_t>(stream));
+}
+
 size_t dv_gather_transposed_gemv_workspace_bytes(int B, int N, int M) {
   if (B < 1 || N < 1 || M < 0) return 0;
   return B > kColsVecMaxBatch ? cols_mfma_workspace_bytes(B, N, M) : cols_workspace_bytes(B, N, M);
@@ -807,6 +941,27 @@ int dv_qkv_proj_batch_f16(const void* x, int64_t ldx, const void* W, const void*
   if (B <= 16) DV_QB(1);
   else DV_QB(2);
 #undef DV_QB
+  return launch_status();
+}
+
+int dv_prefill_attention_f16(const void* qkv, int B, int T, int H, int hd, float scale, void* ctx, void* k_cache,
+                             void* v_cache, int pos0, int S, void* stream) {
+  if (!qkv || !ctx || B < 1 || T < 0 || H <= 0 || ((k_cache == nullptr) != (v_cache == nullptr)) ||
+      (k_cache && (S <= 0 || pos0 < 0 || pos0 + T > S)))
+    return DV_ERR_INVALID_ARG;
+  if (hd != 64 && hd != 128) return DV_ERR_UNSUPPORTED;
+  if (!aligned16(qkv) || (k_cache && (!aligned16(k_cache) || !aligned16(v_cache)))) return DV_ERR_ALIGNMENT;
+  if (T == 0) return DV_OK;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const dim3 grid((T + kPfWaves * 16 - 1) / (kPfWaves * 16), H, B);
+  if (hd == 128)
+    hipLaunchKernelGGL(prefill_attn_kernel<128>, grid, dim3(kPfWaves * 64), 0, s, reinterpret_cast<const half_t*>(qkv),
+                       T, H, scale, reinterpret_cast<half_t*>(ctx), reinterpret_cast<half_t*>(k_cache),
+                       reinterpret_cast<half_t*>(v_cache), pos0, S);
+  else
+    hipLaunchKernelGGL(prefill_attn_kernel<64>, grid, dim3(kPfWaves * 64), 0, s, reinterpret_cast<const half_t*>(qkv),
+                       T, H, scale, reinterpret_cast<half_t*>(ctx), reinterpret_cast<half_t*>(k_cache),
+                       reinterpret_cast<half_t*>(v_cache), pos0, S);
   return launch_status();
 }
 

@@ -1,0 +1,219 @@
+// Y[b, m] = act( sum_n X[b, n] * W[row(m), n] + bias[row(m)] ) for a block of X rows that is
+// SHARED through LDS by the whole workgroup, on the matrix cores: batched fc1 (17..64 rows),
+// batched predictor products and the dense products of the prompt phase (128 rows per block).
+//
+// gather_rows_mfma_kernel gives every workgroup 16 weight rows and lets each wavefront fetch its
+// own X operands, so X travels from L2 once per 16-row tile: B/16 times the weight bytes.  Here a
+// workgroup of eight wavefronts owns 128 * WT weight rows (16 * WT per wavefront) and walks the
+// columns in chunks of KC; per chunk the 16 * BT x KC block of X is staged ONCE into LDS by all
+// 512 threads (double-buffered: one workgroup barrier per chunk) and every wavefront multiplies
+// its private weight tile, staged through LDS as in the other MFMA kernels, against it.  X then
+// travels once per 128 * WT rows.  One workgroup fills a compute unit's LDS, so every wavefront
+// keeps TWO chunks of weights in flight (register stages A / B).
+// Because that leaves few workgroups for short matrices, the columns are also split over gridDim.z (split-K): split s handles chunks [s * cps, (s + 1) * cps)
+// and writes raw fp32 sums to partial[(s * B + b) * M + m]; gemm_split_reduce_kernel adds the splits
+// in ascending order, then bias and activation.  With one split the result is written directly.
+//
+// Operands per v_mfma_f32_16x16x32_f16: A = 16 weight rows x 32 columns, B = 16 X rows x the same
+// 32 columns; value v of lane l is weight row 4 * (l / 16) + v, X row l % 16: a lane ends with four
+// consecutive m of one batch row (one 8-byte store).
+// Grid: x = blocks of 16 * BT X rows (fastest: workgroups that share a weight tile are dispatched
+// together), y = groups of 128 * WT weight rows, z = column splits.
+// idx == nullptr: no gather (row m of W).  N % 8 == 0, ldx % 8 == 0, ldw % 8 == 0.
+#pragma once
+#include "common.hpp"
+#include "gemm_mfma.hpp"
+
+namespace dv {
+
+constexpr int kTgWaves = 8;
+constexpr int kTgPad = 8;  // halfs of padding per LDS row (bank spread)
+
+template <int BT, int WT, int KC>
+constexpr size_t tiled_lds_bytes() {
+  return (size_t)(2 * 16 * BT + kTgWaves * 16 * WT) * (KC + kTgPad) * sizeof(half_t);
+}
+
+template <int BT, int WT, int KC>
+__global__ __launch_bounds__(kTgWaves * 64) void gemm_tiled_mfma_kernel(
+    const half_t* __restrict__ X, int64_t ldx, const half_t* __restrict__ W, int64_t ldw,
+    const half_t* __restrict__ bias, const void* __restrict__ idx, int idx_bytes, int B, int N, int Z, int M,
+    half_t* __restrict__ Y, int64_t ldy, int relu, int chunks_per_split, float* __restrict__ partial) {
+  const bool SPLIT = chunks_per_split > 0;  // uniform
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  constexpr int LD = KC + kTgPad;
+  constexpr int XROWS = 16 * BT, WROWS = 16 * WT;
+  constexpr int VPR = KC / 8;                      // 16-byte vectors per staged row
+  constexpr int XV = XROWS * VPR / (kTgWaves * 64);  // X vectors per thread and chunk
+  constexpr int WV = WROWS * VPR / 64;               // weight vectors per lane and chunk
+  static_assert(XROWS * VPR % (kTgWaves * 64) == 0 && WROWS * VPR % 64 == 0, "staging does not tile");
+  half_t* xs = reinterpret_cast<half_t*>(smem_raw);                       // [2][XROWS][LD]
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  half_t* ws = xs + (size_t)2 * XROWS * LD + (size_t)wave * WROWS * LD;  // [WROWS][LD], wavefront-private
+  const int l16 = lane & 15, kg = lane >> 4;
+
+  const int b0 = blockIdx.x * XROWS;
+  const int m0 = (blockIdx.y * kTgWaves + wave) * WROWS;  // first output row of this wavefront
+  const int nchunks = (N + KC - 1) / KC;
+  const int c_begin = SPLIT ? (int)blockIdx.z * chunks_per_split : 0;
+  const int c_end = SPLIT ? (c_begin + chunks_per_split < nchunks ? c_begin + chunks_per_split : nchunks) : nchunks;
+
+  // weight row of output row m0 + lane (lanes < WROWS), -1 when out of range
+  int rid_mine = -1;
+  if (lane < WROWS && m0 + lane < M) {
+    const int m = m0 + lane;
+    const int64_t id = idx == nullptr ? (int64_t)m : load_index(idx, idx_bytes, m);
+    rid_mine = (id >= 0 && id < Z) ? (int)id : -1;
+  }
+  // staging coordinates: weight vector q of a lane is row q * (64 / VPR) + lane / VPR, columns (lane % VPR) * 8
+  const int wv_row = lane / VPR, wv_col = (lane % VPR) * 8;
+  const half_t* wrow[WV];
+  unsigned wrow_ok = 0;
+#pragma unroll
+  for (int q = 0; q < WV; ++q) {
+    const int rid = __shfl(rid_mine, q * (64 / VPR) + wv_row, kWave);
+    wrow[q] = W + (int64_t)(rid >= 0 ? rid : 0) * ldw;
+    wrow_ok |= (unsigned)(rid >= 0) << q;
+  }
+  // X vector p of a thread is row (p * 512 + tid) / VPR of the block, columns (tid % VPR) * 8
+  const half_t* xrow[XV];
+#pragma unroll
+  for (int p = 0; p < XV; ++p) {
+    const int b = b0 + (p * kTgWaves * 64 + tid) / VPR;
+    xrow[p] = X + (int64_t)(b < B ? b : b0) * ldx;  // rows past B re-read the block's first row; never stored
+  }
+  const int xv_col = (tid % VPR) * 8;
+
+  float4_t acc[WT][BT];
+#pragma unroll
+  for (int wt = 0; wt < WT; ++wt)
+#pragma unroll
+    for (int bt = 0; bt < BT; ++bt) acc[wt][bt] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  // All loads are unconditional so that the compiler can count them (two chunks stay in flight): a
+  // chunk past the end of this split reads one fixed line instead (never stored).
+  auto load_stage = [&](half8_t (&wstage)[WV], half8_t (&xstage)[XV], int c) {
+    const bool live = c < c_end;
+    int wc = c * KC + wv_col, xc = c * KC + xv_col;
+    if (wc >= N) wc = 0;  // zeroed when stored
+    if (xc >= N) xc = 0;
+#pragma unroll
+    for (int p = 0; p < XV; ++p) xstage[p] = load8(live ? xrow[p] + xc : X);
+#pragma unroll
+    for (int q = 0; q < WV; ++q) wstage[q] = load8_stream(live ? wrow[q] + wc : W);
+  };
+  auto store_stage = [&](const half8_t (&wstage)[WV], const half8_t (&xstage)[XV], int c, int buf) {
+    const bool w_ok = c * KC + wv_col < N, x_ok = c * KC + xv_col < N;
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");  // this wavefront's reads of its weight tile are done
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int q = 0; q < WV; ++q)
+      store8(ws + (q * (64 / VPR) + wv_row) * LD + wv_col, (w_ok && ((wrow_ok >> q) & 1u)) ? wstage[q] : zero8());
+    half_t* xb = xs + (size_t)buf * XROWS * LD;
+#pragma unroll
+    for (int p = 0; p < XV; ++p)
+      store8(xb + ((p * kTgWaves * 64 + tid) / VPR) * LD + xv_col, x_ok ? xstage[p] : zero8());
+  };
+  auto multiply = [&](int buf) {
+    const half_t* xb = xs + (size_t)buf * XROWS * LD;
+#pragma unroll
+    for (int ks = 0; ks < KC / 32; ++ks) {
+      half8_t a[WT];
+#pragma unroll
+      for (int wt = 0; wt < WT; ++wt) a[wt] = load8(ws + (wt * 16 + l16) * LD + ks * 32 + kg * 8);
+#pragma unroll
+      for (int bt = 0; bt < BT; ++bt) {
+        const half8_t b = load8(xb + (bt * 16 + l16) * LD + ks * 32 + kg * 8);
+#pragma unroll
+        for (int wt = 0; wt < WT; ++wt) acc[wt][bt] = mfma_16x16x32(a[wt], b, acc[wt][bt]);
+      }
+    }
+  };
+  // One chunk: store its stage (weights: wavefront-private tile; X: buffer `buf`), one workgroup barrier
+  // (the X block is complete, and every wavefront has finished the multiplies of the chunk before, so the
+  // other X buffer may be overwritten next time), request the chunk two ahead, multiply.
+  auto step = [&](half8_t (&wstage)[WV], half8_t (&xstage)[XV], int c, int buf) {
+    store_stage(wstage, xstage, c, buf);
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+    load_stage(wstage, xstage, c + 2);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(buf);
+  };
+
+  half8_t wa[WV], xa[XV], wb[WV], xb2[XV];
+  if (c_begin < c_end) {
+    load_stage(wa, xa, c_begin);
+    load_stage(wb, xb2, c_begin + 1);
+    int c = c_begin;
+    for (; c + 1 < c_end; c += 2) {
+      step(wa, xa, c, 0);
+      step(wb, xb2, c + 1, 1);
+    }
+    if (c < c_end) step(wa, xa, c, 0);
+  }
+
+  // value v of a lane: output row m0 + wt * 16 + 4 * kg + v, batch row b0 + bt * 16 + l16
+#pragma unroll
+  for (int wt = 0; wt < WT; ++wt) {
+    const int mrow = m0 + wt * 16 + 4 * kg;
+    int rid[4];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) rid[v] = __shfl(rid_mine, wt * 16 + 4 * kg + v, kWave);
+#pragma unroll
+    for (int bt = 0; bt < BT; ++bt) {
+      const int b = b0 + bt * 16 + l16;
+      if (b >= B || mrow >= M) continue;
+      float val[4];
+#pragma unroll
+      for (int v = 0; v < 4; ++v) val[v] = rid[v] >= 0 ? acc[wt][bt][v] : 0.f;
+      if (SPLIT) {
+        float* dst = partial + ((int64_t)blockIdx.z * B + b) * M + mrow;
+        if (mrow + 3 < M && (M & 3) == 0) {
+          *reinterpret_cast<float4_t*>(dst) = float4_t{val[0], val[1], val[2], val[3]};
+        } else {
+#pragma unroll
+          for (int v = 0; v < 4; ++v)
+            if (mrow + v < M) dst[v] = val[v];
+        }
+        continue;
+      }
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        if (bias != nullptr && rid[v] >= 0) val[v] += (float)bias[rid[v]];
+        if (relu) val[v] = relu_f(val[v]);
+      }
+      half_t* dst = Y + (int64_t)b * ldy + mrow;
+      if (mrow + 3 < M && (ldy & 3) == 0 && (reinterpret_cast<uintptr_t>(Y) & 7) == 0) {
+        half4_t o = {(half_t)val[0], (half_t)val[1], (half_t)val[2], (half_t)val[3]};
+        *reinterpret_cast<half4_t*>(dst) = o;
+      } else {
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+          if (mrow + v < M) dst[v] = (half_t)val[v];
+      }
+    }
+  }
+}
+
+// Y[b, m] = act(sum_s partial[(s * B + b) * M + m] + bias[row(m)]), splits added in ascending order.
+__global__ __launch_bounds__(256) void gemm_split_reduce_kernel(
+    const float* __restrict__ partial, int nsplit, int B, int M, const half_t* __restrict__ bias,
+    const void* __restrict__ idx, int idx_bytes, int Z, int relu, half_t* __restrict__ Y, int64_t ldy) {
+  const int64_t total = (int64_t)B * M;
+  const int64_t o = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (o >= total) return;
+  const int b = (int)(o / M), m = (int)(o - (int64_t)b * M);
+  float s = 0.f;
+  for (int y = 0; y < nsplit; ++y) s += partial[(int64_t)y * total + o];
+  if (bias != nullptr) {
+    const int64_t id = idx == nullptr ? (int64_t)m : load_index(idx, idx_bytes, m);
+    if (id >= 0 && id < Z) s += (float)bias[id];
+  }
+  if (relu) s = relu_f(s);
+  Y[(int64_t)b * ldy + m] = (half_t)s;
+}
+
+}  // namespace dv

@@ -35,6 +35,10 @@ from ._lib import check, lib
 # module path: 322 tokens/s with the side stream, 357 without; eager 792 -> 765 ms).
 USE_SIDE_STREAM = False
 
+# Prompt phase on this package's own kernels (dense products: dv_dense_linear_f16; causal attention
+# + cache fill: dv_prefill_attention_f16).  False: PyTorch's library GEMM and attention.
+USE_HIP_PROMPT = True
+
 _side_streams: dict = {}
 
 
@@ -209,11 +213,26 @@ class ParallelFusedMLPDejavu(nn.Module):
 def decode_linear(linear: nn.Linear, x: torch.Tensor, activation: str = "id") -> torch.Tensor:
     """``linear(x)`` (+ ReLU).  The few rows of a decode step (x: (B, 1, d), fp16, on the GPU) are
     streamed by the row GEMV kernels; anything else (the prompt phase) goes to the library GEMM."""
-    if x.is_cuda and x.dtype == torch.float16 and x.dim() == 3 and x.shape[1] == 1 and x.shape[0] <= 64 \
-            and linear.weight.dtype == torch.float16 and x.shape[-1] % 8 == 0:
+    on_hip = x.is_cuda and x.dtype == torch.float16 and linear.weight.dtype == torch.float16 and x.shape[-1] % 8 == 0
+    if on_hip and x.dim() == 3 and x.shape[1] == 1 and x.shape[0] <= 16:
         return ops.dense_decode_linear(x, linear.weight, linear.bias, activation)
+    if on_hip and USE_HIP_PROMPT:
+        # many rows (the prompt, or a large decode batch): blocks of X shared through LDS on the matrix cores
+        return ops.dense_linear(x, linear.weight, linear.bias, activation)
     y = linear(x)
     return F.relu(y) if activation == "relu" else y
+
+
+def _kv_caches(inference_params, layer_idx, H, hd, dtype, device):
+    """The layer's (k_cache, v_cache), created on first use: packed keys (B, H, hd/8, S, 8) and values
+    (B, H, S, hd) (Dejavu/src/models/modules/mha_dejavu.py:404-446, fused_ft_kernel layout)."""
+    if layer_idx not in inference_params.key_value_memory_dict:
+        k_cache = torch.zeros(inference_params.max_batch_size, H, hd // 8, inference_params.max_sequence_len, 8,
+                              dtype=dtype, device=device)
+        v_cache = torch.zeros(inference_params.max_batch_size, H, inference_params.max_sequence_len, hd,
+                              dtype=dtype, device=device)
+        inference_params.key_value_memory_dict[layer_idx] = (k_cache, v_cache)
+    return inference_params.key_value_memory_dict[layer_idx]
 
 
 def _update_kv_cache(kv, inference_params, layer_idx):
@@ -271,11 +290,22 @@ class _MHABase(nn.Module):
         B, s = qkv.shape[0], qkv.shape[1]
         scale = self.softmax_scale
         if inference_params is None or inference_params.sequence_len_offset == 0:
+            causal = self.causal if inference_params is None else True
+            if USE_HIP_PROMPT and qkv.is_cuda and qkv.dtype == torch.float16 and qkv.shape[-1] in (64, 128) \
+                    and (causal or s == 1):
+                # causal attention and the cache fill in one launch (no permuted copy of K / V)
+                kc = vc = None
+                if inference_params is not None:
+                    assert self.layer_idx is not None, "Generation requires layer_idx in the constructor"
+                    k_cache, v_cache = _kv_caches(inference_params, self.layer_idx, self.num_heads, self.head_dim,
+                                                  qkv.dtype, qkv.device)
+                    b0 = inference_params.batch_size_offset
+                    kc, vc = k_cache[b0:b0 + B], v_cache[b0:b0 + B]
+                return ops.prefill_attention(qkv.contiguous(), kc, vc, 0, scale)
             if inference_params is not None:
                 assert self.layer_idx is not None, "Generation requires layer_idx in the constructor"
                 _update_kv_cache(qkv[:, :, 1:], inference_params, self.layer_idx)
             q, k, v = (t.transpose(1, 2) for t in qkv.unbind(dim=2))  # (B, H, s, hd)
-            causal = self.causal if inference_params is None else True
             ctx = F.scaled_dot_product_attention(q, k, v, is_causal=causal and s > 1, scale=scale)
             return ctx.transpose(1, 2).reshape(B, s, -1)
         assert s == 1, "decode processes one token at a time"

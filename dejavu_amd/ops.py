@@ -202,10 +202,45 @@ def gather_gemv(x: torch.Tensor, weight: torch.Tensor, idx: Optional[torch.Tenso
         assert x.dtype == bias.dtype, f"Input and bias must have the same dtype, got {x.dtype} and {bias.dtype}"
     idx = None if idx is None else idx.contiguous()
     output = torch.empty(batch, M, device=x.device, dtype=x.dtype)
-    check(lib.dv_gather_gemv_f16(_ptr(x), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(idx),
-                                 8 if idx is None else _idx_bytes(idx),
-                                 batch, N, Z, M, _ACT[activation], _ptr(output), _stream()), "dv_gather_gemv_f16")
+    nbytes = lib.dv_gather_gemv_workspace_bytes(batch, N, M)  # 0 below 17 rows
+    ws = _workspace(x.device, nbytes) if nbytes else None
+    check(lib.dv_gather_gemv_ws_f16(_ptr(x), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(idx),
+                                    8 if idx is None else _idx_bytes(idx), batch, N, Z, M, _ACT[activation],
+                                    _ptr(output), _ptr(ws), 0 if ws is None else ws.numel(), _stream()),
+          "dv_gather_gemv_ws_f16")
     return output
+
+
+def dense_linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                 activation: str = "id", out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``activation(F.linear(x, weight, bias))`` for any number of rows on the matrix cores: the dense
+    products of the prompt phase.  x: (..., N) fp16 with a contiguous last dimension (rows may be
+    strided after flattening); weight: (M, N); returns (..., M)."""
+    if activation not in _ACT:
+        raise NotImplementedError(f"activation {activation!r}: 'relu' / 'id' only")
+    _require_device(x, weight, bias, out)
+    M, N = weight.shape
+    assert x.shape[-1] == N and x.dtype == weight.dtype == torch.float16
+    lead = x.shape[:-1]
+    x2 = x.reshape(-1, N)
+    if x2.stride(1) != 1 or x2.stride(0) % 8 or x2.data_ptr() % 16:
+        x2 = x2.contiguous()
+    if weight.stride(1) != 1:
+        weight = weight.contiguous()
+    rows = x2.shape[0]
+    if bias is not None:
+        bias = bias.contiguous()
+        assert bias.shape == (M,) and bias.dtype == x.dtype
+    if out is None:
+        out = torch.empty(rows, M, device=x.device, dtype=x.dtype)
+    else:
+        assert out.shape == (rows, M) and out.stride(1) == 1 and out.dtype == x.dtype
+    nbytes = lib.dv_dense_linear_workspace_bytes(rows, N, M)
+    ws = _workspace(x.device, nbytes) if nbytes else None
+    check(lib.dv_dense_linear_f16(_ptr(x2), x2.stride(0) if rows > 1 else N, _ptr(weight), weight.stride(0),
+                                  _ptr(bias), rows, N, M, _ACT[activation], _ptr(out), out.stride(0) if rows > 1 else M,
+                                  _ptr(ws), 0 if ws is None else ws.numel(), _stream()), "dv_dense_linear_f16")
+    return out.view(*lead, M) if out.is_contiguous() else out
 
 
 def dense_decode_linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
@@ -561,6 +596,33 @@ def single_query_attention(q: torch.Tensor, k: Optional[torch.Tensor], v: Option
                                       _ptr(lengths_per_sample), n_len, B, H, hd, S, scale, _ptr(out), out.stride(0),
                                       _ptr(ws), ws.numel(), _stream()), "dv_decode_attention_f16")
     return out
+
+
+def prefill_attention(qkv: torch.Tensor, k_cache: Optional[torch.Tensor] = None,
+                      v_cache: Optional[torch.Tensor] = None, pos0: int = 0,
+                      softmax_scale: Optional[float] = None) -> torch.Tensor:
+    """Causal attention over the prompt; with caches, the prompt's K / V rows are also written to
+    positions ``pos0 .. pos0 + T - 1`` of the (packed) decode caches by the same launch.
+
+    qkv: (B, T, 3, H, hd) fp16 contiguous -> context (B, T, H * hd).
+    k_cache (B, H, hd / 8, S, 8), v_cache (B, H, S, hd).
+    """
+    _require_device(qkv, k_cache, v_cache)
+    B, T, three, H, hd = qkv.shape
+    assert three == 3 and hd in [64, 128], "the prompt attention kernel is built for head_dim 64 and 128"
+    assert qkv.dtype == torch.float16 and qkv.is_contiguous()
+    S = 0
+    if k_cache is not None:
+        assert v_cache is not None
+        S = v_cache.shape[2]
+        assert v_cache.shape == (B, H, S, hd) and k_cache.shape == (B, H, hd // 8, S, 8)
+        assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dtype == v_cache.dtype == qkv.dtype
+        assert 0 <= pos0 and pos0 + T <= S
+    ctx = torch.empty(B, T, H * hd, device=qkv.device, dtype=qkv.dtype)
+    scale = float(hd ** -0.5 if softmax_scale is None else softmax_scale)
+    check(lib.dv_prefill_attention_f16(_ptr(qkv), B, T, H, hd, scale, _ptr(ctx), _ptr(k_cache), _ptr(v_cache),
+                                       int(pos0), S, _stream()), "dv_prefill_attention_f16")
+    return ctx
 
 
 _attn_workspaces: dict = {}

@@ -114,6 +114,34 @@ DV_API int dv_gather_gemv_f16(const void* x, const void* W, int64_t ldw, const v
                        void* y, void* stream);
 
 /*
+ * dv_gather_gemv_f16 with a workspace: from 17 batch rows on, the whole workgroup shares each block
+ * of X through LDS (X leaves L2 once per 128 gathered rows instead of once per 16) and the columns
+ * are also split over workgroups, each split writing fp32 partial sums that a second launch adds in
+ * ascending order (deterministic) before bias and activation.
+ *   workspace: dv_gather_gemv_workspace_bytes(B, N, M) bytes, 16-byte aligned, no initialisation
+ *   needed; with NULL / too small a workspace, or fewer than 17 rows, the call is dv_gather_gemv_f16.
+ */
+DV_API size_t dv_gather_gemv_workspace_bytes(int B, int N, int M);
+DV_API int dv_gather_gemv_ws_f16(const void* x, const void* W, int64_t ldw, const void* bias,
+                                 const void* idx, int idx_bytes, int B, int N, int Z, int M, int act,
+                                 void* y, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * y = act(x . W^T + bias) for any number of rows, on the matrix cores: the dense products of the
+ * prompt phase (Wqkv, out_proj, fc1 + activation, fc2), which the reference runs through
+ * nn.Linear / fused_dense_lib (Dejavu/src/ops/fused_dense_sparse_dejavu.py:924-936 fused_mlp_func,
+ * Dejavu/src/models/modules/mha_dejavu.py:1494-1496 Wqkv / out_proj of the dense branch).
+ * Blocks of up to 128 rows of x are shared through LDS by a workgroup that streams 256 weight rows;
+ * short matrices are also split over the columns (fp32 partial sums, added in ascending order).
+ *   x (rows, N) row stride ldx; W (M, N) row stride ldw; bias (M,) or NULL; y (rows, M) row stride
+ *   ldy; workspace: dv_dense_linear_workspace_bytes(rows, N, M) bytes (may be 0), 16-byte aligned.
+ */
+DV_API size_t dv_dense_linear_workspace_bytes(int rows, int N, int M);
+DV_API int dv_dense_linear_f16(const void* x, int64_t ldx, const void* W, int64_t ldw, const void* bias,
+                               int rows, int N, int M, int act, void* y, int64_t ldy, void* workspace,
+                               size_t workspace_bytes, void* stream);
+
+/*
  * y = x . W[idx] + bias.  Replaces gather_transposed_gemv,
  * Dejavu/src/ops/triton/gather_gemv.py:572-644 (deterministic: fixed-order
  * split over row groups instead of floating-point atomics).
@@ -192,6 +220,20 @@ DV_API int dv_qkv_proj_batch_f16(const void* x, int64_t ldx, const void* W, cons
                                  const void* head_idx, const void* live, int live_stride, int nnz, int B,
                                  int d, int H, int hd, void* y, void* k_cache, void* v_cache,
                                  const void* positions, int per_sample, int pos_add, int S, void* stream);
+
+/*
+ * Causal attention over the prompt, and the prompt's K / V rows written into the decode caches:
+ *   ctx[b, t, h, :] = softmax_{s <= t}(q[b, t, h] . k[b, s, h] * scale) . v[b, s, h]
+ *   k_cache[b, h, j / 8, pos0 + t, j % 8] = k[b, t, h, j];  v_cache[b, h, pos0 + t, j] = v[b, t, h, j]
+ * fp32 scores and online softmax, fp16 probabilities into the second product.  Replaces the prompt
+ * branch of the attention modules: _update_kv_cache (Dejavu/src/models/modules/mha_dejavu.py:385-447,
+ * the permuted cache fill) followed by causal flash attention (mha_dejavu.py:1393-1410).
+ *   qkv (B, T, 3, H, hd) contiguous, the output of the Wqkv product; ctx (B, T, H * hd);
+ *   k_cache (B, H, hd/8, S, 8), v_cache (B, H, S, hd): both or neither NULL, pos0 + T <= S;
+ *   hd in {64, 128}.
+ */
+DV_API int dv_prefill_attention_f16(const void* qkv, int B, int T, int H, int hd, float scale, void* ctx,
+                                    void* k_cache, void* v_cache, int pos0, int S, void* stream);
 
 /*
  * Scatter of (re)computed keys / values into the caches:

@@ -43,6 +43,8 @@ How each function is pinned (see tests/test_oracle.py):
   single-sequence functions run on sequence b alone with the shared selections
   (bit-equal), against per-sequence float64 attention + head-masked out_proj,
   and B = 1 against ``block_decode_step`` (bit-equal).
+* ``prompt_attention``: against torch's causal scaled_dot_product_attention in float64
+  and, for the cache fill, against ``unpack_k_cache`` round trips.
 * ``WindowTracker``: against a literal index-by-index replay of the reference's
   ParallelTracker calls over several windows.
 * top-k tie order: the reference (``torch.topk(sorted=False)`` on CUDA) leaves
@@ -663,6 +665,34 @@ def new_decode_state(params, max_len):
     return {"caches": caches, "pos": 0, "window": 0}
 
 
+def prompt_attention(qkv, k_cache=None, v_cache=None, pos0=0, softmax_scale=None):
+    """Causal attention over the T prompt tokens of one sequence, and the prompt's K / V rows
+    written to positions pos0 .. pos0 + T - 1 of the caches.
+
+    Prompt branch of the attention modules, Dejavu/src/models/modules/mha_dejavu.py:385-447
+    (_update_kv_cache: keys packed as (H, hd/8, S, 8), values as (H, S, hd)) and :1393-1410
+    (causal attention, causal=True at gpt_dejavu.py:236); arithmetic as CrossAttention /
+    SelfAttention.forward, mha_dejavu.py:264-375: fp32 scores, softmax, fp16 result.
+    qkv: (T, 3, H, hd) fp16; k_cache (H, hd/8, S, 8), v_cache (H, S, hd) or None.  Returns ctx (T, H, hd) fp16.
+    """
+    qkv = np.asarray(qkv, F16)
+    T, _, H, hd = qkv.shape
+    if k_cache is not None:
+        k_cache[:, :, pos0:pos0 + T, :] = pack_k_cache(qkv[None, :, 1])[0]
+        v_cache[:, pos0:pos0 + T, :] = qkv[:, 2].transpose(1, 0, 2)
+    scale = F32(hd ** -0.5 if softmax_scale is None else softmax_scale)
+    ctx = np.zeros((T, H, hd), F16)
+    mask = np.triu(np.ones((T, T), bool), 1)
+    for h in range(H):
+        q, k, v = (qkv[:, j, h].astype(F32) for j in range(3))
+        sc = (q @ k.T) * scale
+        sc[mask] = -np.inf
+        pr = np.exp(sc - sc.max(axis=-1, keepdims=True))
+        pr = pr / pr.sum(axis=-1, keepdims=True, dtype=F32)
+        ctx[:, h] = (pr @ v).astype(F16)
+    return ctx
+
+
 def model_prompt(params, state, input_ids):
     """Dense forward over the prompt, filling the caches; returns the fp16 logits
     of the last prompt token.
@@ -683,18 +713,7 @@ def model_prompt(params, state, input_ids):
         residual = hidden if residual is None else _add_f16(hidden, residual)
         x = layer_norm(residual, p["ln1_w"], p["ln1_b"])
         qkv = _linear_f16(x, p["Wqkv"].reshape(3 * H * hd, d), p["bqkv"].reshape(-1)).reshape(T, 3, H, hd)
-        k_cache[0, :, :, :T, :] = pack_k_cache(qkv[None, :, 1])[0]
-        v_cache[0, :, :T, :] = qkv[:, 2].transpose(1, 0, 2)
-        scale = F32(hd ** -0.5)
-        ctx = np.zeros((T, H, hd), F16)
-        mask = np.triu(np.ones((T, T), bool), 1)
-        for h in range(H):
-            q, k, v = (qkv[:, j, h].astype(F32) for j in range(3))
-            sc = (q @ k.T) * scale
-            sc[mask] = -np.inf
-            pr = np.exp(sc - sc.max(axis=-1, keepdims=True))
-            pr = pr / pr.sum(axis=-1, keepdims=True, dtype=F32)
-            ctx[:, h] = (pr @ v).astype(F16)
+        ctx = prompt_attention(qkv, k_cache[0], v_cache[0])
         attn_out = _linear_f16(ctx.reshape(T, H * hd), p["Wout"].reshape(d, H * hd), p["bout"])
         residual = _add_f16(attn_out, residual)
         x2 = layer_norm(residual, p["ln2_w"], p["ln2_b"])

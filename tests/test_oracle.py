@@ -609,3 +609,33 @@ def test_block_decode_step_batched_shares_selections_and_keeps_rows_independent(
             assert np.array_equal(one[key][0].view(np.uint16), bat[key][b].view(np.uint16)), (key, b)
         assert np.array_equal(one["next_mlp_logit"].view(np.uint16), bat["next_mlp_logit"][b].view(np.uint16))
         assert np.array_equal(k_cache[b], kb[0]) and np.array_equal(v_cache[b], vb[0])
+
+
+# ----------------------------------------------------------------- prompt phase
+def test_prompt_attention_matches_causal_sdpa_and_fills_caches():
+    g = rng(28)
+    T, H, hd, S, pos0 = 37, 3, 16, 48, 5
+    qkv = randn16(g, T, 3, H, hd)
+    k_cache = np.zeros((H, hd // 8, S, 8), F16)
+    v_cache = np.zeros((H, S, hd), F16)
+    ctx = O.prompt_attention(qkv, k_cache, v_cache, pos0=pos0)
+    q, k, v = (torch.from_numpy(qkv[:, j].astype(np.float64)).permute(1, 0, 2).unsqueeze(0) for j in range(3))
+    ref = torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True)[0].permute(1, 0, 2).numpy()
+    assert np.abs(ctx.astype(np.float64) - ref).max() <= 2e-3
+    # the first token attends to itself only
+    assert np.array_equal(ctx[0], qkv[0, 2])
+    # caches: rows pos0 .. pos0 + T - 1 hold K / V, nothing else is written
+    ku = O.unpack_k_cache(k_cache[None])[0]  # (H, S, hd)
+    assert np.array_equal(ku[:, pos0:pos0 + T], qkv[:, 1].transpose(1, 0, 2))
+    assert np.array_equal(v_cache[:, pos0:pos0 + T], qkv[:, 2].transpose(1, 0, 2))
+    assert np.all(ku[:, :pos0] == 0) and np.all(ku[:, pos0 + T:] == 0) and np.all(v_cache[:, pos0 + T:] == 0)
+    # a decode step over the filled cache continues the prompt: the newest query sees every cached key
+    q_new, k_new, v_new = (randn16(g, 1, H, hd) for _ in range(3))
+    out = O.single_query_attention(q_new, k_new, v_new, k_cache[None].copy(), v_cache[None].copy(), pos0 + T)
+    K = np.concatenate([qkv[:, 1], k_new], 0).astype(np.float64)[None].transpose(0, 2, 1, 3)
+    V = np.concatenate([qkv[:, 2], v_new], 0).astype(np.float64)[None].transpose(0, 2, 1, 3)
+    K = np.concatenate([np.zeros((1, H, pos0, hd)), K], 2)  # positions before pos0 hold zeros in this test
+    V = np.concatenate([np.zeros((1, H, pos0, hd)), V], 2)
+    ref2 = torch.nn.functional.scaled_dot_product_attention(
+        torch.from_numpy(q_new.astype(np.float64)).unsqueeze(2), torch.from_numpy(K), torch.from_numpy(V)).squeeze(2).numpy()
+    assert np.abs(out.astype(np.float64) - ref2).max() <= 2e-3
