@@ -366,7 +366,7 @@ int rows_short_mfma(const half_t* x, const half_t* W, int64_t ldw, int B, int N,
 
 // ---- X-shared split-K products (gemm_tiled.hpp) ---------------------------------
 struct TiledPlan {
-  int bt, wt, kc, xblocks, row_groups, nsplit, chunks_per_split;
+  int bt, wt, kc, waves, xblocks, row_groups, nsplit, chunks_per_split;
 };
 
 TiledPlan plan_tiled(int B, int N, int M) {
@@ -375,33 +375,47 @@ TiledPlan plan_tiled(int B, int N, int M) {
   p.kc = p.bt == 8 ? 128 : 256;
   p.xblocks = (B + 16 * p.bt - 1) / (16 * p.bt);
   const int cus = compute_units();
-  // 32 rows per wavefront halve the LDS reads of X per weight byte; worth it when the matrix still
-  // gives every compute unit a workgroup
-  // (LDS holds 32-row wavefront tiles next to one or eight batch tiles of X, not next to two or four)
-  p.wt = (p.bt == 8 || (p.bt == 1 && (int64_t)M * p.xblocks >= (int64_t)256 * cus)) ? 2 : 1;
-  p.row_groups = (M + kTgWaves * 16 * p.wt - 1) / (kTgWaves * 16 * p.wt);
   const int nchunks = (N + p.kc - 1) / p.kc;
-  // one workgroup per compute unit is resident: pick the split count whose workgroups fill whole
-  // rounds of the device best, charging each split for the partial sums it writes and reads back
-  const int64_t base = (int64_t)p.row_groups * p.xblocks;
-  int best = 1;
+  // 32 rows per wavefront halve the LDS reads of X per weight byte (LDS holds such tiles next to one or
+  // eight batch tiles of X, not next to two or four); worth it when the matrix still fills the device
+  p.wt = (p.bt == 8 || (p.bt == 1 && (int64_t)M * p.xblocks >= (int64_t)256 * cus)) ? 2 : 1;
+  // Workgroup size (8 wavefronts = 128 * wt rows, or 4) and column splits.  Measured at the OPT-175B
+  // shapes (QKV of 32 heads: 12288 rows; fc1: 4096 rows; batch 16 / 32): what counts is one round of
+  // workgroups over the device with loops as long as possible -- 192 workgroups of 24 chunks beat 768
+  // of 6 (61 against 70 us), and workgroups of 4 wavefronts are only worth it when several are
+  // resident per compute unit or when they double the chunks per workgroup (fc1: 24.2 against 25.9 us).
   double best_score = -1.0;
+  p.waves = 8;
+  p.nsplit = 1;
   const int max_split = nchunks / 4 > 1 ? (nchunks / 4 < 16 ? nchunks / 4 : 16) : 1;
-  for (int ns = 1; ns <= max_split; ++ns) {
-    const int cps = (nchunks + ns - 1) / ns;
-    if ((nchunks + cps - 1) / cps != ns) continue;  // this count cannot be realised with whole chunks
-    const int64_t wgs = base * ns;
-    const int64_t rounds = (wgs + cus - 1) / cus;
-    const double fill = (double)wgs / (double)(rounds * cus);
-    const double extra = ns > 1 ? 8.0 * ns * (16.0 * p.bt * p.xblocks) / (2.0 * N) : 0.0;  // partial bytes / weight bytes
-    const double score = fill / (1.0 + extra);
-    if (score > best_score + 1e-9) {
-      best_score = score;
-      best = ns;
+  for (int waves = 8; waves >= (p.bt == 8 ? 8 : 4); waves -= 4) {
+    const size_t lds = (size_t)(2 * 16 * p.bt + waves * 16 * p.wt) * (p.kc + kTgPad) * sizeof(half_t);
+    const int resident = (int)((size_t)160 * 1024 / lds) > 0 ? (int)((size_t)160 * 1024 / lds) : 1;
+    const int64_t groups = (M + waves * 16 * p.wt - 1) / (waves * 16 * p.wt);
+    for (int ns = 1; ns <= max_split; ++ns) {
+      const int cps = (nchunks + ns - 1) / ns;
+      if ((nchunks + cps - 1) / cps != ns) continue;  // not realisable with whole chunks
+      const int64_t wgs = groups * p.xblocks * ns;
+      double fill;
+      if (wgs <= cus) {
+        fill = (double)wgs / cus;
+      } else {
+        const int64_t slots = (int64_t)cus * resident;
+        fill = (double)wgs / (double)((wgs + slots - 1) / slots * slots);
+      }
+      const double loop = (double)cps / (cps + 4.0);  // start-up and drain of a workgroup, in chunks
+      const double few_waves = (waves == 4 && wgs <= cus) ? 0.85 : 1.0;  // half the bytes in flight per unit
+      const double extra = ns > 1 ? 4.0 * ns * (16.0 * p.bt * p.xblocks) / N : 0.0;  // partial bytes / weight bytes
+      const double score = fill * loop * few_waves / (1.0 + extra);
+      if (score > best_score + 1e-9) {
+        best_score = score;
+        p.waves = waves;
+        p.nsplit = ns;
+      }
     }
   }
-  p.nsplit = best;
-  p.chunks_per_split = (nchunks + best - 1) / best;
+  p.row_groups = (M + p.waves * 16 * p.wt - 1) / (p.waves * 16 * p.wt);
+  p.chunks_per_split = (nchunks + p.nsplit - 1) / p.nsplit;
   return p;
 }
 
@@ -410,18 +424,58 @@ size_t tiled_workspace_bytes(int B, int N, int M) {
   return p.nsplit > 1 ? (size_t)p.nsplit * B * M * sizeof(float) : 0;
 }
 
-template <int BT, int WT, int KC>
+template <int BT, int WT, int KC, int WAVES>
 int launch_tiled(const TiledPlan& p, const half_t* X, int64_t ldx, const half_t* W, int64_t ldw, const half_t* bias,
                  const void* idx, int idx_bytes, int B, int N, int Z, int M, half_t* Y, int64_t ldy, int relu,
                  float* partial, hipStream_t s) {
-  auto kern = gemm_tiled_mfma_kernel<BT, WT, KC>;
-  constexpr size_t lds = tiled_lds_bytes<BT, WT, KC>();
+  auto kern = gemm_tiled_mfma_kernel<BT, WT, KC, false, WAVES>;
+  constexpr size_t lds = tiled_lds_bytes<BT, WT, KC, WAVES>();
   static LdsGrant grant;
   if (int rc = grant.ensure(reinterpret_cast<const void*>(kern), lds); rc != DV_OK) return rc;
   const dim3 grid(p.xblocks, p.row_groups, p.nsplit);
-  hipLaunchKernelGGL(kern, grid, dim3(kTgWaves * 64), lds, s, X, ldx, W, ldw, bias, idx, idx_bytes, B, N, Z, M, Y,
-                     ldy, relu, p.nsplit > 1 ? p.chunks_per_split : 0, partial);
+  hipLaunchKernelGGL(kern, grid, dim3(WAVES * 64), lds, s, X, ldx, W, ldw, bias, idx, idx_bytes, B, N, Z, M, Y,
+                     ldy, relu, p.nsplit > 1 ? p.chunks_per_split : 0, partial, QkvScatter{});
   return DV_OK;
+}
+
+// QKV of the selected heads for B rows (see QkvScatter): M = 3 * Hk * hd output rows
+int gemm_tiled_qkv(const half_t* X, int64_t ldx, const half_t* W, const half_t* bias, int B, int d, half_t* Y,
+                   const QkvScatter& qs, void* workspace, size_t workspace_bytes, hipStream_t s) {
+  const int M = 3 * qs.Hk * qs.hd, Z = 3 * qs.H * qs.hd;
+  const TiledPlan p = plan_tiled(B, d, M);
+  float* partial = nullptr;
+  if (p.nsplit > 1) {
+    if (workspace == nullptr || !aligned16(workspace) || workspace_bytes < tiled_workspace_bytes(B, d, M))
+      return DV_ERR_WORKSPACE;
+    partial = reinterpret_cast<float*>(workspace);
+  }
+  const dim3 grid(p.xblocks, p.row_groups, p.nsplit);
+  const int cps = p.nsplit > 1 ? p.chunks_per_split : 0;
+#define DV_TQW(BT, WT, WAVES)                                                                                  \
+  do {                                                                                                         \
+    auto kern = gemm_tiled_mfma_kernel<BT, WT, 256, true, WAVES>;                                              \
+    constexpr size_t lds = tiled_lds_bytes<BT, WT, 256, WAVES>();                                              \
+    static LdsGrant grant;                                                                                     \
+    if (int rc = grant.ensure(reinterpret_cast<const void*>(kern), lds); rc != DV_OK) return rc;               \
+    hipLaunchKernelGGL(kern, grid, dim3(WAVES * 64), lds, s, X, ldx, W, (int64_t)d, bias,                      \
+                       (const void*)nullptr, 4, B, d, Z, M, Y, (int64_t)Z, 0, cps, partial, qs);              \
+  } while (0)
+#define DV_TQ(BT, WT)                  \
+  do {                                 \
+    if (p.waves == 4) DV_TQW(BT, WT, 4); \
+    else DV_TQW(BT, WT, 8);            \
+  } while (0)
+  if (p.bt == 1) { if (p.wt == 2) DV_TQ(1, 2); else DV_TQ(1, 1); }
+  else if (p.bt == 2) DV_TQ(2, 1);
+  else return DV_ERR_UNSUPPORTED;
+#undef DV_TQW
+#undef DV_TQ
+  if (p.nsplit > 1) {
+    const int64_t total = (int64_t)B * M;
+    hipLaunchKernelGGL(qkv_split_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, partial,
+                       p.nsplit, B, M, bias, Y, qs);
+  }
+  return launch_status();
 }
 
 // Y (B, M) row stride ldy = act(X (B, N) . W[idx]^T + bias[idx]); idx == nullptr: rows 0..M-1 of W.
@@ -437,12 +491,17 @@ int gemm_tiled(const half_t* X, int64_t ldx, const half_t* W, int64_t ldw, const
   }
   const int relu = act == DV_ACT_RELU;
   int rc;
-#define DV_TG(BT, WT, KC) \
-  rc = launch_tiled<BT, WT, KC>(p, X, ldx, W, ldw, bias, idx, idx_bytes, B, N, Z, M, Y, ldy, relu, partial, s)
+#define DV_TG(BT, WT, KC)                                                                                          \
+  do {                                                                                                             \
+    if (p.waves == 4)                                                                                              \
+      rc = launch_tiled<BT, WT, KC, 4>(p, X, ldx, W, ldw, bias, idx, idx_bytes, B, N, Z, M, Y, ldy, relu, partial, s); \
+    else                                                                                                           \
+      rc = launch_tiled<BT, WT, KC, 8>(p, X, ldx, W, ldw, bias, idx, idx_bytes, B, N, Z, M, Y, ldy, relu, partial, s); \
+  } while (0)
   if (p.bt == 1) { if (p.wt == 2) DV_TG(1, 2, 256); else DV_TG(1, 1, 256); }
   else if (p.bt == 2) DV_TG(2, 1, 256);
   else if (p.bt == 4) DV_TG(4, 1, 256);
-  else DV_TG(8, 2, 128);
+  else rc = launch_tiled<8, 2, 128, 8>(p, X, ldx, W, ldw, bias, idx, idx_bytes, B, N, Z, M, Y, ldy, relu, partial, s);
 #undef DV_TG
   if (rc != DV_OK) return rc;
   if (p.nsplit > 1) {
@@ -918,10 +977,18 @@ int dv_qkv_proj_sparse_f16(const void* x, const void* W, const void* bias, const
                                       nullptr, nullptr, 0, stream);
 }
 
+// Batches from which the X-shared split-K kernel takes over from the one that fetches X per 16-row tile
+constexpr int kQkvTiledMinBatch = 9;
+
+size_t dv_qkv_proj_batch_workspace_bytes(int B, int d, int nnz, int hd) {
+  if (B < kQkvTiledMinBatch || B > 32 || d <= 0 || nnz <= 0 || hd <= 0) return 0;
+  return tiled_workspace_bytes(B, d, 3 * nnz * hd);
+}
+
 int dv_qkv_proj_batch_f16(const void* x, int64_t ldx, const void* W, const void* bias, const void* head_idx,
                           const void* live, int live_stride, int nnz, int B, int d, int H, int hd, void* y,
                           void* k_cache, void* v_cache, const void* positions, int per_sample, int pos_add,
-                          int S, void* stream) {
+                          int S, void* workspace, size_t workspace_bytes, void* stream) {
   if (!x || !W || !y || B < 1 || d <= 0 || H <= 0 || nnz < 0 || (nnz > 0 && !head_idx) ||
       ((k_cache == nullptr) != (v_cache == nullptr)) || (k_cache && S <= 0) || (live && live_stride < 1))
     return DV_ERR_INVALID_ARG;
@@ -929,6 +996,16 @@ int dv_qkv_proj_batch_f16(const void* x, int64_t ldx, const void* W, const void*
   if (d % 8 || ldx % 8 || ldx < d || !aligned16(x) || !aligned16(W)) return DV_ERR_ALIGNMENT;
   if (nnz == 0) return DV_OK;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (B >= kQkvTiledMinBatch && (dv_qkv_proj_batch_workspace_bytes(B, d, nnz, hd) == 0 ||
+                                 (workspace != nullptr && aligned16(workspace) &&
+                                  workspace_bytes >= dv_qkv_proj_batch_workspace_bytes(B, d, nnz, hd)))) {
+    const QkvScatter qs{reinterpret_cast<const int*>(head_idx), reinterpret_cast<const int*>(live), live_stride, nnz, H,
+                        hd, reinterpret_cast<half_t*>(k_cache), reinterpret_cast<half_t*>(v_cache),
+                        reinterpret_cast<const int*>(positions), per_sample, pos_add, S};
+    return gemm_tiled_qkv(reinterpret_cast<const half_t*>(x), ldx, reinterpret_cast<const half_t*>(W),
+                          reinterpret_cast<const half_t*>(bias), B, d, reinterpret_cast<half_t*>(y), qs, workspace,
+                          workspace_bytes, s);
+  }
   const dim3 grid(nnz * 3 * (hd / 16));
 #define DV_QB(XT)                                                                                          \
   hipLaunchKernelGGL((qkv_batch_mfma_kernel<kQkvMfmaWaves, XT>), grid, dim3(kQkvMfmaWaves * 64), 0, s,      \

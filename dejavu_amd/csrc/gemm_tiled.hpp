@@ -26,27 +26,69 @@
 
 namespace dv {
 
-constexpr int kTgWaves = 8;
+constexpr int kTgWaves = 8;  // default; 4-wavefront workgroups (64 * WT rows) when more of them must be resident
 constexpr int kTgPad = 8;  // halfs of padding per LDS row (bank spread)
 
-template <int BT, int WT, int KC>
+template <int BT, int WT, int KC, int WAVES = kTgWaves>
 constexpr size_t tiled_lds_bytes() {
-  return (size_t)(2 * 16 * BT + kTgWaves * 16 * WT) * (KC + kTgPad) * sizeof(half_t);
+  return (size_t)(2 * 16 * BT + WAVES * 16 * WT) * (KC + kTgPad) * sizeof(half_t);
 }
 
-template <int BT, int WT, int KC>
-__global__ __launch_bounds__(kTgWaves * 64) void gemm_tiled_mfma_kernel(
+// QKV mode: the M = 3 * Hk * hd output rows are the q, k, v rows of the selected heads
+// (m = (t * Hk + i) * hd + j -> weight row (t * H + head_idx[i]) * hd + j, skipped when the head is out of
+// range or live[i * live_stride] < 0), the result goes to column `weight row` of Y (B, 3, H, hd) and the
+// K / V rows are also appended to the per-sequence caches k_cache (B, H, hd/8, S, 8), v_cache (B, H, S, hd)
+// at position positions[per_sample ? b : 0] + pos_add.
+struct QkvScatter {
+  const int* head_idx;
+  const int* live;
+  int live_stride, Hk, H, hd;
+  half_t* k_cache;
+  half_t* v_cache;
+  const int* positions;
+  int per_sample, pos_add, S;
+};
+
+__device__ __forceinline__ int qkv_row_of(const QkvScatter& q, int m) {
+  const int t = m / (q.Hk * q.hd);
+  const int rem = m - t * q.Hk * q.hd;
+  const int i = rem / q.hd, j = rem - i * q.hd;
+  const int h = q.head_idx[i];
+  if (h < 0 || h >= q.H || t > 2) return -1;
+  if (q.live != nullptr && q.live[(int64_t)i * q.live_stride] < 0) return -1;
+  return (t * q.H + h) * q.hd + j;
+}
+
+// stores one finished value: Y[b, weight row] and, for K / V rows, the cache entry
+__device__ __forceinline__ void qkv_store(const QkvScatter& q, half_t* __restrict__ Y, int b, int rid, half_t hv) {
+  Y[(int64_t)b * 3 * q.H * q.hd + rid] = hv;
+  if (q.k_cache == nullptr) return;
+  const int t = rid / (q.H * q.hd);
+  if (t == 0) return;
+  const int rem = rid - t * q.H * q.hd;
+  const int h = rem / q.hd, j = rem - h * q.hd;
+  const int dst = (q.positions ? q.positions[q.per_sample ? b : 0] : 0) + q.pos_add;
+  if (dst < 0 || dst >= q.S) return;
+  if (t == 1)
+    q.k_cache[((((int64_t)b * q.H + h) * (q.hd / 8) + j / 8) * q.S + dst) * 8 + (j & 7)] = hv;
+  else
+    q.v_cache[(((int64_t)b * q.H + h) * q.S + dst) * q.hd + j] = hv;
+}
+
+template <int BT, int WT, int KC, bool QKV = false, int WAVES = kTgWaves>
+__global__ __launch_bounds__(WAVES * 64) void gemm_tiled_mfma_kernel(
     const half_t* __restrict__ X, int64_t ldx, const half_t* __restrict__ W, int64_t ldw,
     const half_t* __restrict__ bias, const void* __restrict__ idx, int idx_bytes, int B, int N, int Z, int M,
-    half_t* __restrict__ Y, int64_t ldy, int relu, int chunks_per_split, float* __restrict__ partial) {
+    half_t* __restrict__ Y, int64_t ldy, int relu, int chunks_per_split, float* __restrict__ partial,
+    QkvScatter qs) {
   const bool SPLIT = chunks_per_split > 0;  // uniform
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   constexpr int LD = KC + kTgPad;
   constexpr int XROWS = 16 * BT, WROWS = 16 * WT;
   constexpr int VPR = KC / 8;                      // 16-byte vectors per staged row
-  constexpr int XV = XROWS * VPR / (kTgWaves * 64);  // X vectors per thread and chunk
+  constexpr int XV = XROWS * VPR / (WAVES * 64);  // X vectors per thread and chunk
   constexpr int WV = WROWS * VPR / 64;               // weight vectors per lane and chunk
-  static_assert(XROWS * VPR % (kTgWaves * 64) == 0 && WROWS * VPR % 64 == 0, "staging does not tile");
+  static_assert(XROWS * VPR % (WAVES * 64) == 0 && WROWS * VPR % 64 == 0, "staging does not tile");
   half_t* xs = reinterpret_cast<half_t*>(smem_raw);                       // [2][XROWS][LD]
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -55,7 +97,7 @@ __global__ __launch_bounds__(kTgWaves * 64) void gemm_tiled_mfma_kernel(
   const int l16 = lane & 15, kg = lane >> 4;
 
   const int b0 = blockIdx.x * XROWS;
-  const int m0 = (blockIdx.y * kTgWaves + wave) * WROWS;  // first output row of this wavefront
+  const int m0 = (blockIdx.y * WAVES + wave) * WROWS;  // first output row of this wavefront
   const int nchunks = (N + KC - 1) / KC;
   const int c_begin = SPLIT ? (int)blockIdx.z * chunks_per_split : 0;
   const int c_end = SPLIT ? (c_begin + chunks_per_split < nchunks ? c_begin + chunks_per_split : nchunks) : nchunks;
@@ -64,8 +106,12 @@ __global__ __launch_bounds__(kTgWaves * 64) void gemm_tiled_mfma_kernel(
   int rid_mine = -1;
   if (lane < WROWS && m0 + lane < M) {
     const int m = m0 + lane;
-    const int64_t id = idx == nullptr ? (int64_t)m : load_index(idx, idx_bytes, m);
-    rid_mine = (id >= 0 && id < Z) ? (int)id : -1;
+    if (QKV) {
+      rid_mine = qkv_row_of(qs, m);
+    } else {
+      const int64_t id = idx == nullptr ? (int64_t)m : load_index(idx, idx_bytes, m);
+      rid_mine = (id >= 0 && id < Z) ? (int)id : -1;
+    }
   }
   // staging coordinates: weight vector q of a lane is row q * (64 / VPR) + lane / VPR, columns (lane % VPR) * 8
   const int wv_row = lane / VPR, wv_col = (lane % VPR) * 8;
@@ -81,7 +127,7 @@ __global__ __launch_bounds__(kTgWaves * 64) void gemm_tiled_mfma_kernel(
   const half_t* xrow[XV];
 #pragma unroll
   for (int p = 0; p < XV; ++p) {
-    const int b = b0 + (p * kTgWaves * 64 + tid) / VPR;
+    const int b = b0 + (p * WAVES * 64 + tid) / VPR;
     xrow[p] = X + (int64_t)(b < B ? b : b0) * ldx;  // rows past B re-read the block's first row; never stored
   }
   const int xv_col = (tid % VPR) * 8;
@@ -114,7 +160,7 @@ __global__ __launch_bounds__(kTgWaves * 64) void gemm_tiled_mfma_kernel(
     half_t* xb = xs + (size_t)buf * XROWS * LD;
 #pragma unroll
     for (int p = 0; p < XV; ++p)
-      store8(xb + ((p * kTgWaves * 64 + tid) / VPR) * LD + xv_col, x_ok ? xstage[p] : zero8());
+      store8(xb + ((p * WAVES * 64 + tid) / VPR) * LD + xv_col, x_ok ? xstage[p] : zero8());
   };
   auto multiply = [&](int buf) {
     const half_t* xb = xs + (size_t)buf * XROWS * LD;
@@ -185,6 +231,12 @@ __global__ __launch_bounds__(kTgWaves * 64) void gemm_tiled_mfma_kernel(
         if (bias != nullptr && rid[v] >= 0) val[v] += (float)bias[rid[v]];
         if (relu) val[v] = relu_f(val[v]);
       }
+      if (QKV) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+          if (mrow + v < M && rid[v] >= 0) qkv_store(qs, Y, b, rid[v], (half_t)val[v]);
+        continue;
+      }
       half_t* dst = Y + (int64_t)b * ldy + mrow;
       if (mrow + 3 < M && (ldy & 3) == 0 && (reinterpret_cast<uintptr_t>(Y) & 7) == 0) {
         half4_t o = {(half_t)val[0], (half_t)val[1], (half_t)val[2], (half_t)val[3]};
@@ -214,6 +266,22 @@ __global__ __launch_bounds__(256) void gemm_split_reduce_kernel(
   }
   if (relu) s = relu_f(s);
   Y[(int64_t)b * ldy + m] = (half_t)s;
+}
+
+// QKV mode: sums the splits, adds the bias and scatters (Y and the caches).
+__global__ __launch_bounds__(256) void qkv_split_reduce_kernel(const float* __restrict__ partial, int nsplit, int B,
+                                                               int M, const half_t* __restrict__ bias,
+                                                               half_t* __restrict__ Y, QkvScatter qs) {
+  const int64_t total = (int64_t)B * M;
+  const int64_t o = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (o >= total) return;
+  const int b = (int)(o / M), m = (int)(o - (int64_t)b * M);
+  const int rid = qkv_row_of(qs, m);
+  if (rid < 0) return;
+  float s = 0.f;
+  for (int y = 0; y < nsplit; ++y) s += partial[(int64_t)y * total + o];
+  if (bias != nullptr) s += (float)bias[rid];
+  qkv_store(qs, Y, b, rid, (half_t)s);
 }
 
 }  // namespace dv

@@ -367,7 +367,7 @@ def qkv_proj_batch(x: torch.Tensor, weight: torch.Tensor, head_idx: torch.Tensor
                    bias: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
                    k_cache: Optional[torch.Tensor] = None, v_cache: Optional[torch.Tensor] = None,
                    positions: Optional[torch.Tensor] = None, pos_add: int = 0,
-                   live: Optional[torch.Tensor] = None) -> torch.Tensor:
+                   live: Optional[torch.Tensor] = None, use_workspace: bool = True) -> torch.Tensor:
     """QKV of the active heads for one token of each of B sequences (one shared head set), on the
     matrix cores, the weights streamed once for the whole batch; with caches the K / V rows are
     appended to sequence b's cache at ``positions[b] + pos_add`` (``positions``: int32, (B,) per
@@ -379,6 +379,7 @@ def qkv_proj_batch(x: torch.Tensor, weight: torch.Tensor, head_idx: torch.Tensor
     :param live: optional int32 vector or strided column, one entry per active head: heads with a
         negative entry are skipped (back-fill passes)
     :param k_cache, v_cache: (B, nheads, head_dim / 8, S, 8), (B, nheads, S, head_dim)
+    :param use_workspace: False keeps the kernel that needs no scratch memory also from 9 rows on
     :return: (B, 3, nheads, head_dim); rows of inactive / skipped heads keep the content of ``out``
     """
     _require_device(x, weight, head_idx, bias, k_cache, v_cache, positions, live)
@@ -408,9 +409,12 @@ def qkv_proj_batch(x: torch.Tensor, weight: torch.Tensor, head_idx: torch.Tensor
     if live is not None:
         assert live.dtype == torch.int32 and live.dim() == 1 and live.shape[0] == n_active
         live_stride = live.stride(0)
+    nbytes = lib.dv_qkv_proj_batch_workspace_bytes(B, hidden_dim, n_active, head_dim) if use_workspace else 0
+    ws = _workspace(x.device, nbytes) if nbytes else None
     check(lib.dv_qkv_proj_batch_f16(_ptr(x), x.stride(0), _ptr(weight), _ptr(bias), _ptr(head_idx), _ptr(live),
                                     live_stride, n_active, B, hidden_dim, nheads, head_dim, _ptr(out), _ptr(k_cache),
-                                    _ptr(v_cache), _ptr(positions), per_sample, int(pos_add), S, _stream()),
+                                    _ptr(v_cache), _ptr(positions), per_sample, int(pos_add), S, _ptr(ws),
+                                    0 if ws is None else ws.numel(), _stream()),
           "dv_qkv_proj_batch_f16")
     return out
 

@@ -215,11 +215,17 @@ DV_API int dv_qkv_proj_sparse_cache_f16(const void* x, const void* W, const void
  *   k_cache (B, H, hd/8, S, 8), v_cache (B, H, S, hd): both or neither NULL; positions: device
  *   int32, (B,) when per_sample != 0, else (1,), or NULL (= 0); rows whose position is outside
  *   [0, S) are projected but not cached.  hd in {32, 64, 128}.
+ *   workspace: dv_qkv_proj_batch_workspace_bytes(B, d, nnz, hd) bytes (0 up to 8 rows), 16-byte
+ *   aligned, no initialisation needed: from 9 rows on the block of X is shared through LDS by a
+ *   workgroup that owns 128 weight rows, and the columns are split over workgroups (fp32 partial
+ *   sums added in ascending order by a second launch); without it every 16-row tile fetches X itself.
  */
+DV_API size_t dv_qkv_proj_batch_workspace_bytes(int B, int d, int nnz, int hd);
 DV_API int dv_qkv_proj_batch_f16(const void* x, int64_t ldx, const void* W, const void* bias,
                                  const void* head_idx, const void* live, int live_stride, int nnz, int B,
                                  int d, int H, int hd, void* y, void* k_cache, void* v_cache,
-                                 const void* positions, int per_sample, int pos_add, int S, void* stream);
+                                 const void* positions, int per_sample, int pos_add, int S,
+                                 void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Causal attention over the prompt, and the prompt's K / V rows written into the decode caches:
