@@ -82,7 +82,11 @@ int launch_canonical(const half_t* X, const half_t* W, int64_t ldw, int B, int r
   // group; batch 4: 98 us per MLP block with R = 1 against 102 us with R = 4; batch 8: 122 against 121.
   const size_t xlds = (size_t)B * n * sizeof(float);
   const bool use_xlds = LANES == 16 && xlds <= 48 * 1024;
-  const int xr = B >= 5 ? 4 : (B == 1 ? 2 : 1);
+  // Few rows (the head predictor's second product: 96 rows): one row per lane group, so that the rows
+  // spread over as many wavefronts as possible (16 us -> a few us at batch 8: four rows per group left
+  // six wavefronts with long dependent chains).
+  const bool few_rows = B >= 5 && rows < RW * 4 * 4 * compute_units();
+  const int xr = B >= 5 ? (few_rows ? 1 : 4) : (B == 1 ? 2 : 1);
   if (use_xlds) {
     blocks = ((rows + RW * xr - 1) / (RW * xr) + 3) / 4;
     if (blocks > cap) blocks = cap;
@@ -90,7 +94,10 @@ int launch_canonical(const half_t* X, const half_t* W, int64_t ldw, int B, int r
   }
 #define DV_CASE(BB)                                                                                \
   case BB:                                                                                         \
-    if (use_xlds)                                                                                  \
+    if (use_xlds && few_rows)                                                                      \
+      hipLaunchKernelGGL((canonical_gemv_xlds_kernel<LANES, BB, (BB >= 5 ? 4 : 8), 1>), dim3(blocks), \
+                         dim3(256), xlds, s, X, W, ldw, rows, n, Y);                               \
+    else if (use_xlds)                                                                             \
       hipLaunchKernelGGL((canonical_gemv_xlds_kernel<LANES, BB, (BB >= 5 ? 4 : 8), (BB >= 5 ? 4 : (BB == 1 ? 2 : 1))>), dim3(blocks), \
                          dim3(256), xlds, s, X, W, ldw, rows, n, Y);                               \
     else                                                                                           \
@@ -106,9 +113,34 @@ int launch_canonical(const half_t* X, const half_t* W, int64_t ldw, int B, int r
   return launch_status();
 }
 
+// Long rows, three or more batch rows: the slices kernel (X shared through LDS); same bits.
+template <int B>
+int launch_canonical_slices(const half_t* X, const half_t* W, int64_t ldw, int rows, int n, half_t* Y,
+                            hipStream_t s) {
+  const size_t lds = (size_t)2 * B * kCanonSlice * sizeof(half_t);
+  static LdsGrant grant;
+  if (int rc = grant.ensure(reinterpret_cast<const void*>(canonical_gemv_slices_kernel<B>), lds); rc != DV_OK)
+    return rc;
+  int blocks = (rows + 3) / 4;
+  const int cap = compute_units() * 4;
+  if (blocks > cap) blocks = cap;
+  if (blocks < 1) blocks = 1;
+  hipLaunchKernelGGL((canonical_gemv_slices_kernel<B>), dim3(blocks), dim3(256), lds, s, X, W, ldw, rows, n, Y);
+  return launch_status();
+}
+
 int canonical_gemv(const half_t* X, const half_t* W, int64_t ldw, int B, int rows, int n,
                    half_t* Y, hipStream_t s) {
   if (dv_canonical_lanes(n) == 16) return launch_canonical<16, 8>(X, W, ldw, B, rows, n, Y, s);
+  switch (B) {  // measured at the OPT-175B predictor (1000 rows of 12288): see the kernel's header
+    case 3: return launch_canonical_slices<3>(X, W, ldw, rows, n, Y, s);
+    case 4: return launch_canonical_slices<4>(X, W, ldw, rows, n, Y, s);
+    case 5: return launch_canonical_slices<5>(X, W, ldw, rows, n, Y, s);
+    case 6: return launch_canonical_slices<6>(X, W, ldw, rows, n, Y, s);
+    case 7: return launch_canonical_slices<7>(X, W, ldw, rows, n, Y, s);
+    case 8: return launch_canonical_slices<8>(X, W, ldw, rows, n, Y, s);
+    default: break;
+  }
   return launch_canonical<64, 8>(X, W, ldw, B, rows, n, Y, s);
 }
 

@@ -179,6 +179,89 @@ __global__ __launch_bounds__(256) void canonical_gemv_xlds_kernel(
   canonical_gemv_lds_body<LANES, B, U, R>(xf, W, ldw, rows, n, Y, blockIdx.x, gridDim.x);
 }
 
+// Long rows (64 lanes per row), several batch rows: canonical_gemv_body re-reads B x 16 bytes of X
+// from L2 for every 16 bytes of weights (B rows of X do not fit LDS at n = 12288).  Here the
+// workgroup walks the columns in slices of kCanonSlice elements; all its wavefronts (one weight row
+// each) share the slice of X, staged as fp16 in LDS (double-buffered, one barrier per slice), and
+// the next slice's weights and X are requested before the current slice is multiplied.  Per output
+// the products are folded in the same (chunk, element) order and the same butterfly as
+// canonical_gemv_body (chunks past the row end contribute w = x = 0): the same bits.
+// Dynamic LDS: 2 * B * kCanonSlice halfs.  n % 8 == 0, ldw % 8 == 0.
+constexpr int kCanonSlice = 2048;  // four chunks of 8 * 64 elements
+
+template <int B>
+__global__ __launch_bounds__(256) void canonical_gemv_slices_kernel(
+    const half_t* __restrict__ X, const half_t* __restrict__ W, int64_t ldw, int rows, int n,
+    half_t* __restrict__ Y) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  half_t* xs = reinterpret_cast<half_t*>(smem_raw);  // [2][B][kCanonSlice]
+  constexpr int CH = 8 * kWave;
+  constexpr int U = kCanonSlice / CH;               // chunks per slice
+  constexpr int XV = B * kCanonSlice / 8 / 256;     // X vectors per thread and slice
+  static_assert(B * kCanonSlice / 8 % 256 == 0, "slice staging does not tile");
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int nslices = (n + kCanonSlice - 1) / kCanonSlice;
+  // X vector p of a thread: batch row (p * 256 + tid) / (kCanonSlice / 8), columns ((p * 256 + tid) % (kCanonSlice / 8)) * 8
+  auto load_x = [&](half8_t (&xv)[XV], int sl) {
+#pragma unroll
+    for (int p = 0; p < XV; ++p) {
+      const int o = p * 256 + tid;
+      const int b = o / (kCanonSlice / 8), col = sl * kCanonSlice + (o % (kCanonSlice / 8)) * 8;
+      xv[p] = col < n ? load8(X + (int64_t)b * n + col) : zero8();
+    }
+  };
+  auto store_x = [&](const half8_t (&xv)[XV], int buf) {
+#pragma unroll
+    for (int p = 0; p < XV; ++p) store8(xs + (size_t)buf * B * kCanonSlice + (size_t)(p * 256 + tid) * 8, xv[p]);
+  };
+  for (int row0 = blockIdx.x * 4; row0 < rows; row0 += gridDim.x * 4) {  // uniform over the workgroup
+    const int row = row0 + wave;
+    const bool valid = row < rows;
+    const half_t* wr = W + (int64_t)(valid ? row : 0) * ldw + lane * 8;
+    auto load_w = [&](half8_t (&w)[U], int sl) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int col = sl * kCanonSlice + u * CH + lane * 8;
+        w[u] = col < n ? load8_stream(wr + sl * kCanonSlice + u * CH) : zero8();
+      }
+    };
+    float acc[B];
+#pragma unroll
+    for (int b = 0; b < B; ++b) acc[b] = 0.f;
+    half8_t w[U], wn[U], xv[XV];
+    __syncthreads();  // the previous row group's reads of the X buffers are done
+    load_x(xv, 0);
+    load_w(w, 0);
+    store_x(xv, 0);
+    for (int sl = 0; sl < nslices; ++sl) {
+      const int buf = sl & 1;
+      __syncthreads();  // slice sl is in LDS; every wavefront is done with slice sl - 1 (the other buffer)
+      if (sl + 1 < nslices) {
+        load_x(xv, sl + 1);
+        load_w(wn, sl + 1);
+      }
+      const half_t* xb = xs + (size_t)buf * B * kCanonSlice + lane * 8;
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+#pragma unroll
+        for (int b = 0; b < B; ++b) acc[b] = fma8_ordered(w[u], load8(xb + b * kCanonSlice + u * CH), acc[b]);
+      }
+      if (sl + 1 < nslices) {
+        store_x(xv, buf ^ 1);
+#pragma unroll
+        for (int u = 0; u < U; ++u) w[u] = wn[u];
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < B; ++b) {
+      const float v = butterfly_sum<kWave>(acc[b]);
+      if (valid && lane == 0) Y[(int64_t)b * rows + row] = (half_t)v;
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Y[b, m] = act( sum_i W[idx[m], i] * X[b, i] + bias[idx[m]] ), fp16 out.
 // One wavefront owns R gathered rows at a time (R independent load streams);

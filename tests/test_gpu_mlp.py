@@ -291,3 +291,21 @@ def test_opt67b_block_batch_by_k_grid(ops, batch, K):
                  "mlp_sparse")
     if batch == 8 and K == 16384:
         _GRID_CACHE.clear()
+
+
+@pytest.mark.parametrize("B,d,r", [(3, 5128, 72), (5, 2056, 40), (8, 12288, 64), (6, 1032, 24)])
+def test_predictor_first_product_long_rows_several_batch_rows_bit_exact(ops, B, d, r):
+    """Rows longer than 1024 with 3..8 batch rows: X slices shared through LDS.  Same fixed summation
+    order as the single-row kernel (bit-exact against the oracle); row lengths that are not multiples
+    of the 2048-element slice or of the 512-element chunk, more rows than one pass of the grid."""
+    g = torch.Generator().manual_seed(B * 31 + d)
+    x = torch.randn(B, d, generator=g).half()
+    Wa = (torch.randn(r, d, generator=g) * 0.05).half()
+    Wb = (torch.randn(96, r, generator=g) * 0.05).half()
+    print(f"case predictor long rows B={B} d={d} r={r}", flush=True)
+    hidden = torch.empty(B, r, dtype=torch.float16, device="cuda")
+    got = ops.predictor_logits(x.cuda(), Wa.cuda(), Wb.cuda(), hidden=hidden)
+    torch.cuda.synchronize()
+    h_ref, l_ref = O.predictor_logits(x.numpy(), Wa.numpy(), Wb.numpy())
+    assert np.array_equal(np16(hidden).view(np.uint16), h_ref.view(np.uint16)), "hidden vector differs"
+    assert np.array_equal(np16(got).view(np.uint16), l_ref.view(np.uint16)), "logits differ"
