@@ -51,15 +51,19 @@ TRAFFIC_JSON = os.path.join(ROOT, "profiles", "traffic.json")
 CSRC_DIR = os.path.join(ROOT, "dejavu_amd", "csrc")
 
 
+# sources of the kernels whose traffic is recorded (the QKV projection, stand-alone and inside the fused layer)
+TRAFFIC_SOURCES = ("attention.hpp", "common.hpp", "gemm_mfma.hpp", "layer_fused.hpp", "qkv_mfma.hpp")
+
+
 def csrc_digest():
-    """SHA-256 over the kernel sources: ties a counter measurement to the code it was taken on."""
+    """SHA-256 over the sources of the measured kernels: ties a counter measurement to the code it was
+    taken on."""
     import hashlib
 
     h = hashlib.sha256()
-    for name in sorted(os.listdir(CSRC_DIR)):
-        if name.endswith((".hip", ".hpp")):
-            with open(os.path.join(CSRC_DIR, name), "rb") as f:
-                h.update(name.encode() + b"\0" + f.read())
+    for name in TRAFFIC_SOURCES:
+        with open(os.path.join(CSRC_DIR, name), "rb") as f:
+            h.update(name.encode() + b"\0" + f.read())
     return h.hexdigest()
 
 
@@ -113,7 +117,8 @@ def write_traffic(fetch_csv, write_csv):
                                 text=True).stdout.strip()
     except OSError:
         commit = ""
-    doc = {"csrc_sha256": csrc_digest(), "commit": commit, "unit": "HBM bytes per launch (read + written)",
+    doc = {"csrc_sha256": csrc_digest(), "sources": list(TRAFFIC_SOURCES), "commit": commit,
+           "unit": "HBM bytes per launch (read + written)",
            "scale": {"FETCH_SIZE": round(f_scale, 4), "WRITE_SIZE": round(w_scale, 4),
                      "calibration": "1 GiB device-to-device copy in the same run"},
            "bytes_per_launch": out}
