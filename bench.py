@@ -101,11 +101,21 @@ def write_traffic(fetch_csv, write_csv):
         hits = [v for k, v in table.items() if needle in k]
         return hits[0] if hits else None
 
+    def largest(path, counter, needle):
+        best = 0.0
+        with open(path, newline="") as f:
+            for row in csv.DictReader(f):
+                if row.get("Counter_Name") == counter and needle in row["Kernel_Name"]:
+                    best = max(best, float(row["Counter_Value"]))
+        return best
+
     fetch, write = per_kernel(fetch_csv, "FETCH_SIZE"), per_kernel(write_csv, "WRITE_SIZE")
+    # the calibration copy is the largest dispatch of the runtime's buffer-copy kernel (1 GiB read and written)
     copy_kib = float(1 << 20)
-    f_scale = copy_kib / find(fetch, "copyBuffer")
-    w_scale = copy_kib / find(write, "copyBuffer")
-    names = {"qkv_sparse_kernel": "qkv_sparse", "layer_l2_kernel<1>": "qkv_l2_one_token",
+    f_scale = copy_kib / largest(fetch_csv, "FETCH_SIZE", "copyBuffer")
+    w_scale = copy_kib / largest(write_csv, "WRITE_SIZE", "copyBuffer")
+    names = {"qkv_sparse_kernel": "qkv_sparse", "qkv_window_mfma_kernelILi4ELi1E": "qkv_window_mfma",
+             "qkv_window_mfma_kernelILi4ELi2E": "qkv_flush_mfma", "layer_l2_kernel<1>": "qkv_l2_one_token",
              "layer_l2_kernel<0>": "qkv_l2_mfma", "layer_l2_kernel<-1>": "qkv_l2_flush"}
     out = {}
     for needle, key in names.items():
@@ -805,11 +815,15 @@ def main():
                         "(flush); the fused layer runs the same bodies as layer_l2_kernel<1>, <0>, <-1>",
                         "achieved": round(mix_bytes / mix_us / 1e3, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                         "frac": round(mix_bytes / mix_us / 1e3 / HBM_PEAK_GBPS, 4),
-                        "traffic": measured_traffic(args.config, batch, "qkv_sparse"),
-                        "traffic_kernel": "qkv_sparse_kernel",
+                        "traffic": None,
                         "bytes_per_launch": round(mix_bytes / launches), "us_per_launch": round(mix_us / launches, 2),
                         "launch_mix": {k: n for k, n in mix},
                         "standalone": {k: table[k] for k, _ in mix}}
+            # HBM bytes per launch from the last counter run (profiles/traffic.json), same launch mix
+            per = {k: measured_traffic(args.config, batch, k) for k, n in mix if n}
+            if per and all(v is not None for v in per.values()):
+                roofline["traffic"] = round(sum(per[k] * n for k, n in mix if n) / launches)
+                roofline["traffic_per_kernel"] = per
         else:
             dom = "decode_attn" if nbytes["decode_attn"] >= nbytes["qkv_sparse"] else "qkv_batch"
             roofline = {"bound": "hbm", "kernel": {"decode_attn": "decode_attn_kernel", "qkv_batch":
