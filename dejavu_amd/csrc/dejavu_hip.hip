@@ -693,7 +693,11 @@ int dv_canonical_lanes(int n) { return n <= 1024 ? 16 : 64; }
 
 size_t dv_predictor_workspace_bytes(int B, int d, int r) {
   if (B <= 8 || B > 64 || d <= 0 || r <= 0) return 0;
-  return rows_split_workspace_bytes(B, d, r);
+  // the first product's column splits; the second product (rows of r elements) splits only when r is long,
+  // allow for as many partial sums again
+  const size_t first = tiled_workspace_bytes(B, d, r);
+  const size_t floor_bytes = (size_t)1 << 20;
+  return 2 * (first > floor_bytes ? first : floor_bytes);
 }
 
 int dv_predictor_logits_ws_f16(const void* x, const void* Wa, int64_t ldwa, const void* Wb, int64_t ldwb,
@@ -706,6 +710,36 @@ int dv_predictor_logits_ws_f16(const void* x, const void* Wa, int64_t ldwa, cons
       !aligned16(Wa) || !aligned16(Wb) || !aligned16(hidden))
     return DV_ERR_ALIGNMENT;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (B > 8 && workspace != nullptr && aligned16(workspace) &&
+      workspace_bytes >= dv_predictor_workspace_bytes(B, d, r) && ldwa >= d) {
+    // more rows than the fixed-order kernel keeps accumulators for: both products on the matrix cores
+    // (fp32 accumulation in the MFMA's own order).  First product (r rows of d elements: few row tiles):
+    // the X-shared split-K kernel (measured at the OPT-175B predictor, batch 16 / 32: 33.6 / 38.8 us for
+    // the whole MLP predictor against 37.2 / 44.1 us with one 16-row tile per workgroup).  Second
+    // product: many short rows -> whole tiles per wavefront with X in LDS (rows_short); few rows (the
+    // head predictor: 96) -> the X-shared kernel again (head predictor 17.7 / 21.6 against 18.7 / 25.3 us).
+    int rc = gemm_tiled(reinterpret_cast<const half_t*>(x), d, reinterpret_cast<const half_t*>(Wa), ldwa, nullptr,
+                        nullptr, 4, B, d, r, r, DV_ACT_ID, reinterpret_cast<half_t*>(hidden), r, workspace,
+                        workspace_bytes, s);
+    if (rc != DV_OK) return rc;
+    const int pass_rows = B <= 32 ? B : 32;
+    if (rows_short_fits(pass_rows, r, n_out) && aligned16(logits) && ((int64_t)32 * n_out) % 8 == 0) {
+      for (int b0 = 0; b0 < B && rc == DV_OK; b0 += 32) {
+        const int nb = B - b0 < 32 ? B - b0 : 32;
+        rc = rows_short_mfma(reinterpret_cast<const half_t*>(hidden) + (int64_t)b0 * r,
+                             reinterpret_cast<const half_t*>(Wb), ldwb, nb, r, n_out,
+                             reinterpret_cast<half_t*>(logits) + (int64_t)b0 * n_out, s);
+      }
+      if (rc != DV_ERR_UNSUPPORTED) return rc;
+    }
+    if (tiled_workspace_bytes(B, r, n_out) <= workspace_bytes)
+      return gemm_tiled(reinterpret_cast<const half_t*>(hidden), r, reinterpret_cast<const half_t*>(Wb), ldwb,
+                        nullptr, nullptr, 4, B, r, n_out, n_out, DV_ACT_ID, reinterpret_cast<half_t*>(logits),
+                        n_out, workspace, workspace_bytes, s);
+    return gather_rows_mfma(reinterpret_cast<const half_t*>(hidden), reinterpret_cast<const half_t*>(Wb), ldwb,
+                            nullptr, nullptr, 4, B, r, n_out, n_out, DV_ACT_ID,
+                            reinterpret_cast<half_t*>(logits), s);
+  }
   if (B > 8) {
     // more rows than the fixed-order kernel keeps accumulators for: both products on the
     // matrix cores (no gather, no bias), fp32 accumulation in the MFMA's own order.  The

@@ -192,9 +192,15 @@ __global__ __launch_bounds__(256) void topk_small_kernel(const half_t* __restric
   __shared__ unsigned s_sel[1024];
   for (int i = threadIdx.x; i < n; i += blockDim.x) {
     unsigned key = 0u;
-    for (int b = 0; b < B; ++b) {
-      const unsigned kk = topk_key(logits[(int64_t)b * n + i]);
-      key = kk > key ? kk : key;
+    for (int b0 = 0; b0 < B; b0 += 8) {  // eight rows requested at once (a batch is a chain of latencies otherwise)
+      half_t v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = logits[(int64_t)(b0 + u < B ? b0 + u : B - 1) * n + i];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const unsigned kk = topk_key(v[u]);
+        key = kk > key ? kk : key;
+      }
     }
     s_key[i] = key;
   }

@@ -105,7 +105,7 @@ def predictor_logits(x: torch.Tensor, fc0_weight: torch.Tensor, fc1_weight: torc
         ws = _workspace(x.device, nbytes) if nbytes else None
         check(lib.dv_predictor_logits_ws_f16(_ptr(x[b0:]), _ptr(fc0_weight), fc0_weight.stride(0), _ptr(fc1_weight),
                                              fc1_weight.stride(0), nb, d, r, n_out, _ptr(hidden[b0:]),
-                                             _ptr(logits[b0:]), _ptr(ws), nbytes, _stream()),
+                                             _ptr(logits[b0:]), _ptr(ws), 0 if ws is None else ws.numel(), _stream()),
               "dv_predictor_logits_ws_f16")
     return logits
 

@@ -65,8 +65,9 @@ DV_API int dv_predictor_logits_f16(const void* x, const void* Wa, int64_t ldwa, 
 
 /*
  * The same with a workspace: for 9..64 rows the first product (r rows of d
- * elements: few 16-row tiles) is also split over the columns, each split writing
- * fp32 partial sums that a second launch adds in ascending order (deterministic).
+ * elements: few row tiles) shares each block of x through LDS and is split over
+ * the columns, each split writing fp32 partial sums that a second launch adds in
+ * ascending order (deterministic); so is the second product when it has few rows.
  * workspace: dv_predictor_workspace_bytes(B, d, r) bytes, 16-byte aligned; with
  * NULL / 0 the call behaves like dv_predictor_logits_f16.  Up to 8 rows the
  * workspace is not used.
