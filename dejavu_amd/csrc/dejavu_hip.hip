@@ -555,7 +555,7 @@ ColsMfmaPlan plan_cols_mfma(int B, int N, int M) {
   // unit measured best for batch 8..64.  Up to batch 32 a workgroup's four wavefronts split the
   // group's rows and add their sums through LDS (a quarter of the partials: fc2 at the OPT-175B
   // shape 3 us faster at batch 16 and 32); above, they split the columns.
-  const int waves_per_cu = 3;
+  const int waves_per_cu = 3;  // 4..16 measured 30-50 % slower for batch 5..32 (fc2, OPT-175B shape)
   const bool split_rows = B <= 32;
   const int col_tile = mfma_col_tile(split_rows ? 1 : 2);
   p.col_tiles = (N + col_tile - 1) / col_tile;

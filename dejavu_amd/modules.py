@@ -34,12 +34,22 @@ from ._lib import check, lib
 # graph down (greedy decode of the 40-layer OPT-13B shape, only the dense first block on the
 # module path: 322 tokens/s with the side stream, 357 without; eager 792 -> 765 ms).
 USE_SIDE_STREAM = False
+# From this many sequences on the side stream is used regardless: a batched layer step goes module by
+# module, its predictors and top-ks are a dozen short launches beside kernels of 50-170 us, and
+# overlapping them pays (OPT-175B shape: 279.9 -> 255.3 us/layer at batch 8, 425.1 -> 385.0 us at
+# batch 32).  None: never.
+SIDE_STREAM_MIN_BATCH = 2
 
 # Prompt phase on this package's own kernels (dense products: dv_dense_linear_f16; causal attention
 # + cache fill: dv_prefill_attention_f16).  False: PyTorch's library GEMM and attention.
 USE_HIP_PROMPT = True
 
 _side_streams: dict = {}
+_side_pending = False  # work was enqueued on the side stream since the last join_side_stream()
+
+
+def side_stream_enabled(batch: int = 1) -> bool:
+    return bool(USE_SIDE_STREAM) or (SIDE_STREAM_MIN_BATCH is not None and batch >= SIDE_STREAM_MIN_BATCH)
 
 
 def side_stream(device=None) -> "torch.cuda.Stream":
@@ -59,7 +69,9 @@ def side_stream(device=None) -> "torch.cuda.Stream":
 def join_side_stream() -> None:
     """Makes the current stream wait for everything enqueued on the side stream so far
     (e.g. before a graph capture that used the side stream ends)."""
-    if USE_SIDE_STREAM and _side_streams:
+    global _side_pending
+    if _side_pending and _side_streams:
+        _side_pending = False
         ev = torch.cuda.Event(enable_timing=False, blocking=False)
         st = side_stream()
         st.record_event(ev)
@@ -182,8 +194,10 @@ class ParallelFusedMLPDejavu(nn.Module):
         # stream while fc1 / fc2 run (the reference starts it after the MLP, to
         # overlap the tensor-parallel all-reduce that one GPU does not have).
         mlp_logit = None
-        side = do_token_generation and USE_SIDE_STREAM
+        side = do_token_generation and side_stream_enabled(x.shape[0])
         if side:
+            global _side_pending
+            _side_pending = True
             curr_stream.record_event(self.event_mlp)
             with torch.cuda.stream(self.sp_stream):
                 self.sp_stream.wait_event(self.event_mlp)
@@ -327,13 +341,16 @@ class _MHABase(nn.Module):
         self._side_used = False
         if mlp_sp_logit is None and att_sp is None:
             return mlp_idx, att_idx
-        if not USE_SIDE_STREAM:
+        batch = residual.shape[0] if residual is not None else (mlp_sp_logit.shape[0] if mlp_sp_logit.dim() > 1 else 1)
+        if not side_stream_enabled(batch):
             if att_sp is not None:
                 att_idx = ops.topk_indices(att_sp(residual), att_k, dtype=torch.int32, out=att_idx_out)
             if mlp_sp_logit is not None:
                 mlp_idx = ops.topk_indices(mlp_sp_logit, self.mlp_k)
             return mlp_idx, att_idx
         self._side_used = True
+        global _side_pending
+        _side_pending = True
         torch.cuda.current_stream().record_event(self.event_in)
         with torch.cuda.stream(self.sp_stream):
             self.sp_stream.wait_event(self.event_in)

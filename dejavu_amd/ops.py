@@ -53,7 +53,9 @@ _retired_workspaces: list = []
 
 
 def _grown(cache: dict, device: torch.device, nbytes: int, floor: int) -> torch.Tensor:
-    key = (device.type, device.index)
+    # one buffer per (device, stream): ops enqueued on different streams (the modules' side stream)
+    # may run at the same time and must not share partial sums
+    key = (device.type, device.index, torch.cuda.current_stream(device).cuda_stream)
     ws = cache.get(key)
     if ws is None or ws.numel() < nbytes:
         if ws is not None:
@@ -64,8 +66,7 @@ def _grown(cache: dict, device: torch.device, nbytes: int, floor: int) -> torch.
 
 
 def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
-    """Per-device scratch, grown on demand (the kernels write every word before they read it).
-    Ops that share it must not run concurrently on different streams."""
+    """Scratch per device and stream, grown on demand (the kernels write every word before they read it)."""
     return _grown(_workspaces, device, nbytes, 8 << 20)
 
 
@@ -114,8 +115,8 @@ _topk_workspaces: dict = {}
 
 
 def _topk_workspace(device: torch.device) -> torch.Tensor:
-    """Histogram scratch per device.  Top-k calls that share it must not overlap."""
-    key = (device.type, device.index)
+    """Histogram scratch per device and stream.  Top-k calls that share it must not overlap."""
+    key = (device.type, device.index, torch.cuda.current_stream(device).cuda_stream)
     ws = _topk_workspaces.get(key)
     if ws is None:
         ws = torch.empty(lib.dv_topk_workspace_bytes(65536) // 4, dtype=torch.int32, device=device)

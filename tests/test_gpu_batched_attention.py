@@ -245,3 +245,51 @@ def test_batched_sparse_block_decode_step_matches_oracle(cfg, B):
         vcd[b, sel, t] = v0[b, sel, t]
         kcd[b, sel, :, t] = k0[b, sel, :, t]
     assert torch.equal(vcd, v0) and torch.equal(kcd, k0), "cache entries other than the appended rows changed"
+
+
+def test_batched_block_step_same_bits_with_and_without_the_side_stream():
+    """From two sequences on, the predictors and top-ks of a layer step run on the modules' side stream
+    (their scratch buffers are per stream); the results must not depend on it."""
+    import copy
+
+    import dejavu_amd.modules as M
+    from dejavu_amd.block import create_sparse_block, init_block_synthetic
+    from dejavu_amd.modules import InferenceParams
+    from dejavu_amd.workloads import pack_k_cache
+
+    B, d, ffn, H, r, K, Hk, S = 12, 1024, 4096, 8, 1000, 512, 3, 64
+    hd = d // H
+    blk = create_sparse_block(d, ffn, H, r, K, r, Hk, layer_idx=0)
+    init_block_synthetic(blk, seed=7)
+    g = torch.Generator().manual_seed(77)
+    kc = pack_k_cache(torch.randn(B, H, S, hd, generator=g).half())
+    vc = torch.randn(B, H, S, hd, generator=g).half()
+    assert M.SIDE_STREAM_MIN_BATCH == 2
+    results = []
+    try:
+        for min_batch in (2, None):
+            M.SIDE_STREAM_MIN_BATCH = min_batch
+            b = copy.deepcopy(blk)
+            ip = InferenceParams(max_sequence_len=S, max_batch_size=B, sequence_len_offset=40)
+            ip.key_value_memory_dict[0] = (kc.clone().cuda(), vc.clone().cuda())
+            gg = torch.Generator().manual_seed(78)
+            outs = []
+            for step in range(3):
+                hs = torch.randn(B, 1, d, generator=gg).half().cuda()
+                res = torch.randn(B, 1, d, generator=gg).half().cuda()
+                head_idx = torch.sort(torch.randperm(H, generator=gg)[:Hk]).values.int().cuda()
+                logit = (torch.randn(B, ffn, generator=gg) * 4).half().cuda()
+                print(f"case batched block, side stream from batch {min_batch}, step {step}", flush=True)
+                with torch.no_grad():
+                    outs.append(b(hs, res, mixer_kwargs={"inference_params": ip}, head_idx=head_idx, mlp_sp_logit=logit))
+                M.join_side_stream()
+                torch.cuda.synchronize()
+                ip.sequence_len_offset += 1
+            results.append((outs, ip.key_value_memory_dict[0]))
+    finally:
+        M.SIDE_STREAM_MIN_BATCH = 2
+    for oa, ob in zip(results[0][0], results[1][0]):
+        for xa, xb in zip(oa, ob):
+            assert torch.equal(xa, xb)
+    for ca, cb in zip(results[0][1], results[1][1]):
+        assert torch.equal(ca, cb)
