@@ -36,6 +36,23 @@ def _idx_bytes(idx: torch.Tensor) -> int:
     return 4 if idx.dtype == torch.int32 else 8
 
 
+def _expect(ok: bool, what: str) -> None:
+    """Precondition failures are ``AssertionError``s, as in the reference's wrappers."""
+    if not ok:
+        raise AssertionError(what)
+
+
+def _same_f16(name_a: str, a: torch.Tensor, name_b: str, b: Optional[torch.Tensor]) -> None:
+    if b is not None:
+        _expect(a.dtype == b.dtype, f"{name_a} is {a.dtype} but {name_b} is {b.dtype}: they must agree")
+    _expect(a.dtype == torch.float16, f"{name_a} is {a.dtype}: the kernels are fp16 only")
+
+
+def _int32_vector(name: str, t: torch.Tensor, n: int) -> None:
+    _expect(t.dtype == torch.int32 and tuple(t.shape) == (n,), f"{name} must be an int32 vector of {n} entries, "
+            f"got {t.dtype} {tuple(t.shape)}")
+
+
 def _require_device(*tensors: Optional[torch.Tensor]) -> None:
     for t in tensors:
         if t is not None and not t.is_cuda:
@@ -178,30 +195,35 @@ def greedy_advance(logits: torch.Tensor, token: torch.Tensor, position: torch.Te
 # ---------------------------------------------------------------------------
 def gather_gemv(x: torch.Tensor, weight: torch.Tensor, idx: Optional[torch.Tensor],
                 bias: Optional[torch.Tensor] = None, activation: str = "id") -> torch.Tensor:
-    """Compute y = activation(x @ weight[idx, :].T + bias[idx]).
+    """Rows ``idx`` of ``weight`` applied to every row of ``x``:
+    ``y[b, m] = activation(weight[idx[m]] . x[b] + bias[idx[m]])`` (the fc1 of the sparse MLP;
+    interface of gather_gemv.py:198-261).
 
-    x: (batch, N); weight: (Z, N); idx: (M,); bias: (Z,) -> (batch, M).
-    idx=None: every row (a dense product, M = Z).
+    Shapes: x (batch, N), weight (Z, N), idx (M,) int32 / int64, bias (Z,); returns (batch, M).
+    ``idx=None`` takes all Z rows in order (a dense product).  batch may go up to 64 (the
+    reference's kernel stops at 4; from 3 rows on the product runs on the matrix cores).
     """
-    assert activation in ["id", "relu", "gelu", "gelu_approx", "squared_relu"]
+    _expect(activation in ("id", "relu", "gelu", "gelu_approx", "squared_relu"), f"unknown activation {activation!r}")
     if activation not in _ACT:
         raise NotImplementedError(f"activation {activation!r}: the OPT decode path uses 'relu' / 'id' only")
     _require_device(x, weight, idx, bias)
-    Z, N = weight.shape
-    batch, _ = x.shape
-    assert x.shape == (batch, N)
-    assert 1 <= batch <= 64  # the reference stops at 4; larger batches run on the matrix cores
-    M = Z if idx is None else idx.shape[0]
-    x = x.contiguous()
-    if weight.stride(1) > 1:
-        weight = weight.contiguous()
-    assert x.dtype == weight.dtype, f"Input and weight must have the same dtype, got {x.dtype} and {weight.dtype}"
-    assert x.dtype == torch.float16, "kernels are built for fp16"
+    _expect(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
+            f"x {tuple(x.shape)} and weight {tuple(weight.shape)} must share their last dimension")
+    batch, N = x.shape
+    Z = weight.shape[0]
+    _expect(1 <= batch <= 64, f"batch {batch} outside 1..64")
+    _same_f16("x", x, "weight", weight)
     if bias is not None:
+        _expect(tuple(bias.shape) == (Z,), f"bias {tuple(bias.shape)} does not match the {Z} weight rows")
+        _same_f16("x", x, "bias", bias)
         bias = bias.contiguous()
-        assert bias.shape == (Z,), "Incompatible dimensions in between weight and bias"
-        assert x.dtype == bias.dtype, f"Input and bias must have the same dtype, got {x.dtype} and {bias.dtype}"
-    idx = None if idx is None else idx.contiguous()
+    x = x.contiguous()
+    if weight.stride(1) != 1:
+        weight = weight.contiguous()
+    M = Z
+    if idx is not None:
+        idx = idx.contiguous()
+        M = idx.shape[0]
     output = torch.empty(batch, M, device=x.device, dtype=x.dtype)
     nbytes = lib.dv_gather_gemv_workspace_bytes(batch, N, M)  # 0 below 17 rows
     ws = _workspace(x.device, nbytes) if nbytes else None
@@ -256,25 +278,27 @@ def dense_decode_linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[to
 
 def gather_transposed_gemv(x: torch.Tensor, weight: torch.Tensor, idx: torch.Tensor,
                            bias: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Compute y = weight[idx, :]^T @ x + bias.
+    """Gathered rows of ``weight`` combined with the coefficients in ``x``:
+    ``y[b, :] = sum_m x[b, m] * weight[idx[m], :] + bias`` (the fc2 of the sparse MLP over the
+    transposed weight; interface of gather_gemv.py:572-636).
 
-    x: (batch, M); weight: (Z, N); idx: (M,); bias: (N,) -> (batch, N).
+    Shapes: x (batch, M), weight (Z, N), idx (M,), bias (N,); returns (batch, N); batch 1..64.
+    The split reduction has a fixed order: the result does not change from run to run.
     """
     _require_device(x, weight, idx, bias)
+    _expect(x.dim() == 2 and weight.dim() == 2 and idx.dim() == 1 and x.shape[1] == idx.shape[0],
+            f"x {tuple(x.shape)} needs one column per entry of idx {tuple(idx.shape)}")
+    batch, M = x.shape
     Z, N = weight.shape
-    (M,) = idx.shape
-    batch, _ = x.shape
-    assert x.shape == (batch, M)
-    assert 1 <= batch <= 64  # the reference stops at 4; larger batches run on the matrix cores
-    x = x.contiguous()
-    if weight.stride(1) > 1:
-        weight = weight.contiguous()
-    assert x.dtype == weight.dtype, f"Input and weight must have the same dtype, got {x.dtype} and {weight.dtype}"
-    assert x.dtype == torch.float16, "kernels are built for fp16"
+    _expect(1 <= batch <= 64, f"batch {batch} outside 1..64")
+    _same_f16("x", x, "weight", weight)
     if bias is not None:
+        _expect(tuple(bias.shape) == (N,), f"bias {tuple(bias.shape)} does not match the {N} output columns")
+        _same_f16("x", x, "bias", bias)
         bias = bias.contiguous()
-        assert bias.shape == (N,), "Incompatible dimensions in between weight and bias"
-        assert x.dtype == bias.dtype, f"Input and bias must have the same dtype, got {x.dtype} and {bias.dtype}"
+    x = x.contiguous()
+    if weight.stride(1) != 1:
+        weight = weight.contiguous()
     idx = idx.contiguous()
     output = torch.empty(batch, N, device=x.device, dtype=x.dtype)
     nbytes = lib.dv_gather_transposed_gemv_workspace_bytes(batch, N, M)
@@ -286,16 +310,11 @@ def gather_transposed_gemv(x: torch.Tensor, weight: torch.Tensor, idx: torch.Ten
 
 
 def mlp_sparse(x, W1, W2t, idx, bias1=None, bias2=None):
-    """
-    x: (batch, d)
-    W1: (4d, d)
-    W2t: (4d, d). This is the transpose of W2, contiguous so that gathered rows stream.
-    bias1: (4d)
-    bias2: (d)
-    """
-    x = gather_gemv(x, W1, idx, bias1, activation="relu")
-    x = gather_transposed_gemv(x, W2t, idx, bias2)
-    return x
+    """The sparse MLP on the neurons ``idx``: ReLU(fc1) then fc2, two gathered products
+    (gather_gemv.py:647-657).  x (batch, d); W1 and W2t both (ffn, d), W2t being fc2.weight
+    transposed so that a neuron's fc2 column is a contiguous row; bias1 (ffn,), bias2 (d,)."""
+    hidden = gather_gemv(x, W1, idx, bias1, activation="relu")
+    return gather_transposed_gemv(hidden, W2t, idx, bias2)
 
 
 # ---------------------------------------------------------------------------
@@ -305,44 +324,38 @@ def qkv_proj_sparse(x: torch.Tensor, weight: torch.Tensor, head_idx: torch.Tenso
                     bias: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
                     k_cache: Optional[torch.Tensor] = None, v_cache: Optional[torch.Tensor] = None,
                     padding: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """
-    Compute y = torch.einsum("bm,thdm->bthd", x, weight), but only for the active heads in @head_idx
-    and only for the batch indices in @batch_idx. Negative indices in batch_idx will be ignored.
-    :param x: input tensor, (batch_size, hidden_dim)
-    :param weight: weight matrix, (3, nheads, head_dim, hidden_dim)
-    :param head_idx: int32, (nnz,)
-    :param batch_idx: int32, (nnz, batch_size). Negative indices are ignored.
-    :param bias: indices, (3, nheads, head_dim)
-    :param k_cache, v_cache, padding: optional; when given, the computed K / V rows are also scattered
-        into the caches exactly as ``k_cache_copy_sparse`` / ``v_cache_copy_sparse`` would with
-        ``seqlen_idx = batch_idx`` (one launch instead of three)
-    :return: result tensor, (batch_size, 3, nheads, head_dim); entries of inactive heads /
-        skipped rows are uninitialised (or keep the content of ``out`` when it is given)
+    """Head-sparse QKV projection of up to 16 window tokens (interface of
+    attention_proj_sparse.py:110-190): for every listed head ``h = head_idx[i]`` and every row
+    ``r = batch_idx[i, s] >= 0`` the three vectors ``y[r, t, h, :] = weight[t, h] @ x[r] + bias[t, h]``
+    (t = q, k, v) are written; negative entries of ``batch_idx`` skip that (head, row) pair.
+
+    Shapes: x (rows, hidden), rows <= 16; weight (3, nheads, head_dim, hidden); head_idx (nnz,)
+    int32; batch_idx (nnz, rows) int32; bias (3, nheads, head_dim).  Returns (rows, 3, nheads,
+    head_dim); what is not written is uninitialised memory, or keeps the content of ``out``.
+
+    With ``k_cache`` / ``v_cache`` (and the int32 ``padding`` offset) the same launch also stores
+    the new K / V rows at cache position ``r + padding[0]``, which is what the two cache-copy ops
+    would do with ``seqlen_idx = batch_idx``.
     """
     _require_device(x, weight, head_idx, batch_idx, bias)
-    three, nheads, head_dim, hidden_dim = weight.shape
-    assert three == 3
-    assert head_dim in [32, 64, 128]
-    assert hidden_dim % 128 == 0
-    batch_size, _ = x.shape
-    assert batch_size <= 16
-    assert x.shape == (batch_size, hidden_dim)
+    _expect(weight.dim() == 4 and weight.shape[0] == 3, f"weight {tuple(weight.shape)} is not (3, nheads, head_dim, hidden)")
+    _, nheads, head_dim, hidden_dim = weight.shape
+    _expect(head_dim in (32, 64, 128), f"head_dim {head_dim} not in 32 / 64 / 128")
+    _expect(hidden_dim % 128 == 0, f"hidden size {hidden_dim} is not a multiple of 128")
+    batch_size = x.shape[0]
+    _expect(tuple(x.shape) == (batch_size, hidden_dim) and batch_size <= 16,
+            f"x {tuple(x.shape)} must be (rows <= 16, {hidden_dim})")
     n_active = head_idx.shape[0]
-    assert n_active <= nheads
-    assert head_idx.shape == (n_active,)
-    assert head_idx.dtype == torch.int32
-    assert batch_idx.shape == (n_active, batch_size)
-    assert batch_idx.dtype == torch.int32
-    x = x.contiguous()
-    weight = weight.contiguous()
-    head_idx = head_idx.contiguous()
-    batch_idx = batch_idx.contiguous()
-    assert x.dtype == weight.dtype, f"Input and weight must have the same dtype, got {x.dtype} and {weight.dtype}"
-    assert x.dtype == torch.float16, "kernels are built for fp16"
+    _expect(n_active <= nheads, f"{n_active} heads listed, the layer has {nheads}")
+    _int32_vector("head_idx", head_idx, n_active)
+    _expect(batch_idx.dtype == torch.int32 and tuple(batch_idx.shape) == (n_active, batch_size),
+            f"batch_idx must be int32 ({n_active}, {batch_size}), got {batch_idx.dtype} {tuple(batch_idx.shape)}")
+    _same_f16("x", x, "weight", weight)
     if bias is not None:
+        _expect(tuple(bias.shape) == (3, nheads, head_dim), f"bias {tuple(bias.shape)} is not (3, {nheads}, {head_dim})")
+        _same_f16("x", x, "bias", bias)
         bias = bias.contiguous()
-        assert bias.shape == (3, nheads, head_dim), "Incompatible dimensions in between weight and bias"
-        assert x.dtype == bias.dtype, f"Input and bias must have the same dtype, got {x.dtype} and {bias.dtype}"
+    x, weight, head_idx, batch_idx = x.contiguous(), weight.contiguous(), head_idx.contiguous(), batch_idx.contiguous()
     if out is None:
         out = torch.empty(batch_size, 3, nheads, head_dim, device=x.device, dtype=x.dtype)
     else:
@@ -422,33 +435,30 @@ def qkv_proj_batch(x: torch.Tensor, weight: torch.Tensor, head_idx: torch.Tensor
 
 def out_proj_sparse(x: torch.Tensor, weight: torch.Tensor, head_idx: torch.Tensor,
                     bias: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """
-    Compute y = torch.einsum("bhd,nhd->bn", x, weight), but only for the active heads in @head_idx.
-    :param x: input tensor, (batch, nheads, head_dim)
-    :param weight: weight matrix, (hidden_dim, nheads, head_dim)
-    :param head_idx: int32, (nnz,)
-    :param bias: indices, (hidden_dim)
-    :return: result tensor, (batch, hidden_dim)
+    """Output projection over the listed heads only (interface of attention_proj_sparse.py:274-335):
+    ``y[b, n] = sum_{h in head_idx} weight[n, h, :] . x[b, h, :] + bias[n]``; the context of every
+    other head is never read.
+
+    Shapes: x (batch <= 16, nheads, head_dim); weight (hidden, nheads, head_dim), the reference's
+    layout; head_idx (nnz,) int32; bias (hidden,).  Returns (batch, hidden).  ``out_proj_sparse_t``
+    gives the same result from the transposed weight in one pass per batch.
     """
     _require_device(x, weight, head_idx, bias)
+    _expect(weight.dim() == 3 and x.dim() == 3, "x must be (batch, nheads, head_dim), weight (hidden, nheads, head_dim)")
     hidden_dim, nheads, head_dim = weight.shape
-    assert head_dim in [32, 64, 128]
-    assert hidden_dim % 128 == 0
-    batch, _, _ = x.shape
-    assert x.shape == (batch, nheads, head_dim)
+    _expect(head_dim in (32, 64, 128), f"head_dim {head_dim} not in 32 / 64 / 128")
+    _expect(hidden_dim % 128 == 0, f"hidden size {hidden_dim} is not a multiple of 128")
+    batch = x.shape[0]
+    _expect(tuple(x.shape) == (batch, nheads, head_dim) and batch <= 16,
+            f"x {tuple(x.shape)} must be (batch <= 16, {nheads}, {head_dim})")
     n_active = head_idx.shape[0]
-    assert head_idx.shape == (n_active,)
-    assert head_idx.dtype == torch.int32
-    assert batch <= 16
-    x = x.contiguous()
-    weight = weight.contiguous()
-    assert x.dtype == weight.dtype, f"Input and weight must have the same dtype, got {x.dtype} and {weight.dtype}"
-    assert x.dtype == torch.float16, "kernels are built for fp16"
+    _int32_vector("head_idx", head_idx, n_active)
+    _same_f16("x", x, "weight", weight)
     if bias is not None:
+        _expect(tuple(bias.shape) == (hidden_dim,), f"bias {tuple(bias.shape)} does not match hidden size {hidden_dim}")
+        _same_f16("x", x, "bias", bias)
         bias = bias.contiguous()
-        assert bias.shape == (hidden_dim,), "Incompatible dimensions in between weight and bias"
-        assert x.dtype == bias.dtype, f"Input and bias must have the same dtype, got {x.dtype} and {bias.dtype}"
-    head_idx = head_idx.contiguous()
+    x, weight, head_idx = x.contiguous(), weight.contiguous(), head_idx.contiguous()
     output = torch.empty(batch, hidden_dim, device=x.device, dtype=x.dtype)
     check(lib.dv_out_proj_sparse_f16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(head_idx), n_active, batch, nheads,
                                      head_dim, hidden_dim, _ptr(output), _stream()), "dv_out_proj_sparse_f16")
@@ -490,35 +500,32 @@ def out_proj_sparse_t(x: torch.Tensor, weight_t: torch.Tensor, head_idx: torch.T
 def _cache_copy(k, v, k_cache, v_cache, head_idx, seqlen_idx, padding):
     src = k if k is not None else v
     _require_device(src, k_cache, v_cache, head_idx, seqlen_idx, padding)
+    _expect(src.dim() == 3, "k / v must be (tokens, nheads, head_dim)")
     nnz_seqlen, nheads, head_dim = src.shape
-    assert head_dim in [32, 64, 128]
-    assert nnz_seqlen <= 16
+    _expect(head_dim in (32, 64, 128), f"head_dim {head_dim} not in 32 / 64 / 128")
+    _expect(nnz_seqlen <= 16, f"{nnz_seqlen} tokens: a back-fill window holds at most 16")
+    _expect(src.stride(2) == 1 and src.stride(1) == head_dim, "the heads of a k / v row must be contiguous")
     n_active = head_idx.shape[0]
-    assert n_active <= nheads
-    assert head_idx.shape == (n_active,)
-    assert head_idx.dtype == torch.int32
-    assert seqlen_idx.shape == (n_active, nnz_seqlen)
-    assert seqlen_idx.dtype == torch.int32
-    assert src.stride(2) == 1 and src.stride(1) == head_dim, "k / v must be (n, nheads, head_dim) with contiguous heads"
-    head_idx = head_idx.contiguous()
-    seqlen_idx = seqlen_idx.contiguous()
+    _expect(n_active <= nheads, f"{n_active} heads listed, the layer has {nheads}")
+    _int32_vector("head_idx", head_idx, n_active)
+    _expect(seqlen_idx.dtype == torch.int32 and tuple(seqlen_idx.shape) == (n_active, nnz_seqlen),
+            f"seqlen_idx must be int32 ({n_active}, {nnz_seqlen}), got {seqlen_idx.dtype} {tuple(seqlen_idx.shape)}")
     if padding is not None:
-        assert padding.shape == (1,)
-        assert padding.dtype == torch.int32
+        _int32_vector("padding", padding, 1)
+    head_idx, seqlen_idx = head_idx.contiguous(), seqlen_idx.contiguous()
+    seqlen = 0
     if k_cache is not None:
-        packsize = 8
-        assert k.dtype == torch.float16, "kernels are built for fp16"
-        _, _, _, seqlen, _ = k_cache.shape
-        assert k_cache.shape == (1, nheads, head_dim // packsize, seqlen, packsize)
-        assert k_cache.is_contiguous()
-        assert k.dtype == k_cache.dtype, f"k and k_cache must have the same dtype, got {k.dtype} and {k_cache.dtype}"
+        _same_f16("k", k, "k_cache", k_cache)
+        seqlen = k_cache.shape[3]
+        _expect(tuple(k_cache.shape) == (1, nheads, head_dim // 8, seqlen, 8) and k_cache.is_contiguous(),
+                f"k_cache {tuple(k_cache.shape)} is not a contiguous (1, {nheads}, {head_dim // 8}, S, 8) tensor")
     if v_cache is not None:
-        _, _, seqlen, _ = v_cache.shape
-        assert v_cache.shape == (1, nheads, seqlen, head_dim)
-        assert v_cache.is_contiguous()
-        assert v.dtype == v_cache.dtype, f"v and v_cache must have the same dtype, got {v.dtype} and {v_cache.dtype}"
+        _same_f16("v", v, "v_cache", v_cache)
+        seqlen = v_cache.shape[2]
+        _expect(tuple(v_cache.shape) == (1, nheads, seqlen, head_dim) and v_cache.is_contiguous(),
+                f"v_cache {tuple(v_cache.shape)} is not a contiguous (1, {nheads}, S, {head_dim}) tensor")
     if k is not None and v is not None:
-        assert k.stride(0) == v.stride(0)
+        _expect(k.stride(0) == v.stride(0), "k and v must have the same row stride")
     check(lib.dv_kv_cache_copy_sparse_f16(_ptr(k), _ptr(v), src.stride(0), nnz_seqlen, _ptr(k_cache), _ptr(v_cache),
                                           _ptr(head_idx), _ptr(seqlen_idx), n_active, nnz_seqlen, _ptr(padding),
                                           nheads, head_dim, seqlen, _stream()), "dv_kv_cache_copy_sparse_f16")
@@ -526,25 +533,18 @@ def _cache_copy(k, v, k_cache, v_cache, head_idx, seqlen_idx, padding):
 
 def k_cache_copy_sparse(k: torch.Tensor, k_cache: torch.Tensor, head_idx: torch.Tensor, seqlen_idx: torch.Tensor,
                         padding: torch.Tensor = None) -> None:
-    """
-    :param k: input tensor, (nnz_seqlen, nheads, head_dim)
-    :param k_cache: input tensor, (1, nheads, headdim / PACKSIZE, seqlen, PACKSIZE), PACKSIZE = 8 (fp16)
-    :param head_idx: int32, (nnz,)
-    :param seqlen_idx: int32, (nnz, nnz_seqlen). Negative indices are ignored.
-    :param padding: int32, (1). Padding is added to indices in seqlen_idx before writing to k_cache
-    """
+    """Stores window tokens' K rows of the listed heads into the packed key cache (interface of
+    attention_proj_sparse.py:525-590): for ``h = head_idx[i]`` and ``s = seqlen_idx[i, j] >= 0``,
+    ``k_cache[0, h, c // 8, s + padding[0], c % 8] = k[s, h, c]``.  k (tokens <= 16, nheads,
+    head_dim); k_cache (1, nheads, head_dim / 8, S, 8); head_idx (nnz,), seqlen_idx (nnz, tokens)
+    and padding (1,) int32."""
     _cache_copy(k, None, k_cache, None, head_idx, seqlen_idx, padding)
 
 
 def v_cache_copy_sparse(v: torch.Tensor, v_cache: torch.Tensor, head_idx: torch.Tensor, seqlen_idx: torch.Tensor,
                         padding: torch.Tensor = None) -> None:
-    """
-    :param v: input tensor, (nnz_seqlen, nheads, head_dim)
-    :param v_cache: input tensor, (1, nheads, seqlen, head_dim)
-    :param head_idx: int32, (nnz,)
-    :param seqlen_idx: int32, (nnz, nnz_seqlen). Negative indices are ignored.
-    :param padding: int32, (1). Padding is added to indices in seqlen_idx before writing to v_cache
-    """
+    """The value-cache counterpart of ``k_cache_copy_sparse`` (attention_proj_sparse.py:396-459):
+    ``v_cache[0, h, s + padding[0], :] = v[s, h, :]``; v_cache is (1, nheads, S, head_dim)."""
     _cache_copy(None, v, None, v_cache, head_idx, seqlen_idx, padding)
 
 
