@@ -10,6 +10,7 @@
 
 #include "attention.hpp"
 #include "common.hpp"
+#include "gemm_cols16.hpp"
 #include "gemm_mfma.hpp"
 #include "gemm_tiled.hpp"
 #include "gemv_cols.hpp"
@@ -573,9 +574,50 @@ ColsMfmaPlan plan_cols_mfma(int B, int N, int M) {
   return p;
 }
 
+// plan of gather_cols_mfma16_kernel (batch <= 32): 128 columns per workgroup of 4 wavefronts whose shares
+// are whole double steps (64 rows).  One batch tile: about three workgroups per compute unit (fc2 at the
+// OPT-175B shape, batch 8: 22.7 us with 8 row groups, 24.4 with 4, 24.2 with 2; the 32x32x16 kernel: 26.7);
+// two batch tiles write twice the partial sums per group: about one workgroup per compute unit
+// (batch 32: 30.6 us with 2 groups, 32.3 with 4, 33.0 with 8; the 32x32x16 kernel: 32.2).
+struct Cols16Plan {
+  int col_tiles, groups, rows_per_block, rows_per_wave;
+};
+constexpr int kC16Waves = 4;
+
+Cols16Plan plan_cols16(int B, int N, int M) {
+  Cols16Plan p;
+  p.col_tiles = (N + kC16Cols - 1) / kC16Cols;
+  int groups = (B <= 16 ? 3 : 1) * compute_units() / p.col_tiles;
+  if (groups < 1) groups = 1;
+  const int unit = kC16Waves * 2 * kC16Step;
+  int rpb = ((M + groups - 1) / groups + unit - 1) / unit * unit;
+  if (rpb > kC16Waves * kC16MaxRows) rpb = kC16Waves * kC16MaxRows;
+  if (rpb < unit) rpb = unit;
+  p.rows_per_block = rpb;
+  p.rows_per_wave = rpb / kC16Waves;
+  p.groups = M > 0 ? (M + rpb - 1) / rpb : 1;
+  return p;
+}
+
 size_t cols_mfma_workspace_bytes(int B, int N, int M) {
   const ColsMfmaPlan p = plan_cols_mfma(B, N, M);
-  return (size_t)p.groups * B * N * sizeof(float);
+  const Cols16Plan q = plan_cols16(B, N, M);
+  const int groups = p.groups > q.groups ? p.groups : q.groups;
+  return (size_t)groups * B * N * sizeof(float);
+}
+
+template <int BT, bool IDX64, bool BLOCKED>
+void launch_cols16(const Cols16Plan& p, const half_t* h, int64_t ldh, int x_expanded, const half_t* W, int64_t ldw,
+                   const half_t* bias, const void* idx, int blk, int B, int N, int Z, int M, float* partial,
+                   half_t* y, hipStream_t s) {
+  hipLaunchKernelGGL((gather_cols_mfma16_kernel<BT, kC16Waves, IDX64, BLOCKED>), dim3(p.col_tiles, p.groups),
+                     dim3(kC16Waves * 64), 0, s, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M,
+                     p.rows_per_block, p.rows_per_wave, partial, y);
+  if (p.groups > 1) {
+    const int64_t total = (int64_t)B * N;
+    hipLaunchKernelGGL(cols_reduce_kernel, dim3((unsigned)((total + 63) / 64)), dim3(256), 0, s, partial,
+                       bias, p.groups, B, N, y);
+  }
 }
 
 template <int BT, bool IDX64, bool BLOCKED, bool HVEC>
@@ -599,6 +641,25 @@ int gather_cols_mfma(const half_t* h, int64_t ldh, int x_expanded, const half_t*
   float* partial = reinterpret_cast<float*>(workspace);
   const bool i64 = idx_bytes == 8, blocked = blk != 1;
   const bool hvec = M % 8 == 0 && ldh % 8 == 0 && aligned16(h) && (!x_expanded || blk % 8 == 0);
+  // up to 32 rows: the 16x16x32 kernel (it needs vector loads of H and, for a blocked row map, blocks
+  // that are multiples of 8 rows)
+  if (B <= 32 && hvec && M >= 8 && (blocked ? blk % 8 == 0 : !x_expanded)) {
+    const Cols16Plan q = plan_cols16(B, N, M);
+#define DV_C16(BT)                                                                                                   \
+  do {                                                                                                               \
+    if (blocked) {                                                                                                   \
+      if (i64) launch_cols16<BT, true, true>(q, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M, partial, y, s);  \
+      else launch_cols16<BT, false, true>(q, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M, partial, y, s);     \
+    } else {                                                                                                         \
+      if (i64) launch_cols16<BT, true, false>(q, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M, partial, y, s); \
+      else launch_cols16<BT, false, false>(q, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M, partial, y, s);    \
+    }                                                                                                                \
+  } while (0)
+    if (B <= 16) DV_C16(1);
+    else DV_C16(2);
+#undef DV_C16
+    return launch_status();
+  }
 #define DV_ARGS p, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M, partial, y, s
 #define DV_CM3(BT, I64, BLK)                                   \
   do {                                                         \
