@@ -591,6 +591,43 @@ def mlp_bench(args):
         "batches": results}))
 
 
+def other_workloads():
+    """Runs `bench.py --batch 8 / 16 / 32` and `bench.py --workload decode` as child processes (one at a
+    time, each bounded) and returns the figures of their JSON lines; a leg that fails is reported as
+    such and never fails the headline run."""
+    import subprocess
+
+    def child(argv, limit):
+        cmd = [sys.executable, os.path.abspath(__file__), *argv, "--no-cpu-baseline"]
+        t0 = time.perf_counter()
+        try:
+            r = subprocess.run(cmd, capture_output=True, text=True, timeout=limit)
+            lines = [ln for ln in r.stdout.strip().splitlines() if ln.startswith("{")]
+            if r.returncode != 0 or not lines:
+                return {"error": f"exit {r.returncode}: {r.stderr.strip()[-200:]}"}, time.perf_counter() - t0
+            return json.loads(lines[-1]), time.perf_counter() - t0
+        except subprocess.TimeoutExpired:
+            return {"error": f"no result within {limit} s"}, time.perf_counter() - t0
+
+    out = {"batched_layer": {}, "how": "child processes of this script, run before the headline measurement"}
+    for b in (8, 16, 32):
+        d, secs = child(["--batch", str(b), "--steps", "96", "--warmup", "24"], 300)
+        if "error" in d:
+            out["batched_layer"][str(b)] = d
+        else:
+            out["batched_layer"][str(b)] = dict(d["layer"], wall_s=round(secs, 1), steps=d["steps"],
+                                                workload=d["config"]["workload"])
+    d, secs = child(["--workload", "decode"], 420)
+    if "error" in d:
+        out["decode"] = d
+    else:
+        out["decode"] = {"metric": d["metric"], "tokens_per_s": d["value"], "ms_per_token": d["ms_per_step"],
+                         "us_per_layer": d["us_per_layer"], "prompt_ms": d["prompt_ms"],
+                         "frac_of_hbm_peak": d["frac_of_hbm_peak"], "graph_equals_eager": d["graph_equals_eager"],
+                         "new_tokens": d["steps"], "wall_s": round(secs, 1)}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -616,6 +653,8 @@ def main():
                     help="layer: the headline sparse decode layer; decode: end-to-end greedy generation "
                          "(40-layer OPT-13B shape, --steps = new tokens, default 256)")
     ap.add_argument("--decode-layers", type=int, default=40)
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="default run only: skip the batched-layer (batch 8 / 16 / 32) and greedy-decode legs")
     ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"), default=None,
                     help="no GPU work: read the counter CSVs of two `rocprofv3 --pmc` runs of `bench.py "
                          "--pmc-calibration` (FETCH_SIZE, then WRITE_SIZE) and write profiles/traffic.json")
@@ -626,6 +665,14 @@ def main():
         sys.exit(2)
     if args.traffic_from:
         return write_traffic(*args.traffic_from)
+
+    # The headline run also reports the other BASELINE workloads (batched layer, end-to-end decode), each
+    # measured by a child process of this script that runs BEFORE this process touches the GPU
+    # (a child started later would be forked from a process that holds the device).
+    others = None
+    if (args.workload == "layer" and args.batch == 1 and args.config == "opt-175b" and not args.no_other_workloads
+            and not args.pmc_calibration and not args.no_graph and args.window == "cycle"):
+        others = other_workloads()
 
     import torch
 
@@ -877,6 +924,8 @@ def main():
         "spread": spread,
         "kernels": table,
     }
+    if others is not None:
+        out["other_workloads"] = others
     print(json.dumps(out))
 
 

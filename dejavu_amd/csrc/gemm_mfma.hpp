@@ -1,8 +1,8 @@
 // Batched (5 <= B <= 64) gathered GEMMs on the matrix cores.  The gathered weight
 // rows are streamed with coalesced 128-bit loads into LDS and read back in MFMA
 // operand layout.  fc1 (rows kernel) uses v_mfma_f32_16x16x32_f16 with the batch
-// padded to tiles of 16; fc2 (columns kernel) uses v_mfma_f32_32x32x16_f16 with
-// the batch padded to tiles of 32.
+// padded to tiles of 16; fc2 (columns kernel, here for 33..64 rows; up to 32 rows
+// gemm_cols16.hpp) uses v_mfma_f32_32x32x16_f16 with the batch padded to tiles of 32.
 //
 // Operand layout of the 32x32x16 fp16 MFMA (64 lanes): lane l holds, for the A
 // operand, 8 consecutive-k values of row (l % 32), k-group (l / 32); for the B
