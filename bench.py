@@ -591,6 +591,20 @@ def mlp_bench(args):
         "batches": results}))
 
 
+def holds_gpu():
+    """True when this process already has the GPU's device node open (the compute driver's /dev/kfd)."""
+    try:
+        for fd in os.listdir("/proc/self/fd"):
+            try:
+                if os.readlink(f"/proc/self/fd/{fd}") == "/dev/kfd":
+                    return True
+            except OSError:
+                pass
+    except OSError:
+        pass
+    return False
+
+
 def other_workloads():
     """Runs `bench.py --batch 8 / 16 / 32` and `bench.py --workload decode` as child processes (one at a
     time, each bounded) and returns the figures of their JSON lines; a leg that fails is reported as
@@ -672,7 +686,11 @@ def main():
     others = None
     if (args.workload == "layer" and args.batch == 1 and args.config == "opt-175b" and not args.no_other_workloads
             and not args.pmc_calibration and not args.no_graph and args.window == "cycle"):
-        others = other_workloads()
+        if holds_gpu():  # e.g. under a profiler whose preloaded library opened the device: start no child
+            others = {"skipped": "this process held the GPU before the measurement started; run the legs with "
+                                 "--batch 8 / 16 / 32 and --workload decode"}
+        else:
+            others = other_workloads()
 
     import torch
 
