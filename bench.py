@@ -647,9 +647,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None, help="default 960 (20 windows of 3 layers x 16 positions)")
     ap.add_argument("--warmup", type=int, default=None, help="default 192")
-    ap.add_argument("--window", default="cycle", choices=["cycle", "start"],
-                    help="cycle: steps walk through whole 16-token back-fill windows; "
-                         "start: only the first position of a window (no back-fill)")
+    ap.add_argument("--window", default=None, choices=["cycle", "start"],
+                    help="cycle: steps walk through whole 16-token back-fill windows (default at batch 1); "
+                         "start: only the first position of a window, no back-fill (default at batch > 1)")
     ap.add_argument("--config", default="opt-175b")
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -685,7 +685,7 @@ def main():
     # (a child started later would be forked from a process that holds the device).
     others = None
     if (args.workload == "layer" and args.batch == 1 and args.config == "opt-175b" and not args.no_other_workloads
-            and not args.pmc_calibration and not args.no_graph and args.window == "cycle"):
+            and not args.pmc_calibration and not args.no_graph and args.window in (None, "cycle")):
         if holds_gpu():  # e.g. under a profiler whose preloaded library opened the device: start no child
             others = {"skipped": "this process held the GPU before the measurement started; run the legs with "
                                  "--batch 8 / 16 / 32 and --workload decode"}
@@ -719,8 +719,8 @@ def main():
     if not 1 <= batch <= 32:
         print("bench.py: --batch must be in 1..32", file=sys.stderr)
         sys.exit(2)
-    if batch > 1:
-        args.window = "start"  # B sequences in lockstep: every step at the first position of a window
+    if args.window is None:
+        args.window = "cycle" if batch == 1 else "start"
     device = torch.device("cuda:0")
     layers = build_layers(cfg, batch, device)
     cycle = args.window == "cycle"

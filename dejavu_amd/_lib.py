@@ -77,6 +77,11 @@ SIGNATURES = {
         _c_int,
         [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr,
          _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_size, _c_ptr]),
+    "dv_qkv_window_batch_workspace_bytes": (_c_size, [_c_int, _c_int, _c_int, _c_int, _c_int]),
+    "dv_qkv_window_batch_f16": (
+        _c_int,
+        [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr,
+         _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_size, _c_ptr]),
     "dv_prefill_attention_f16": (
         _c_int,
         [_c_ptr, _c_int, _c_int, _c_int, _c_int, ctypes.c_float, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr]),

@@ -405,13 +405,18 @@ struct TiledPlan {
 TiledPlan plan_tiled(int B, int N, int M) {
   TiledPlan p;
   p.bt = B <= 16 ? 1 : (B <= 32 ? 2 : (B <= 64 ? 4 : 8));
-  p.kc = p.bt == 8 ? 128 : 256;
+  // Two and four batch tiles: 32 weight rows per wavefront and chunks of 128 columns (fewer LDS reads per
+  // MFMA) once the matrix has rows enough to fill the device that way (QKV of 32 heads at 32 rows: 65.6 ->
+  // 59.0 us; 64 rows: 96 -> 69 us); short matrices (fc1: 4096 rows, a predictor's 1000) keep 16 rows per
+  // wavefront, chunks of 256 and more workgroups.
+  const bool wide = p.bt >= 4 || (p.bt == 2 && M >= 32 * compute_units());
+  p.kc = wide ? 128 : 256;
   p.xblocks = (B + 16 * p.bt - 1) / (16 * p.bt);
   const int cus = compute_units();
   const int nchunks = (N + p.kc - 1) / p.kc;
-  // 32 rows per wavefront halve the LDS reads of X per weight byte (LDS holds such tiles next to one or
-  // eight batch tiles of X, not next to two or four); worth it when the matrix still fills the device
-  p.wt = (p.bt == 8 || (p.bt == 1 && (int64_t)M * p.xblocks >= (int64_t)256 * cus)) ? 2 : 1;
+  // one batch tile: 32 rows per wavefront halve the LDS reads of X per weight byte; worth it when the
+  // matrix still fills the device
+  p.wt = (wide || (p.bt == 1 && (int64_t)M * p.xblocks >= (int64_t)256 * cus)) ? 2 : 1;
   // Workgroup size (8 wavefronts = 128 * wt rows, or 4) and column splits.  Measured at the OPT-175B
   // shapes (QKV of 32 heads: 12288 rows; fc1: 4096 rows; batch 16 / 32): what counts is one round of
   // workgroups over the device with loops as long as possible -- 192 workgroups of 24 chunks beat 768
@@ -421,7 +426,7 @@ TiledPlan plan_tiled(int B, int N, int M) {
   p.waves = 8;
   p.nsplit = 1;
   const int max_split = nchunks / 4 > 1 ? (nchunks / 4 < 16 ? nchunks / 4 : 16) : 1;
-  for (int waves = 8; waves >= (p.bt == 8 ? 8 : 4); waves -= 4) {
+  for (int waves = 8; waves >= (wide ? 8 : 4); waves -= 4) {
     const size_t lds = (size_t)(2 * 16 * p.bt + waves * 16 * p.wt) * (p.kc + kTgPad) * sizeof(half_t);
     const int resident = (int)((size_t)160 * 1024 / lds) > 0 ? (int)((size_t)160 * 1024 / lds) : 1;
     const int64_t groups = (M + waves * 16 * p.wt - 1) / (waves * 16 * p.wt);
@@ -484,23 +489,24 @@ int gemm_tiled_qkv(const half_t* X, int64_t ldx, const half_t* W, const half_t* 
   }
   const dim3 grid(p.xblocks, p.row_groups, p.nsplit);
   const int cps = p.nsplit > 1 ? p.chunks_per_split : 0;
-#define DV_TQW(BT, WT, WAVES)                                                                                  \
+#define DV_TQW(BT, WT, KC, WAVES)                                                                              \
   do {                                                                                                         \
-    auto kern = gemm_tiled_mfma_kernel<BT, WT, 256, true, WAVES>;                                              \
-    constexpr size_t lds = tiled_lds_bytes<BT, WT, 256, WAVES>();                                              \
+    auto kern = gemm_tiled_mfma_kernel<BT, WT, KC, true, WAVES>;                                               \
+    constexpr size_t lds = tiled_lds_bytes<BT, WT, KC, WAVES>();                                               \
     static LdsGrant grant;                                                                                     \
     if (int rc = grant.ensure(reinterpret_cast<const void*>(kern), lds); rc != DV_OK) return rc;               \
     hipLaunchKernelGGL(kern, grid, dim3(WAVES * 64), lds, s, X, ldx, W, (int64_t)d, bias,                      \
                        (const void*)nullptr, 4, B, d, Z, M, Y, (int64_t)Z, 0, cps, partial, qs);              \
   } while (0)
-#define DV_TQ(BT, WT)                  \
-  do {                                 \
-    if (p.waves == 4) DV_TQW(BT, WT, 4); \
-    else DV_TQW(BT, WT, 8);            \
+#define DV_TQ(BT, WT)                       \
+  do {                                      \
+    if (p.waves == 4) DV_TQW(BT, WT, 256, 4); \
+    else DV_TQW(BT, WT, 256, 8);            \
   } while (0)
   if (p.bt == 1) { if (p.wt == 2) DV_TQ(1, 2); else DV_TQ(1, 1); }
-  else if (p.bt == 2) DV_TQ(2, 1);
-  else return DV_ERR_UNSUPPORTED;
+  else if (p.bt == 2) { if (p.wt == 2) DV_TQW(2, 2, 128, 8); else DV_TQ(2, 1); }
+  else if (p.bt == 4) DV_TQW(4, 2, 128, 8);
+  else DV_TQW(8, 2, 128, 8);
 #undef DV_TQW
 #undef DV_TQ
   if (p.nsplit > 1) {
@@ -532,8 +538,11 @@ int gemm_tiled(const half_t* X, int64_t ldx, const half_t* W, int64_t ldw, const
       rc = launch_tiled<BT, WT, KC, 8>(p, X, ldx, W, ldw, bias, idx, idx_bytes, B, N, Z, M, Y, ldy, relu, partial, s); \
   } while (0)
   if (p.bt == 1) { if (p.wt == 2) DV_TG(1, 2, 256); else DV_TG(1, 1, 256); }
-  else if (p.bt == 2) DV_TG(2, 1, 256);
-  else if (p.bt == 4) DV_TG(4, 1, 256);
+  else if (p.bt == 2) {
+    if (p.wt == 2) rc = launch_tiled<2, 2, 128, 8>(p, X, ldx, W, ldw, bias, idx, idx_bytes, B, N, Z, M, Y, ldy, relu, partial, s);
+    else DV_TG(2, 1, 256);
+  }
+  else if (p.bt == 4) rc = launch_tiled<4, 2, 128, 8>(p, X, ldx, W, ldw, bias, idx, idx_bytes, B, N, Z, M, Y, ldy, relu, partial, s);
   else rc = launch_tiled<8, 2, 128, 8>(p, X, ldx, W, ldw, bias, idx, idx_bytes, B, N, Z, M, Y, ldy, relu, partial, s);
 #undef DV_TG
   if (rc != DV_OK) return rc;
@@ -1128,7 +1137,7 @@ int dv_qkv_proj_batch_f16(const void* x, int64_t ldx, const void* W, const void*
                                   workspace_bytes >= dv_qkv_proj_batch_workspace_bytes(B, d, nnz, hd)))) {
     const QkvScatter qs{reinterpret_cast<const int*>(head_idx), reinterpret_cast<const int*>(live), live_stride, nnz, H,
                         hd, reinterpret_cast<half_t*>(k_cache), reinterpret_cast<half_t*>(v_cache),
-                        reinterpret_cast<const int*>(positions), per_sample, pos_add, S};
+                        reinterpret_cast<const int*>(positions), per_sample, pos_add, S, B, 1, 0, 0};
     return gemm_tiled_qkv(reinterpret_cast<const half_t*>(x), ldx, reinterpret_cast<const half_t*>(W),
                           reinterpret_cast<const half_t*>(bias), B, d, reinterpret_cast<half_t*>(y), qs, workspace,
                           workspace_bytes, s);
@@ -1457,6 +1466,29 @@ int dv_out_proj_sparse_t_f16(const void* x, const void* Wt, int64_t ldw, const v
                      reinterpret_cast<const half_t*>(Wt), ldw, reinterpret_cast<const half_t*>(bias),
                      head_idx, 4, hd, B, N, H * hd, nnz * hd, reinterpret_cast<half_t*>(y),
                      workspace, workspace_bytes, reinterpret_cast<hipStream_t>(stream));
+}
+
+size_t dv_qkv_window_batch_workspace_bytes(int tokens, int nseq, int d, int nnz, int hd) {
+  if (tokens < 1 || tokens > 16 || nseq < 1 || nseq > 32 || d <= 0 || nnz <= 0 || hd <= 0) return 0;
+  return tiled_workspace_bytes(tokens * nseq, d, 3 * nnz * hd);
+}
+
+int dv_qkv_window_batch_f16(const void* x, int64_t ldx, const void* W, const void* bias, const void* head_idx,
+                            const void* batch_idx, int nnz, int tokens, int nseq, int d, int H, int hd, void* y,
+                            void* k_cache, void* v_cache, const void* positions, int per_sample, int pos_add,
+                            int S, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!x || !W || !y || !batch_idx || tokens < 1 || nseq < 1 || d <= 0 || H <= 0 || nnz < 0 ||
+      (nnz > 0 && !head_idx) || ((k_cache == nullptr) != (v_cache == nullptr)) || (k_cache && S <= 0))
+    return DV_ERR_INVALID_ARG;
+  if (tokens > 16 || nseq > 32 || (hd != 32 && hd != 64 && hd != 128)) return DV_ERR_UNSUPPORTED;
+  if (d % 8 || ldx % 8 || ldx < d || !aligned16(x) || !aligned16(W)) return DV_ERR_ALIGNMENT;
+  if (nnz == 0) return DV_OK;
+  const QkvScatter qs{reinterpret_cast<const int*>(head_idx), reinterpret_cast<const int*>(batch_idx), tokens, nnz, H,
+                      hd, reinterpret_cast<half_t*>(k_cache), reinterpret_cast<half_t*>(v_cache),
+                      reinterpret_cast<const int*>(positions), per_sample, pos_add, S, nseq, tokens, 1, tokens - 1};
+  return gemm_tiled_qkv(reinterpret_cast<const half_t*>(x), ldx, reinterpret_cast<const half_t*>(W),
+                        reinterpret_cast<const half_t*>(bias), tokens * nseq, d, reinterpret_cast<half_t*>(y), qs,
+                        workspace, workspace_bytes, reinterpret_cast<hipStream_t>(stream));
 }
 
 int dv_add_layer_norm_f16(const void* h, const void* residual, const void* gamma, const void* beta,

@@ -35,10 +35,13 @@ constexpr size_t tiled_lds_bytes() {
 }
 
 // QKV mode: the M = 3 * Hk * hd output rows are the q, k, v rows of the selected heads
-// (m = (t * Hk + i) * hd + j -> weight row (t * H + head_idx[i]) * hd + j, skipped when the head is out of
-// range or live[i * live_stride] < 0), the result goes to column `weight row` of Y (B, 3, H, hd) and the
-// K / V rows are also appended to the per-sequence caches k_cache (B, H, hd/8, S, 8), v_cache (B, H, S, hd)
-// at position positions[per_sample ? b : 0] + pos_add.
+// (m = (t * Hk + i) * hd + j -> weight row (t * H + head_idx[i]) * hd + j).  The X rows are `tokens`
+// window tokens of `nseq` sequences each, row r = s * nseq + b (tokens == 1: one token per sequence).
+// live[i * live_stride + s * live_tstride] < 0 skips (head i, token s); a head with no live token, or out
+// of range, is skipped altogether.  The result of token y_token goes to column `weight row` of
+// Y (nseq, 3, H, hd); the K / V rows of every live (head, token) are appended to the per-sequence caches
+// k_cache (nseq, H, hd/8, S, 8), v_cache (nseq, H, S, hd) at position
+// positions[per_sample ? b : 0] + pos_add + s.
 struct QkvScatter {
   const int* head_idx;
   const int* live;
@@ -47,6 +50,7 @@ struct QkvScatter {
   half_t* v_cache;
   const int* positions;
   int per_sample, pos_add, S;
+  int nseq, tokens, live_tstride, y_token;
 };
 
 __device__ __forceinline__ int qkv_row_of(const QkvScatter& q, int m) {
@@ -55,24 +59,61 @@ __device__ __forceinline__ int qkv_row_of(const QkvScatter& q, int m) {
   const int i = rem / q.hd, j = rem - i * q.hd;
   const int h = q.head_idx[i];
   if (h < 0 || h >= q.H || t > 2) return -1;
-  if (q.live != nullptr && q.live[(int64_t)i * q.live_stride] < 0) return -1;
+  if (q.live != nullptr) {
+    bool any = false;
+    for (int s = 0; s < q.tokens; ++s)
+      any |= q.live[(int64_t)i * q.live_stride + (int64_t)s * q.live_tstride] >= 0;
+    if (!any) return -1;
+  }
   return (t * q.H + h) * q.hd + j;
 }
 
-// stores one finished value: Y[b, weight row] and, for K / V rows, the cache entry
-__device__ __forceinline__ void qkv_store(const QkvScatter& q, half_t* __restrict__ Y, int b, int rid, half_t hv) {
-  Y[(int64_t)b * 3 * q.H * q.hd + rid] = hv;
+// stores one finished value of X row r, output row m (weight row rid): Y[b, weight row] for the token
+// that is wanted there and, for K / V rows, the cache entry
+__device__ __forceinline__ void qkv_store(const QkvScatter& q, half_t* __restrict__ Y, int r, int m, int rid,
+                                          half_t hv) {
+  const int s = q.tokens > 1 ? r / q.nseq : 0;
+  const int b = r - s * q.nseq;
+  if (q.live != nullptr && q.tokens > 1) {  // with one token a dead head has no weight row at all
+    const int i = (m % (q.Hk * q.hd)) / q.hd;
+    if (q.live[(int64_t)i * q.live_stride + (int64_t)s * q.live_tstride] < 0) return;
+  }
+  if (s == q.y_token) Y[(int64_t)b * 3 * q.H * q.hd + rid] = hv;
   if (q.k_cache == nullptr) return;
   const int t = rid / (q.H * q.hd);
   if (t == 0) return;
   const int rem = rid - t * q.H * q.hd;
   const int h = rem / q.hd, j = rem - h * q.hd;
-  const int dst = (q.positions ? q.positions[q.per_sample ? b : 0] : 0) + q.pos_add;
+  const int dst = (q.positions ? q.positions[q.per_sample ? b : 0] : 0) + q.pos_add + s;
   if (dst < 0 || dst >= q.S) return;
   if (t == 1)
     q.k_cache[((((int64_t)b * q.H + h) * (q.hd / 8) + j / 8) * q.S + dst) * 8 + (j & 7)] = hv;
   else
     q.v_cache[(((int64_t)b * q.H + h) * q.S + dst) * q.hd + j] = hv;
+}
+
+// four consecutive output rows m .. m + 3 of X row r (m % 4 == 0, so they belong to one head and one
+// 8-pack of the key cache): one 8-byte store each to Y and to the cache
+__device__ __forceinline__ void qkv_store4(const QkvScatter& q, half_t* __restrict__ Y, int r, int m, int rid,
+                                           const float (&val)[4]) {
+  const int s = q.tokens > 1 ? r / q.nseq : 0;
+  const int b = r - s * q.nseq;
+  if (q.live != nullptr && q.tokens > 1) {
+    const int i = (m % (q.Hk * q.hd)) / q.hd;
+    if (q.live[(int64_t)i * q.live_stride + (int64_t)s * q.live_tstride] < 0) return;
+  }
+  const half4_t o = {(half_t)val[0], (half_t)val[1], (half_t)val[2], (half_t)val[3]};
+  if (s == q.y_token) *reinterpret_cast<half4_t*>(Y + (int64_t)b * 3 * q.H * q.hd + rid) = o;
+  if (q.k_cache == nullptr) return;
+  const int t = rid / (q.H * q.hd);
+  if (t == 0) return;
+  const int rem = rid - t * q.H * q.hd;
+  const int h = rem / q.hd, j = rem - h * q.hd;
+  const int dst = (q.positions ? q.positions[q.per_sample ? b : 0] : 0) + q.pos_add + s;
+  if (dst < 0 || dst >= q.S) return;
+  half_t* p = t == 1 ? q.k_cache + ((((int64_t)b * q.H + h) * (q.hd / 8) + j / 8) * q.S + dst) * 8 + (j & 7)
+                     : q.v_cache + (((int64_t)b * q.H + h) * q.S + dst) * q.hd + j;
+  *reinterpret_cast<half4_t*>(p) = o;
 }
 
 template <int BT, int WT, int KC, bool QKV = false, int WAVES = kTgWaves>
@@ -162,19 +203,36 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_tiled_mfma_kernel(
     for (int p = 0; p < XV; ++p)
       store8(xb + ((p * WAVES * 64 + tid) / VPR) * LD + xv_col, x_ok ? xstage[p] : zero8());
   };
+  // Per k-step all WT + BT operand reads are issued before the first MFMA (the compiler otherwise
+  // alternates one LDS read, a full wait and two MFMAs: with many batch tiles the kernel is then
+  // bound by LDS latency, not by the weight stream).  With few operands per step the next step's are
+  // requested while the MFMAs of this one run (two register sets); with many (eight batch tiles) there
+  // is one set and the other wavefront of the SIMD covers the wait.
   auto multiply = [&](int buf) {
     const half_t* xb = xs + (size_t)buf * XROWS * LD;
+    constexpr int KS = KC / 32;
+    constexpr int SETS = (WT + BT) <= 6 ? 2 : 1;
+    half8_t a[SETS][WT], b[SETS][BT];
+    auto fetch = [&](int ks, int slot) {
 #pragma unroll
-    for (int ks = 0; ks < KC / 32; ++ks) {
-      half8_t a[WT];
+      for (int wt = 0; wt < WT; ++wt) a[slot][wt] = load8(ws + (wt * 16 + l16) * LD + ks * 32 + kg * 8);
 #pragma unroll
-      for (int wt = 0; wt < WT; ++wt) a[wt] = load8(ws + (wt * 16 + l16) * LD + ks * 32 + kg * 8);
+      for (int bt = 0; bt < BT; ++bt) b[slot][bt] = load8(xb + (bt * 16 + l16) * LD + ks * 32 + kg * 8);
+    };
+    if (SETS == 2) fetch(0, 0);
 #pragma unroll
-      for (int bt = 0; bt < BT; ++bt) {
-        const half8_t b = load8(xb + (bt * 16 + l16) * LD + ks * 32 + kg * 8);
+    for (int ks = 0; ks < KS; ++ks) {
+      const int cur = SETS == 2 ? (ks & 1) : 0;
+      __builtin_amdgcn_sched_barrier(0);
+      if (SETS == 1)
+        fetch(ks, 0);
+      else if (ks + 1 < KS)
+        fetch(ks + 1, cur ^ 1);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int wt = 0; wt < WT; ++wt) acc[wt][bt] = mfma_16x16x32(a[wt], b, acc[wt][bt]);
-      }
+      for (int bt = 0; bt < BT; ++bt)
+#pragma unroll
+        for (int wt = 0; wt < WT; ++wt) acc[wt][bt] = mfma_16x16x32(a[cur][wt], b[cur][bt], acc[wt][bt]);
     }
   };
   // One chunk: store its stage (weights: wavefront-private tile; X: buffer `buf`), one workgroup barrier
@@ -232,9 +290,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_tiled_mfma_kernel(
         if (relu) val[v] = relu_f(val[v]);
       }
       if (QKV) {
-#pragma unroll
-        for (int v = 0; v < 4; ++v)
-          if (mrow + v < M && rid[v] >= 0) qkv_store(qs, Y, b, rid[v], (half_t)val[v]);
+        // the four values of a lane are four consecutive rows of one (q|k|v, head): hd % 4 == 0
+        if (rid[0] >= 0) qkv_store4(qs, Y, b, mrow, rid[0], val);
         continue;
       }
       half_t* dst = Y + (int64_t)b * ldy + mrow;
@@ -281,7 +338,7 @@ __global__ __launch_bounds__(256) void qkv_split_reduce_kernel(const float* __re
   float s = 0.f;
   for (int y = 0; y < nsplit; ++y) s += partial[(int64_t)y * total + o];
   if (bias != nullptr) s += (float)bias[rid];
-  qkv_store(qs, Y, b, rid, (half_t)s);
+  qkv_store(qs, Y, b, m, rid, (half_t)s);
 }
 
 }  // namespace dv

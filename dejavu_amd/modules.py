@@ -469,10 +469,10 @@ class ParallelMHASparseAttMlp(_MHABase):
         """x: (B, 1, d), B > 1 sequences that decode in lockstep and share the head set and the
         back-fill window (the reference's sparse attention is single-sequence, mha_dejavu.py:1469;
         this is its batch extension).  The window buffer holds the B LayerNorm rows of each of
-        the 16 window tokens; the tracker is the one of the single-sequence path.  The newest
-        token's QKV is one pass over the active heads' weights for all B rows; each earlier
-        window token that some active head still misses costs one more pass restricted to
-        those heads (the flush step: 16 passes over every head)."""
+        the 16 window tokens; the tracker is the one of the single-sequence path.  At the first
+        window position the QKV is one pass over the active heads' weights for the B rows; later
+        positions multiply all window tokens of all sequences (up to 16 B rows) in one pass and
+        store, per head, the tokens that head still misses (the flush step: every head, 16 B rows)."""
         dev = x.device
         assert x.dtype == torch.float16 and x.is_contiguous()
         B, d, H, hd = x.shape[0], self.embed_dim, self.num_heads, self.head_dim
@@ -499,12 +499,14 @@ class ParallelMHASparseAttMlp(_MHABase):
         weight = self.Wqkv.weight.view(3, H, hd, d)
         bias = None if self.Wqkv.bias is None else self.Wqkv.bias.view(3, H, hd)
         qkv = torch.empty(B, 3, H, hd, dtype=torch.float16, device=dev)
-        scratch = qkv if nb == 1 else torch.empty_like(qkv)
-        for s in range(nb):  # window token s: position cache_offset + s, or lengths[b] - (counter - s)
-            ops.qkv_proj_batch(self.x_cache_batch[s].view(B, d), weight, head_idx, bias,
-                               out=qkv if s == nb - 1 else scratch, k_cache=kc, v_cache=vc,
-                               positions=self.cache_offset if lengths is None else lengths,
-                               pos_add=s if lengths is None else s - self.counter, live=batch_idx[:, s])
+        # window token s goes to cache position cache_offset + s, or lengths[b] - (counter - s)
+        positions = self.cache_offset if lengths is None else lengths
+        if nb == 1:
+            ops.qkv_proj_batch(self.x_cache_batch[0].view(B, d), weight, head_idx, bias, out=qkv, k_cache=kc,
+                               v_cache=vc, positions=positions, pos_add=0, live=batch_idx[:, 0])
+        else:  # all window tokens of all sequences in one pass over the weights
+            ops.qkv_window_batch(self.x_cache_batch, weight, head_idx, batch_idx, B, bias, out=qkv, k_cache=kc,
+                                 v_cache=vc, positions=positions, pos_add=0 if lengths is None else -self.counter)
         self.counter += 1
         return qkv, head_idx, kc, vc
 

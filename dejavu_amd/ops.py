@@ -433,6 +433,64 @@ def qkv_proj_batch(x: torch.Tensor, weight: torch.Tensor, head_idx: torch.Tensor
     return out
 
 
+def qkv_window_batch(x_window: torch.Tensor, weight: torch.Tensor, head_idx: torch.Tensor, batch_idx: torch.Tensor,
+                     nseq: int, bias: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+                     k_cache: Optional[torch.Tensor] = None, v_cache: Optional[torch.Tensor] = None,
+                     positions: Optional[torch.Tensor] = None, pos_add: int = 0) -> torch.Tensor:
+    """QKV of the active heads for every token of a back-fill window shared by ``nseq`` sequences, in ONE
+    pass over the weights (``qkv_proj_batch`` once per window token would stream them once per token).
+
+    :param x_window: (tokens, nseq * hidden) or (tokens * nseq, hidden): LayerNorm rows of the window,
+        token-major; tokens <= 16, nseq <= 32
+    :param batch_idx: int32 (nnz, tokens), the tracker's output: (head i, token s) is computed when
+        ``batch_idx[i, s] >= 0``
+    :param positions, pos_add: token s of sequence b is cached at ``positions[b] + pos_add + s``
+        (``positions``: int32, (nseq,) per sequence or (1,) for all; None = 0)
+    :return: (nseq, 3, nheads, head_dim) with the rows of the newest token (s = tokens - 1); rows of
+        heads that were not computed for it keep the content of ``out``
+    """
+    _require_device(x_window, weight, head_idx, batch_idx, bias, k_cache, v_cache, positions)
+    _expect(weight.dim() == 4 and weight.shape[0] == 3, f"weight {tuple(weight.shape)} is not (3, nheads, head_dim, hidden)")
+    _, nheads, head_dim, hidden_dim = weight.shape
+    n_active = head_idx.shape[0]
+    _int32_vector("head_idx", head_idx, n_active)
+    _expect(batch_idx.dtype == torch.int32 and batch_idx.dim() == 2 and batch_idx.shape[0] == n_active
+            and batch_idx.is_contiguous(), "batch_idx must be a contiguous int32 (nnz, tokens) matrix")
+    tokens = batch_idx.shape[1]
+    _expect(1 <= tokens <= 16 and 1 <= nseq <= 32, f"{tokens} tokens x {nseq} sequences outside 16 x 32")
+    x2 = x_window.reshape(-1, hidden_dim)
+    _expect(x2.shape[0] >= tokens * nseq and x2.is_contiguous(), "x_window must hold tokens * nseq contiguous rows")
+    _same_f16("x_window", x2, "weight", weight)
+    _expect(weight.is_contiguous() and head_idx.is_contiguous(), "weight and head_idx must be contiguous")
+    if bias is not None:
+        _expect(tuple(bias.shape) == (3, nheads, head_dim) and bias.is_contiguous() and bias.dtype == x2.dtype,
+                f"bias {tuple(bias.shape)} is not a contiguous fp16 (3, {nheads}, {head_dim}) tensor")
+    if out is None:
+        out = torch.empty(nseq, 3, nheads, head_dim, device=x2.device, dtype=x2.dtype)
+    else:
+        _expect(tuple(out.shape) == (nseq, 3, nheads, head_dim) and out.is_contiguous() and out.dtype == x2.dtype,
+                "out must be a contiguous fp16 (nseq, 3, nheads, head_dim) tensor")
+    S, per_sample = 0, 0
+    if k_cache is not None:
+        _expect(v_cache is not None, "k_cache without v_cache")
+        S = v_cache.shape[2]
+        _expect(tuple(v_cache.shape) == (nseq, nheads, S, head_dim)
+                and tuple(k_cache.shape) == (nseq, nheads, head_dim // 8, S, 8)
+                and k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dtype == v_cache.dtype == x2.dtype,
+                "caches must be contiguous fp16 (nseq, H, hd/8, S, 8) and (nseq, H, S, hd)")
+    if positions is not None:
+        _expect(positions.dtype == torch.int32 and positions.is_contiguous() and positions.numel() in (1, nseq),
+                "positions must be int32 with one entry, or one per sequence")
+        per_sample = int(positions.numel() == nseq and nseq > 1)
+    nbytes = lib.dv_qkv_window_batch_workspace_bytes(tokens, nseq, hidden_dim, n_active, head_dim)
+    ws = _workspace(x2.device, nbytes) if nbytes else None
+    check(lib.dv_qkv_window_batch_f16(_ptr(x2), hidden_dim, _ptr(weight), _ptr(bias), _ptr(head_idx), _ptr(batch_idx),
+                                      n_active, tokens, nseq, hidden_dim, nheads, head_dim, _ptr(out), _ptr(k_cache),
+                                      _ptr(v_cache), _ptr(positions), per_sample, int(pos_add), S, _ptr(ws),
+                                      0 if ws is None else ws.numel(), _stream()), "dv_qkv_window_batch_f16")
+    return out
+
+
 def out_proj_sparse(x: torch.Tensor, weight: torch.Tensor, head_idx: torch.Tensor,
                     bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Output projection over the listed heads only (interface of attention_proj_sparse.py:274-335):

@@ -229,6 +229,27 @@ DV_API int dv_qkv_proj_batch_f16(const void* x, int64_t ldx, const void* W, cons
                                  void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * The same projection for ALL tokens of a shared back-fill window in one pass over the weights:
+ *   x row s * nseq + b is window token s (< tokens <= 16) of sequence b (< nseq <= 32), row stride ldx;
+ *   batch_idx (nnz, tokens) int32: (head i, token s) is computed when batch_idx[i, s] >= 0 (the
+ *   tracker's output, Dejavu/src/models/modules/mha_dejavu.py:1124-1149, 1318-1329), a head with no
+ *   such token is skipped altogether;
+ *   y (nseq, 3, H, hd) receives the rows of the newest token (s = tokens - 1) only;
+ *   the K / V rows of every computed (head, token) go to the caches at position
+ *   positions[per_sample ? b : 0] + pos_add + s.
+ * It replaces one dv_qkv_proj_batch_f16 pass per window token (the reference recomputes skipped
+ * K / V rows of a single sequence through qkv_proj_sparse with up to 16 rows,
+ * mha_dejavu.py:1333-1352): tokens * nseq rows are multiplied against each weight tile in blocks of
+ * up to 128 rows.  workspace: dv_qkv_window_batch_workspace_bytes(...) bytes, 16-byte aligned.
+ */
+DV_API size_t dv_qkv_window_batch_workspace_bytes(int tokens, int nseq, int d, int nnz, int hd);
+DV_API int dv_qkv_window_batch_f16(const void* x, int64_t ldx, const void* W, const void* bias,
+                                   const void* head_idx, const void* batch_idx, int nnz, int tokens, int nseq,
+                                   int d, int H, int hd, void* y, void* k_cache, void* v_cache,
+                                   const void* positions, int per_sample, int pos_add, int S,
+                                   void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Causal attention over the prompt, and the prompt's K / V rows written into the decode caches:
  *   ctx[b, t, h, :] = softmax_{s <= t}(q[b, t, h] . k[b, s, h] * scale) . v[b, s, h]
  *   k_cache[b, h, j / 8, pos0 + t, j % 8] = k[b, t, h, j];  v_cache[b, h, pos0 + t, j] = v[b, t, h, j]

@@ -90,6 +90,68 @@ def test_qkv_proj_batch_matches_oracle(B, H, hd, d, S):
     assert np.array_equal(np16(v2)[:, :, keep], vc0.numpy()[:, :, keep])
 
 
+@pytest.mark.parametrize("tokens,nseq,H,hd,d,S,per_sample", [
+    (2, 3, 4, 64, 512, 40, True), (5, 8, 6, 128, 776, 64, False), (16, 8, 4, 64, 512, 48, True),
+    (9, 17, 3, 32, 264, 40, True), (16, 32, 3, 128, 520, 40, False)])
+def test_qkv_window_batch_matches_oracle(tokens, nseq, H, hd, d, S, per_sample):
+    """All tokens of a shared back-fill window in one pass: (head, token) pairs the tracker marks are
+    projected for every sequence and cached at position + token; the newest token's rows also go to
+    `out`; everything else stays untouched.  Row counts cover one to four blocks of 128 rows, ragged
+    last column chunks and every batch-tile count of the kernel (6 .. 512 rows)."""
+    from dejavu_amd import ops
+    from dejavu_amd.workloads import pack_k_cache
+
+    g = torch.Generator().manual_seed(tokens * 1000 + nseq)
+    xw = randh(g, 16, nseq * d)  # the whole window buffer; rows past `tokens` must not be read into results
+    W = randh(g, 3, H, hd, d, std=0.05)
+    bias = randh(g, 3, H, hd, std=0.1)
+    head_idx = torch.sort(torch.randperm(H, generator=g)[: max(2, H - 1)]).values.int()
+    nnz = head_idx.numel()
+    batch_idx = torch.where(torch.rand(nnz, tokens, generator=g) < 0.6,
+                            torch.arange(tokens).expand(nnz, tokens), torch.full((nnz, tokens), -1)).int()
+    batch_idx[0, tokens - 1] = tokens - 1  # head 0 computes the newest token
+    batch_idx[1, :] = -1                   # head 1 computes nothing
+    if per_sample:
+        positions = torch.randint(0, S - tokens, (nseq,), generator=g).int()
+    else:
+        positions = torch.tensor([S - tokens - 2], dtype=torch.int32)
+    pos_add = 1
+    kc0, vc0 = randh(g, nseq, H, S, hd), randh(g, nseq, H, S, hd)
+    k_cache, v_cache = pack_k_cache(kc0).cuda(), vc0.clone().cuda()
+    out = torch.full((nseq, 3, H, hd), 7.0, dtype=torch.float16, device="cuda")
+    print(f"case qkv window batch tokens={tokens} nseq={nseq} H={H} hd={hd} d={d}", flush=True)
+    ops.qkv_window_batch(xw.cuda(), W.cuda(), head_idx.cuda(), batch_idx.cuda(), nseq, bias.cuda(), out=out,
+                         k_cache=k_cache, v_cache=v_cache, positions=positions.cuda(), pos_add=pos_add)
+    torch.cuda.synchronize()
+    x_rows = xw[:tokens].reshape(tokens * nseq, d).float()
+    full = torch.einsum("rn,thjn->rthj", x_rows, W.float()) + bias.float()  # (rows, 3, H, hd), fp32
+    full = full.half().numpy().reshape(tokens, nseq, 3, H, hd)
+    got, kn, vn = np16(out), O.unpack_k_cache(np16(k_cache)), np16(v_cache)
+    want_k, want_v = kc0.numpy().copy(), vc0.numpy().copy()
+    written = np.zeros((nseq, H, S), dtype=bool)
+    for i, h in enumerate(int(v) for v in head_idx):
+        for s_ in range(tokens):
+            if batch_idx[i, s_] < 0:
+                continue
+            for b in range(nseq):
+                p = int(positions[b if per_sample else 0]) + pos_add + s_
+                want_k[b, h, p], want_v[b, h, p] = full[s_, b, 1, h], full[s_, b, 2, h]
+                written[b, h, p] = True
+    # values agree within tolerance where something was written, bit-for-bit elsewhere
+    assert_close(kn[written], want_k[written], "cached K rows")
+    assert np.array_equal(kn[~written], want_k[~written]), "K cache entries outside the marked (head, token) pairs changed"
+    assert_close(vn[written], want_v[written], "cached V rows")
+    assert np.array_equal(vn[~written], want_v[~written]), "V cache entries outside the marked (head, token) pairs changed"
+    newest = [int(h) for i, h in enumerate(head_idx) if batch_idx[i, tokens - 1] >= 0]
+    assert_close(got[:, :, newest], full[tokens - 1][:, :, newest], "rows of the newest token")
+    rest = [h for h in range(H) if h not in newest]
+    assert np.all(got[:, :, rest] == 7.0), "heads without the newest token must not be written"
+    # what the cache holds for the newest token is exactly what `out` holds
+    for b in range(nseq):
+        p = int(positions[b if per_sample else 0]) + pos_add + tokens - 1
+        assert np.array_equal(kn[b, newest, p], got[b, 1, newest]) and np.array_equal(vn[b, newest, p], got[b, 2, newest])
+
+
 def build_attention(g, d, H, r, Hk, mlp_k, layer_idx=1):
     from dejavu_amd.modules import ParallelMHASparseAttMlp
 
