@@ -510,8 +510,8 @@ int gemm_tiled_qkv(const half_t* X, int64_t ldx, const half_t* W, const half_t* 
 #undef DV_TQW
 #undef DV_TQ
   if (p.nsplit > 1) {
-    const int64_t total = (int64_t)B * M;
-    hipLaunchKernelGGL(qkv_split_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, partial,
+    const int64_t quads = (int64_t)B * M / 4;  // M = 3 * Hk * hd is a multiple of 4
+    hipLaunchKernelGGL(qkv_split_reduce_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, partial,
                        p.nsplit, B, M, bias, Y, qs);
   }
   return launch_status();

@@ -68,32 +68,9 @@ __device__ __forceinline__ int qkv_row_of(const QkvScatter& q, int m) {
   return (t * q.H + h) * q.hd + j;
 }
 
-// stores one finished value of X row r, output row m (weight row rid): Y[b, weight row] for the token
-// that is wanted there and, for K / V rows, the cache entry
-__device__ __forceinline__ void qkv_store(const QkvScatter& q, half_t* __restrict__ Y, int r, int m, int rid,
-                                          half_t hv) {
-  const int s = q.tokens > 1 ? r / q.nseq : 0;
-  const int b = r - s * q.nseq;
-  if (q.live != nullptr && q.tokens > 1) {  // with one token a dead head has no weight row at all
-    const int i = (m % (q.Hk * q.hd)) / q.hd;
-    if (q.live[(int64_t)i * q.live_stride + (int64_t)s * q.live_tstride] < 0) return;
-  }
-  if (s == q.y_token) Y[(int64_t)b * 3 * q.H * q.hd + rid] = hv;
-  if (q.k_cache == nullptr) return;
-  const int t = rid / (q.H * q.hd);
-  if (t == 0) return;
-  const int rem = rid - t * q.H * q.hd;
-  const int h = rem / q.hd, j = rem - h * q.hd;
-  const int dst = (q.positions ? q.positions[q.per_sample ? b : 0] : 0) + q.pos_add + s;
-  if (dst < 0 || dst >= q.S) return;
-  if (t == 1)
-    q.k_cache[((((int64_t)b * q.H + h) * (q.hd / 8) + j / 8) * q.S + dst) * 8 + (j & 7)] = hv;
-  else
-    q.v_cache[(((int64_t)b * q.H + h) * q.S + dst) * q.hd + j] = hv;
-}
-
-// four consecutive output rows m .. m + 3 of X row r (m % 4 == 0, so they belong to one head and one
-// 8-pack of the key cache): one 8-byte store each to Y and to the cache
+// stores four finished values: consecutive output rows m .. m + 3 of X row r (m % 4 == 0, so they belong to
+// one head and one 8-pack of the key cache; weight rows rid .. rid + 3): one 8-byte store to Y for the token
+// that is wanted there and, for K / V rows, one to the cache
 __device__ __forceinline__ void qkv_store4(const QkvScatter& q, half_t* __restrict__ Y, int r, int m, int rid,
                                            const float (&val)[4]) {
   const int s = q.tokens > 1 ? r / q.nseq : 0;
@@ -325,20 +302,25 @@ __global__ __launch_bounds__(256) void gemm_split_reduce_kernel(
   Y[(int64_t)b * ldy + m] = (half_t)s;
 }
 
-// QKV mode: sums the splits, adds the bias and scatters (Y and the caches).
+// QKV mode: sums the splits, adds the bias and scatters (Y and the caches).  A thread takes four
+// consecutive output rows (one head, M % 4 == 0): 16-byte loads of the partial sums, 8-byte stores.
 __global__ __launch_bounds__(256) void qkv_split_reduce_kernel(const float* __restrict__ partial, int nsplit, int B,
                                                                int M, const half_t* __restrict__ bias,
                                                                half_t* __restrict__ Y, QkvScatter qs) {
   const int64_t total = (int64_t)B * M;
-  const int64_t o = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t o = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
   if (o >= total) return;
   const int b = (int)(o / M), m = (int)(o - (int64_t)b * M);
   const int rid = qkv_row_of(qs, m);
   if (rid < 0) return;
-  float s = 0.f;
-  for (int y = 0; y < nsplit; ++y) s += partial[(int64_t)y * total + o];
-  if (bias != nullptr) s += (float)bias[rid];
-  qkv_store(qs, Y, b, m, rid, (half_t)s);
+  float4_t s = {0.f, 0.f, 0.f, 0.f};
+  for (int y = 0; y < nsplit; ++y) s += *reinterpret_cast<const float4_t*>(partial + (int64_t)y * total + o);
+  float val[4] = {s[0], s[1], s[2], s[3]};
+  if (bias != nullptr) {
+#pragma unroll
+    for (int v = 0; v < 4; ++v) val[v] += (float)bias[rid + v];
+  }
+  qkv_store4(qs, Y, b, m, rid, val);
 }
 
 }  // namespace dv
