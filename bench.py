@@ -606,8 +606,8 @@ def holds_gpu():
 
 
 def other_workloads():
-    """Runs `bench.py --batch 8 / 16 / 32` and `bench.py --workload decode` as child processes (one at a
-    time, each bounded) and returns the figures of their JSON lines; a leg that fails is reported as
+    """Runs `bench.py --batch 8 / 16 / 32 --window cycle` and `bench.py --workload decode` as child processes
+    (one at a time, each bounded) and returns the figures of their JSON lines; a leg that fails is reported as
     such and never fails the headline run."""
     import subprocess
 
@@ -625,12 +625,14 @@ def other_workloads():
 
     out = {"batched_layer": {}, "how": "child processes of this script, run before the headline measurement"}
     for b in (8, 16, 32):
-        d, secs = child(["--batch", str(b), "--steps", "96", "--warmup", "24"], 300)
+        # two whole windows per layer: the window average, and the first window position measured beside it
+        d, secs = child(["--batch", str(b), "--window", "cycle", "--steps", "96", "--warmup", "48"], 300)
         if "error" in d:
             out["batched_layer"][str(b)] = d
         else:
-            out["batched_layer"][str(b)] = dict(d["layer"], wall_s=round(secs, 1), steps=d["steps"],
-                                                workload=d["config"]["workload"])
+            out["batched_layer"][str(b)] = {"window_start": d["window_start"],
+                                            "window_average": dict(d["layer"], steps=d["steps"]),
+                                            "workload": d["config"]["workload"], "wall_s": round(secs, 1)}
     d, secs = child(["--workload", "decode"], 420)
     if "error" in d:
         out["decode"] = d
