@@ -44,6 +44,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+MFMA_PEAK_TFLOPS = 2500.0  # dense fp16
 N_LAYERS = 3
 WINDOW = 16
 MAX_GRAPH_STEPS = 192  # steps per HIP graph (four schedule periods)
@@ -311,6 +312,13 @@ def kernel_table(torch, cfg, batch, layers):
         table[name] = {"us": round(us, 2), "MB": round(nbytes[name] / 1e6, 2),
                        "GB/s": round(nbytes[name] / us / 1e3, 1),
                        "frac": round(nbytes[name] / us / 1e3 / HBM_PEAK_GBPS, 4)}
+        if batch > 1 and name != "decode_attn":
+            # a weight product at a batch: 2 B flop per fp16 weight = B flop per byte, on the matrix cores
+            # from 3 (fc1), 5 (fc2 / out_proj) and 9 (predictors) rows on; utilisation against the dense
+            # fp16 MFMA peak (the product stays bound by the weight stream: 8 TB/s x B flop/byte)
+            tflops = batch * nbytes[name] / us / 1e6
+            table[name]["TFLOP/s"] = round(tflops, 1)
+            table[name]["mfma_frac_of_peak"] = round(tflops / MFMA_PEAK_TFLOPS, 4)
     # fc1 -> fc2 -> split reduction, back to back as in a layer step: 4 K d bytes
     us = time_kernel(torch, lambda L: ops.mlp_sparse(x, f(L).fc1.weight, f(L).fc2_weight_t, idx, f(L).fc1.bias,
                                                      f(L).fc2.bias), layers)
