@@ -1,4 +1,4 @@
-"""Host-side logic of bench.py (no GPU): the byte model of the scope table, the one-GPU rule, the
+"""Host-side logic of bench.py (no GPU): the byte model of a layer step, the one-GPU rule, the
 counter reduction that writes profiles/traffic.json, and the guard that keeps child processes away from
 a process that already holds the device."""
 import csv
@@ -16,7 +16,7 @@ import bench  # noqa: E402
 from dejavu_amd.workloads import CONFIGS  # noqa: E402
 
 
-def test_algorithmic_bytes_match_the_scope_table():
+def test_algorithmic_bytes_of_a_layer_step():
     """OPT-175B layer, batch 1: 785.2 MB per step (4 K d = 201.33 MB for the MLP pair, 301.99 MB QKV,
     33.55 MB KV of the selected heads, 100.66 MB out_proj, 122.88 + 24.77 MB predictors)."""
     cfg = CONFIGS["opt-175b"]
