@@ -115,6 +115,55 @@ def test_head_sparse_projections_against_library(ops, gen):
     close(ops.out_proj_sparse(ctx, Wout_t.t().contiguous().view(D, H, HD), head_idx, bout), ref, "out_proj, (d, H, hd)")
 
 
+def test_batched_window_projection_against_library(ops, gen):
+    """One pass over the active heads' weights for all 16 tokens of a shared back-fill window of 8
+    sequences (128 rows) and for 2 tokens of 32 sequences: the newest token's rows and the cached K / V
+    rows of the marked (head, token) pairs against fp32 einsum; a batched out_proj / fc2 at 8 and 32 rows."""
+    S = 64
+    Wqkv, bqkv = randn(gen, 3, H, HD, D, std=0.02), randn(gen, 3, H, HD, std=0.02)
+    head_idx = torch.sort(torch.randperm(H, device="cuda", generator=gen)[:HK]).values.int()
+    hi = head_idx.long()
+    for tokens, nseq in ((16, 8), (2, 32)):
+        print(f"case full-size window projection tokens={tokens} nseq={nseq}", flush=True)
+        xw = randn(gen, 16, nseq * D)
+        batch_idx = torch.arange(tokens, device="cuda", dtype=torch.int32).repeat(HK, 1)
+        drop = torch.rand(HK, tokens, device="cuda", generator=gen) < 0.3
+        drop[:, tokens - 1] = False
+        batch_idx = torch.where(drop, torch.full_like(batch_idx, -1), batch_idx).contiguous()
+        k_cache = torch.zeros(nseq, H, HD // 8, S, 8, dtype=torch.float16, device="cuda")
+        v_cache = torch.zeros(nseq, H, S, HD, dtype=torch.float16, device="cuda")
+        positions = torch.randint(0, S - tokens, (nseq,), device="cuda", generator=gen).int()
+        out = torch.zeros(nseq, 3, H, HD, dtype=torch.float16, device="cuda")
+        ops.qkv_window_batch(xw, Wqkv, head_idx, batch_idx, nseq, bqkv, out=out, k_cache=k_cache, v_cache=v_cache,
+                             positions=positions)
+        rows = xw[:tokens].reshape(tokens * nseq, D).float()
+        ref = torch.einsum("thjn,rn->rthj", Wqkv[:, hi].float(), rows) + bqkv[:, hi].float()
+        ref = ref.view(tokens, nseq, 3, HK, HD)
+        close(out[:, :, hi], ref[tokens - 1], "rows of the newest token")
+        k_plain = k_cache.permute(0, 1, 3, 2, 4).reshape(nseq, H, S, HD)
+        seqs = torch.arange(nseq, device="cuda")
+        for s_ in range(tokens):
+            live = (batch_idx[:, s_] >= 0)
+            pos = (positions + s_).long()
+            got_k = k_plain[seqs[:, None], hi[None, :], pos[:, None]]  # (nseq, HK, HD)
+            got_v = v_cache[seqs[:, None], hi[None, :], pos[:, None]]
+            close(got_k[:, live], ref[s_, :, 1][:, live], f"cached K rows of token {s_}")
+            close(got_v[:, live], ref[s_, :, 2][:, live], f"cached V rows of token {s_}")
+            assert not got_k[:, ~live].any() and not got_v[:, ~live].any(), "unmarked (head, token) pairs were cached"
+    Wout_t, bout = randn(gen, H * HD, D, std=0.02), randn(gen, D, std=0.02)
+    W2t, b2 = randn(gen, FFN, D, std=0.02), randn(gen, D, std=0.02)
+    idx = torch.sort(torch.randperm(FFN, device="cuda", generator=gen)[:K]).values
+    rows = (hi[:, None] * HD + torch.arange(HD, device="cuda")[None, :]).flatten()
+    for B in (8, 32):
+        print(f"case full-size batched out_proj / fc2 B={B}", flush=True)
+        ctx = randn(gen, B, H, HD)
+        ref = ctx.view(B, H * HD)[:, rows].float() @ Wout_t.index_select(0, rows).float() + bout.float()
+        close(ops.out_proj_sparse_t(ctx, Wout_t, head_idx, bout), ref, f"out_proj, {B} rows")
+        hmid = randn(gen, B, K)
+        ref = hmid.float() @ W2t.index_select(0, idx).float() + b2.float()
+        close(ops.gather_transposed_gemv(hmid, W2t, idx, b2), ref, f"fc2, {B} rows")
+
+
 def test_decode_attention_against_sdpa(ops, gen):
     S, t = 2048, 2047
     from dejavu_amd.workloads import pack_k_cache
