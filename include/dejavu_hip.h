@@ -107,7 +107,7 @@ DV_API int dv_topk_search_f16(const void* logits, int B, int n, int k, void* idx
  *   y (B, M) fp16.  1 <= B <= 64 (the reference stops at 4): B <= 2 runs as a
  *   bandwidth-bound GEMV on the vector ALUs; 3 <= B <= 64 stages the gathered
  *   rows through LDS into 16x16x32 fp16 MFMA tiles.
-  * idx == NULL: no gather, row m of W (a dense product y = act(x W[:M]^T + bias), M <= Z),
+ * idx == NULL: no gather, row m of W (a dense product y = act(x W[:M]^T + bias), M <= Z),
  * as the one-token decode step of a dense block or of the lm_head needs it.
  */
 DV_API int dv_gather_gemv_f16(const void* x, const void* W, int64_t ldw, const void* bias,
@@ -147,7 +147,8 @@ DV_API int dv_dense_linear_f16(const void* x, int64_t ldx, const void* W, int64_
  * Dejavu/src/ops/triton/gather_gemv.py:572-644 (deterministic: fixed-order
  * split over row groups instead of floating-point atomics).
  *   x (B, M); W (Z, N) row stride ldw; bias (N,) or NULL; idx (M,);
- *   y (B, N) fp16.  1 <= B <= 64 (vector ALUs up to 4, MFMA tiles above).
+ *   y (B, N) fp16.  1 <= B <= 64 (vector ALUs up to 4; above, the weight tile is transposed in
+ *   registers into 16x16x32 MFMA operands up to 32 rows, 32x32x16 operands up to 64).
  *   workspace: dv_gather_transposed_gemv_workspace_bytes(B, N, M) bytes, no
  *   initialisation needed; calls sharing it must not overlap.
  */
