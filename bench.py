@@ -631,7 +631,7 @@ def other_workloads():
         except subprocess.TimeoutExpired:
             return {"error": f"no result within {limit} s"}, time.perf_counter() - t0
 
-    out = {"batched_layer": {}, "how": "child processes of this script, run before the headline measurement"}
+    out = {"batched_layer": {}, "how": "child processes of this script, run after the headline leg"}
     for b in (8, 16, 32):
         # two whole windows per layer: the window average, and the first window position measured beside it
         d, secs = child(["--batch", str(b), "--window", "cycle", "--steps", "96", "--warmup", "48"], 300)
@@ -650,6 +650,22 @@ def other_workloads():
                          "frac_of_hbm_peak": d["frac_of_hbm_peak"], "graph_equals_eager": d["graph_equals_eager"],
                          "new_tokens": d["steps"], "wall_s": round(secs, 1)}
     return out
+
+
+def coordinate_legs():
+    """The headline leg (this command line + --no-other-workloads) as a child process, then the other
+    workloads; prints the headline leg's JSON line with `other_workloads` added."""
+    import subprocess
+
+    cmd = [sys.executable, os.path.abspath(__file__), *sys.argv[1:], "--no-other-workloads"]
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, text=True)  # stderr passes through
+    lines = [ln for ln in r.stdout.strip().splitlines() if ln.startswith("{")]
+    if r.returncode != 0 or not lines:
+        sys.stdout.write(r.stdout)
+        sys.exit(r.returncode or 1)
+    out = json.loads(lines[-1])
+    out["other_workloads"] = other_workloads()
+    print(json.dumps(out))
 
 
 def main():
@@ -690,9 +706,10 @@ def main():
     if args.traffic_from:
         return write_traffic(*args.traffic_from)
 
-    # The headline run also reports the other BASELINE workloads (batched layer, end-to-end decode), each
-    # measured by a child process of this script that runs BEFORE this process touches the GPU
-    # (a child started later would be forked from a process that holds the device).
+    # The headline run also reports the other BASELINE workloads (batched layer, end-to-end decode).  Every
+    # leg, the headline one first, is then a child process of this script and this process never touches
+    # the GPU (a child must not be forked from a process that holds the device, and the headline figure is
+    # taken before the other legs have heated the part: measured after them it read 3 % higher).
     others = None
     if (args.workload == "layer" and args.batch == 1 and args.config == "opt-175b" and not args.no_other_workloads
             and not args.pmc_calibration and not args.no_graph and args.window in (None, "cycle")):
@@ -700,7 +717,7 @@ def main():
             others = {"skipped": "this process held the GPU before the measurement started; run the legs with "
                                  "--batch 8 / 16 / 32 and --workload decode"}
         else:
-            others = other_workloads()
+            return coordinate_legs()
 
     import torch
 
