@@ -202,19 +202,25 @@ def build_layers(cfg, batch, device):
     return layers
 
 
-def layer_step(L):
-    """One decode step of one block in the state 'first token of a back-fill
-    window': every active head computes Q, K, V of the newest token only."""
+def layer_step_inputs(L):
+    """Host-side state of 'first token of a back-fill window' (every active head computes Q, K, V of
+    the newest token only); returns the predictions the step consumes."""
     mixer = L["block"].mixer
     mixer.counter = 0  # the window step re-initialises the tracker at counter 0
     L["ip"].sequence_len_offset = L["S"] - 1  # mixer.cache_offset must hold S - 1 (set by the caller)
+    return L["att_idx_in"], L["mlp_logit_in"]
+
+
+def layer_step(L):
+    """One decode step of one block at the first position of a back-fill window."""
+    head_idx, logit = layer_step_inputs(L)
     return L["block"](L["hidden"], L["residual"], mixer_kwargs={"inference_params": L["ip"]},
-                      head_idx=L["att_idx_in"], mlp_sp_logit=L["mlp_logit_in"])
+                      head_idx=head_idx, mlp_sp_logit=logit)
 
 
-def window_step(L, c):
-    """Decode step at window position c (0..15) of a window that occupies the last 16 cache
-    positions; heads drawn for this (layer, position).  Position 15 flushes the window."""
+def window_step_inputs(L, c):
+    """Host-side state of the decode step at window position c (0..15) of a window that occupies the
+    last 16 cache positions; heads drawn for this (layer, position).  Position 15 flushes the window."""
     mixer = L["block"].mixer
     S = L["S"]
     if c == 0:
@@ -224,8 +230,13 @@ def window_step(L, c):
             L["offset_mode"] = "window"
     assert mixer.counter == c
     L["ip"].sequence_len_offset = S - WINDOW + c
+    return L["heads"][c], L["mlp_logit_in"]
+
+
+def window_step(L, c):
+    head_idx, logit = window_step_inputs(L, c)
     return L["block"](L["hidden"], L["residual"], mixer_kwargs={"inference_params": L["ip"]},
-                      head_idx=L["heads"][c], mlp_sp_logit=L["mlp_logit_in"])
+                      head_idx=head_idx, mlp_sp_logit=logit)
 
 
 def time_kernel(torch, fn, layers, launches=30, replays=5):
@@ -680,6 +691,9 @@ def main():
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying HIP graphs")
+    ap.add_argument("--no-chain", action="store_true",
+                    help="batch 1: one dv_sparse_layer_decode_f16 call per step (seven launches, every step from the "
+                         "same fixed input) instead of chaining the steps of a graph in one call (six launches each)")
     ap.add_argument("--side-stream", action="store_true",
                     help="module path: predictors / top-k on a side stream, as the reference's sp_stream (slower here)")
     ap.add_argument("--pmc-calibration", action="store_true",
@@ -760,6 +774,34 @@ def main():
             return window_step(layers[l], c)
         return layer_step(layers[i % N_LAYERS])
 
+    chained = batch == 1 and not args.no_chain
+
+    def run_steps(first, count):
+        """Enqueues steps first .. first+count-1.  Batch 1: as ONE call for consecutive blocks of a
+        model (dv_sparse_layers_decode_f16): the residual stream of a step feeds the next step, the
+        layers forming a ring, and the launch that ends a step prepares the next; the predictions a
+        step consumes are the schedule's own (heads re-drawn per position)."""
+        if not chained:
+            for i in range(first, first + count):
+                step_fn(i)
+            return
+        from dejavu_amd.fused_layer import LayerChain
+
+        chain = LayerChain()
+        for i in range(first, first + count):
+            if cycle:
+                c, l = divmod(i % period, N_LAYERS)
+                L = layers[l]
+                head_idx, logit = window_step_inputs(L, c)
+            else:
+                L = layers[i % N_LAYERS]
+                head_idx, logit = layer_step_inputs(L)
+            if len(chain) == 0:
+                chain.add(L["block"], head_idx, logit, L["ip"], L["hidden"], L["residual"])
+            else:
+                chain.add(L["block"], head_idx, logit, L["ip"])
+        chain.run()
+
     graphs = {}
     primed = set()
 
@@ -775,8 +817,7 @@ def main():
                     L["block"].mixer.counter = c0 + (1 if l < (first % period) % N_LAYERS else 0)
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g):
-                for i in range(first, first + count):
-                    step_fn(i)
+                run_steps(first, count)
                 dv_modules.join_side_stream()
             graphs[key] = g
         return graphs[key]
@@ -958,7 +999,12 @@ def main():
         "config": {"workload": f"{args.config} sparse decode layer, batch {batch}, " + what, "d": cfg["d"],
                    "ffn": cfg["ffn"], "heads": cfg["H"], "head_dim": cfg["hd"], "K": cfg["K"],
                    "active_heads": cfg["Hk"], "predictor_rank": cfg["r"], "kv_len": cfg["S"], "batch": batch,
-                   "layers_cycled": N_LAYERS, "window": args.window, "hip_graph": graph_mode},
+                   "layers_cycled": N_LAYERS, "window": args.window, "hip_graph": graph_mode,
+                   "entry_point": ("dv_sparse_layers_decode_f16: the steps of a graph are consecutive blocks of one "
+                                   "call, the residual stream of a step feeds the next (six launches per step)"
+                                   if chained and not args.no_graph else
+                                   "dv_sparse_layer_decode_f16 per step (seven launches)" if batch == 1 else
+                                   "module path")},
         "positions": {"steps_per_window_position": positions, "schedule_period": period},
         "roofline": roofline,
         "mlp_pair": table["mlp_pair"],

@@ -11,6 +11,7 @@
 //   positions reads 1 KiB contiguous per load;  v_cache (B, H, S, hd).
 #pragma once
 #include "common.hpp"
+#include "norm.hpp"
 
 namespace dv {
 
@@ -134,6 +135,160 @@ __global__ __launch_bounds__(256) void qkv_sparse_kernel(
     half_t* __restrict__ v_cache, const int* __restrict__ padding, int S) {
   qkv_sparse_body<NBMAX, R, U>(X, W, bias, head_idx, batch_idx, nb, d, H, hd, nnz, Y, k_cache, v_cache,
                                padding, S, blockIdx.x, gridDim.x);
+}
+
+// The newest token of a back-fill window whose LayerNorm has not been applied yet: the residual
+// stream row, the statistics pairs of its 64-element parts (norm.hpp) and the LayerNorm
+// parameters.  A QKV workgroup normalises the row itself; workgroup 0 also stores the
+// normalised row to `x_row_out` (the token's row of the window buffer).
+struct QkvLnArgs {
+  const half_t* R1;
+  const float2* parts;
+  const half_t* gamma;
+  const half_t* beta;
+  float eps;
+  half_t* x_row_out;
+  int token;  // index of the token in the window (its Y row and cache position offset)
+};
+
+// QKV of the active heads for that one token (every active head computes it: the first position
+// of a window, where nothing is back-filled).  The whole workgroup normalises the row into LDS
+// (xs: d halves) from the precomputed statistics, then every wavefront runs the dot products of
+// qkv_sparse_body<1, R, U> (same products in the same order: the same bits) with x from LDS.
+// NP: statistics pairs per lane (d <= 4096 * NP).
+template <int R, int U, int NP>
+__device__ __forceinline__ void qkv_ln_token_body(
+    const QkvLnArgs& ln, const half_t* __restrict__ W, const half_t* __restrict__ bias,
+    const int* __restrict__ head_idx, int d, int H, int hd, int nnz, half_t* __restrict__ Y,
+    half_t* __restrict__ k_cache, half_t* __restrict__ v_cache, const int* __restrict__ padding, int S,
+    half_t* xs, int block_id, int nblocks) {
+  constexpr int CH = 8 * kWave;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int waves_per_block = blockDim.x >> 6;
+  const int groups_per_head = hd / R;
+  const int ntasks = nnz * 3 * groups_per_head;
+  const int task0 = block_id * waves_per_block + wave;
+
+  // Requests in this order: the statistics pairs and the row (cache hits), then the first batch
+  // of this wavefront's weights.  The load counter retires in order, so the row can be normalised
+  // while the weights are still on their way.
+  const int nvec = d / 8;
+  const int P = (d + kLnPart - 1) / kLnPart;
+  const LnParts<NP> lp = ln_load_parts<NP>(ln.parts, P);
+  constexpr int VB = 3;  // vectors per thread and round; one round when d <= 8 * VB * blockDim.x
+  half8_t xr[VB], xg[VB], xb[VB];
+#pragma unroll
+  for (int j = 0; j < VB; ++j) {
+    const int i = j * blockDim.x + threadIdx.x;
+    if (i < nvec) {
+      xr[j] = load8(ln.R1 + i * 8);
+      xg[j] = load8(ln.gamma + i * 8);
+      xb[j] = load8(ln.beta + i * 8);
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  // first task's first batch (a full batch exists when d >= U * CH; shorter rows start in the loop)
+  constexpr int PRE = U / 2;  // chunks of the first batch requested this early (registers are short here)
+  half8_t w0[PRE][R];
+  bool have_w0 = false;
+  {
+    const int i = task0 < ntasks ? task0 / (3 * groups_per_head) : 0;
+    const int h = task0 < ntasks ? head_idx[i] : -1;
+    if (h >= 0 && h < H && U * CH <= d) {
+      const int rem = task0 - i * 3 * groups_per_head;
+      const int t = rem / groups_per_head;
+      const half_t* wr = W + (((int64_t)t * H + h) * hd + (rem - t * groups_per_head) * R) * d + lane * 8;
+#pragma unroll
+      for (int u = 0; u < PRE; ++u)
+#pragma unroll
+        for (int r = 0; r < R; ++r) w0[u][r] = load8_stream(wr + (int64_t)r * d + u * CH);
+      have_w0 = true;
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  const LnStats st = ln_combine_loaded(lp, P, d, ln.eps);
+#pragma unroll
+  for (int j = 0; j < VB; ++j) {
+    const int i = j * blockDim.x + threadIdx.x;
+    if (i < nvec) {
+      const half8_t o = ln_apply(xr[j], xg[j], xb[j], st);
+      store8(xs + i * 8, o);
+      if (block_id == 0) store8(ln.x_row_out + i * 8, o);
+    }
+  }
+  for (int i = VB * blockDim.x + threadIdx.x; i < nvec; i += blockDim.x) {  // longer rows
+    const half8_t o = ln_apply(load8(ln.R1 + i * 8), load8(ln.gamma + i * 8), load8(ln.beta + i * 8), st);
+    store8(xs + i * 8, o);
+    if (block_id == 0) store8(ln.x_row_out + i * 8, o);
+  }
+  __syncthreads();
+
+  for (int task = task0; task < ntasks; task += nblocks * waves_per_block) {
+    const int i = task / (3 * groups_per_head);
+    const int rem = task - i * 3 * groups_per_head;
+    const int t = rem / groups_per_head;
+    const int j0 = (rem - t * groups_per_head) * R;
+    const int h = head_idx[i];
+    if (h < 0 || h >= H) continue;
+    const int64_t row0 = ((int64_t)t * H + h) * hd + j0;
+    const half_t* wr = W + row0 * d + lane * 8;
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = 0.f;
+    int base = 0;
+    for (; base + U * CH <= d; base += U * CH) {
+      half8_t w[U][R];
+      if (have_w0) {  // part of the batch was requested before the row was normalised
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+          for (int r = 0; r < R; ++r)
+            w[u][r] = u < PRE ? w0[u < PRE ? u : 0][r] : load8_stream(wr + (int64_t)r * d + base + u * CH);
+        have_w0 = false;
+      } else {
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+          for (int r = 0; r < R; ++r) w[u][r] = load8_stream(wr + (int64_t)r * d + base + u * CH);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const half8_t xv = load8(xs + base + u * CH + lane * 8);
+#pragma unroll
+        for (int r = 0; r < R; ++r) acc[r] = dot8_fast(w[u][r], xv, acc[r]);
+      }
+    }
+    for (; base < d; base += CH) {
+      if (base + lane * 8 < d) {
+        half8_t w[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) w[r] = load8_stream(wr + (int64_t)r * d + base);
+        const half8_t xv = load8(xs + base + lane * 8);
+#pragma unroll
+        for (int r = 0; r < R; ++r) acc[r] = dot8_fast(w[r], xv, acc[r]);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      float v = butterfly_sum<kWave>(acc[r]);
+      if (bias != nullptr) v += (float)bias[row0 + r];
+      if (lane == 0) {
+        const half_t hv = (half_t)v;
+        Y[(int64_t)ln.token * 3 * H * hd + row0 + r] = hv;
+        if (t != 0 && k_cache != nullptr) {
+          const int dst = ln.token + (padding ? padding[0] : 0);
+          const int j = j0 + r;
+          if (dst >= 0 && dst < S) {
+            if (t == 1)
+              k_cache[(((int64_t)h * (hd / 8) + j / 8) * S + dst) * 8 + (j & 7)] = hv;
+            else
+              v_cache[((int64_t)h * S + dst) * hd + j] = hv;
+          }
+        }
+      }
+    }
+  }
 }
 
 // ---------------------------------------------------------------------------

@@ -73,6 +73,13 @@ __device__ __forceinline__ int64_t load_index(const void* idx, int idx_bytes, in
                         : (int64_t) reinterpret_cast<const int32_t*>(idx)[i];
 }
 
+// Fixed-point form of an fp32 partial sum: v * 2^32 rounded to the nearest integer.  Integer
+// additions commute, so partial sums added in this form give the same bits in any order.
+__device__ __forceinline__ long long to_fixed(float v) { return __float2ll_rn(v * 4294967296.f); }
+__device__ __forceinline__ float from_fixed(long long a) {
+  return (float)(__ll2double_rn(a) * 2.3283064365386963e-10);
+}
+
 __device__ __forceinline__ float relu_f(float x) { return x >= 0.f ? x : 0.f; }
 
 }  // namespace dv

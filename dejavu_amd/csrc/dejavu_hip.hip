@@ -222,8 +222,8 @@ void launch_cols(const ColsPlan& p, const half_t* x, int64_t ldx, int x_expanded
                      bias, idx, blk, N, Z, M, p.rows_per_block, partial, y);
   if (p.groups > 1) {
     const int64_t total = (int64_t)B * N;
-    hipLaunchKernelGGL(cols_reduce_kernel, dim3((unsigned)((total + 63) / 64)), dim3(256), 0, s,
-                       partial, bias, p.groups, B, N, y);
+    hipLaunchKernelGGL(cols_reduce_kernel<false>, dim3((unsigned)((total + 63) / 64)), dim3(256), 0, s,
+                       partial, bias, p.groups, B, N, y, (const half_t*)nullptr, (half_t*)nullptr);
   }
 }
 
@@ -624,8 +624,8 @@ void launch_cols16(const Cols16Plan& p, const half_t* h, int64_t ldh, int x_expa
                      p.rows_per_block, p.rows_per_wave, partial, y);
   if (p.groups > 1) {
     const int64_t total = (int64_t)B * N;
-    hipLaunchKernelGGL(cols_reduce_kernel, dim3((unsigned)((total + 63) / 64)), dim3(256), 0, s, partial,
-                       bias, p.groups, B, N, y);
+    hipLaunchKernelGGL(cols_reduce_kernel<false>, dim3((unsigned)((total + 63) / 64)), dim3(256), 0, s, partial,
+                       bias, p.groups, B, N, y, (const half_t*)nullptr, (half_t*)nullptr);
   }
 }
 
@@ -637,8 +637,8 @@ void launch_cols_mfma(const ColsMfmaPlan& p, const half_t* h, int64_t ldh, int x
                      s, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M, p.rows_per_block, partial, y);
   if (p.groups > 1) {
     const int64_t total = (int64_t)B * N;
-    hipLaunchKernelGGL(cols_reduce_kernel, dim3((unsigned)((total + 63) / 64)), dim3(256), 0, s, partial,
-                       bias, p.groups, B, N, y);
+    hipLaunchKernelGGL(cols_reduce_kernel<false>, dim3((unsigned)((total + 63) / 64)), dim3(256), 0, s, partial,
+                       bias, p.groups, B, N, y, (const half_t*)nullptr, (half_t*)nullptr);
   }
 }
 
@@ -1392,7 +1392,7 @@ int dv_attention_out_proj_f16(const void* q, int64_t ldq, const void* k_cache, c
 #define DV_AO(BB)                                                                                 \
   hipLaunchKernelGGL((gather_cols_kernel<BB, 8, false, true, true>), grid, dim3(256), 0, s, \
                      (const half_t*)nullptr, (int64_t)0, 1, ww, ldw, bb, head_idx, hd, N, H * hd, M, \
-                     p.rows_per_block, partial, yy, part, nsplit)
+                     p.rows_per_block, partial, yy, part, nsplit, 1)
   switch (B) {
     case 1: DV_AO(1); break;
     case 2: DV_AO(2); break;
@@ -1400,11 +1400,11 @@ int dv_attention_out_proj_f16(const void* q, int64_t ldq, const void* k_cache, c
     default: DV_AO(4); break;
   }
 #undef DV_AO
-  if (p.groups > 1) {
-    const int64_t total = (int64_t)B * N;
-    hipLaunchKernelGGL(cols_reduce_kernel, dim3((unsigned)((total + 63) / 64)), dim3(256), 0, s,
-                       partial, bb, p.groups, B, N, yy);
-  }
+  // the row groups' partial sums are added in fixed point: the same bits as the fused layer step,
+  // which adds them with integer atomics
+  const int64_t total = (int64_t)B * N;
+  hipLaunchKernelGGL(cols_reduce_kernel<true>, dim3((unsigned)((total + 63) / 64)), dim3(256), 0, s, partial, bb,
+                     p.groups, B, N, yy, (const half_t*)nullptr, (half_t*)nullptr);
   return launch_status();
 }
 
@@ -1521,8 +1521,8 @@ int dv_add_layer_norm_f16(const void* h, const void* residual, const void* gamma
 
 namespace {
 struct LayerPlan {
-  size_t off_topk, off_x, off_res1, off_attn_out, off_x2, off_qkv, off_batch_idx, off_hp_hidden,
-      off_mp_hidden, off_h, off_head_logits, off_attn_part, off_cols_part, total;
+  size_t off_topk, off_res1, off_parts, off_acc, off_qkv, off_batch_idx, off_hp_hidden, off_mp_hidden, off_h,
+      off_head_logits, off_attn_part, off_cols_part, total;
   int nsplit;
   ColsPlan out_cols, fc2_cols;
 };
@@ -1534,10 +1534,9 @@ LayerPlan plan_layer(const dvSparseLayerArgs& a) {
   size_t o = 0;
   p.off_topk = o;
   o = align_up(o + dv_topk_workspace_bytes(a.ffn > 1024 ? a.ffn : 2048));
-  p.off_x = o;            o = align_up(o + (size_t)a.d * 2);
   p.off_res1 = o;         o = align_up(o + (size_t)a.d * 2);
-  p.off_attn_out = o;     o = align_up(o + (size_t)a.d * 2);
-  p.off_x2 = o;           o = align_up(o + (size_t)a.d * 2);
+  p.off_parts = o;        o = align_up(o + (size_t)((a.d + kLnPart - 1) / kLnPart) * sizeof(float2));
+  p.off_acc = o;          o = align_up(o + (size_t)a.d * sizeof(long long));
   p.off_qkv = o;          o = align_up(o + (size_t)16 * 3 * a.H * a.hd * 2);
   p.off_batch_idx = o;    o = align_up(o + (size_t)a.H * 16 * 4);
   p.off_hp_hidden = o;    o = align_up(o + (size_t)a.r_att * 2);
@@ -1548,27 +1547,37 @@ LayerPlan plan_layer(const dvSparseLayerArgs& a) {
   p.off_attn_part = o;    o = align_up(o + (size_t)a.Hk * p.nsplit * (a.hd + 2) * 4);
   p.out_cols = plan_cols(a.d, a.Hk * a.hd);
   p.fc2_cols = plan_cols(a.d, a.K);
-  const int g = p.out_cols.groups > p.fc2_cols.groups ? p.out_cols.groups : p.fc2_cols.groups;
-  p.off_cols_part = o;    o = align_up(o + (size_t)g * a.d * 4);
+  p.off_cols_part = o;    o = align_up(o + (size_t)p.fc2_cols.groups * a.d * 4);
   p.total = o;
   return p;
 }
 
-int check_layer_args(const dvSparseLayerArgs& a) {
-  if (!a.hidden || !a.ln1_w || !a.ln1_b || !a.ln2_w || !a.ln2_b || !a.Wqkv || !a.Wout_t || !a.att_Wa ||
+int check_layer_args(const dvSparseLayerArgs& a, bool first) {
+  if (!a.ln1_w || !a.ln1_b || !a.ln2_w || !a.ln2_b || !a.Wqkv || !a.Wout_t || !a.att_Wa ||
       !a.att_Wb || !a.W1 || !a.W2t || !a.mlp_Wa || !a.mlp_Wb || !a.head_idx || !a.mlp_logit_in ||
       !a.cache_offset || !a.k_cache || !a.v_cache || !a.x_cache || !a.tracker || !a.hidden_out ||
-      !a.residual_out || !a.mlp_logit_out || !a.att_idx_out || !a.mlp_idx_out || !a.workspace)
+      !a.residual_out || !a.mlp_logit_out || !a.att_idx_out || !a.mlp_idx_out)
     return DV_ERR_INVALID_ARG;
+  if (first && (!a.hidden || !a.workspace)) return DV_ERR_INVALID_ARG;
   if (a.d <= 0 || a.ffn <= 0 || a.H <= 0 || a.Hk < 1 || a.Hk > a.H || a.att_k < 1 || a.att_k > a.H ||
       a.K < 1 || a.K > a.ffn || a.r_att <= 0 || a.r_mlp <= 0 || a.S <= 0 || a.n_len < 1 || a.n_len > a.S ||
       a.counter < 0 || a.counter > 15 || (a.counter == 15 && a.Hk != a.H))
     return DV_ERR_INVALID_ARG;
   if ((a.hd != 64 && a.hd != 128) || a.H * a.hd != a.d || a.H > 1024 || a.ffn > 65536 || a.ffn <= 1024 ||
-      a.d > 1024 * 8 * 4 || (size_t)a.d * 2 > 160 * 1024)
+      a.d > 1024 * 8 * 4 || (size_t)a.d * 2 > 144 * 1024)
     return DV_ERR_UNSUPPORTED;
   if (a.d % 8 || a.ffn % 8 || a.r_att % 8 || a.r_mlp % 8) return DV_ERR_ALIGNMENT;
   return DV_OK;
+}
+
+// the scratch of a call is the first block's; every block of the call needs no more than it holds
+size_t layers_workspace_bytes(const dvSparseLayerArgs* layers, int n) {
+  size_t need = 0;
+  for (int l = 0; l < n; ++l) {
+    const size_t t = plan_layer(layers[l]).total;
+    if (t > need) need = t;
+  }
+  return need;
 }
 }  // namespace
 
@@ -1577,149 +1586,194 @@ size_t dv_sparse_layer_workspace_bytes(const dvSparseLayerArgs* args) {
   return plan_layer(*args).total;
 }
 
-int dv_sparse_layer_decode_f16(const dvSparseLayerArgs* args, void* stream) {
-  if (!args) return DV_ERR_INVALID_ARG;
-  const dvSparseLayerArgs& a = *args;
-  int rc = check_layer_args(a);
-  if (rc != DV_OK) return rc;
-  const LayerPlan p = plan_layer(a);
-  if (a.workspace_bytes < p.total || !aligned16(a.workspace)) return DV_ERR_WORKSPACE;
+int dv_sparse_layers_decode_f16(const dvSparseLayerArgs* layers, int n_layers, void* stream) {
+  if (!layers || n_layers < 1) return DV_ERR_INVALID_ARG;
+  for (int l = 0; l < n_layers; ++l) {
+    const int rc = check_layer_args(layers[l], l == 0);
+    if (rc != DV_OK) return rc;
+    // one residual stream, and the scratch regions that travel from a block to the next at fixed offsets
+    if (layers[l].d != layers[0].d || layers[l].ffn != layers[0].ffn || layers[l].H != layers[0].H)
+      return DV_ERR_INVALID_ARG;
+  }
+  if (layers[0].workspace_bytes < layers_workspace_bytes(layers, n_layers) || !aligned16(layers[0].workspace))
+    return DV_ERR_WORKSPACE;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  unsigned char* ws = reinterpret_cast<unsigned char*>(a.workspace);
-  auto H16 = [&](size_t off) { return reinterpret_cast<half_t*>(ws + off); };
+  unsigned char* ws = reinterpret_cast<unsigned char*>(layers[0].workspace);
   auto CH = [](const void* q) { return reinterpret_cast<const half_t*>(q); };
-  unsigned* topk_ws = reinterpret_cast<unsigned*>(ws + p.off_topk);
-  int* batch_idx = reinterpret_cast<int*>(ws + p.off_batch_idx);
-  float* attn_part = reinterpret_cast<float*>(ws + p.off_attn_part);
-  float* cols_part = reinterpret_cast<float*>(ws + p.off_cols_part);
-  half_t* x = H16(p.off_x);
-  half_t* res1 = H16(p.off_res1);
-  half_t* attn_out = H16(p.off_attn_out);
-  half_t* qkv = H16(p.off_qkv);
-  half_t* hp_hidden = H16(p.off_hp_hidden);
-  half_t* mp_hidden = H16(p.off_mp_hidden);
-  half_t* hbuf = H16(p.off_h);
-  half_t* head_logits = H16(p.off_head_logits);
-  half_t* x_cache = reinterpret_cast<half_t*>(a.x_cache);
-  const int* head_idx = reinterpret_cast<const int*>(a.head_idx);
   const int cus = compute_units();
-  const int nb = a.counter + 1;
-  const int topk_blocks = (a.ffn + kTopkItemsPerBlock - 1) / kTopkItemsPerBlock;
+  const int d = layers[0].d;
+  const int nred = (d + 63) / 64;
 
-  // L1: add + LayerNorm 1 + window step | key histogram of this layer's MLP logits
-  {
-    const int hist_blocks = topk_blocks;  // 256 * 8 columns each
-#define DV_L1(V)                                                                                      \
-  hipLaunchKernelGGL((layer_l1_kernel<V>), dim3(1 + hist_blocks), dim3(kLnThreads), 0, s, CH(a.hidden),   \
-                     CH(a.residual), CH(a.ln1_w), CH(a.ln1_b), a.eps1, a.d, x, res1,                     \
-                     x_cache + (size_t)a.counter * a.d, reinterpret_cast<int*>(a.tracker), head_idx, a.Hk, \
-                     a.H, a.counter, a.counter == 15 ? 1 : 0, batch_idx, CH(a.mlp_logit_in), a.ffn, topk_ws)
-    if (a.d <= kLnThreads * 8) DV_L1(1);
-    else if (a.d <= kLnThreads * 16) DV_L1(2);
-    else DV_L1(4);
-#undef DV_L1
-  }
-  // L2: QKV + cache scatter
-  {
-    QkvArgs q{x_cache, CH(a.Wqkv), CH(a.bqkv), head_idx, batch_idx, nb, a.d, a.H, a.hd, a.Hk, qkv,
-              reinterpret_cast<half_t*>(a.k_cache), reinterpret_cast<half_t*>(a.v_cache),
-              reinterpret_cast<const int*>(a.cache_offset), a.S};
-    const bool mfma = qkv_use_mfma(nb);
-    const int ntasks = a.Hk * 3 * (a.hd / 2);
-    int nq = (ntasks + 3) / 4;
-    if (nq > cus * 8) nq = cus * 8;
-    const bool two = mfma && qkv_mfma_two_tiles(a.Hk, a.hd);
-    if (mfma) nq = a.Hk * 3 * (a.hd / (two ? 32 : 16));
-    const dim3 grid(nq);
-#define DV_L2(NB) hipLaunchKernelGGL((layer_l2_kernel<NB>), grid, dim3(256), 0, s, q)
-    if (two) DV_L2(-1);
-    else if (mfma) DV_L2(0);
-    else DV_L2(1);
-#undef DV_L2
-  }
-  // L3: attention partials | head predictor fc0 | top-k threshold and counts.  The head predictor
-  // (input: the residual stream after L1, output: only needed at the end of the step) runs one
-  // launch later than it could: the QKV launch is the fullest one, this one has bandwidth to spare.
-  const int nsplit = a.seq_pos ? p.nsplit : attn_splits(a.n_len);
-  {
-    AttnArgs at{qkv + (size_t)a.counter * 3 * a.H * a.hd, (int64_t)3 * a.H * a.hd,
-                reinterpret_cast<const half_t*>(a.k_cache), reinterpret_cast<const half_t*>(a.v_cache),
-                head_idx, reinterpret_cast<const int*>(a.seq_pos), a.n_len, a.H, a.S, nsplit, a.Hk,
-                a.softmax_scale, attn_part};
-    CanonArgs hp0{res1, CH(a.att_Wa), (int64_t)a.d, a.r_att, a.d, hp_hidden};
-    const int na = nsplit * a.Hk;
-    const int rw0 = a.d <= 1024 ? 4 * kCanonShortRows : 1;
-    const int nh = ((a.r_att + rw0 - 1) / rw0 + 3) / 4;
-    const dim3 grid(na + nh + topk_blocks);
-    int* advance_ptr = (a.counter == 15 && a.advance_window) ? reinterpret_cast<int*>(a.cache_offset) : nullptr;
-    if (a.hd == 128)
-      hipLaunchKernelGGL((layer_l3_kernel<128>), grid, dim3(256), 0, s, at, na, hp0, nh, CH(a.mlp_logit_in),
-                         a.ffn, a.K, topk_ws, advance_ptr, 16);
-    else
-      hipLaunchKernelGGL((layer_l3_kernel<64>), grid, dim3(256), 0, s, at, na, hp0, nh, CH(a.mlp_logit_in),
-                         a.ffn, a.K, topk_ws, advance_ptr, 16);
-  }
-  // L4 + L5: out_proj from the attention partials | head predictor fc1 | top-k emission; split reduction
-  {
-    const ColsPlan& c = p.out_cols;
-    OutProjArgs o{CH(a.Wout_t), (int64_t)a.d, CH(a.bout), head_idx, a.hd, a.d, a.H * a.hd, a.Hk * a.hd,
-                  c.rows_per_block, c.col_tiles, c.groups, cols_part, attn_out, attn_part, nsplit};
-    CanonArgs hp1{hp_hidden, CH(a.att_Wb), (int64_t)a.r_att, a.H, a.r_att, head_logits};
-    const int rw1 = a.r_att <= 1024 ? 4 * kCanonShortRows : 1;
-    const int nh1 = ((a.H + rw1 - 1) / rw1 + 3) / 4;
-    const int no = c.col_tiles * c.groups;
-    hipLaunchKernelGGL(layer_l4_kernel, dim3(no + nh1 + topk_blocks), dim3(256), 0, s, o, no, hp1, nh1,
-                       CH(a.mlp_logit_in), a.ffn, a.K, topk_ws, reinterpret_cast<int64_t*>(a.mlp_idx_out),
-                       topk_blocks);
-    // L5: split reduction + bias, and the residual stream advanced by the attention output
-    hipLaunchKernelGGL(cols_reduce_kernel, dim3((unsigned)((a.d + 63) / 64)), dim3(256), 0, s,
-                       c.groups > 1 ? cols_part : nullptr, CH(a.bout), c.groups, 1, a.d, attn_out, res1,
-                       reinterpret_cast<half_t*>(a.residual_out));
-  }
-  const half_t* res2 = reinterpret_cast<const half_t*>(a.residual_out);
-  const int64_t* mlp_idx = reinterpret_cast<const int64_t*>(a.mlp_idx_out);
-  // L7: LayerNorm 2 + fc1 gather | MLP predictor fc0 | head top-k
-  {
-    RowsArgs f{res2, CH(a.ln2_w), CH(a.ln2_b), a.eps2, CH(a.W1), CH(a.b1), mlp_idx, a.d, (int64_t)a.d, a.ffn,
-               a.K, hbuf};
-    int nf = ((a.K + 1) / 2 + 3) / 4;
-    if (nf > cus * 8) nf = cus * 8;
-    CanonArgs mp0{res2, CH(a.mlp_Wa), (int64_t)a.d, a.r_mlp, a.d, mp_hidden};
-    const int rw0 = a.d <= 1024 ? 4 * kCanonShortRows : 1;
-    const int nm = ((a.r_mlp + rw0 - 1) / rw0 + 3) / 4;
-    const size_t lds = (size_t)a.d * sizeof(half_t);
-    const int v = a.d <= 8192 ? 0 : (a.d <= 16384 ? 1 : 2);
-    const void* l7[3] = {reinterpret_cast<const void*>(layer_l7_kernel<1>),
-                         reinterpret_cast<const void*>(layer_l7_kernel<2>),
-                         reinterpret_cast<const void*>(layer_l7_kernel<4>)};
-    static LdsGrant grant[3];
-    if (int rc = grant[v].ensure(l7[v], lds); rc != DV_OK) return rc;
-    int* att_out = reinterpret_cast<int*>(a.att_idx_out);
-    const dim3 grid(nf + nm + 1);  // + the head top-k
-    if (v == 0)
-      hipLaunchKernelGGL(layer_l7_kernel<1>, grid, dim3(256), lds, s, f, nf, mp0, nm, head_logits, a.H, a.att_k, att_out);
-    else if (v == 1)
-      hipLaunchKernelGGL(layer_l7_kernel<2>, grid, dim3(256), lds, s, f, nf, mp0, nm, head_logits, a.H, a.att_k, att_out);
-    else
-      hipLaunchKernelGGL(layer_l7_kernel<4>, grid, dim3(256), lds, s, f, nf, mp0, nm, head_logits, a.H, a.att_k, att_out);
-  }
-  // L8 + L9: fc2 gather | MLP predictor fc1, then the split reduction
-  {
+  // P of block l: residual add (or the split reduction of block l - 1's fc2) + part statistics |
+  // key histogram of block l's MLP logits | block l's window step.  prev == nullptr: the call's input.
+  auto launch_pre = [&](const dvSparseLayerArgs* prev, const dvSparseLayerArgs& a) {
+    const LayerPlan p = plan_layer(a);
+    PreArgs pa;
+    if (prev == nullptr) {
+      pa.partial = nullptr;
+      pa.bias = nullptr;
+      pa.G = 1;
+      pa.Y = const_cast<half_t*>(CH(a.hidden));
+      pa.R = CH(a.residual);
+    } else {
+      const LayerPlan pp = plan_layer(*prev);
+      // a single row group has stored the finished row itself
+      pa.partial = pp.fc2_cols.groups > 1 ? reinterpret_cast<const float*>(ws + pp.off_cols_part) : nullptr;
+      pa.bias = CH(prev->b2);
+      pa.G = pp.fc2_cols.groups;
+      pa.Y = reinterpret_cast<half_t*>(prev->hidden_out);
+      pa.R = CH(prev->residual_out);
+    }
+    pa.d = d;
+    pa.Rout = reinterpret_cast<half_t*>(ws + p.off_res1);
+    pa.parts = reinterpret_cast<float2*>(ws + p.off_parts);
+    pa.mlp_logits = CH(a.mlp_logit_in);
+    pa.ffn = a.ffn;
+    pa.topk_ws = reinterpret_cast<unsigned*>(ws + p.off_topk);
+    pa.tracker = reinterpret_cast<int*>(a.tracker);
+    pa.head_idx = reinterpret_cast<const int*>(a.head_idx);
+    pa.nnz = a.Hk;
+    pa.H = a.H;
+    pa.counter = a.counter;
+    pa.flush = a.counter == 15 ? 1 : 0;
+    pa.batch_idx = reinterpret_cast<int*>(ws + p.off_batch_idx);
+    const int nhist = (a.ffn + kTopkItemsPerBlock - 1) / kTopkItemsPerBlock;
+    hipLaunchKernelGGL(layer_pre_kernel, dim3(nred + nhist + 1), dim3(256), 0, s, pa, nred, nhist);
+  };
+
+  for (int l = 0; l < n_layers; ++l) {
+    const dvSparseLayerArgs& a = layers[l];
+    const LayerPlan p = plan_layer(a);
+    auto H16 = [&](size_t off) { return reinterpret_cast<half_t*>(ws + off); };
+    unsigned* topk_ws = reinterpret_cast<unsigned*>(ws + p.off_topk);
+    int* batch_idx = reinterpret_cast<int*>(ws + p.off_batch_idx);
+    float* attn_part = reinterpret_cast<float*>(ws + p.off_attn_part);
+    float* cols_part = reinterpret_cast<float*>(ws + p.off_cols_part);
+    long long* acc = reinterpret_cast<long long*>(ws + p.off_acc);
+    half_t* res1 = H16(p.off_res1);
+    half_t* qkv = H16(p.off_qkv);
+    half_t* hp_hidden = H16(p.off_hp_hidden);
+    half_t* mp_hidden = H16(p.off_mp_hidden);
+    half_t* hbuf = H16(p.off_h);
+    half_t* head_logits = H16(p.off_head_logits);
+    half_t* x_cache = reinterpret_cast<half_t*>(a.x_cache);
+    const int* head_idx = reinterpret_cast<const int*>(a.head_idx);
+    const int nb = a.counter + 1;
+    const int topk_blocks = (a.ffn + kTopkItemsPerBlock - 1) / kTopkItemsPerBlock;
+
+    if (l == 0) launch_pre(nullptr, a);
+    // L2: LayerNorm 1 + QKV + cache scatter
+    {
+      QkvArgs q{x_cache, CH(a.Wqkv), CH(a.bqkv), head_idx, batch_idx, nb, a.d, a.H, a.hd, a.Hk, qkv,
+                reinterpret_cast<half_t*>(a.k_cache), reinterpret_cast<half_t*>(a.v_cache),
+                reinterpret_cast<const int*>(a.cache_offset), a.S,
+                QkvLnArgs{res1, reinterpret_cast<const float2*>(ws + p.off_parts), CH(a.ln1_w), CH(a.ln1_b), a.eps1,
+                          x_cache + (size_t)a.counter * a.d, a.counter}};
+      const bool mfma = qkv_use_mfma(nb);
+      const bool two = mfma && qkv_mfma_two_tiles(a.Hk, a.hd);
+      if (mfma) {
+        const dim3 grid(a.Hk * 3 * (a.hd / (two ? 32 : 16)));
+        if (two) hipLaunchKernelGGL((layer_l2_kernel<-1>), grid, dim3(256), 0, s, q);
+        else hipLaunchKernelGGL((layer_l2_kernel<0>), grid, dim3(256), 0, s, q);
+      } else {
+        // one task (two weight rows) per wavefront; workgroups of eight wavefronts when that still
+        // leaves two per compute unit (fewer copies of the row to normalise), else of four
+        const int ntasks = a.Hk * 3 * (a.hd / 2);
+        const int waves = ntasks >= cus * 16 ? 8 : 4;
+        int nq = (ntasks + waves - 1) / waves;
+        if (nq > cus * (24 / waves)) nq = cus * (24 / waves);
+        const size_t lds = (size_t)a.d * sizeof(half_t);
+        static LdsGrant grant[2];
+        if (a.d <= 16384) {
+          if (int rc = grant[0].ensure(reinterpret_cast<const void*>(layer_l2_kernel<1>), lds); rc != DV_OK) return rc;
+          hipLaunchKernelGGL((layer_l2_kernel<1>), dim3(nq), dim3(waves * 64), lds, s, q);
+        } else {
+          if (int rc = grant[1].ensure(reinterpret_cast<const void*>(layer_l2_kernel<2>), lds); rc != DV_OK) return rc;
+          hipLaunchKernelGGL((layer_l2_kernel<2>), dim3(nq), dim3(waves * 64), lds, s, q);
+        }
+      }
+    }
+    // L3: attention partials | head predictor fc0 | top-k threshold and counts | accumulator reset.
+    // The head predictor (input: the residual stream, output: only needed at the end of the step)
+    // runs one launch later than it could: the QKV launch is the fullest one, this one has
+    // bandwidth to spare.
+    const int nsplit = a.seq_pos ? p.nsplit : attn_splits(a.n_len);
+    {
+      AttnArgs at{qkv + (size_t)a.counter * 3 * a.H * a.hd, (int64_t)3 * a.H * a.hd,
+                  reinterpret_cast<const half_t*>(a.k_cache), reinterpret_cast<const half_t*>(a.v_cache),
+                  head_idx, reinterpret_cast<const int*>(a.seq_pos), a.n_len, a.H, a.S, nsplit, a.Hk,
+                  a.softmax_scale, attn_part};
+      CanonArgs hp0{res1, CH(a.att_Wa), (int64_t)a.d, a.r_att, a.d, hp_hidden};
+      const int na = nsplit * a.Hk;
+      const int rw0 = a.d <= 1024 ? 4 * kCanonShortRows : 1;
+      const int nh = ((a.r_att + rw0 - 1) / rw0 + 3) / 4;
+      const dim3 grid(na + nh + topk_blocks + 1);
+      int* advance_ptr = (a.counter == 15 && a.advance_window) ? reinterpret_cast<int*>(a.cache_offset) : nullptr;
+      if (a.hd == 128)
+        hipLaunchKernelGGL((layer_l3_kernel<128>), grid, dim3(256), 0, s, at, na, hp0, nh, CH(a.mlp_logit_in),
+                           a.ffn, a.K, topk_ws, advance_ptr, 16, acc, a.d);
+      else
+        hipLaunchKernelGGL((layer_l3_kernel<64>), grid, dim3(256), 0, s, at, na, hp0, nh, CH(a.mlp_logit_in),
+                           a.ffn, a.K, topk_ws, advance_ptr, 16, acc, a.d);
+    }
+    // L4: out_proj from the attention partials, sums added in fixed point | head predictor fc1 | top-k emission
+    {
+      const ColsPlan& c = p.out_cols;
+      OutProjArgs o{CH(a.Wout_t), (int64_t)a.d, CH(a.bout), head_idx, a.hd, a.d, a.H * a.hd, a.Hk * a.hd,
+                    c.rows_per_block, c.col_tiles, c.groups, acc, attn_part, nsplit};
+      CanonArgs hp1{hp_hidden, CH(a.att_Wb), (int64_t)a.r_att, a.H, a.r_att, head_logits};
+      const int rw1 = a.r_att <= 1024 ? 4 * kCanonShortRows : 1;
+      const int nh1 = ((a.H + rw1 - 1) / rw1 + 3) / 4;
+      const int no = c.col_tiles * c.groups;
+      hipLaunchKernelGGL(layer_l4_kernel, dim3(no + nh1 + topk_blocks), dim3(256), 0, s, o, no, hp1, nh1,
+                         CH(a.mlp_logit_in), a.ffn, a.K, topk_ws, reinterpret_cast<int64_t*>(a.mlp_idx_out),
+                         topk_blocks);
+    }
+    const half_t* res2 = reinterpret_cast<const half_t*>(a.residual_out);
+    const int64_t* mlp_idx = reinterpret_cast<const int64_t*>(a.mlp_idx_out);
+    // L7: residual add + LayerNorm 2 + fc1 gather | MLP predictor fc0 | head top-k
+    {
+      RowsArgs f{acc, CH(a.bout), res1, reinterpret_cast<half_t*>(a.residual_out), CH(a.ln2_w), CH(a.ln2_b), a.eps2,
+                 CH(a.W1), CH(a.b1), mlp_idx, a.d, (int64_t)a.d, a.ffn, a.K, hbuf};
+      const int tasks = (a.K + 1) / 2;  // two gathered rows per wavefront
+      const int waves = tasks >= cus * 8 ? 8 : 4;
+      int nf = (tasks + waves - 1) / waves;
+      if (nf > cus * (32 / waves)) nf = cus * (32 / waves);
+      CanonArgs mp0{res2, CH(a.mlp_Wa), (int64_t)a.d, a.r_mlp, a.d, mp_hidden};
+      const int rw0 = a.d <= 1024 ? 4 * kCanonShortRows : 1;
+      const int nm = ((a.r_mlp + rw0 - 1) / rw0 + waves - 1) / waves;
+      const size_t lds = (size_t)a.d * sizeof(half_t);
+      static LdsGrant grant;
+      if (int rc = grant.ensure(reinterpret_cast<const void*>(layer_l7_kernel), lds); rc != DV_OK) return rc;
+      hipLaunchKernelGGL(layer_l7_kernel, dim3(nf + nm + 1), dim3(waves * 64), lds, s, f, nf, mp0, nm, head_logits,
+                         a.H, a.att_k, reinterpret_cast<int*>(a.att_idx_out));
+    }
+    // L8: fc2 gather | MLP predictor fc1
     const ColsPlan& c = p.fc2_cols;
-    ColsArgs cc{hbuf, CH(a.W2t), (int64_t)a.d, mlp_idx, a.d, a.ffn, a.K, c.rows_per_block, c.col_tiles, c.groups,
-                cols_part, reinterpret_cast<half_t*>(a.hidden_out), CH(a.b2)};
-    CanonArgs mp1{mp_hidden, CH(a.mlp_Wb), (int64_t)a.r_mlp, a.ffn, a.r_mlp,
-                  reinterpret_cast<half_t*>(a.mlp_logit_out)};
-    const int rw1 = a.r_mlp <= 1024 ? 4 * kCanonShortRows : 1;
-    int nm = ((a.ffn + rw1 - 1) / rw1 + 3) / 4;
-    if (nm > cus * 16) nm = cus * 16;
-    const int nf = c.col_tiles * c.groups;
-    hipLaunchKernelGGL(layer_l8_kernel, dim3(nf + nm), dim3(256), 0, s, cc, nf, mp1, nm);
-    if (c.groups > 1)
-      hipLaunchKernelGGL(cols_reduce_kernel, dim3((unsigned)((a.d + 63) / 64)), dim3(256), 0, s, cols_part,
-                         CH(a.b2), c.groups, 1, a.d, reinterpret_cast<half_t*>(a.hidden_out));
+    {
+      ColsArgs cc{hbuf, CH(a.W2t), (int64_t)a.d, mlp_idx, a.d, a.ffn, a.K, c.rows_per_block, c.col_tiles, c.groups,
+                  cols_part, reinterpret_cast<half_t*>(a.hidden_out), CH(a.b2)};
+      CanonArgs mp1{mp_hidden, CH(a.mlp_Wb), (int64_t)a.r_mlp, a.ffn, a.r_mlp,
+                    reinterpret_cast<half_t*>(a.mlp_logit_out)};
+      const int rw1 = a.r_mlp <= 1024 ? 4 * kCanonShortRows : 1;
+      int nm = ((a.ffn + rw1 - 1) / rw1 + 3) / 4;
+      if (nm > cus * 16) nm = cus * 16;
+      const int nf = c.col_tiles * c.groups;
+      hipLaunchKernelGGL(layer_l8_kernel, dim3(nf + nm), dim3(256), 0, s, cc, nf, mp1, nm);
+    }
+    // L9: the split reduction; with another block behind it, that block's P
+    if (l + 1 < n_layers)
+      launch_pre(&a, layers[l + 1]);
+    else if (c.groups > 1)
+      hipLaunchKernelGGL(cols_reduce_kernel<false>, dim3((unsigned)nred), dim3(256), 0, s, cols_part, CH(a.b2),
+                         c.groups, 1, a.d, reinterpret_cast<half_t*>(a.hidden_out), (const half_t*)nullptr,
+                         (half_t*)nullptr);
   }
   return launch_status();
+}
+
+int dv_sparse_layer_decode_f16(const dvSparseLayerArgs* args, void* stream) {
+  return dv_sparse_layers_decode_f16(args, 1, stream);
 }
 
 }  // extern "C"

@@ -8,6 +8,7 @@
 // against 20.2 us for fc2 at the OPT-175B shape.)
 #pragma once
 #include "common.hpp"
+#include "norm.hpp"
 
 namespace dv {
 
@@ -21,13 +22,16 @@ constexpr int kColTile = 8 * kWave;  // 512 columns per workgroup
 // fly from the un-normalised attention partials { max, sum, o[blk] } of
 // decode_attn_kernel (attn_nsplit splits per head), rounded to fp16 as a
 // stored context vector would be.
-template <int B, int U, bool IDX64, bool BLOCKED, bool ATTN>
+// FIXED: the workgroup adds its partial sums, in fixed point, to acc_fixed (B, N) with 64-bit
+// integer atomics instead of storing an fp32 partial per row group; acc_fixed must hold zeros
+// when the launch starts.
+template <int B, int U, bool IDX64, bool BLOCKED, bool ATTN, bool FIXED = false>
 __device__ __forceinline__ void gather_cols_body(
     const half_t* __restrict__ X, int64_t ldx, int x_expanded, const half_t* __restrict__ W,
     int64_t ldw, const half_t* __restrict__ bias, const void* __restrict__ idx, int blk, int N,
     int Z, int M, int rows_per_block, float* __restrict__ partial,
     half_t* __restrict__ Y, const float* __restrict__ attn_part, int attn_nsplit, int ct, int g,
-    int G) {
+    int G, long long* __restrict__ acc_fixed = nullptr) {
   __shared__ float red[4][B][kColTile];
 
   const int tid = threadIdx.x;
@@ -199,6 +203,18 @@ __device__ __forceinline__ void gather_cols_body(
     sum[j] = (red[0][b][c] + red[1][b][c]) + (red[2][b][c] + red[3][b][c]);
   }
 
+  if constexpr (FIXED) {
+#pragma unroll
+    for (int j = 0; j < PER_THREAD; ++j) {
+      const int o = j * 256 + tid;
+      const int b = o / kColTile, c = ct * kColTile + o % kColTile;
+      if (c < N)
+        __hip_atomic_fetch_add(reinterpret_cast<unsigned long long*>(acc_fixed) + (int64_t)b * N + c,
+                               (unsigned long long)to_fixed(sum[j]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    return;
+  }
+
   if (G == 1) {
 #pragma unroll
     for (int j = 0; j < PER_THREAD; ++j) {
@@ -222,59 +238,107 @@ __global__ __launch_bounds__(256) void gather_cols_kernel(
     const half_t* __restrict__ X, int64_t ldx, int x_expanded, const half_t* __restrict__ W,
     int64_t ldw, const half_t* __restrict__ bias, const void* __restrict__ idx, int blk, int N,
     int Z, int M, int rows_per_block, float* __restrict__ partial,
-    half_t* __restrict__ Y, const float* __restrict__ attn_part = nullptr, int attn_nsplit = 0) {
+    half_t* __restrict__ Y, const float* __restrict__ attn_part = nullptr, int attn_nsplit = 0,
+    int always_partial = 0) {
+  // always_partial: a single row group also stores its partial (the caller runs the reduction)
   gather_cols_body<B, U, IDX64, BLOCKED, ATTN>(X, ldx, x_expanded, W, ldw, bias, idx, blk, N, Z, M,
                                                      rows_per_block, partial, Y, attn_part,
-                                                     attn_nsplit, blockIdx.x, blockIdx.y, gridDim.y);
+                                                     attn_nsplit, blockIdx.x, blockIdx.y,
+                                                     always_partial ? 0 : (int)gridDim.y);
 }
 
 // Second pass of the non-fused path: Y[b, c] = fp16(sum_g partial[g, b, c] + bias[c]).
 // A workgroup owns 64 outputs; its four wavefronts each add every fourth group
 // (ascending), and the four slice sums are combined in a fixed order.
+// FIXED: every partial is first brought to fixed point (to_fixed) and the sum is an integer sum:
+// the same bits as the partials added with integer atomics in any order (gather_cols_body<FIXED>).
 // With R / Rout (optional) the residual stream is advanced in the same pass:
-// Rout[b, c] = fp16(Y[b, c] + R[b, c]), the rounded sum of the two fp16 values.
+// Rout[b, c] = fp16(Y[b, c] + R[b, c]), the rounded sum of the two fp16 values (R == nullptr: Rout = Y).
 // partial == nullptr: Y already holds the result, only the residual add is done.
+// parts (optional, B == 1): the LayerNorm statistics pair of the 64 values this workgroup stored
+// to Rout (norm.hpp), parts[block_id].
+template <bool FIXED>
+__device__ __forceinline__ void cols_reduce_body(const float* __restrict__ partial,
+                                                 const half_t* __restrict__ bias, int G, int B, int N,
+                                                 half_t* __restrict__ Y, const half_t* __restrict__ R,
+                                                 half_t* __restrict__ Rout, float2* __restrict__ parts,
+                                                 int block_id) {
+  __shared__ float red[4][kWave];
+  __shared__ long long redq[FIXED ? 4 : 1][FIXED ? kWave : 1];
+  __shared__ __attribute__((aligned(16))) half_t s_row[kWave];
+  const int lane = threadIdx.x & 63;
+  const int slice = threadIdx.x >> 6;
+  const int64_t total = (int64_t)B * N;
+  const int64_t o = (int64_t)block_id * kWave + lane;
+  half_t out = (half_t)0.f;  // the value stored to Rout (slice 0)
+  if (partial == nullptr) {  // Y is complete already (single row group): only the residual add
+    if (slice != 0) return;
+    if (o < total && Rout != nullptr) {
+      out = R != nullptr ? (half_t)((float)Y[o] + (float)R[o]) : Y[o];
+      Rout[o] = out;
+    }
+  } else {
+    // bias and residual are requested together with the partial sums, not after the barrier
+    float bv = 0.f, rv = 0.f;
+    if (slice == 0 && o < total) {
+      if (bias != nullptr) bv = (float)bias[o % N];
+      if (Rout != nullptr && R != nullptr) rv = (float)R[o];
+    }
+    float s = 0.f;
+    long long sq = 0;
+    if (o < total) {
+      const float* p = partial + o;
+      int gg = slice;
+      for (; gg + 28 < G; gg += 32) {
+        float v[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) v[q] = p[(int64_t)(gg + 4 * q) * total];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+          if (FIXED) sq += to_fixed(v[q]);
+          else s += v[q];
+        }
+      }
+      for (; gg < G; gg += 4) {
+        if (FIXED) sq += to_fixed(p[(int64_t)gg * total]);
+        else s += p[(int64_t)gg * total];
+      }
+    }
+    if (FIXED) redq[slice][lane] = sq;
+    else red[slice][lane] = s;
+    __syncthreads();
+    if (slice != 0) return;
+    if (o < total) {
+      const float r = FIXED ? from_fixed((redq[0][lane] + redq[1][lane]) + (redq[2][lane] + redq[3][lane]))
+                            : (red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]);
+      const half_t y = (half_t)(r + bv);
+      if (Y != nullptr) Y[o] = y;
+      if (Rout != nullptr) {
+        out = R != nullptr ? (half_t)((float)y + rv) : y;
+        Rout[o] = out;
+      }
+    }
+  }
+  if (parts != nullptr) {  // wavefront 0 only (B == 1)
+    s_row[lane] = out;  // lanes past the row end hold 0 and are not counted
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    int n_p = N - block_id * kWave;
+    if (n_p > kWave) n_p = kWave;
+    const bool present = lane < 8 && lane * 8 < n_p;
+    const half8_t v = present ? load8(s_row + lane * 8) : zero8();
+    const float2 st = ln_part_stats_lanes8(v, present, n_p);
+    if (lane == 0) parts[block_id] = st;
+  }
+}
+
+template <bool FIXED = false>
 __global__ __launch_bounds__(256) void cols_reduce_kernel(const float* __restrict__ partial,
                                                           const half_t* __restrict__ bias, int G,
                                                           int B, int N, half_t* __restrict__ Y,
                                                           const half_t* __restrict__ R = nullptr,
                                                           half_t* __restrict__ Rout = nullptr) {
-  __shared__ float red[4][kWave];
-  const int lane = threadIdx.x & 63;
-  const int slice = threadIdx.x >> 6;
-  const int64_t total = (int64_t)B * N;
-  const int64_t o = (int64_t)blockIdx.x * kWave + lane;
-  if (partial == nullptr) {  // Y is complete already (single row group): only the residual add
-    if (slice == 0 && o < total && Rout != nullptr) Rout[o] = (half_t)((float)Y[o] + (float)R[o]);
-    return;
-  }
-  // bias and residual are requested together with the partial sums, not after the barrier
-  float bv = 0.f, rv = 0.f;
-  if (slice == 0 && o < total) {
-    if (bias != nullptr) bv = (float)bias[o % N];
-    if (Rout != nullptr) rv = (float)R[o];
-  }
-  float s = 0.f;
-  if (o < total) {
-    const float* p = partial + o;
-    int gg = slice;
-    for (; gg + 28 < G; gg += 32) {
-      float v[8];
-#pragma unroll
-      for (int q = 0; q < 8; ++q) v[q] = p[(int64_t)(gg + 4 * q) * total];
-#pragma unroll
-      for (int q = 0; q < 8; ++q) s += v[q];
-    }
-    for (; gg < G; gg += 4) s += p[(int64_t)gg * total];
-  }
-  red[slice][lane] = s;
-  __syncthreads();
-  if (slice == 0 && o < total) {
-    const float r = (red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]);
-    const half_t y = (half_t)(r + bv);
-    Y[o] = y;
-    if (Rout != nullptr) Rout[o] = (half_t)((float)y + rv);
-  }
+  cols_reduce_body<FIXED>(partial, bias, G, B, N, Y, R, Rout, nullptr, blockIdx.x);
 }
 
 }  // namespace dv

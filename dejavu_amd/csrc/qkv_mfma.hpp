@@ -24,6 +24,7 @@
 // where the x reads are as large as the weight reads).  Each accumulator sees
 // the same operands in the same order as with TILES = 1: identical bits.
 #pragma once
+#include "attention.hpp"
 #include "common.hpp"
 #include "gemm_mfma.hpp"
 
@@ -31,15 +32,22 @@ namespace dv {
 
 constexpr int kQkvMfmaWaves = 4;
 
-template <int WAVES, int TILES = 1>
+//
+// LN: the newest window token (slot ln.token) is not in X yet: its row is the residual stream row
+// ln.R1, normalised on the fly from the precomputed statistics (QkvLnArgs).  Per chunk, the lower
+// half of each wavefront normalises the chunk's 256 columns into a wavefront-private LDS row, from
+// which the lanes of that slot take their operands; workgroup 0 also stores the normalised row
+// to ln.x_row_out.  Same values as a stored LayerNorm row, so the same bits as without LN.
+template <int WAVES, int TILES = 1, bool LN = false>
 __device__ __forceinline__ void qkv_window_mfma_body(
     const half_t* __restrict__ X, const half_t* __restrict__ W, const half_t* __restrict__ bias,
     const int* __restrict__ head_idx, const int* __restrict__ batch_idx, int nb, int d, int H,
     int hd, int nnz, half_t* __restrict__ Y, half_t* __restrict__ k_cache,
     half_t* __restrict__ v_cache, const int* __restrict__ padding, int S, int block_id,
-    int nblocks) {
+    int nblocks, const QkvLnArgs& ln = QkvLnArgs{}) {
   constexpr int kTile = kMfmaRows * kMfmaLdsRow;  // halves per 16-row tile
   __shared__ __attribute__((aligned(16))) half_t s_tiles[WAVES][TILES * kTile];
+  __shared__ __attribute__((aligned(16))) half_t s_xnew[LN ? WAVES : 1][LN ? kMfmaKC : 8];
   static_assert(sizeof(half_t) * TILES * kTile >= TILES * 256 * sizeof(float), "tile too small for the reduction");
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -51,6 +59,8 @@ __device__ __forceinline__ void qkv_window_mfma_body(
   const int ntasks = nnz * 3 * groups_per_head;
   const int nchunks = (d + kMfmaKC - 1) / kMfmaKC;
   constexpr int KS = kMfmaKC / 32;
+  LnStats st{0.f, 0.f};
+  if (LN) st = ln_combine(ln.parts, (d + kLnPart - 1) / kLnPart, d, ln.eps);
 
   for (int task = block_id; task < ntasks; task += nblocks) {
     const int i = task / (3 * groups_per_head);
@@ -63,9 +73,11 @@ __device__ __forceinline__ void qkv_window_mfma_body(
     if (slot >= nb) slot = -1;
     if (__ballot(slot >= 0) == 0) continue;  // every wavefront sees the same 16 slots
     const int64_t row0 = ((int64_t)t * H + h) * hd + j0;
+    const bool is_new = LN && slot == ln.token;  // operands come from the LDS row
     // dead slots: every such lane reads the start of row 0 (one line per instruction)
-    const half_t* xrow = X + (slot >= 0 ? (int64_t)slot * d : 0);
-    const bool live = slot >= 0;
+    const bool live = slot >= 0 && !is_new;
+    const half_t* xrow = X + (live ? (int64_t)slot * d : 0);
+    const bool store_row = LN && block_id == 0 && task == 0;
 
     float4_t acc[TILES];
 #pragma unroll
@@ -106,6 +118,40 @@ __device__ __forceinline__ void qkv_window_mfma_body(
         }
       }
     };
+    // newest token: the chunk's 256 columns of the residual row and of the LayerNorm parameters,
+    // four per lane
+    half4_t nr, ng, nbt;
+    auto load_new = [&](int c) {
+      if (LN) {
+        int col = c * kMfmaKC + lane * 4;
+        if (col >= d) col = 0;  // masked when stored
+        nr = *reinterpret_cast<const half4_t*>(ln.R1 + col);
+        ng = *reinterpret_cast<const half4_t*>(ln.gamma + col);
+        nbt = *reinterpret_cast<const half4_t*>(ln.beta + col);
+      }
+    };
+    auto stage_new = [&](int c) {
+      if (LN) {
+        half_t* xn = s_xnew[wave];
+        const int col = c * kMfmaKC + lane * 4;
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");  // the previous chunk's row fully read
+        __builtin_amdgcn_wave_barrier();
+        half4_t o = {0, 0, 0, 0};
+        if (col < d) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            o[e] = (half_t)__builtin_fmaf(((float)nr[e] - st.mean) * st.rstd, (float)ng[e], (float)nbt[e]);
+        }
+        *reinterpret_cast<half4_t*>(xn + lane * 4) = o;
+        if (store_row && col < d) *reinterpret_cast<half4_t*>(ln.x_row_out + col) = o;
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        if (is_new) {  // LDS reads: they do not take part in the count of outstanding memory loads
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) xb[ks] = load8(xn + ks * 32 + kg * 8);
+        }
+      }
+    };
 
     int c = wave;
     if (c < nchunks) {
@@ -116,13 +162,17 @@ __device__ __forceinline__ void qkv_window_mfma_body(
         // swap them: the load counter retires in order, so the multiplies can then wait for x
         // alone while the weight loads stay in flight
         load_x(c);
+        load_new(c);
         __builtin_amdgcn_sched_barrier(0);
         load_stage(c + WAVES);
         __builtin_amdgcn_sched_barrier(0);
+        stage_new(c);
         multiply();
       }
       store_stage(c);
       load_x(c);
+      load_new(c);
+      stage_new(c);
       multiply();
     }
     __syncthreads();  // every wavefront is done with its tile: reuse it for the reduction

@@ -3,7 +3,8 @@
 ``BlockMlpAttSparse.forward`` takes it when the step is an ordinary head-sparse decode step
 (batch 1, one token, fp16, predictions available), the window-flush step included; everything else
 goes through the modules' own forwards.  Same results either way: the fused entry point runs
-the same kernel bodies in eight launches instead of about twenty.
+the same kernel bodies in seven launches instead of about twenty (six per block when consecutive
+blocks go through ``sparse_layers_decode``).
 """
 from __future__ import annotations
 
@@ -43,6 +44,8 @@ lib.dv_sparse_layer_workspace_bytes.restype = ctypes.c_size_t
 lib.dv_sparse_layer_workspace_bytes.argtypes = [ctypes.POINTER(SparseLayerArgs)]
 lib.dv_sparse_layer_decode_f16.restype = ctypes.c_int
 lib.dv_sparse_layer_decode_f16.argtypes = [ctypes.POINTER(SparseLayerArgs), ctypes.c_void_p]
+lib.dv_sparse_layers_decode_f16.restype = ctypes.c_int
+lib.dv_sparse_layers_decode_f16.argtypes = [ctypes.POINTER(SparseLayerArgs), ctypes.c_int, ctypes.c_void_p]
 
 _workspaces: dict = {}
 
@@ -81,10 +84,13 @@ def eligible(block, hidden_states, residual, head_idx, mlp_sp_logit, inference_p
     return head_idx.dtype == torch.int32 and mlp_sp_logit.dtype == torch.float16
 
 
-def sparse_layer_decode(block, hidden_states, residual, head_idx, mlp_sp_logit, inference_params):
-    """Returns (hidden_states, residual, next_mlp_sp_logit, next_att_idx) like the block's forward."""
+def _fill_args(a, block, hidden_states, residual, head_idx, mlp_sp_logit, inference_params):
+    """Fills one ``SparseLayerArgs`` for ``block`` and returns its output tensors
+    (hidden_out, residual_out, logit_out, att_idx_out, mlp_idx_out) plus the tensors that must stay
+    alive until the launches are enqueued.  ``hidden_states`` / ``head_idx`` / ``mlp_sp_logit`` may be
+    None for a block that follows another one in the same call."""
     m, f = block.mixer, block.mlp
-    dev = hidden_states.device
+    dev = m.Wqkv.weight.device
     d, H, hd = m.embed_dim, m.num_heads, m.head_dim
     ffn = f.fc1.out_features
     f.transposed_fc2()
@@ -100,20 +106,19 @@ def sparse_layer_decode(block, hidden_states, residual, head_idx, mlp_sp_logit, 
     b0 = inference_params.batch_size_offset
     kc, vc = k_cache[b0:b0 + 1], v_cache[b0:b0 + 1]
     assert kc.is_contiguous() and vc.is_contiguous()
-    hidden_states = hidden_states.contiguous()
+    hidden_states = None if hidden_states is None else hidden_states.contiguous()
     residual = None if residual is None else residual.contiguous()
     head_idx = head_idx.contiguous()
     mlp_sp_logit = mlp_sp_logit.contiguous()
 
-    hidden_out = torch.empty_like(hidden_states)
-    residual_out = torch.empty_like(hidden_states)
+    hidden_out = torch.empty(1, 1, d, dtype=torch.float16, device=dev)
+    residual_out = torch.empty(1, 1, d, dtype=torch.float16, device=dev)
     logit_out = f.sp.logits_out if f.sp.logits_out is not None else \
         torch.empty(ffn, dtype=torch.float16, device=dev)
     att_idx_out = m.att_idx_out if m.att_idx_out is not None else \
         torch.empty(m.att_k, dtype=torch.int32, device=dev)
     mlp_idx_out = torch.empty(m.mlp_k, dtype=torch.int64, device=dev)
 
-    a = SparseLayerArgs()
     a.d, a.ffn, a.H, a.hd = d, ffn, H, hd
     a.r_att, a.r_mlp = m.sp.fc0.out_features, f.sp.fc0.out_features
     a.K, a.Hk, a.att_k = m.mlp_k, head_idx.shape[0], m.att_k
@@ -137,13 +142,85 @@ def sparse_layer_decode(block, hidden_states, residual, head_idx, mlp_sp_logit, 
     a.k_cache, a.v_cache, a.x_cache, a.tracker = _ptr(kc), _ptr(vc), _ptr(m.x_cache), _ptr(m.tracker)
     a.hidden_out, a.residual_out = _ptr(hidden_out), _ptr(residual_out)
     a.mlp_logit_out, a.att_idx_out, a.mlp_idx_out = _ptr(logit_out), _ptr(att_idx_out), _ptr(mlp_idx_out)
-    nbytes = lib.dv_sparse_layer_workspace_bytes(ctypes.byref(a))
-    ws = _workspace(dev, nbytes)
-    a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
-    check(lib.dv_sparse_layer_decode_f16(ctypes.byref(a), torch.cuda.current_stream().cuda_stream),
-          "dv_sparse_layer_decode_f16")
+    keep = (hidden_states, residual, head_idx, mlp_sp_logit, kc, vc)
+    return (hidden_out, residual_out, logit_out, att_idx_out, mlp_idx_out), keep, flush
+
+
+def _advance_window(m, flush):
     m.counter += 1
     if flush:  # window complete: start the next one (cache_offset was advanced on the device)
         m.counter = 0
+
+
+def sparse_layer_decode(block, hidden_states, residual, head_idx, mlp_sp_logit, inference_params):
+    """Returns (hidden_states, residual, next_mlp_sp_logit, next_att_idx) like the block's forward."""
+    a = SparseLayerArgs()
+    outs, keep, flush = _fill_args(a, block, hidden_states, residual, head_idx, mlp_sp_logit, inference_params)
+    hidden_out, residual_out, logit_out, att_idx_out, mlp_idx_out = outs
+    nbytes = lib.dv_sparse_layer_workspace_bytes(ctypes.byref(a))
+    ws = _workspace(hidden_out.device, nbytes)
+    a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+    check(lib.dv_sparse_layer_decode_f16(ctypes.byref(a), torch.cuda.current_stream().cuda_stream),
+          "dv_sparse_layer_decode_f16")
+    _advance_window(block.mixer, flush)
     block.last_mlp_idx = mlp_idx_out
-    return hidden_out, residual_out, logit_out.view(-1), att_idx_out
+    return hidden_out.view_as(hidden_states), residual_out.view_as(hidden_states), logit_out.view(-1), att_idx_out
+
+
+class LayerChain:
+    """Decode steps of consecutive blocks gathered into ONE ``dv_sparse_layers_decode_f16`` call: block
+    l + 1 consumes the residual stream block l produces, and the launch that finishes block l also
+    prepares block l + 1.  ``add`` reads the block's window state as it is at that moment and
+    advances it, exactly as the block's own forward would; ``run`` enqueues the launches."""
+
+    def __init__(self):
+        self._args = []
+        self._keep = []
+        self.outputs = []  # per block: (hidden_out, residual_out, logit_out, att_idx_out, mlp_idx_out)
+        self._nbytes = 0
+
+    def __len__(self):
+        return len(self._args)
+
+    def add(self, block, head_idx, mlp_sp_logit, inference_params, hidden_states=None, residual=None):
+        """Appends a block.  The first block needs ``hidden_states`` (and ``residual`` unless it is the
+        model's first block); the others take the stream from the block before them.  Returns the
+        block's output tensors (complete once ``run`` has been called and the stream has got there)."""
+        first = not self._args
+        assert first == (hidden_states is not None), "only the first block of a chain is given the stream"
+        a = SparseLayerArgs()
+        outs, keep, flush = _fill_args(a, block, hidden_states, residual, head_idx, mlp_sp_logit, inference_params)
+        self._nbytes = max(self._nbytes, lib.dv_sparse_layer_workspace_bytes(ctypes.byref(a)))
+        _advance_window(block.mixer, flush)
+        block.last_mlp_idx = outs[4]
+        self._args.append(a)
+        self._keep.append(keep)
+        self.outputs.append(outs)
+        return outs
+
+    def run(self):
+        n = len(self._args)
+        assert n > 0
+        arr = (SparseLayerArgs * n)(*self._args)
+        ws = _workspace(self.outputs[0][0].device, self._nbytes)
+        arr[0].workspace, arr[0].workspace_bytes = ws.data_ptr(), ws.numel()
+        check(lib.dv_sparse_layers_decode_f16(arr, n, torch.cuda.current_stream().cuda_stream),
+              "dv_sparse_layers_decode_f16")
+        return self.outputs[-1]
+
+
+def sparse_layers_decode(blocks, hidden_states, residual, head_idx, mlp_sp_logit, inference_params):
+    """The decode step of consecutive blocks of a model in one call; every block must be ``eligible``.
+    ``head_idx`` / ``mlp_sp_logit`` feed the first block, the others take the predictions of the
+    block before them.  Returns (hidden_states, residual, next_mlp_sp_logit, next_att_idx) of the last
+    block and the list of per-block (head_idx, mlp_sp_logit) inputs."""
+    chain = LayerChain()
+    consumed = []
+    for l, block in enumerate(blocks):
+        consumed.append((head_idx, mlp_sp_logit))
+        outs = chain.add(block, head_idx, mlp_sp_logit, inference_params,
+                         hidden_states if l == 0 else None, residual if l == 0 else None)
+        mlp_sp_logit, head_idx = outs[2].view(-1), outs[3]
+    hidden_out, residual_out, logit_out, att_idx_out, _ = chain.run()
+    return (hidden_out.view_as(hidden_states), residual_out.view_as(hidden_states), logit_out.view(-1),
+            att_idx_out, consumed)

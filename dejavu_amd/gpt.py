@@ -32,7 +32,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from . import modules as dv_modules
-from . import ops
+from . import fused_layer, ops
 from .block import BlockDejavu, BlockMlpAttSparse
 from .modules import (InferenceParams, ParallelFusedMLPDejavu, ParallelMHADejavu, ParallelMHASparseAttMlp,
                       decode_linear)
@@ -152,6 +152,8 @@ class GPTModel(nn.Module):
         # when a list, every decode forward appends, per block, the lookahead inputs it
         # consumed: (head_idx, mlp_sp_logit) clones (None for the first block)
         self.record = None
+        # False: every block through its own forward (one fused call per block)
+        self.chain_layers = True
 
     def forward(self, input_ids, position_ids=None, inference_params=None):
         """Dejavu/src/models/gpt_dejavu.py:552-623."""
@@ -163,10 +165,28 @@ class GPTModel(nn.Module):
         # attention idx & mlp logit are passed on to the next layer
         next_mlp_sp_logit = None
         next_att_idx = None
+        # Consecutive head-sparse decode steps go through ONE call (fused_layer.LayerChain: the launch
+        # that ends a block also prepares the next one).  Not while recording: the record clones each
+        # block's inputs when the block is reached, and a chain only enqueues them at its end.
+        chain = None
+        chaining = (self.chain_layers and self.att_sparse and self.record is None and input_ids.shape[1] == 1
+                    and input_ids.shape[0] == 1)
         for layer in self.layers:
             if self.record is not None and input_ids.shape[1] == 1:
                 self.record.append((None if next_att_idx is None else next_att_idx.clone(),
                                     None if next_mlp_sp_logit is None else next_mlp_sp_logit.clone()))
+            if chaining and getattr(layer, "use_fused_layer", False) and fused_layer.eligible(
+                    layer, hidden_states, residual, next_att_idx, next_mlp_sp_logit, inference_params):
+                if chain is None:
+                    chain = fused_layer.LayerChain()
+                    outs = chain.add(layer, next_att_idx, next_mlp_sp_logit, inference_params, hidden_states, residual)
+                else:
+                    outs = chain.add(layer, next_att_idx, next_mlp_sp_logit, inference_params)
+                hidden_states, residual, next_mlp_sp_logit, next_att_idx = outs[0], outs[1], outs[2].view(-1), outs[3]
+                continue
+            if chain is not None:
+                chain.run()
+                chain = None
             if self.att_sparse:
                 hidden_states, residual, next_mlp_sp_logit, next_att_idx = layer(
                     hidden_states, residual, head_idx=next_att_idx, mlp_sp_logit=next_mlp_sp_logit,
@@ -174,6 +194,8 @@ class GPTModel(nn.Module):
             else:
                 hidden_states, residual, next_mlp_sp_logit = layer(
                     hidden_states, residual, mlp_sp_logit=next_mlp_sp_logit, mixer_kwargs=mixer_kwargs)
+        if chain is not None:
+            chain.run()
         if hidden_states.is_cuda and hidden_states.dtype == torch.float16:
             hidden_states, _ = ops.add_layer_norm(hidden_states, residual, self.ln_f.weight, self.ln_f.bias,
                                                   self.ln_f.eps)

@@ -474,6 +474,23 @@ typedef struct dvSparseLayerArgs {
 DV_API size_t dv_sparse_layer_workspace_bytes(const dvSparseLayerArgs* args);
 DV_API int dv_sparse_layer_decode_f16(const dvSparseLayerArgs* args, void* stream);
 
+/*
+ * The same step for n_layers consecutive blocks of a model, the loop over the layers of
+ * GPTModel.forward (Dejavu/src/models/gpt_dejavu.py:595-612) for one decode token:
+ * block l + 1 takes (hidden_out, residual_out) of block l, whatever its own `hidden` /
+ * `residual` say (they may be NULL for l > 0).  Equivalent to n_layers calls of
+ * dv_sparse_layer_decode_f16, bit for bit, but the launch that finishes block l's MLP
+ * output also does the residual add, the LayerNorm statistics, the key histogram and the
+ * window step of block l + 1 (six launches per block instead of seven).
+ * All blocks share d, ffn and H; the scratch is layers[0].workspace, at least the largest
+ * dv_sparse_layer_workspace_bytes() of the blocks (the other blocks' workspace fields are
+ * not read).  Every block's outputs are stored as documented above.  The predictions a
+ * block consumes must be complete when its turn comes: buffers written by the block
+ * before it (mlp_logit_out / att_idx_out of block l as mlp_logit_in / head_idx of block
+ * l + 1) or by earlier work on the stream.
+ */
+DV_API int dv_sparse_layers_decode_f16(const dvSparseLayerArgs* layers, int n_layers, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

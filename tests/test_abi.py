@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
 
     from dejavu_amd import fused_layer  # noqa: F401  (binds the struct-taking entry points)
 
-    struct_entry_points = {"dv_sparse_layer_workspace_bytes", "dv_sparse_layer_decode_f16"}
+    struct_entry_points = {"dv_sparse_layer_workspace_bytes", "dv_sparse_layer_decode_f16", "dv_sparse_layers_decode_f16"}
     for name in declared_symbols():
         assert hasattr(_lib.lib, name), f"{name} declared in the header but not exported"
         assert name in _lib.SIGNATURES or name in struct_entry_points, f"{name} has no ctypes signature"

@@ -164,3 +164,78 @@ def test_fused_layer_equals_module_by_module_path(d, H, ffn, r, K, Hk):
             assert torch.equal(ca, cb), f"step {step}: caches differ"
         for ip in ips:
             ip.sequence_len_offset += 1
+
+
+@pytest.mark.parametrize("d,H,ffn,r,K,Hk", [(768, 12, 3072, 128, 512, 3), (5120, 40, 20480, 1000, 2048, 16),
+                                            (12288, 96, 49152, 1000, 4096, 32)])
+def test_chained_layers_equal_layer_by_layer(d, H, ffn, r, K, Hk):
+    """Three consecutive blocks through ONE dv_sparse_layers_decode_f16 call (the launch that ends a
+    block also prepares the next one) against the same blocks stepped one by one through the module
+    path: outputs, predictions, caches and window state bit for bit, over a window and into the
+    next one, with poisoned scratch."""
+    import copy
+
+    from dejavu_amd import fused_layer, ops
+    from dejavu_amd.block import create_sparse_block, init_block_synthetic
+    from dejavu_amd.modules import InferenceParams
+    from dejavu_amd.workloads import pack_k_cache
+
+    S, L = 64, 3
+    hd = d // H
+    g = torch.Generator().manual_seed(21)
+    chain, single = [], []
+    for l in range(L):
+        blk = create_sparse_block(d, ffn, H, r, K, r, Hk, layer_idx=l)
+        init_block_synthetic(blk, seed=30 + l)
+        with torch.no_grad():
+            for n in (blk.norm1, blk.norm2):
+                n.weight.copy_((1 + 0.1 * torch.randn(d, generator=g)).half())
+                n.bias.copy_((0.1 * torch.randn(d, generator=g)).half())
+            blk.mixer.Wqkv.bias.copy_((0.1 * torch.randn(3 * d, generator=g)).half())
+            blk.mixer.out_proj.bias.copy_((0.1 * torch.randn(d, generator=g)).half())
+            blk.mlp.fc2.bias.copy_((0.1 * torch.randn(d, generator=g)).half())
+        chain.append(blk)
+        other = copy.deepcopy(blk)
+        other.use_fused_layer = False
+        single.append(other)
+    t0 = 20
+    ips = []
+    for _ in range(2):
+        ip = InferenceParams(max_sequence_len=S, max_batch_size=1, sequence_len_offset=t0)
+        gk = torch.Generator().manual_seed(22)
+        for l in range(L):
+            ip.key_value_memory_dict[l] = (pack_k_cache(torch.randn(1, H, S, hd, generator=gk).half()).cuda(),
+                                           torch.randn(1, H, S, hd, generator=gk).half().cuda())
+        ips.append(ip)
+    for step in range(19):
+        hs = torch.randn(1, 1, d, generator=g).half().cuda()
+        res = torch.randn(1, 1, d, generator=g).half().cuda()
+        head_idx = torch.sort(torch.randperm(H, generator=g)[:Hk]).values.int().cuda()
+        logit = (torch.randn(ffn, generator=g) * 4).half().cuda()
+        print(f"case chained layers d={d} step={step} counter={chain[0].mixer.counter}", flush=True)
+        for cache in (ops._workspaces, ops._topk_workspaces, ops._attn_workspaces, fused_layer._workspaces):
+            for ws in cache.values():
+                ws.view(torch.uint8).fill_(255)
+        with torch.no_grad():
+            got = fused_layer.sparse_layers_decode(chain, hs, res, head_idx, logit, ips[0])
+            h, rr, lg, hi = hs, res, logit, head_idx
+            inputs = []
+            for blk in single:
+                inputs.append((hi, lg))
+                h, rr, lg, hi = blk(h, rr, mixer_kwargs={"inference_params": ips[1]}, head_idx=hi, mlp_sp_logit=lg)
+        torch.cuda.synchronize()
+        for name, xa, xb in zip(("hidden", "residual", "next_logit", "next_att_idx"), got[:4], (h, rr, lg, hi)):
+            assert torch.equal(xa.reshape(-1), xb.reshape(-1)), f"step {step}: {name} differs"
+        for l, ((hi_c, lg_c), (hi_s, lg_s)) in enumerate(zip(got[4], inputs)):
+            flush = single[l].mixer.counter == 0  # the step just taken closed a window: every head was active
+            assert flush or torch.equal(hi_c, hi_s), f"step {step}: heads fed to block {l} differ"
+            assert torch.equal(lg_c.reshape(-1), lg_s.reshape(-1)), f"step {step}: MLP logits fed to block {l} differ"
+        for l in range(L):
+            ma, mb = chain[l].mixer, single[l].mixer
+            assert ma.counter == mb.counter and torch.equal(ma.cache_offset, mb.cache_offset)
+            assert torch.equal(ma.tracker, mb.tracker), f"step {step}: tracker of block {l} differs"
+            assert torch.equal(ma.x_cache[:max(1, ma.counter)], mb.x_cache[:max(1, mb.counter)])
+            for ca, cb in zip(ips[0].key_value_memory_dict[l], ips[1].key_value_memory_dict[l]):
+                assert torch.equal(ca, cb), f"step {step}: caches of block {l} differ"
+        for ip in ips:
+            ip.sequence_len_offset += 1
