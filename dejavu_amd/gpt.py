@@ -152,6 +152,9 @@ class GPTModel(nn.Module):
         # when a list, every decode forward appends, per block, the lookahead inputs it
         # consumed: (head_idx, mlp_sp_logit) clones (None for the first block)
         self.record = None
+        # when a list (together with `record`), every decode forward also appends, per block, the MLP
+        # neurons the block selected (None for a block without a selection)
+        self.record_mlp_idx = None
         # False: every block through its own forward (one fused call per block)
         self.chain_layers = True
 
@@ -194,6 +197,9 @@ class GPTModel(nn.Module):
             else:
                 hidden_states, residual, next_mlp_sp_logit = layer(
                     hidden_states, residual, mlp_sp_logit=next_mlp_sp_logit, mixer_kwargs=mixer_kwargs)
+            if self.record is not None and self.record_mlp_idx is not None and input_ids.shape[1] == 1:
+                idx = getattr(layer, "last_mlp_idx", None)
+                self.record_mlp_idx.append(None if idx is None else idx.clone())
         if chain is not None:
             chain.run()
         if hidden_states.is_cuda and hidden_states.dtype == torch.float16:

@@ -54,3 +54,34 @@ def load_model_params(model, params):
         layer.mlp.fc2_weight_t = None
         layer.mixer.out_proj_weight_t = None
     model.tie_weights()
+
+
+def fp16_steps_from(value, reference):
+    """|value - reference| in units of the fp16 spacing at `reference` (normal range)."""
+    ref = abs(float(reference))
+    step = 2.0 ** (np.floor(np.log2(max(ref, 2.0 ** -14))) - 10)
+    return abs(float(value) - float(reference)) / step
+
+
+def index_set_against_oracle(device_idx, oracle_logits, k, what, max_steps):
+    """Compares a device-side top-k set with the oracle's own selection on the ORACLE's logits
+    ((n,) or (B, n): a column's score is its maximum over the rows).  The sets may differ only at
+    the threshold: every index that is in one set and not in the other must have an oracle score
+    within `max_steps` fp16 steps of the oracle's k-th largest score.  Returns (number of differing
+    indices, largest distance in fp16 steps) and prints them."""
+    from oracle import dejavu_oracle as O
+
+    logits = np.asarray(oracle_logits)
+    score = logits.astype(np.float32)
+    if score.ndim == 2:
+        score = score.max(axis=0)
+    want = np.asarray(O.topk_lower_index(logits, k)).astype(np.int64)
+    got = np.asarray(device_idx).astype(np.int64)
+    assert got.size == k and np.unique(got).size == k, f"{what}: not {k} distinct indices"
+    kth = np.sort(score)[-k]
+    diff = np.setxor1d(got, want)
+    worst = max((fp16_steps_from(score[i], kth) for i in diff), default=0.0)
+    print(f"index sets, {what}: {diff.size // 2} of {k} indices differ from the oracle's selection, "
+          f"farthest {worst:.2f} fp16 steps from the k-th score {float(kth):.4g}", flush=True)
+    assert worst <= max_steps, f"{what}: an index {worst:.2f} fp16 steps away from the threshold was swapped"
+    return diff.size // 2, worst

@@ -10,12 +10,20 @@ from oracle import dejavu_oracle as O
 
 pytestmark = pytest.mark.gpu
 
+# From 9 batch rows on the predictor logits come from the matrix cores (another fp32 order than the
+# oracle's), so a selection may swap columns whose oracle scores sit at the threshold: at most this
+# many fp16 steps away from the k-th score (the tests print what they measure; at the OPT-66B shape with 16
+# rows and the OPT-175B shape with 32 rows the sets are identical to the oracle's).
+INDEX_SET_MAX_STEPS = 1.0
+
 
 def assert_close(got, want, what="", max_abs_tol=2e-2, rel_tol=1e-3):
     got = np.asarray(got, dtype=np.float64)
     want = np.asarray(want, dtype=np.float64)
     max_abs = np.max(np.abs(got - want)) if got.size else 0.0
     rel = np.linalg.norm(got - want) / max(np.linalg.norm(want), 1e-30)
+    if (max_abs_tol, rel_tol) != (2e-2, 1e-3):  # a bound other than the per-operator one: say what was measured
+        print(f"measured {what}: max_abs={max_abs:.3e} rel_l2={rel:.3e} (bounds {max_abs_tol:g} / {rel_tol:g})", flush=True)
     assert max_abs <= max_abs_tol and rel <= rel_tol, f"{what}: max_abs={max_abs:.3e} rel_l2={rel:.3e}"
 
 
@@ -207,7 +215,7 @@ def test_batched_sparse_attention_module_backfills_skipped_heads(B, d, H, Hk, pr
         used = np.arange(H) if step % 16 == 15 else head_idx.numpy()
         for b in range(B):
             want, _ = O.sparse_attention_step_dense_kv(xs[b, : t + 1].numpy(), Wqkv, bqkv, Wout, bout, used, hd ** -0.5)
-            assert_close(np16(out)[b, 0], want, f"step {step} row {b}", max_abs_tol=3e-2, rel_tol=3e-3)
+            assert_close(np16(out)[b, 0], want, f"step {step} row {b}")
         assert np.array_equal(np16(mlp_idx), O.topk_lower_index(np16(mlp_sp_logit), mlp_k))
         dev_logits = att.sp(residual)  # (B, H) as the module computed them
         assert np.array_equal(np16(att_idx).astype(np.int64), O.topk_lower_index(np16(dev_logits), Hk))
@@ -236,7 +244,8 @@ def test_batched_sparse_block_decode_step_matches_oracle(cfg, B):
     """One decode step of a whole block for B sequences (OPT-66B shape at batch 16, OPT-175B shape at
     batch 8 and 32, full-size weights and caches) against block_decode_step_batched.  Up to 8 rows
     the predictors are bit-exact; above, their logits come from the matrix cores and are compared
-    within tolerance, the selections being checked as the exact top-k of the device's own logits."""
+    within tolerance, the selections being checked as the exact top-k of the device's own logits
+    AND against the oracle's selections (differences only at the threshold, counted and bounded)."""
     from dejavu_amd.block import create_sparse_block, init_block_synthetic
     from dejavu_amd.modules import InferenceParams
     from dejavu_amd.workloads import CONFIGS, pack_k_cache
@@ -281,7 +290,7 @@ def test_batched_sparse_block_decode_step_matches_oracle(cfg, B):
     want = O.block_decode_step_batched(p, hs.numpy()[:, 0], res.numpy()[:, 0], head_idx.numpy(), mlp_sp_logit.numpy(),
                                        kn, vn, lengths.numpy(), residual2_override=np16(residual)[:, 0])
     assert_close(np16(residual)[:, 0], want["residual"], "residual stream after attention")
-    assert_close(np16(hidden)[:, 0], want["hidden"], "block output", max_abs_tol=3e-2, rel_tol=3e-3)
+    assert_close(np16(hidden)[:, 0], want["hidden"], "block output")
     assert np.array_equal(np16(next_att).astype(np.int64), O.topk_lower_index(np16(dev_head_logits), Hk)), \
         "next heads are not the top-k of the batch maxima of the device's head logits"
     if B <= 8:
@@ -296,6 +305,17 @@ def test_batched_sparse_block_decode_step_matches_oracle(cfg, B):
             top = float(np.abs(want_l.astype(np.float32)).max())
             two_steps = 2.0 * 2.0 ** (np.floor(np.log2(max(top, 1e-3))) - 10)
             assert_close(np16(got_l), want_l, what + " (matrix-core order)", max_abs_tol=max(2e-2, two_steps))
+        # ... and the selections made from them against the oracle's selections on the ORACLE's logits:
+        # the sets may differ only by columns whose oracle score sits at the threshold
+        from tests.model_utils import index_set_against_oracle
+
+        index_set_against_oracle(np16(next_att), want["att_logit"], Hk, f"{cfg} B={B} next heads", max_steps=INDEX_SET_MAX_STEPS)
+        from dejavu_amd import ops as ops_mod
+
+        dev_mlp_idx = ops_mod.topk_indices(next_logit, K)
+        torch.cuda.synchronize()
+        index_set_against_oracle(np16(dev_mlp_idx), want["next_mlp_logit"], K, f"{cfg} B={B} next neurons",
+                                 max_steps=INDEX_SET_MAX_STEPS)
     # the appended K / V rows are projections (within tolerance of the oracle's); every other cache
     # entry is untouched bit for bit
     kcd, vcd = ip.key_value_memory_dict[2]

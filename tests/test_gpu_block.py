@@ -14,6 +14,8 @@ def assert_close(got, want, what="", max_abs_tol=2e-2, rel_tol=1e-3):
     want = np.asarray(want, dtype=np.float64)
     max_abs = np.max(np.abs(got - want)) if got.size else 0.0
     rel = np.linalg.norm(got - want) / max(np.linalg.norm(want), 1e-30)
+    if (max_abs_tol, rel_tol) != (2e-2, 1e-3):  # a bound other than the per-operator one: say what was measured
+        print(f"measured {what}: max_abs={max_abs:.3e} rel_l2={rel:.3e} (bounds {max_abs_tol:g} / {rel_tol:g})", flush=True)
     assert max_abs <= max_abs_tol and rel <= rel_tol, f"{what}: max_abs={max_abs:.3e} rel_l2={rel:.3e}"
 
 
@@ -44,8 +46,9 @@ def test_add_layer_norm(rows, d):
 
 
 @pytest.mark.parametrize("d,ffn,H,r,K,Hk,S", [(768, 3072, 12, 128, 1024, 4, 128),
+                                              (9216, 36864, 72, 1000, 4096, 24, 1024),
                                               (12288, 49152, 96, 1000, 4096, 32, 2048)],
-                         ids=["opt-125m-shape", "opt-175b-shape"])
+                         ids=["opt-125m-shape", "opt-66b-shape", "opt-175b-shape"])
 def test_sparse_block_decode_step_matches_oracle(d, ffn, H, r, K, Hk, S):
     """One decode step of a whole block against the oracle, at a small shape and at the
     headline shape (full-size weights, 2048-token caches)."""
@@ -89,7 +92,7 @@ def test_sparse_block_decode_step_matches_oracle(d, ffn, H, r, K, Hk, S):
     want = O.block_decode_step(p, hs.numpy()[0], res.numpy()[0], head_idx.numpy(), mlp_sp_logit.numpy(), kn, vn, t,
                                residual2_override=np16(residual)[0])
     assert_close(np16(residual)[0], want["residual"], "residual stream after attention")
-    assert_close(np16(hidden)[0], want["hidden"], "block output", max_abs_tol=3e-2, rel_tol=3e-3)
+    assert_close(np16(hidden)[0], want["hidden"], "block output")
     assert np.array_equal(np16(next_att).astype(np.int64), want["next_att_idx"].astype(np.int64)), "next heads differ"
     assert np.array_equal(np16(next_logit).view(np.uint16), want["next_mlp_logit"].view(np.uint16)), \
         "next-layer MLP logits not bit-exact"

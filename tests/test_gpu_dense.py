@@ -12,6 +12,8 @@ def assert_close(got, want, what="", max_abs_tol=2e-2, rel_tol=1e-3):
     want = np.asarray(want, dtype=np.float64)
     max_abs = np.max(np.abs(got - want)) if got.size else 0.0
     rel = np.linalg.norm(got - want) / max(np.linalg.norm(want), 1e-30)
+    if (max_abs_tol, rel_tol) != (2e-2, 1e-3):  # a bound other than the per-operator one: say what was measured
+        print(f"measured {what}: max_abs={max_abs:.3e} rel_l2={rel:.3e} (bounds {max_abs_tol:g} / {rel_tol:g})", flush=True)
     assert max_abs <= max_abs_tol and rel <= rel_tol, f"{what}: max_abs={max_abs:.3e} rel_l2={rel:.3e}"
 
 
@@ -120,9 +122,9 @@ def test_prompt_runs_on_the_hip_kernels_and_matches_the_library_path():
         M.USE_HIP_PROMPT = True
     state = O.new_decode_state(params, 64)
     want = O.model_prompt(params, state, prompt).astype(np.float32)
-    assert_close(outs[0], want, "prompt logits, hip kernels vs oracle", rel_tol=2.5e-3)
-    assert_close(outs[1], want, "prompt logits, library path vs oracle", rel_tol=2.5e-3)
+    assert_close(outs[0], want, "prompt logits, hip kernels vs oracle", rel_tol=1.3e-3)
+    assert_close(outs[1], want, "prompt logits, library path vs oracle", rel_tol=1.3e-3)
     for l in range(L):
         for got, ref, o in zip(caches[0][l], caches[1][l], state["caches"][l]):
-            assert_close(got, o.astype(np.float32), f"layer {l} cache vs oracle", rel_tol=2.5e-3)
-            assert_close(got, ref, f"layer {l} cache, hip vs library path", rel_tol=2.5e-3)
+            assert_close(got, o.astype(np.float32), f"layer {l} cache vs oracle")
+            assert_close(got, ref, f"layer {l} cache, hip vs library path")

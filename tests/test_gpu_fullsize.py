@@ -18,6 +18,8 @@ def close(got, want, what, max_abs_tol=MAX_ABS, rel_tol=REL_L2):
     got, want = got.double(), want.double()
     max_abs = (got - want).abs().max().item()
     rel = ((got - want).norm() / want.norm().clamp_min(1e-30)).item()
+    if (max_abs_tol, rel_tol) != (MAX_ABS, REL_L2):  # a bound other than the per-operator one: say what was measured
+        print(f"measured {what}: max_abs={max_abs:.3e} rel_l2={rel:.3e} (bounds {max_abs_tol:g} / {rel_tol:g})", flush=True)
     assert max_abs <= max_abs_tol and rel <= rel_tol, f"{what}: max_abs={max_abs:.3e} rel_l2={rel:.3e}"
 
 
@@ -55,7 +57,7 @@ def test_sparse_mlp_against_library_and_linearity(ops, gen):
     # fc2 is linear in h (no bias): f(h1 + h2) = f(h1) + f(h2) up to fp16 rounding of the three results
     h2 = randn(gen, 1, K).abs()
     f = lambda v: ops.gather_transposed_gemv(v, W2t, idx, None).float()
-    close(f((h.float() + h2.float()).half()), f(h) + f(h2), "fc2 linearity", max_abs_tol=3e-2, rel_tol=3e-3)
+    close(f((h.float() + h2.float()).half()), f(h) + f(h2), "fc2 linearity")
     # the same neurons in another order: the same sum up to fp32 re-association
     perm = torch.randperm(K, device="cuda", generator=gen)
     close(ops.gather_transposed_gemv(h[:, perm].contiguous(), W2t, idx[perm].contiguous(), b2), y_ref,

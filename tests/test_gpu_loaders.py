@@ -97,6 +97,6 @@ def test_remapped_checkpoint_generates_like_the_oracle_on_the_same_tensors():
     max_abs = float(np.abs(got - want).max())
     rel = max(float(np.linalg.norm(g - w) / np.linalg.norm(w)) for g, w in zip(got, want))
     print(f"checkpoint generate: max-abs {max_abs:.3g} rel-L2 {rel:.3g}")
-    assert max_abs <= 2e-2 and rel <= 2.5e-3
+    assert max_abs <= 2e-2 and rel <= 1.8e-3
     agree = sum(int(np.argmax(w)) == t for w, t in zip(want, seq[len(prompt):]))
     assert agree >= n_new - 2  # near-ties aside, the greedy tokens are the oracle's

@@ -86,6 +86,10 @@ def test_predictor_more_than_eight_rows_runs_on_the_matrix_cores(ops, cfg, batch
     want_logits = (np16(hidden).astype(np.float32) @ np16(t["mlp_Wb"]).astype(np.float32).T)
     assert_close(np16(got), want_logits, "predictor logits")
     assert np.array_equal(np16(idx), O.topk_lower_index(np16(got), k)), "union top-k of the device logits"
+    # against the oracle's selection on the oracle's own logits: differences only at the threshold
+    from tests.model_utils import index_set_against_oracle
+
+    index_set_against_oracle(np16(idx), l_ref, k, f"{cfg} B={batch} MLP neurons", max_steps=1.0)
 
 
 @pytest.mark.parametrize("B,r,n_out", [(17, 520, 16390), (32, 1000, 20480), (12, 8, 16384), (32, 1024, 16386),

@@ -81,7 +81,7 @@ def test_greedy_generation_matches_oracle_with_replayed_selections(mlp_K, att_K)
             checked += 1
     print(f"logits: worst max-abs {worst_abs:.4g}, worst rel-L2 {worst_rel:.4g}, tokens checked {checked}")
     # three blocks + lm_head of fp16-rounded intermediates against the oracle's own fp16 rounding
-    assert worst_abs <= 2e-2 and worst_rel <= 2.5e-3
+    assert worst_abs <= 2e-2 and worst_rel <= 1.8e-3
     assert checked >= n_new // 2
 
 
@@ -221,3 +221,68 @@ def test_greedy_advance_matches_torch_argmax_and_bookkeeping(vocab):
         ops.greedy_advance(shifted, token, position, seq_pos, sequences, out_index)
         torch.cuda.synchronize()
         assert int(token) == want and int(out_index) == 6
+
+
+def test_opt13b_shaped_model_at_full_size_graphs_equal_eager_and_selections_are_exact():
+    """The end-to-end configuration at its real size: 40 layers of the OPT-13B shape (d = 5120, ffn = 20480,
+    40 heads, K = 2048 neurons, 16 heads, vocabulary 50272), a 128-token prompt and 48 generated tokens.
+    Size-independent properties (the numpy oracle would take hours here): generation replayed from HIP
+    graphs equals eager generation bit for bit (sequences and scores), the chained layer calls equal one
+    call per block, and every selection a block consumed is well-formed: the MLP neurons are the exact
+    top-k (ties to the lower index) of the logits the block was given, the heads are distinct and ascending."""
+    from dejavu_amd.block import init_block_synthetic
+    from dejavu_amd.gpt import GPTLMHeadModel, SparseGPTConfig
+    from dejavu_amd.workloads import CONFIGS
+
+    cfg = CONFIGS["opt-13b"]
+    L, vocab, prompt_len, n_new = 40, 50272, 128, 48
+    conf = SparseGPTConfig(hidden_size=cfg["d"], num_attention_heads=cfg["H"], num_hidden_layers=L,
+                           vocab_size=vocab, n_inner=cfg["ffn"], max_position_embeddings=2048, mlp_K=cfg["K"],
+                           mlp_sp_dim=cfg["r"], att_K=[cfg["Hk"], cfg["Hk"]], att_sp_dim=cfg["r"],
+                           pad_vocab_size_multiple=8)
+    print("case full-size OPT-13B-shaped model: build", flush=True)
+    model = GPTLMHeadModel(conf, device="cuda", dtype=torch.float16).eval()
+    with torch.no_grad():
+        gen = torch.Generator(device="cuda")
+        gen.manual_seed(7)
+        for l, blk in enumerate(model.transformer.layers):
+            init_block_synthetic(blk, seed=100 + l)
+        for emb in (model.transformer.embeddings.word_embeddings, model.transformer.embeddings.position_embeddings):
+            tmp = torch.empty(emb.weight.shape, dtype=torch.float32, device="cuda")
+            tmp.normal_(0.0, 0.02, generator=gen)
+            emb.weight.copy_(tmp)
+        model.tie_weights()
+        ids = torch.randint(0, vocab, (1, prompt_len), generator=gen, device="cuda")
+    max_length = prompt_len + n_new
+    tr = model.transformer
+    print("case full-size model: eager generation, one call per block, recording", flush=True)
+    tr.record, tr.record_mlp_idx = [], []
+    rec = model.generate(ids, max_length=max_length, vocab_size=vocab, return_dict_in_generate=True, output_scores=True)
+    torch.cuda.synchronize()
+    record, used = tr.record, tr.record_mlp_idx
+    tr.record = tr.record_mlp_idx = None
+    steps = n_new - 1
+    assert len(record) == steps * L and len(used) == steps * L
+    checked = 0
+    for s in range(steps):
+        for l in range(1, L):
+            hi, lg = record[s * L + l]
+            idx = used[s * L + l]
+            assert hi.numel() == cfg["Hk"] and bool(torch.all(hi[1:] > hi[:-1])) and 0 <= int(hi[0]) and int(hi[-1]) < cfg["H"]
+            if s % 6 == 0 or s == steps - 1:  # the exact top-k on the host, for a sample of the steps
+                want = O.topk_lower_index(lg.cpu().numpy(), cfg["K"])
+                np.testing.assert_array_equal(idx.cpu().numpy(), want, err_msg=f"step {s} block {l}")
+                checked += 1
+    print(f"full-size model: {checked} neuron selections equal the exact top-k of their logits", flush=True)
+    print("case full-size model: eager generation, chained blocks", flush=True)
+    eager = model.generate(ids, max_length=max_length, vocab_size=vocab, return_dict_in_generate=True, output_scores=True)
+    torch.cuda.synchronize()
+    assert torch.equal(eager.sequences, rec.sequences) and torch.equal(eager.scores, rec.scores)
+    for attempt in ("first call (captures)", "second call (replays only)"):
+        print(f"case full-size model: cg=True, {attempt}", flush=True)
+        g = model.generate(ids, max_length=max_length, cg=True, vocab_size=vocab, return_dict_in_generate=True,
+                           output_scores=True)
+        torch.cuda.synchronize()
+        assert torch.equal(g.sequences, eager.sequences), attempt
+        assert torch.equal(g.scores, eager.scores), attempt
+    assert "window" in model._decoding_cache.graphs

@@ -17,6 +17,8 @@ def assert_close(got, want, what="", max_abs_tol=MAX_ABS, rel_tol=REL_L2):
     want = np.asarray(want, dtype=np.float64)
     max_abs = np.max(np.abs(got - want)) if got.size else 0.0
     rel = np.linalg.norm(got - want) / max(np.linalg.norm(want), 1e-30)
+    if (max_abs_tol, rel_tol) != (2e-2, 1e-3):  # a bound other than the per-operator one: say what was measured
+        print(f"measured {what}: max_abs={max_abs:.3e} rel_l2={rel:.3e} (bounds {max_abs_tol:g} / {rel_tol:g})", flush=True)
     assert max_abs <= max_abs_tol and rel <= rel_tol, f"{what}: max_abs={max_abs:.3e} rel_l2={rel:.3e}"
 
 
@@ -124,7 +126,7 @@ def test_sparse_attention_module_backfills_skipped_heads(d, H, Hk, prompt, steps
         want, _ = O.sparse_attention_step_dense_kv(xs[: t + 1].numpy(), Wqkv, bqkv, Wout, bout, used, hd ** -0.5)
         got = np16(out)[0, 0]
         worst = max(worst, float(np.max(np.abs(got.astype(np.float64) - want.astype(np.float64)))))
-        assert_close(got, want, f"step {step}", max_abs_tol=3e-2, rel_tol=3e-3)
+        assert_close(got, want, f"step {step}")
         assert mlp_idx.dtype == torch.int64 and att_idx.dtype == torch.int32
         assert np.array_equal(np16(mlp_idx), O.topk_lower_index(np16(mlp_sp_logit), mlp_k))
         _, l_ref = O.predictor_logits(np16(residual)[0], np16(att.sp.fc0.weight), np16(att.sp.fc1.weight))
@@ -160,7 +162,7 @@ def test_dense_decode_attention_module_matches_dense_kv():
     torch.cuda.synchronize()
     # last prompt row is causal attention over the whole prompt
     want, _ = O.sparse_attention_step_dense_kv(xs[:prompt].numpy(), Wqkv, bqkv, Wout, bout, np.arange(H))
-    assert_close(np16(out_p)[0, -1], want, "prompt last row", max_abs_tol=3e-2, rel_tol=3e-3)
+    assert_close(np16(out_p)[0, -1], want, "prompt last row")
     ip.sequence_len_offset = prompt
     for step in range(steps):
         t = prompt + step
@@ -169,6 +171,6 @@ def test_dense_decode_attention_module_matches_dense_kv():
             out, mlp_idx = att(xs[t].cuda().view(1, 1, d), mlp_sp_logit=logit, inference_params=ip)
         torch.cuda.synchronize()
         want, _ = O.sparse_attention_step_dense_kv(xs[: t + 1].numpy(), Wqkv, bqkv, Wout, bout, np.arange(H))
-        assert_close(np16(out)[0, 0], want, f"dense decode step {step}", max_abs_tol=3e-2, rel_tol=3e-3)
+        assert_close(np16(out)[0, 0], want, f"dense decode step {step}")
         assert np.array_equal(np16(mlp_idx), O.topk_lower_index(np16(logit), 64))
         ip.sequence_len_offset += 1

@@ -639,3 +639,53 @@ def test_prompt_attention_matches_causal_sdpa_and_fills_caches():
     ref2 = torch.nn.functional.scaled_dot_product_attention(
         torch.from_numpy(q_new.astype(np.float64)).unsqueeze(2), torch.from_numpy(K), torch.from_numpy(V)).squeeze(2).numpy()
     assert np.abs(out.astype(np.float64) - ref2).max() <= 2e-3
+
+
+def assert_close(got, want, what, max_abs_tol=2e-2, rel_tol=1e-3):
+    got = np.asarray(got, dtype=np.float64)
+    want = np.asarray(want, dtype=np.float64)
+    max_abs = np.max(np.abs(got - want)) if got.size else 0.0
+    rel = np.linalg.norm(got - want) / max(np.linalg.norm(want), 1e-30)
+    assert max_abs <= max_abs_tol and rel <= rel_tol, f"{what}: max_abs={max_abs:.3e} rel_l2={rel:.3e}"
+
+
+def test_cpu_baseline_layer_step_follows_the_oracle():
+    """oracle/cpu_baseline.layer_step (the PyTorch index_select + matmul form that bench.py times on
+    the host cores) against the oracle's functions on a small layer (OPT-125M shape, batch 1 and 3):
+    the same head and neuron sets up to columns at the selection threshold, outputs within the
+    per-operator tolerance."""
+    import torch
+
+    from dejavu_amd.workloads import CONFIGS, make_layer
+    from oracle import cpu_baseline as C
+
+    cfg = CONFIGS["opt-125m"]
+    H, hd, d = cfg["H"], cfg["hd"], cfg["d"]
+    for batch in (1, 3):
+        t = make_layer(cfg, batch=batch, device="cpu", seed=5 + batch)
+        with torch.no_grad():
+            attn, mlp, mlp_idx, head_idx = C.layer_step(t)
+        n = {k: (v.numpy() if torch.is_tensor(v) else v) for k, v in t.items()}
+        _, att_logits = O.predictor_logits(n["residual"], n["att_Wa"], n["att_Wb"])
+        _, mlp_logits = O.predictor_logits(n["residual"], n["mlp_Wa"], n["mlp_Wb"])
+        # the baseline's logits come from the library's own summation order: its selections may differ
+        # from the oracle's only by columns whose oracle score sits at the threshold
+        from tests.model_utils import index_set_against_oracle
+
+        index_set_against_oracle(head_idx.numpy(), att_logits, cfg["Hk"], f"cpu baseline heads, batch {batch}", 2.0)
+        index_set_against_oracle(mlp_idx.numpy(), mlp_logits, cfg["K"], f"cpu baseline neurons, batch {batch}", 2.0)
+        want_heads = np.sort(head_idx.numpy()).astype(np.int32)
+        want_neurons = np.sort(mlp_idx.numpy())
+        # MLP on the same neuron set (the sums do not depend on the order beyond fp32 rounding)
+        want_mlp = O.mlp_sparse(n["x2"], n["W1"], n["W2t"], want_neurons, n["b1"], n["b2"])
+        assert_close(mlp.numpy(), want_mlp, f"cpu baseline MLP, batch {batch}")
+        # attention: oracle QKV of the newest token for the selected heads, appended at S - 1
+        ts = cfg["S"] - 1
+        bidx = np.tile(np.arange(batch, dtype=np.int32), (cfg["Hk"], 1))
+        qkv = O.qkv_proj_sparse(n["x"], n["Wqkv"], want_heads, bidx, n["bqkv"])
+        kc = O.pack_k_cache(np.ascontiguousarray(n["k_cache_bhsd"].transpose(0, 2, 1, 3)))
+        vc = n["v_cache"].copy()
+        ctx = O.single_query_attention(qkv[:, 0], qkv[:, 1], qkv[:, 2], kc, vc, ts, head_idx=want_heads)
+        wout = np.ascontiguousarray(n["Wout_t"].reshape(H, hd, d).transpose(2, 0, 1))  # (d, H, hd)
+        want_attn = O.out_proj_sparse(ctx, wout, want_heads, n["bout"])
+        assert_close(attn.numpy(), want_attn, f"cpu baseline attention, batch {batch}")
