@@ -53,7 +53,7 @@ CSRC_DIR = os.path.join(ROOT, "dejavu_amd", "csrc")
 
 
 # sources of the kernels whose traffic is recorded (the QKV projection, stand-alone and inside the fused layer)
-TRAFFIC_SOURCES = ("attention.hpp", "common.hpp", "gemm_mfma.hpp", "layer_fused.hpp", "qkv_mfma.hpp")
+TRAFFIC_SOURCES = ("attention.hpp", "common.hpp", "gemm_mfma.hpp", "layer_fused.hpp", "norm.hpp", "qkv_mfma.hpp")
 
 
 def csrc_digest():
@@ -314,6 +314,20 @@ def kernel_table(torch, cfg, batch, layers):
         fns["qkv_flush_mfma"] = lambda L: ops.qkv_proj_sparse(xw, W(L), all_heads, bi16, bq(L), out=qkv[:16])
         nbytes["qkv_window_mfma"] = nbytes["qkv_sparse"]
         nbytes["qkv_flush_mfma"] = 3 * H * hd * d * 2
+        # the same three as the fused layer runs them (layer_l2_kernel<1>, <0>, <-1>): every workgroup
+        # also normalises the newest row from the LayerNorm statistics of its 64-column parts
+        blk0 = layers[0]["block"]
+        r1, parts = ops.add_ln_parts(layers[0]["hidden"].view(1, d), layers[0]["residual"].view(1, d))
+        ln = (blk0.norm1.weight, blk0.norm1.bias, blk0.norm1.eps)
+        xw2 = xw.clone()  # the launches store the normalised row into the window buffer they are given
+        fns["qkv_l2_one_token"] = lambda L: ops.ln_qkv_proj_sparse(r1, parts, *ln, xw2, 0, W(L), head_idx, batch_idx,
+                                                                   bq(L), out=qkv[:1])
+        fns["qkv_l2_mfma"] = lambda L: ops.ln_qkv_proj_sparse(r1, parts, *ln, xw2, 7, W(L), head_idx, bi8, bq(L),
+                                                              out=qkv[:8])
+        fns["qkv_l2_flush"] = lambda L: ops.ln_qkv_proj_sparse(r1, parts, *ln, xw2, 15, W(L), all_heads, bi16, bq(L),
+                                                               out=qkv[:16])
+        nbytes["qkv_l2_one_token"] = nbytes["qkv_l2_mfma"] = nbytes["qkv_sparse"]
+        nbytes["qkv_l2_flush"] = nbytes["qkv_flush_mfma"]
     else:
         fns["qkv_batch"] = lambda L: ops.qkv_proj_batch(x, W(L), head_idx, bq(L), out=qkv[:batch])
         nbytes["qkv_batch"] = nbytes["qkv_sparse"]
@@ -624,6 +638,20 @@ def holds_gpu():
     return False
 
 
+def kill_group(p):
+    """Ends a child started with start_new_session=True together with everything it started."""
+    import signal
+
+    try:
+        os.killpg(p.pid, signal.SIGKILL)
+    except (ProcessLookupError, PermissionError):
+        pass
+    try:
+        p.communicate(timeout=30)
+    except Exception:
+        pass
+
+
 def other_workloads():
     """Runs `bench.py --batch 8 / 16 / 32 --window cycle` and `bench.py --workload decode` as child processes
     (one at a time, each bounded) and returns the figures of their JSON lines; a leg that fails is reported as
@@ -633,14 +661,17 @@ def other_workloads():
     def child(argv, limit):
         cmd = [sys.executable, os.path.abspath(__file__), *argv, "--no-cpu-baseline"]
         t0 = time.perf_counter()
+        # a session of its own: on a timeout the whole process group goes, not only the direct child
+        p = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, start_new_session=True)
         try:
-            r = subprocess.run(cmd, capture_output=True, text=True, timeout=limit)
-            lines = [ln for ln in r.stdout.strip().splitlines() if ln.startswith("{")]
-            if r.returncode != 0 or not lines:
-                return {"error": f"exit {r.returncode}: {r.stderr.strip()[-200:]}"}, time.perf_counter() - t0
-            return json.loads(lines[-1]), time.perf_counter() - t0
+            stdout, stderr = p.communicate(timeout=limit)
         except subprocess.TimeoutExpired:
+            kill_group(p)
             return {"error": f"no result within {limit} s"}, time.perf_counter() - t0
+        lines = [ln for ln in stdout.strip().splitlines() if ln.startswith("{")]
+        if p.returncode != 0 or not lines:
+            return {"error": f"exit {p.returncode}: {stderr.strip()[-200:]}"}, time.perf_counter() - t0
+        return json.loads(lines[-1]), time.perf_counter() - t0
 
     out = {"batched_layer": {}, "how": "child processes of this script, run after the headline leg"}
     for b in (8, 16, 32):
@@ -669,11 +700,17 @@ def coordinate_legs():
     import subprocess
 
     cmd = [sys.executable, os.path.abspath(__file__), *sys.argv[1:], "--no-other-workloads"]
-    r = subprocess.run(cmd, stdout=subprocess.PIPE, text=True)  # stderr passes through
-    lines = [ln for ln in r.stdout.strip().splitlines() if ln.startswith("{")]
-    if r.returncode != 0 or not lines:
-        sys.stdout.write(r.stdout)
-        sys.exit(r.returncode or 1)
+    p = subprocess.Popen(cmd, stdout=subprocess.PIPE, text=True, start_new_session=True)  # stderr passes through
+    try:
+        stdout, _ = p.communicate(timeout=1500)
+    except subprocess.TimeoutExpired:
+        kill_group(p)
+        print("bench.py: the headline leg did not finish within 1500 s", file=sys.stderr)
+        sys.exit(1)
+    lines = [ln for ln in stdout.strip().splitlines() if ln.startswith("{")]
+    if p.returncode != 0 or not lines:
+        sys.stdout.write(stdout)
+        sys.exit(p.returncode or 1)
     out = json.loads(lines[-1])
     out["other_workloads"] = other_workloads()
     print(json.dumps(out))
@@ -843,11 +880,14 @@ def main():
         for g in warm:
             g.replay()
         torch.cuda.synchronize()
-        t0 = time.perf_counter()
+        # between two HIP events on the launch stream (the host clock would add a graph launch's latency)
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
         for g in timed:
             g.replay()
+        b.record()
         torch.cuda.synchronize()
-        return (time.perf_counter() - t0) / n_timed * 1e6
+        return a.elapsed_time(b) * 1e3 / n_timed
 
     nbytes = algorithmic_bytes(cfg, batch)
     start_bytes = sum(nbytes.values())
@@ -939,13 +979,14 @@ def main():
             n0 = positions[0] if cycle else args.steps
             n1 = sum(positions[1:WINDOW - 1]) if cycle else 0
             n2 = positions[WINDOW - 1] if cycle else 0
-            mix = (("qkv_sparse", n0), ("qkv_window_mfma", n1), ("qkv_flush_mfma", n2))
+            mix = (("qkv_l2_one_token", n0), ("qkv_l2_mfma", n1), ("qkv_l2_flush", n2))
             mix_bytes = sum(table[k]["MB"] * 1e6 * n for k, n in mix)
             mix_us = sum(table[k]["us"] * n for k, n in mix)
             launches = n0 + n1 + n2
-            roofline = {"bound": "hbm", "kernel": "QKV projection of the timed schedule: qkv_sparse_kernel (window "
-                        "position 0), qkv_window_mfma_kernel<4,1> (positions 1-14), qkv_window_mfma_kernel<4,2> "
-                        "(flush); the fused layer runs the same bodies as layer_l2_kernel<1>, <0>, <-1>",
+            roofline = {"bound": "hbm", "kernel": "QKV projection (LayerNorm 1 applied by its workgroups) of the timed "
+                        "schedule: layer_l2_kernel<1> (window position 0), layer_l2_kernel<0> (positions 1-14, matrix "
+                        "cores), layer_l2_kernel<-1> (flush), each launched alone through "
+                        "dv_ln_qkv_proj_sparse_cache_f16",
                         "achieved": round(mix_bytes / mix_us / 1e3, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                         "frac": round(mix_bytes / mix_us / 1e3 / HBM_PEAK_GBPS, 4),
                         "traffic": None,
@@ -986,6 +1027,8 @@ def main():
         "metric": "us_per_layer, sparse MLP+attn decode, OPT-175B layer K=4096" if args.config == "opt-175b"
         else f"us_per_layer, sparse MLP+attn decode, {args.config}",
         "value": round(us_per_layer, 2),
+        "value_window_average": None if window_average_us is None else round(window_average_us, 2),
+        "value_window_start": None if window_start_us is None else round(window_start_us, 2),
         "unit": "us/layer",
         "n_gpus": 1,
         "steps": args.steps,

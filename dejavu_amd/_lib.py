@@ -98,6 +98,11 @@ SIGNATURES = {
         _c_int,
         [_c_ptr, _c_ptr, _c_i64, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_int, _c_int,
          _c_int, _c_ptr]),
+    "dv_add_ln_parts_f16": (_c_int, [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr]),
+    "dv_ln_qkv_proj_sparse_cache_f16": (
+        _c_int,
+        [_c_ptr, _c_ptr, _c_ptr, _c_ptr, ctypes.c_float, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
+         _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr]),
     "dv_add_layer_norm_f16": (
         _c_int, [_c_ptr, _c_ptr, _c_ptr, _c_ptr, ctypes.c_float, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr]),
     "dv_window_step_f16": (

@@ -1570,6 +1570,36 @@ int check_layer_args(const dvSparseLayerArgs& a, bool first) {
   return DV_OK;
 }
 
+// LayerNorm 1 + QKV (+ cache scatter) of a window position: one token on the vector ALUs, several on
+// the matrix cores
+int launch_ln_qkv(const QkvArgs& q, hipStream_t s) {
+  const int cus = compute_units();
+  const bool mfma = qkv_use_mfma(q.nb);
+  const bool two = mfma && qkv_mfma_two_tiles(q.nnz, q.hd);
+  if (mfma) {
+    const dim3 grid(q.nnz * 3 * (q.hd / (two ? 32 : 16)));
+    if (two) hipLaunchKernelGGL((layer_l2_kernel<-1>), grid, dim3(256), 0, s, q);
+    else hipLaunchKernelGGL((layer_l2_kernel<0>), grid, dim3(256), 0, s, q);
+  } else {
+    // one task (two weight rows) per wavefront; workgroups of eight wavefronts when that still
+    // leaves two per compute unit (fewer copies of the row to normalise), else of four
+    const int ntasks = q.nnz * 3 * (q.hd / 2);
+    const int waves = ntasks >= cus * 16 ? 8 : 4;
+    int nq = (ntasks + waves - 1) / waves;
+    if (nq > cus * (24 / waves)) nq = cus * (24 / waves);
+    const size_t lds = (size_t)q.d * sizeof(half_t);
+    static LdsGrant grant[2];
+    if (q.d <= 16384) {
+      if (int rc = grant[0].ensure(reinterpret_cast<const void*>(layer_l2_kernel<1>), lds); rc != DV_OK) return rc;
+      hipLaunchKernelGGL((layer_l2_kernel<1>), dim3(nq), dim3(waves * 64), lds, s, q);
+    } else {
+      if (int rc = grant[1].ensure(reinterpret_cast<const void*>(layer_l2_kernel<2>), lds); rc != DV_OK) return rc;
+      hipLaunchKernelGGL((layer_l2_kernel<2>), dim3(nq), dim3(waves * 64), lds, s, q);
+    }
+  }
+  return launch_status();
+}
+
 // the scratch of a call is the first block's; every block of the call needs no more than it holds
 size_t layers_workspace_bytes(const dvSparseLayerArgs* layers, int n) {
   size_t need = 0;
@@ -1669,29 +1699,7 @@ int dv_sparse_layers_decode_f16(const dvSparseLayerArgs* layers, int n_layers, v
                 reinterpret_cast<const int*>(a.cache_offset), a.S,
                 QkvLnArgs{res1, reinterpret_cast<const float2*>(ws + p.off_parts), CH(a.ln1_w), CH(a.ln1_b), a.eps1,
                           x_cache + (size_t)a.counter * a.d, a.counter}};
-      const bool mfma = qkv_use_mfma(nb);
-      const bool two = mfma && qkv_mfma_two_tiles(a.Hk, a.hd);
-      if (mfma) {
-        const dim3 grid(a.Hk * 3 * (a.hd / (two ? 32 : 16)));
-        if (two) hipLaunchKernelGGL((layer_l2_kernel<-1>), grid, dim3(256), 0, s, q);
-        else hipLaunchKernelGGL((layer_l2_kernel<0>), grid, dim3(256), 0, s, q);
-      } else {
-        // one task (two weight rows) per wavefront; workgroups of eight wavefronts when that still
-        // leaves two per compute unit (fewer copies of the row to normalise), else of four
-        const int ntasks = a.Hk * 3 * (a.hd / 2);
-        const int waves = ntasks >= cus * 16 ? 8 : 4;
-        int nq = (ntasks + waves - 1) / waves;
-        if (nq > cus * (24 / waves)) nq = cus * (24 / waves);
-        const size_t lds = (size_t)a.d * sizeof(half_t);
-        static LdsGrant grant[2];
-        if (a.d <= 16384) {
-          if (int rc = grant[0].ensure(reinterpret_cast<const void*>(layer_l2_kernel<1>), lds); rc != DV_OK) return rc;
-          hipLaunchKernelGGL((layer_l2_kernel<1>), dim3(nq), dim3(waves * 64), lds, s, q);
-        } else {
-          if (int rc = grant[1].ensure(reinterpret_cast<const void*>(layer_l2_kernel<2>), lds); rc != DV_OK) return rc;
-          hipLaunchKernelGGL((layer_l2_kernel<2>), dim3(nq), dim3(waves * 64), lds, s, q);
-        }
-      }
+      if (int rc = launch_ln_qkv(q, s); rc != DV_OK) return rc;
     }
     // L3: attention partials | head predictor fc0 | top-k threshold and counts | accumulator reset.
     // The head predictor (input: the residual stream, output: only needed at the end of the step)
@@ -1774,6 +1782,52 @@ int dv_sparse_layers_decode_f16(const dvSparseLayerArgs* layers, int n_layers, v
 
 int dv_sparse_layer_decode_f16(const dvSparseLayerArgs* args, void* stream) {
   return dv_sparse_layers_decode_f16(args, 1, stream);
+}
+
+int dv_add_ln_parts_f16(const void* h, const void* residual, int d, void* r_out, void* parts, void* stream) {
+  if (!h || !r_out || !parts || d <= 0) return DV_ERR_INVALID_ARG;
+  if (d % 8 || !aligned16(h) || !aligned16(r_out) || (residual && !aligned16(residual)) ||
+      (reinterpret_cast<uintptr_t>(parts) & 7u))
+    return DV_ERR_ALIGNMENT;
+  if (d > kLnMaxParts * kLnPart) return DV_ERR_UNSUPPORTED;
+  PreArgs pa{};
+  pa.partial = nullptr;
+  pa.bias = nullptr;
+  pa.G = 1;
+  pa.d = d;
+  pa.Y = const_cast<half_t*>(reinterpret_cast<const half_t*>(h));  // read only: no partial sums to finish
+  pa.R = reinterpret_cast<const half_t*>(residual);
+  pa.Rout = reinterpret_cast<half_t*>(r_out);
+  pa.parts = reinterpret_cast<float2*>(parts);
+  const int nred = (d + 63) / 64;
+  hipLaunchKernelGGL(layer_pre_kernel, dim3(nred), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), pa, nred, 0);
+  return launch_status();
+}
+
+int dv_ln_qkv_proj_sparse_cache_f16(const void* r1, const void* parts, const void* gamma, const void* beta,
+                                    float eps, void* x_cache, int token, const void* W, const void* bias,
+                                    const void* head_idx, const void* batch_idx, int nb, int d, int H, int hd,
+                                    int nnz, void* y, void* k_cache, void* v_cache, const void* padding, int S,
+                                    void* stream) {
+  if (!r1 || !parts || !gamma || !beta || !x_cache || !W || !y || nb < 1 || nb > 16 || token != nb - 1 || d <= 0 ||
+      H <= 0 || nnz < 0 || nnz > H || (nnz > 0 && (!head_idx || !batch_idx)) || ((k_cache == nullptr) != (v_cache == nullptr)) ||
+      (k_cache && S <= 0))
+    return DV_ERR_INVALID_ARG;
+  if ((hd != 64 && hd != 128) || d > kLnMaxParts * kLnPart || (size_t)d * 2 > 144 * 1024) return DV_ERR_UNSUPPORTED;
+  if (d % 8 || !aligned16(r1) || !aligned16(gamma) || !aligned16(beta) || !aligned16(x_cache) || !aligned16(W) ||
+      (reinterpret_cast<uintptr_t>(parts) & 7u))
+    return DV_ERR_ALIGNMENT;
+  if (nnz == 0) return DV_OK;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  half_t* xc = reinterpret_cast<half_t*>(x_cache);
+  QkvArgs q{xc, reinterpret_cast<const half_t*>(W), reinterpret_cast<const half_t*>(bias),
+            reinterpret_cast<const int*>(head_idx), reinterpret_cast<const int*>(batch_idx), nb, d, H, hd, nnz,
+            reinterpret_cast<half_t*>(y), reinterpret_cast<half_t*>(k_cache), reinterpret_cast<half_t*>(v_cache),
+            reinterpret_cast<const int*>(padding), S,
+            QkvLnArgs{reinterpret_cast<const half_t*>(r1), reinterpret_cast<const float2*>(parts),
+                      reinterpret_cast<const half_t*>(gamma), reinterpret_cast<const half_t*>(beta), eps,
+                      xc + (size_t)token * d, token}};
+  return launch_ln_qkv(q, s);
 }
 
 }  // extern "C"

@@ -720,6 +720,69 @@ def add_layer_norm(hidden: torch.Tensor, residual: Optional[torch.Tensor], weigh
     return y, r_out
 
 
+def add_ln_parts(hidden: torch.Tensor, residual: Optional[torch.Tensor]):
+    """First half of ``add_layer_norm`` for ONE row when the consumer of the row normalises it itself:
+    ``r = hidden + residual`` (fp16) and the statistics pairs of r's 64-element parts (float32,
+    (ceil(d / 64), 2): sum, sum of squared deviations from the part's mean).  Returns (r, parts)."""
+    _require_device(hidden, residual)
+    assert hidden.dtype == torch.float16
+    d = hidden.shape[-1]
+    assert hidden.numel() == d, "one row"
+    hidden = hidden.contiguous()
+    if residual is not None:
+        assert residual.shape == hidden.shape and residual.dtype == hidden.dtype
+        residual = residual.contiguous()
+    r_out = torch.empty_like(hidden)
+    parts = torch.empty((d + 63) // 64, 2, dtype=torch.float32, device=hidden.device)
+    check(lib.dv_add_ln_parts_f16(_ptr(hidden), _ptr(residual), d, _ptr(r_out), _ptr(parts), _stream()),
+          "dv_add_ln_parts_f16")
+    return r_out, parts
+
+
+def ln_qkv_proj_sparse(r: torch.Tensor, parts: torch.Tensor, ln_weight: torch.Tensor, ln_bias: torch.Tensor,
+                       eps: float, x_cache: torch.Tensor, token: int, weight: torch.Tensor, head_idx: torch.Tensor,
+                       batch_idx: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                       out: Optional[torch.Tensor] = None, k_cache: Optional[torch.Tensor] = None,
+                       v_cache: Optional[torch.Tensor] = None, padding: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``qkv_proj_sparse`` for window position ``token`` with the LayerNorm of the newest row folded
+    in: ``r`` / ``parts`` come from ``add_ln_parts``; the QKV workgroups normalise the row themselves
+    (``ln_weight``, ``ln_bias``, ``eps``), the normalised row lands in ``x_cache[token]`` and rows
+    ``0 .. token - 1`` are read from ``x_cache`` ((16, hidden) window buffer).  Same bits as
+    ``add_layer_norm`` followed by ``qkv_proj_sparse(x_cache[:token + 1], ...)``.  batch_idx:
+    (nnz, token + 1) int32; with token == 0 every listed head is computed."""
+    _require_device(r, parts, ln_weight, ln_bias, x_cache, weight, head_idx, batch_idx, bias)
+    _, nheads, head_dim, hidden_dim = weight.shape
+    nb = token + 1
+    _expect(head_dim in (64, 128), f"head_dim {head_dim} not 64 / 128")
+    _expect(r.numel() == hidden_dim and r.dtype == torch.float16, "r must be one fp16 row")
+    _expect(parts.dtype == torch.float32 and tuple(parts.shape) == ((hidden_dim + 63) // 64, 2), "parts from add_ln_parts")
+    _expect(tuple(x_cache.shape) == (16, hidden_dim) and x_cache.is_contiguous(), "x_cache must be the (16, hidden) window buffer")
+    n_active = head_idx.shape[0]
+    _int32_vector("head_idx", head_idx, n_active)
+    _expect(batch_idx.dtype == torch.int32 and tuple(batch_idx.shape) == (n_active, nb),
+            f"batch_idx must be int32 ({n_active}, {nb})")
+    if bias is not None:
+        bias = bias.contiguous()
+    r, weight, head_idx, batch_idx = r.contiguous(), weight.contiguous(), head_idx.contiguous(), batch_idx.contiguous()
+    if out is None:
+        out = torch.empty(nb, 3, nheads, head_dim, device=r.device, dtype=r.dtype)
+    else:
+        assert out.shape == (nb, 3, nheads, head_dim) and out.is_contiguous() and out.dtype == r.dtype
+    S = 0
+    if k_cache is not None:
+        assert v_cache is not None
+        _require_device(k_cache, v_cache, padding)
+        S = v_cache.shape[2]
+        assert v_cache.shape == (1, nheads, S, head_dim) and k_cache.shape == (1, nheads, head_dim // 8, S, 8)
+        assert k_cache.is_contiguous() and v_cache.is_contiguous()
+    check(lib.dv_ln_qkv_proj_sparse_cache_f16(_ptr(r), _ptr(parts), _ptr(ln_weight.contiguous()),
+                                              _ptr(ln_bias.contiguous()), float(eps), _ptr(x_cache), token,
+                                              _ptr(weight), _ptr(bias), _ptr(head_idx), _ptr(batch_idx), nb, hidden_dim,
+                                              nheads, head_dim, n_active, _ptr(out), _ptr(k_cache), _ptr(v_cache),
+                                              _ptr(padding), S, _stream()), "dv_ln_qkv_proj_sparse_cache_f16")
+    return out
+
+
 def attention_out_proj(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, head_idx: torch.Tensor,
                        timestep: int, weight_t: torch.Tensor, bias: Optional[torch.Tensor] = None,
                        lengths_per_sample: Optional[torch.Tensor] = None,

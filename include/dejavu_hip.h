@@ -381,6 +381,32 @@ DV_API int dv_out_proj_sparse_t_f16(const void* x, const void* Wt, int64_t ldw, 
                                     void* stream);
 
 /*
+ * The two halves of that add + LayerNorm when the LayerNorm is applied by the consumer of the
+ * row (the same reference lines, block_dejavu.py:575-584):
+ *   dv_add_ln_parts_f16: r_out = fp16(h + residual) (h alone when residual is NULL) and, for
+ *     every 64 consecutive elements of r_out, the pair (sum, sum of squared deviations from the
+ *     part's own mean) as two floats: parts (ceil(d / 64), 2).  From these pairs any consumer
+ *     derives mean and variance of the row in a fixed order.
+ *   dv_ln_qkv_proj_sparse_cache_f16: dv_qkv_proj_sparse_cache_f16 (below the reference's
+ *     qkv_proj_sparse, attention_proj_sparse.py:110-194) for window position `token` = nb - 1,
+ *     whose LayerNorm row is not in the window buffer yet: every workgroup normalises r1 itself
+ *     (gamma, beta, eps) from `parts`, the normalised row is also stored to x_cache[token], the
+ *     other nb - 1 rows are read from x_cache.  Bit-identical to dv_add_layer_norm_f16 followed
+ *     by dv_qkv_proj_sparse_cache_f16.  With nb == 1 every head of head_idx is computed (at the
+ *     first window position no head has the token yet; batch_idx is not read).
+ *   h, residual, r_out, r1, gamma, beta: (d,); x_cache: (16, d); d % 8 == 0, d <= 32768;
+ *   hd 64 or 128; the other arguments as dv_qkv_proj_sparse_cache_f16.
+ */
+DV_API int dv_add_ln_parts_f16(const void* h, const void* residual, int d, void* r_out, void* parts,
+                               void* stream);
+DV_API int dv_ln_qkv_proj_sparse_cache_f16(const void* r1, const void* parts, const void* gamma,
+                                           const void* beta, float eps, void* x_cache, int token,
+                                           const void* W, const void* bias, const void* head_idx,
+                                           const void* batch_idx, int nb, int d, int H, int hd, int nnz,
+                                           void* y, void* k_cache, void* v_cache, const void* padding,
+                                           int S, void* stream);
+
+/*
  * Fused residual add + LayerNorm of the pre-norm block:
  *   residual_out = fp16(h + residual)   (h alone when residual is NULL)
  *   y = LayerNorm(residual_out) * gamma + beta, fp32 statistics, fp16 out.

@@ -316,3 +316,52 @@ def test_attention_out_proj_rows_matches_separate_ops(ops, H, hd, d, S, t, nnz):
         ctx_ref[0, h] = (p / p.sum()) @ vn[h, :t + 1]
     ref = O.out_proj_sparse(ctx_ref.astype(np.float16).astype(np.float32), np16(W), hi, np16(bo))
     assert_close(np16(got), ref, "attention+out_proj rows vs oracle")
+
+
+@pytest.mark.parametrize("d,H,Hk", [(1024, 8, 3), (5120, 40, 16), (12288, 96, 32), (4224, 33, 7)])
+def test_layer_norm_folded_into_the_qkv_projection_same_bits(d, H, Hk):
+    """add_ln_parts + ln_qkv_proj_sparse (the QKV workgroups normalise the newest row from the
+    statistics of its 64-element parts) against add_layer_norm + qkv_proj_sparse: projections, cache rows
+    and the stored window row bit for bit, at the first window position (vector kernel), in the
+    middle of a window (matrix cores, some slots dead) and at the flush step (all heads, 16 slots)."""
+    from dejavu_amd import ops
+
+    hd = d // H
+    S = 48
+    g = torch.Generator().manual_seed(d + Hk)
+    W = (torch.randn(3, H, hd, d, generator=g) * 0.02).half().cuda()
+    bias = (torch.randn(3, H, hd, generator=g) * 0.1).half().cuda()
+    ln_w = (1 + 0.1 * torch.randn(d, generator=g)).half().cuda()
+    ln_b = (0.1 * torch.randn(d, generator=g)).half().cuda()
+    window = torch.randn(16, d, generator=g).half().cuda()
+    pad = torch.tensor([20], dtype=torch.int32, device="cuda")
+    for token, heads in ((0, Hk), (6, Hk), (15, H)):
+        nb = token + 1
+        h = (torch.randn(1, d, generator=g) * 2).half().cuda()
+        res = (torch.randn(1, d, generator=g) * 3 + 0.5).half().cuda()
+        head_idx = torch.sort(torch.randperm(H, generator=g)[:heads]).values.int().cuda()
+        bi = torch.arange(nb, dtype=torch.int32).repeat(heads, 1)
+        if 0 < token < 15:  # dead slots: tokens some heads already have (never the newest one)
+            dead = torch.rand(heads, nb, generator=g) < 0.4
+            dead[:, token] = False
+            bi[dead] = -1
+        bi = bi.cuda()
+        print(f"case LayerNorm folded into QKV d={d} token={token} heads={heads}", flush=True)
+        outs = []
+        for folded in (False, True):
+            xc = window.clone()
+            kc = torch.zeros(1, H, hd // 8, S, 8, dtype=torch.float16, device="cuda")
+            vc = torch.zeros(1, H, S, hd, dtype=torch.float16, device="cuda")
+            y = torch.zeros(nb, 3, H, hd, dtype=torch.float16, device="cuda")
+            if folded:
+                r, parts = ops.add_ln_parts(h, res)
+                ops.ln_qkv_proj_sparse(r, parts, ln_w, ln_b, 1e-5, xc, token, W, head_idx, bi, bias, out=y,
+                                       k_cache=kc, v_cache=vc, padding=pad)
+            else:
+                x, r = ops.add_layer_norm(h, res, ln_w, ln_b, 1e-5)
+                xc[token] = x[0]
+                ops.qkv_proj_sparse(xc[:nb], W, head_idx, bi, bias, out=y, k_cache=kc, v_cache=vc, padding=pad)
+            torch.cuda.synchronize()
+            outs.append((r, xc, y, kc, vc))
+        for name, a, b in zip(("residual row", "window buffer", "projections", "key cache", "value cache"), *outs):
+            assert torch.equal(a, b), f"token {token}: {name} differs"
