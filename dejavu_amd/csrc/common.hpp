@@ -23,6 +23,16 @@ __device__ __forceinline__ half8_t load8(const half_t* p) {
 __device__ __forceinline__ half8_t load8_stream(const half_t* p) {
   return __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(p));
 }
+// The same from a pointer that is known to point into LDS (a generic pointer would make the
+// access a flat load, which the hardware cannot order against global loads without waiting for all).
+__device__ __forceinline__ half8_t load8_lds(const half_t* p) {
+  return *(const __attribute__((address_space(3))) half8_t*)(p);
+}
+template <bool LDS>
+__device__ __forceinline__ half8_t load8_from(const half_t* p) {
+  if constexpr (LDS) return load8_lds(p);
+  else return load8(p);
+}
 __device__ __forceinline__ void store8(half_t* p, half8_t v) {
   *reinterpret_cast<half8_t*>(p) = v;
 }
@@ -76,8 +86,13 @@ __device__ __forceinline__ int64_t load_index(const void* idx, int idx_bytes, in
 // Fixed-point form of an fp32 partial sum: v * 2^32 rounded to the nearest integer.  Integer
 // additions commute, so partial sums added in this form give the same bits in any order.
 __device__ __forceinline__ long long to_fixed(float v) { return __float2ll_rn(v * 4294967296.f); }
+// Back to fp32 with three single-precision operations (no 64-bit arithmetic): the integer part is
+// exact in fp32 for every sum of interest, the fraction is rounded to 24 bits, the sum once more.
+// Every consumer of a fixed-point sum uses this function, so all of them see the same bits.
 __device__ __forceinline__ float from_fixed(long long a) {
-  return (float)(__ll2double_rn(a) * 2.3283064365386963e-10);
+  const int hi = (int)(a >> 32);
+  const unsigned lo = (unsigned)a;
+  return __builtin_fmaf((float)lo, 2.3283064365386963e-10f, (float)hi);
 }
 
 __device__ __forceinline__ float relu_f(float x) { return x >= 0.f ? x : 0.f; }

@@ -213,28 +213,32 @@ size_t cols_workspace_bytes(int B, int N, int M) {
   return (size_t)p.groups * B * N * sizeof(float);
 }
 
+// fixed: the row groups' partial sums are added in fixed point (also with a single group), the form
+// the fused layer step uses for out_proj; else in fp32 in a fixed order (fc2)
 template <int B, bool IDX64, bool BLOCKED>
 void launch_cols(const ColsPlan& p, const half_t* x, int64_t ldx, int x_expanded, const half_t* W,
                  int64_t ldw, const half_t* bias, const void* idx, int blk, int N, int Z, int M,
-                 float* partial, half_t* y, hipStream_t s) {
+                 float* partial, half_t* y, bool fixed, hipStream_t s) {
   dim3 grid(p.col_tiles, p.groups);
   hipLaunchKernelGGL((gather_cols_kernel<B, 8, IDX64, BLOCKED>), grid, dim3(256), 0, s, x, ldx, x_expanded, W, ldw,
-                     bias, idx, blk, N, Z, M, p.rows_per_block, partial, y);
-  if (p.groups > 1) {
-    const int64_t total = (int64_t)B * N;
+                     bias, idx, blk, N, Z, M, p.rows_per_block, partial, y, (const float*)nullptr, 0, fixed ? 1 : 0);
+  const int64_t total = (int64_t)B * N;
+  if (fixed)
+    hipLaunchKernelGGL(cols_reduce_kernel<true>, dim3((unsigned)((total + 63) / 64)), dim3(256), 0, s, partial, bias,
+                       p.groups, B, N, y, (const half_t*)nullptr, (half_t*)nullptr);
+  else if (p.groups > 1)
     hipLaunchKernelGGL(cols_reduce_kernel<false>, dim3((unsigned)((total + 63) / 64)), dim3(256), 0, s,
                        partial, bias, p.groups, B, N, y, (const half_t*)nullptr, (half_t*)nullptr);
-  }
 }
 
 int gather_cols(const half_t* x, int64_t ldx, int x_expanded, const half_t* W, int64_t ldw,
                 const half_t* bias, const void* idx, int idx_bytes, int blk, int B, int N, int Z,
-                int M, half_t* y, void* workspace, size_t workspace_bytes, hipStream_t s) {
+                int M, half_t* y, void* workspace, size_t workspace_bytes, hipStream_t s, bool fixed = false) {
   const ColsPlan p = plan_cols(N, M);
   if (workspace == nullptr || workspace_bytes < cols_workspace_bytes(B, N, M))
     return DV_ERR_WORKSPACE;
   float* partial = reinterpret_cast<float*>(workspace);
-#define DV_ARGS p, x, ldx, x_expanded, W, ldw, bias, idx, blk, N, Z, M, partial, y, s
+#define DV_ARGS p, x, ldx, x_expanded, W, ldw, bias, idx, blk, N, Z, M, partial, y, fixed, s
 #define DV_CASE(BB)                                                   \
   case BB:                                                            \
     if (blk == 1) {                                                   \
@@ -1462,10 +1466,12 @@ int dv_out_proj_sparse_t_f16(const void* x, const void* Wt, int64_t ldw, const v
                             reinterpret_cast<const half_t*>(Wt), ldw, reinterpret_cast<const half_t*>(bias),
                             head_idx, 4, hd, B, N, H * hd, nnz * hd, reinterpret_cast<half_t*>(y), workspace,
                             workspace_bytes, reinterpret_cast<hipStream_t>(stream));
+  // up to four rows: partial sums added in fixed point, the bits of dv_attention_out_proj_f16 and of
+  // the fused layer step
   return gather_cols(reinterpret_cast<const half_t*>(x), (int64_t)H * hd, 1,
                      reinterpret_cast<const half_t*>(Wt), ldw, reinterpret_cast<const half_t*>(bias),
                      head_idx, 4, hd, B, N, H * hd, nnz * hd, reinterpret_cast<half_t*>(y),
-                     workspace, workspace_bytes, reinterpret_cast<hipStream_t>(stream));
+                     workspace, workspace_bytes, reinterpret_cast<hipStream_t>(stream), true);
 }
 
 size_t dv_qkv_window_batch_workspace_bytes(int tokens, int nseq, int d, int nnz, int hd) {

@@ -18,7 +18,8 @@ namespace dv {
 // the LANES partials are combined with an xor butterfly (LANES/2 .. 1).
 // Requires n % 8 == 0 and ldw % 8 == 0.
 // ---------------------------------------------------------------------------
-template <int LANES, int B, int U>
+// X_LDS: X points into LDS (a copy of the row the workgroup holds).
+template <int LANES, int B, int U, bool X_LDS = false>
 __device__ __forceinline__ void canonical_gemv_body(
     const half_t* __restrict__ X, const half_t* __restrict__ W, int64_t ldw, int rows, int n,
     half_t* __restrict__ Y, int block_id, int nblocks) {
@@ -47,7 +48,7 @@ __device__ __forceinline__ void canonical_gemv_body(
       for (int u = 0; u < U; ++u) {
 #pragma unroll
         for (int b = 0; b < B; ++b)
-          acc[b] = fma8_ordered(w[u], load8(xr + (int64_t)b * n + base + u * CH), acc[b]);
+          acc[b] = fma8_ordered(w[u], load8_from<X_LDS>(xr + (int64_t)b * n + base + u * CH), acc[b]);
       }
     }
     if (base < n) {
@@ -65,7 +66,7 @@ __device__ __forceinline__ void canonical_gemv_body(
         if (in[u]) {
 #pragma unroll
           for (int b = 0; b < B; ++b)
-            acc[b] = fma8_ordered(w[u], load8(xr + (int64_t)b * n + base + u * CH), acc[b]);
+            acc[b] = fma8_ordered(w[u], load8_from<X_LDS>(xr + (int64_t)b * n + base + u * CH), acc[b]);
         }
       }
     }
@@ -93,9 +94,10 @@ __global__ __launch_bounds__(256) void canonical_gemv_kernel(
 // (t * R + r) * (64 / LANES) + group.  Same products in the same order per output as
 // canonical_gemv_body, so the same bits.  Dynamic LDS: B * n * 4 bytes.
 // count fp16 values (a multiple of 8) -> fp32 in LDS, by the whole workgroup (which then synchronises)
+template <bool X_LDS = false>
 __device__ __forceinline__ void stage_x_f32(const half_t* __restrict__ X, int count, float* xf) {
   for (int i = threadIdx.x * 8; i < count; i += blockDim.x * 8) {
-    const half8_t v = load8(X + i);
+    const half8_t v = load8_from<X_LDS>(X + i);
 #pragma unroll
     for (int e = 0; e < 8; ++e) xf[i + e] = (float)v[e];
   }

@@ -94,16 +94,17 @@ struct CanonArgs {
 // take the variant with x in LDS and two weight rows per lane group (more loads in flight)
 constexpr int kCanonShortRows = 2;
 
-// x: the input row (c.X, or a copy the workgroup holds in LDS)
+// X_LDS: the input row is `x`, a copy the workgroup holds in LDS (else c.X)
+template <bool X_LDS = false>
 __device__ __forceinline__ void canonical_role(const CanonArgs& c, int block_id, int nblocks,
                                                const half_t* x = nullptr) {
-  if (x == nullptr) x = c.X;
+  const half_t* xin = X_LDS ? x : c.X;
   if (c.n <= 1024) {
     __shared__ __attribute__((aligned(16))) float s_xf[1024];
-    stage_x_f32(x, c.n, s_xf);
+    stage_x_f32<X_LDS>(xin, c.n, s_xf);
     canonical_gemv_lds_body<16, 1, 8, kCanonShortRows>(s_xf, c.W, c.ldw, c.rows, c.n, c.Y, block_id, nblocks);
   } else
-    canonical_gemv_body<64, 1, 8>(x, c.W, c.ldw, c.rows, c.n, c.Y, block_id, nblocks);
+    canonical_gemv_body<64, 1, 8, X_LDS>(xin, c.W, c.ldw, c.rows, c.n, c.Y, block_id, nblocks);
 }
 
 // NBMAX 1 (d <= 16384) / 2: one window token on the vector ALUs (workgroups of up to 512 threads,
@@ -261,7 +262,7 @@ __global__ __launch_bounds__(512, 4) void layer_l7_kernel(RowsArgs f, int nblk_f
     half_t* xs = reinterpret_cast<half_t*>(smem_raw);
     fixed_add_layer_norm_body<false>(f.acc_fixed, f.out_bias, f.res1, nullptr, nullptr, 0.f, f.n, xs, nullptr);
     __syncthreads();
-    canonical_role(mp0, bid - nblk_fc1, nblk_mp0, xs);
+    canonical_role<true>(mp0, bid - nblk_fc1, nblk_mp0, xs);
   } else {
     // head top-k for the next layer (rank selection, one workgroup)
     __shared__ unsigned s_key[1024];
