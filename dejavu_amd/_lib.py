@@ -17,6 +17,9 @@ LIB_PATH = os.path.join(_PKG_DIR, "libdejavu_hip.so")
 DV_OK = 0
 DV_ACT_ID = 0
 DV_ACT_RELU = 1
+DV_ACT_GELU = 2
+DV_ACT_GELU_APPROX = 3
+DV_ACT_SQUARED_RELU = 4
 
 _c_int = ctypes.c_int
 _c_i64 = ctypes.c_int64

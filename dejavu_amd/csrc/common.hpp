@@ -97,4 +97,16 @@ __device__ __forceinline__ float from_fixed(long long a) {
 
 __device__ __forceinline__ float relu_f(float x) { return x >= 0.f ? x : 0.f; }
 
+// The activations of the reference's gathered fc1 (Dejavu/src/ops/triton/k_activations.py:73-162),
+// applied to the fp32 sum (+ bias) before it is rounded to fp16.  Codes as DV_ACT_* of the C ABI.
+__device__ __forceinline__ float act_f(float x, int act) {
+  switch (act) {
+    case 1: return relu_f(x);
+    case 2: return x * 0.5f * (1.f + erff(x * 0.70710678118654752440f));                    // gelu
+    case 3: return 0.5f * x * (1.f + tanhf(0.79788456080286535588f * x * (1.f + 0.044715f * x * x)));  // gelu_approx
+    case 4: { const float r = relu_f(x); return r * r; }                                    // squared_relu
+    default: return x;
+  }
+}
+
 }  // namespace dv

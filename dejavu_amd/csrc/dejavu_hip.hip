@@ -26,6 +26,7 @@ using namespace dv;
 namespace {
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline bool aligned8(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 7u) == 0; }  // null passes
 inline bool idx_ok(int idx_bytes) { return idx_bytes == 4 || idx_bytes == 8; }
 
 inline int launch_status() { return hipGetLastError() == hipSuccess ? DV_OK : DV_ERR_LAUNCH; }
@@ -148,7 +149,7 @@ int canonical_gemv(const half_t* X, const half_t* W, int64_t ldw, int B, int row
 // ---- gathered row GEMV (fc1) ----------------------------------------------
 template <int B, int R, int U, bool RELU>
 int launch_gather_rows(const half_t* x, const half_t* W, int64_t ldw, const half_t* bias,
-                       const void* idx, int idx_bytes, int N, int Z, int M, half_t* y,
+                       const void* idx, int idx_bytes, int N, int Z, int M, half_t* y, int act,
                        hipStream_t s) {
   auto kern = gather_rows_kernel<B, R, U, RELU>;
   const size_t lds = (size_t)B * N * sizeof(half_t);
@@ -160,7 +161,7 @@ int launch_gather_rows(const half_t* x, const half_t* W, int64_t ldw, const half
   if (blocks > cap) blocks = cap;
   if (blocks < 1) blocks = 1;
   hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), lds, s, x, W, bias, idx, idx_bytes, N, ldw, Z,
-                     M, y);
+                     M, y, act);
   return launch_status();
 }
 
@@ -169,9 +170,9 @@ int gather_rows_b(const half_t* x, const half_t* W, int64_t ldw, const half_t* b
                   const void* idx, int idx_bytes, int N, int Z, int M, int act, half_t* y,
                   hipStream_t s) {
   constexpr int R = B <= 2 ? 2 : 1;
-  if (act == DV_ACT_RELU)
-    return launch_gather_rows<B, R, 4, true>(x, W, ldw, bias, idx, idx_bytes, N, Z, M, y, s);
-  return launch_gather_rows<B, R, 4, false>(x, W, ldw, bias, idx, idx_bytes, N, Z, M, y, s);
+  if (act != DV_ACT_ID)
+    return launch_gather_rows<B, R, 4, true>(x, W, ldw, bias, idx, idx_bytes, N, Z, M, y, act, s);
+  return launch_gather_rows<B, R, 4, false>(x, W, ldw, bias, idx, idx_bytes, N, Z, M, y, act, s);
 }
 
 // ---- gathered column GEMV (fc2 / out_proj over transposed weights) ----------
@@ -271,7 +272,7 @@ constexpr int kColsVecMaxBatch = 4;
 #endif
 template <int BT, bool IDX64, bool RELU>
 int launch_rows_mfma(const half_t* x, const half_t* W, int64_t ldw, const half_t* bias, const void* idx,
-                     int B, int N, int Z, int M, half_t* y, hipStream_t s) {
+                     int B, int N, int Z, int M, half_t* y, int act, hipStream_t s) {
   constexpr bool XLDS = DV_ROWS_XLDS && BT <= 2;
   auto kern = gather_rows_mfma_kernel<BT, IDX64, RELU, false, XLDS>;
   // one 16 x 256 staging tile per wavefront (two with X staged as well); the same memory later
@@ -286,18 +287,18 @@ int launch_rows_mfma(const half_t* x, const half_t* W, int64_t ldw, const half_t
   if (blocks > cap) blocks = cap;
   if (blocks < 1) blocks = 1;
   hipLaunchKernelGGL(kern, dim3(blocks), dim3(kMfmaWaves * 64), lds, s, x, W, bias, idx, B, N, ldw, Z, M, y, 0,
-                     static_cast<float*>(nullptr));
+                     static_cast<float*>(nullptr), act);
   return launch_status();
 }
 
 int gather_rows_mfma(const half_t* x, const half_t* W, int64_t ldw, const half_t* bias, const void* idx,
                      int idx_bytes, int B, int N, int Z, int M, int act, half_t* y, hipStream_t s) {
-  const bool relu = act == DV_ACT_RELU, i64 = idx_bytes == 8;
+  const bool relu = act != DV_ACT_ID, i64 = idx_bytes == 8;  // relu: an activation is applied (act says which)
 #define DV_RM(BT)                                                                              \
-  (relu ? (i64 ? launch_rows_mfma<BT, true, true>(x, W, ldw, bias, idx, B, N, Z, M, y, s)        \
-               : launch_rows_mfma<BT, false, true>(x, W, ldw, bias, idx, B, N, Z, M, y, s))      \
-        : (i64 ? launch_rows_mfma<BT, true, false>(x, W, ldw, bias, idx, B, N, Z, M, y, s)       \
-               : launch_rows_mfma<BT, false, false>(x, W, ldw, bias, idx, B, N, Z, M, y, s)))
+  (relu ? (i64 ? launch_rows_mfma<BT, true, true>(x, W, ldw, bias, idx, B, N, Z, M, y, act, s)        \
+               : launch_rows_mfma<BT, false, true>(x, W, ldw, bias, idx, B, N, Z, M, y, act, s))      \
+        : (i64 ? launch_rows_mfma<BT, true, false>(x, W, ldw, bias, idx, B, N, Z, M, y, act, s)       \
+               : launch_rows_mfma<BT, false, false>(x, W, ldw, bias, idx, B, N, Z, M, y, act, s)))
   if (B <= 16) return DV_RM(1);
   if (B <= 32) return DV_RM(2);
   return DV_RM(4);
@@ -532,7 +533,7 @@ int gemm_tiled(const half_t* X, int64_t ldx, const half_t* W, int64_t ldw, const
       return DV_ERR_WORKSPACE;
     partial = reinterpret_cast<float*>(workspace);
   }
-  const int relu = act == DV_ACT_RELU;
+  const int relu = act;  // activation code of the epilogue (0: none)
   int rc;
 #define DV_TG(BT, WT, KC)                                                                                          \
   do {                                                                                                             \
@@ -959,7 +960,7 @@ int dv_gather_gemv_f16(const void* x, const void* W, int64_t ldw, const void* bi
                        const void* idx, int idx_bytes, int B, int N, int Z, int M, int act,
                        void* y, void* stream) {
   if (!x || !W || N <= 0 || Z <= 0 || M < 0 || (idx && !idx_ok(idx_bytes)) || (M > 0 && !y) ||
-      (!idx && M > Z) || (act != DV_ACT_ID && act != DV_ACT_RELU))
+      (!idx && M > Z) || act < DV_ACT_ID || act > DV_ACT_SQUARED_RELU)
     return DV_ERR_INVALID_ARG;
   if (B < 1 || B > 64) return DV_ERR_UNSUPPORTED;
   if (N % 8 || ldw % 8 || ldw < N || !aligned16(x) || !aligned16(W)) return DV_ERR_ALIGNMENT;
@@ -994,7 +995,7 @@ int dv_gather_gemv_ws_f16(const void* x, const void* W, int64_t ldw, const void*
       workspace_bytes < dv_gather_gemv_workspace_bytes(B, N, M) || !aligned16(workspace))
     return dv_gather_gemv_f16(x, W, ldw, bias, idx, idx_bytes, B, N, Z, M, act, y, stream);
   if (!x || !W || N <= 0 || Z <= 0 || (idx && !idx_ok(idx_bytes)) || !y || (!idx && M > Z) ||
-      (act != DV_ACT_ID && act != DV_ACT_RELU))
+      act < DV_ACT_ID || act > DV_ACT_SQUARED_RELU)
     return DV_ERR_INVALID_ARG;
   if (N % 8 || ldw % 8 || ldw < N || !aligned16(x) || !aligned16(W)) return DV_ERR_ALIGNMENT;
   return gemm_tiled(reinterpret_cast<const half_t*>(x), N, reinterpret_cast<const half_t*>(W), ldw,
@@ -1010,7 +1011,7 @@ size_t dv_dense_linear_workspace_bytes(int rows, int N, int M) {
 int dv_dense_linear_f16(const void* x, int64_t ldx, const void* W, int64_t ldw, const void* bias, int rows, int N,
                         int M, int act, void* y, int64_t ldy, void* workspace, size_t workspace_bytes,
                         void* stream) {
-  if (!x || !W || !y || rows < 0 || N <= 0 || M <= 0 || (act != DV_ACT_ID && act != DV_ACT_RELU))
+  if (!x || !W || !y || rows < 0 || N <= 0 || M <= 0 || act < DV_ACT_ID || act > DV_ACT_SQUARED_RELU)
     return DV_ERR_INVALID_ARG;
   if (N % 8 || ldx % 8 || ldw % 8 || ldx < N || ldw < N || ldy < M || !aligned16(x) || !aligned16(W))
     return DV_ERR_ALIGNMENT;
@@ -1033,7 +1034,9 @@ int dv_gather_transposed_gemv_f16(const void* x, const void* W, int64_t ldw, con
   if (!W || !y || N <= 0 || Z <= 0 || M < 0 || !idx_ok(idx_bytes) || (M > 0 && (!idx || !x)))
     return DV_ERR_INVALID_ARG;
   if (B < 1 || B > 64) return DV_ERR_UNSUPPORTED;
-  if (N % 8 || ldw % 8 || ldw < N || !aligned16(W)) return DV_ERR_ALIGNMENT;
+  // y and the partial sums are written with 16-byte vector stores
+  if (N % 8 || ldw % 8 || ldw < N || !aligned16(W) || !aligned16(y) || (workspace && !aligned16(workspace)))
+    return DV_ERR_ALIGNMENT;
   if (B > kColsVecMaxBatch)
     return gather_cols_mfma(reinterpret_cast<const half_t*>(x), M, 0, reinterpret_cast<const half_t*>(W),
                             ldw, reinterpret_cast<const half_t*>(bias), idx, idx_bytes, 1, B, N, Z, M,
@@ -1050,12 +1053,30 @@ namespace {
 // Scratch of dv_gather_transposed_gemv_static_f16: one array per device, resident until the
 // process ends.  In host code the array's name is only a handle: the device address comes from
 // hipGetSymbolAddress, once per device, and is what the kernels are given.
-__device__ __align__(256) unsigned char scratch[DV_STATIC_SCRATCH_BYTES];
+// The array is DV_STATIC_SCRATCH_STREAMS slots of DV_STATIC_SCRATCH_BYTES: a stream keeps the slot it
+// was given at its first call (calls on one stream are ordered by the stream), so calls on
+// different streams never share partial sums.
+__device__ __align__(256) unsigned char scratch[(size_t)DV_STATIC_SCRATCH_STREAMS * DV_STATIC_SCRATCH_BYTES];
 std::atomic<void*> scratch_ptr[kMaxDevices];
+std::atomic<uintptr_t> scratch_owner[kMaxDevices][DV_STATIC_SCRATCH_STREAMS];  // stream handle + 1, 0: free
 
-int static_scratch(void** out) {
+// Slot of `stream` on device `dev` (taken on first use), or -1 when every slot belongs to another stream.
+int static_scratch_slot(int dev, void* stream) {
+  const uintptr_t key = reinterpret_cast<uintptr_t>(stream) + 1;
+  for (int i = 0; i < DV_STATIC_SCRATCH_STREAMS; ++i) {
+    uintptr_t cur = scratch_owner[dev][i].load(std::memory_order_acquire);
+    if (cur == key) return i;
+    if (cur == 0 && scratch_owner[dev][i].compare_exchange_strong(cur, key, std::memory_order_acq_rel)) return i;
+    if (cur == key) return i;  // another thread registered the same stream meanwhile
+  }
+  return -1;
+}
+
+int static_scratch(void** out, void* stream) {
   const int dev = current_device();
   if (dev < 0) return DV_ERR_UNSUPPORTED;
+  const int slot = static_scratch_slot(dev, stream);
+  if (slot < 0) return DV_ERR_UNSUPPORTED;
   void* p = scratch_ptr[dev].load(std::memory_order_acquire);
   if (p == nullptr) {
     if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) {
@@ -1064,7 +1085,7 @@ int static_scratch(void** out) {
     }
     scratch_ptr[dev].store(p, std::memory_order_release);
   }
-  *out = p;
+  *out = static_cast<unsigned char*>(p) + (size_t)slot * DV_STATIC_SCRATCH_BYTES;
   return DV_OK;
 }
 }  // namespace
@@ -1079,7 +1100,7 @@ int dv_gather_transposed_gemv_static_f16(const void* x, const void* W, int64_t l
   const size_t need = dv_gather_transposed_gemv_workspace_bytes(B, N, M);
   if (need > (size_t)DV_STATIC_SCRATCH_BYTES) return DV_ERR_WORKSPACE;
   void* ws = nullptr;
-  if (int rc = static_scratch(&ws); rc != DV_OK) return rc;
+  if (int rc = static_scratch(&ws, stream); rc != DV_OK) return rc;
   // every word of the partial sums is written before it is read: nothing to clear between calls
   return dv_gather_transposed_gemv_f16(x, W, ldw, bias, idx, idx_bytes, B, N, Z, M, y, ws,
                                        (size_t)DV_STATIC_SCRATCH_BYTES, stream);
@@ -1133,7 +1154,10 @@ int dv_qkv_proj_batch_f16(const void* x, int64_t ldx, const void* W, const void*
       ((k_cache == nullptr) != (v_cache == nullptr)) || (k_cache && S <= 0) || (live && live_stride < 1))
     return DV_ERR_INVALID_ARG;
   if (B > 32 || (hd != 32 && hd != 64 && hd != 128)) return DV_ERR_UNSUPPORTED;
-  if (d % 8 || ldx % 8 || ldx < d || !aligned16(x) || !aligned16(W)) return DV_ERR_ALIGNMENT;
+  // y and the caches take 8-byte vector stores
+  if (d % 8 || ldx % 8 || ldx < d || !aligned16(x) || !aligned16(W) || !aligned8(y) || !aligned8(k_cache) ||
+      !aligned8(v_cache))
+    return DV_ERR_ALIGNMENT;
   if (nnz == 0) return DV_OK;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (B >= kQkvTiledMinBatch && (dv_qkv_proj_batch_workspace_bytes(B, d, nnz, hd) == 0 ||
@@ -1460,7 +1484,8 @@ int dv_out_proj_sparse_t_f16(const void* x, const void* Wt, int64_t ldw, const v
   if (!x || !Wt || !y || nnz < 0 || B < 1 || H <= 0 || hd <= 0 || N <= 0 || (nnz > 0 && !head_idx))
     return DV_ERR_INVALID_ARG;
   if (B > 64) return DV_ERR_UNSUPPORTED;
-  if (N % 8 || ldw % 8 || ldw < N || !aligned16(Wt)) return DV_ERR_ALIGNMENT;
+  if (N % 8 || ldw % 8 || ldw < N || !aligned16(Wt) || !aligned16(y) || (workspace && !aligned16(workspace)))
+    return DV_ERR_ALIGNMENT;
   if (B > 4)
     return gather_cols_mfma(reinterpret_cast<const half_t*>(x), (int64_t)H * hd, 1,
                             reinterpret_cast<const half_t*>(Wt), ldw, reinterpret_cast<const half_t*>(bias),
@@ -1487,7 +1512,9 @@ int dv_qkv_window_batch_f16(const void* x, int64_t ldx, const void* W, const voi
       (nnz > 0 && !head_idx) || ((k_cache == nullptr) != (v_cache == nullptr)) || (k_cache && S <= 0))
     return DV_ERR_INVALID_ARG;
   if (tokens > 16 || nseq > 32 || (hd != 32 && hd != 64 && hd != 128)) return DV_ERR_UNSUPPORTED;
-  if (d % 8 || ldx % 8 || ldx < d || !aligned16(x) || !aligned16(W)) return DV_ERR_ALIGNMENT;
+  if (d % 8 || ldx % 8 || ldx < d || !aligned16(x) || !aligned16(W) || !aligned8(y) || !aligned8(k_cache) ||
+      !aligned8(v_cache))
+    return DV_ERR_ALIGNMENT;
   if (nnz == 0) return DV_OK;
   const QkvScatter qs{reinterpret_cast<const int*>(head_idx), reinterpret_cast<const int*>(batch_idx), tokens, nnz, H,
                       hd, reinterpret_cast<half_t*>(k_cache), reinterpret_cast<half_t*>(v_cache),

@@ -56,7 +56,7 @@ template <int BT, bool IDX64, bool RELU, bool SPLIT = false, bool XLDS = false>
 __global__ __launch_bounds__(kMfmaWaves * 64) void gather_rows_mfma_kernel(
     const half_t* __restrict__ X, const half_t* __restrict__ W, const half_t* __restrict__ bias,
     const void* __restrict__ idx, int B, int N, int64_t ldw, int Z, int M, half_t* __restrict__ Y,
-    int chunks_per_split = 0, float* __restrict__ partial = nullptr) {
+    int chunks_per_split = 0, float* __restrict__ partial = nullptr, int act = 1) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -222,7 +222,7 @@ __global__ __launch_bounds__(kMfmaWaves * 64) void gather_rows_mfma_kernel(
             continue;
           }
           val += (bias != nullptr && ok) ? (float)bias[rid] : 0.f;
-          if (RELU) val = relu_f(val);
+          if (RELU) val = act_f(val, act);  // RELU: an activation is applied, act says which
           if (!ok) val = 0.f;
           const int b = bt * 16 + l16;
           if (m < M && b < B) Y[(int64_t)b * M + m] = (half_t)val;

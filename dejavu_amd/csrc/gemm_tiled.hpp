@@ -264,7 +264,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_tiled_mfma_kernel(
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
         if (bias != nullptr && rid[v] >= 0) val[v] += (float)bias[rid[v]];
-        if (relu) val[v] = relu_f(val[v]);
+        if (relu) val[v] = act_f(val[v], relu);
       }
       if (QKV) {
         // the four values of a lane are four consecutive rows of one (q|k|v, head): hd % 4 == 0
@@ -298,7 +298,7 @@ __global__ __launch_bounds__(256) void gemm_split_reduce_kernel(
     const int64_t id = idx == nullptr ? (int64_t)m : load_index(idx, idx_bytes, m);
     if (id >= 0 && id < Z) s += (float)bias[id];
   }
-  if (relu) s = relu_f(s);
+  if (relu) s = act_f(s, relu);
   Y[(int64_t)b * ldy + m] = (half_t)s;
 }
 

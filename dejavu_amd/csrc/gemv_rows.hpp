@@ -271,11 +271,12 @@ __global__ __launch_bounds__(256) void canonical_gemv_slices_kernel(
 // instead of a wild read; idx == nullptr means no gather (row m of W: a dense product).  Requires n % 8 == 0 and ldw % 8 == 0.
 // ---------------------------------------------------------------------------
 // STAGED: the caller has already put X into xs (and synchronised the workgroup).
+// RELU: an activation is applied, `act` says which (act_f; ReLU unless told otherwise).
 template <int B, int R, int U, bool RELU, bool STAGED = false>
 __device__ __forceinline__ void gather_rows_body(
     const half_t* __restrict__ X, const half_t* __restrict__ W, const half_t* __restrict__ bias,
     const void* __restrict__ idx, int idx_bytes, int n, int64_t ldw, int Z, int M,
-    half_t* __restrict__ Y, half_t* xs, int block_id, int nblocks) {
+    half_t* __restrict__ Y, half_t* xs, int block_id, int nblocks, int act = 1) {
   if (!STAGED) {
     for (int i = threadIdx.x * 8; i < B * n; i += blockDim.x * 8) store8(xs + i, load8(X + i));
     __syncthreads();
@@ -342,7 +343,7 @@ __device__ __forceinline__ void gather_rows_body(
 #pragma unroll
       for (int b = 0; b < B; ++b) {
         float v = butterfly_sum<kWave>(acc[r][b]) + bv;
-        if (RELU) v = relu_f(v);
+        if (RELU) v = act_f(v, act);
         if (!valid[r]) v = 0.f;
         if (lane == 0 && m < M) Y[(int64_t)b * M + m] = (half_t)v;
       }
@@ -354,10 +355,10 @@ template <int B, int R, int U, bool RELU>
 __global__ __launch_bounds__(256) void gather_rows_kernel(
     const half_t* __restrict__ X, const half_t* __restrict__ W, const half_t* __restrict__ bias,
     const void* __restrict__ idx, int idx_bytes, int n, int64_t ldw, int Z, int M,
-    half_t* __restrict__ Y) {
+    half_t* __restrict__ Y, int act = 1) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   gather_rows_body<B, R, U, RELU>(X, W, bias, idx, idx_bytes, n, ldw, Z, M, Y,
-                                  reinterpret_cast<half_t*>(smem_raw), blockIdx.x, gridDim.x);
+                                  reinterpret_cast<half_t*>(smem_raw), blockIdx.x, gridDim.x, act);
 }
 
 }  // namespace dv

@@ -207,16 +207,11 @@ class ParallelFusedMLPDejavu(nn.Module):
             mlp_logit = self.sp(residual)
         if idx != None:
             assert x.size(1) == 1
-            if self.activation != "relu":
-                raise NotImplementedError("the sparse MLP kernels fuse ReLU (OPT); gelu_approx runs dense only")
             out = ops.mlp_sparse(x.squeeze(1), self.fc1.weight, self.transposed_fc2(), idx, self.fc1.bias,
-                                 self.fc2.bias)
+                                 self.fc2.bias, activation=self.activation)
             out = out.unsqueeze(1)
         else:
-            if self.activation == "relu":
-                h = decode_linear(self.fc1, x, "relu")
-            else:
-                h = F.gelu(F.linear(x, self.fc1.weight, self.fc1.bias), approximate="tanh")
+            h = decode_linear(self.fc1, x, self.activation)
             out = decode_linear(self.fc2, h)
         # (tensor parallel all-reduce of `out` is the identity on one GPU)
         if side:
@@ -225,16 +220,25 @@ class ParallelFusedMLPDejavu(nn.Module):
 
 
 def decode_linear(linear: nn.Linear, x: torch.Tensor, activation: str = "id") -> torch.Tensor:
-    """``linear(x)`` (+ ReLU).  The few rows of a decode step (x: (B, 1, d), fp16, on the GPU) are
-    streamed by the row GEMV kernels; anything else (the prompt phase) goes to the library GEMM."""
+    """``activation(linear(x))``.  The rows of a decode step (x: (B, 1, d) with B <= 64, fp16, on the GPU)
+    always go to this package's row kernels (vector ALUs for one or two rows, matrix cores above).  Many
+    rows (the prompt phase) go to the X-shared matrix-core kernel when ``USE_HIP_PROMPT`` is set, else to
+    the library GEMM."""
     on_hip = x.is_cuda and x.dtype == torch.float16 and linear.weight.dtype == torch.float16 and x.shape[-1] % 8 == 0
-    if on_hip and x.dim() == 3 and x.shape[1] == 1 and x.shape[0] <= 16:
+    if on_hip and x.dim() == 3 and x.shape[1] == 1 and x.shape[0] <= 64:
         return ops.dense_decode_linear(x, linear.weight, linear.bias, activation)
     if on_hip and USE_HIP_PROMPT:
-        # many rows (the prompt, or a large decode batch): blocks of X shared through LDS on the matrix cores
         return ops.dense_linear(x, linear.weight, linear.bias, activation)
     y = linear(x)
-    return F.relu(y) if activation == "relu" else y
+    if activation == "relu":
+        return F.relu(y)
+    if activation == "gelu_approx":
+        return F.gelu(y, approximate="tanh")
+    if activation == "gelu":
+        return F.gelu(y)
+    if activation == "squared_relu":
+        return F.relu(y) ** 2
+    return y
 
 
 def _kv_caches(inference_params, layer_idx, H, hd, dtype, device):

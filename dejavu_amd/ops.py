@@ -20,7 +20,8 @@ import torch
 from . import _lib
 from ._lib import check, lib
 
-_ACT = {"id": _lib.DV_ACT_ID, "relu": _lib.DV_ACT_RELU}
+_ACT = {"id": _lib.DV_ACT_ID, "relu": _lib.DV_ACT_RELU, "gelu": _lib.DV_ACT_GELU,
+        "gelu_approx": _lib.DV_ACT_GELU_APPROX, "squared_relu": _lib.DV_ACT_SQUARED_RELU}
 
 
 def _stream() -> int:
@@ -204,8 +205,6 @@ def gather_gemv(x: torch.Tensor, weight: torch.Tensor, idx: Optional[torch.Tenso
     reference's kernel stops at 4; from 3 rows on the product runs on the matrix cores).
     """
     _expect(activation in ("id", "relu", "gelu", "gelu_approx", "squared_relu"), f"unknown activation {activation!r}")
-    if activation not in _ACT:
-        raise NotImplementedError(f"activation {activation!r}: the OPT decode path uses 'relu' / 'id' only")
     _require_device(x, weight, idx, bias)
     _expect(x.dim() == 2 and weight.dim() == 2 and x.shape[1] == weight.shape[1],
             f"x {tuple(x.shape)} and weight {tuple(weight.shape)} must share their last dimension")
@@ -239,8 +238,7 @@ def dense_linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Ten
     """``activation(F.linear(x, weight, bias))`` for any number of rows on the matrix cores: the dense
     products of the prompt phase.  x: (..., N) fp16 with a contiguous last dimension (rows may be
     strided after flattening); weight: (M, N); returns (..., M)."""
-    if activation not in _ACT:
-        raise NotImplementedError(f"activation {activation!r}: 'relu' / 'id' only")
+    _expect(activation in _ACT, f"unknown activation {activation!r}")
     _require_device(x, weight, bias, out)
     M, N = weight.shape
     assert x.shape[-1] == N and x.dtype == weight.dtype == torch.float16
@@ -309,11 +307,12 @@ def gather_transposed_gemv(x: torch.Tensor, weight: torch.Tensor, idx: torch.Ten
     return output
 
 
-def mlp_sparse(x, W1, W2t, idx, bias1=None, bias2=None):
-    """The sparse MLP on the neurons ``idx``: ReLU(fc1) then fc2, two gathered products
-    (gather_gemv.py:647-657).  x (batch, d); W1 and W2t both (ffn, d), W2t being fc2.weight
-    transposed so that a neuron's fc2 column is a contiguous row; bias1 (ffn,), bias2 (d,)."""
-    hidden = gather_gemv(x, W1, idx, bias1, activation="relu")
+def mlp_sparse(x, W1, W2t, idx, bias1=None, bias2=None, activation="relu"):
+    """The sparse MLP on the neurons ``idx``: activation(fc1) then fc2, two gathered products
+    (gather_gemv.py:647-657, where the activation is ReLU).  x (batch, d); W1 and W2t both (ffn, d),
+    W2t being fc2.weight transposed so that a neuron's fc2 column is a contiguous row; bias1 (ffn,),
+    bias2 (d,)."""
+    hidden = gather_gemv(x, W1, idx, bias1, activation=activation)
     return gather_transposed_gemv(hidden, W2t, idx, bias2)
 
 

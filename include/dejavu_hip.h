@@ -38,6 +38,9 @@ extern "C" {
 
 #define DV_ACT_ID 0
 #define DV_ACT_RELU 1
+#define DV_ACT_GELU 2         /* x * 0.5 * (1 + erf(x / sqrt(2)))               k_activations.py:136-139 */
+#define DV_ACT_GELU_APPROX 3  /* tanh form                                      k_activations.py:148-155 */
+#define DV_ACT_SQUARED_RELU 4 /* relu(x)^2                                      k_activations.py:92-100  */
 
 /* Library version (major*10000 + minor*100 + patch). */
 DV_API int dv_version(void);
@@ -150,7 +153,8 @@ DV_API int dv_dense_linear_f16(const void* x, int64_t ldx, const void* W, int64_
  *   y (B, N) fp16.  1 <= B <= 64 (vector ALUs up to 4; above, the weight tile is transposed in
  *   registers into 16x16x32 MFMA operands up to 32 rows, 32x32x16 operands up to 64).
  *   workspace: dv_gather_transposed_gemv_workspace_bytes(B, N, M) bytes, no
- *   initialisation needed; calls sharing it must not overlap.
+ *   initialisation needed; calls sharing it must not overlap.  y and workspace must be
+ *   16-byte aligned (vector stores), else DV_ERR_ALIGNMENT.
  */
 DV_API size_t dv_gather_transposed_gemv_workspace_bytes(int B, int N, int M);
 DV_API int dv_gather_transposed_gemv_f16(const void* x, const void* W, int64_t ldw, const void* bias,
@@ -167,10 +171,15 @@ DV_API int dv_gather_transposed_gemv_f16(const void* x, const void* W, int64_t l
  * Same kernels and same bits as dv_gather_transposed_gemv_f16.  Shapes whose partial sums
  * exceed the array (dv_gather_transposed_gemv_workspace_bytes(B, N, M) >
  * DV_STATIC_SCRATCH_BYTES: at the OPT shapes, batches above 32) return DV_ERR_WORKSPACE.
- * All calls on one GPU share the array: calls that overlap in time on different streams of one
- * GPU race.  The array needs no clearing between calls (every word is written before it is read).
+ * The array has DV_STATIC_SCRATCH_STREAMS slots of DV_STATIC_SCRATCH_BYTES; a stream keeps the slot
+ * it is given at its first call for the life of the process, so calls on different streams do not
+ * share partial sums (calls on one stream are ordered by the stream).  A call on one more stream
+ * than there are slots returns DV_ERR_UNSUPPORTED; two host threads that launch on the SAME stream
+ * without ordering their calls still race.  Nothing needs clearing between calls (every word is
+ * written before it is read).  y must be 16-byte aligned.
  */
 #define DV_STATIC_SCRATCH_BYTES (8u << 20)
+#define DV_STATIC_SCRATCH_STREAMS 2
 DV_API int dv_gather_transposed_gemv_static_f16(const void* x, const void* W, int64_t ldw,
                                                 const void* bias, const void* idx, int idx_bytes,
                                                 int B, int N, int Z, int M, void* y, void* stream);
@@ -216,7 +225,8 @@ DV_API int dv_qkv_proj_sparse_cache_f16(const void* x, const void* W, const void
  *   pass over one window token computes only the heads that miss it); y (B, 3, H, hd);
  *   k_cache (B, H, hd/8, S, 8), v_cache (B, H, S, hd): both or neither NULL; positions: device
  *   int32, (B,) when per_sample != 0, else (1,), or NULL (= 0); rows whose position is outside
- *   [0, S) are projected but not cached.  hd in {32, 64, 128}.
+ *   [0, S) are projected but not cached.  hd in {32, 64, 128}.  y, k_cache and v_cache must
+ *   be 8-byte aligned (also for dv_qkv_window_batch_f16), else DV_ERR_ALIGNMENT.
  *   workspace: dv_qkv_proj_batch_workspace_bytes(B, d, nnz, hd) bytes (0 up to 8 rows), 16-byte
  *   aligned, no initialisation needed: from 9 rows on the block of X is shared through LDS by a
  *   workgroup that owns 128 weight rows, and the columns are split over workgroups (fp32 partial
@@ -372,7 +382,8 @@ DV_API int dv_out_proj_sparse_f16(const void* x, const void* W, const void* bias
  * gather (the reference does the same for fc2 with fc2_weight_t,
  * Dejavu/src/ops/fused_dense_sparse_dejavu.py:912-913).  Deterministic.
  *   workspace: dv_out_proj_sparse_t_workspace_bytes(...) bytes, no
- *   initialisation needed (may be shared with dv_gather_transposed_gemv_f16).
+ *   initialisation needed (may be shared with dv_gather_transposed_gemv_f16).  y and workspace
+ *   must be 16-byte aligned.
  */
 DV_API size_t dv_out_proj_sparse_t_workspace_bytes(int B, int N, int nnz, int hd);
 DV_API int dv_out_proj_sparse_t_f16(const void* x, const void* Wt, int64_t ldw, const void* bias,

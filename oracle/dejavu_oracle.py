@@ -74,11 +74,25 @@ def relu(a: np.ndarray) -> np.ndarray:
 
 
 def _act(a: np.ndarray, activation: str) -> np.ndarray:
+    """The activations gather_gemv accepts (Dejavu/src/ops/triton/gather_gemv.py:213), as written in
+    Dejavu/src/ops/triton/k_activations.py: relu :73-80, squared_relu :92-100 (relu(x)^2), gelu
+    :136-139 (x * 0.5 * (1 + erf(x / sqrt 2))), gelu_approx :148-155 (0.5 x (1 + tanh(sqrt(2 / pi) *
+    x * (1 + 0.044715 x^2)))).  Evaluated in float64 on the fp32 sums."""
     if activation == "id":
         return a
     if activation == "relu":
         return relu(a)
-    raise ValueError(f"oracle implements 'id' and 'relu' only, got {activation!r}")
+    x = a.astype(np.float64)
+    if activation == "squared_relu":
+        r = np.where(x >= 0, x, 0.0)
+        return (r * r).astype(a.dtype)
+    if activation == "gelu":
+        from math import erf
+
+        return (x * 0.5 * (1.0 + np.vectorize(erf)(x * 0.7071067811865476))).astype(a.dtype)
+    if activation == "gelu_approx":
+        return (0.5 * x * (1.0 + np.tanh(0.7978845608028654 * x * (1.0 + 0.044715 * x * x)))).astype(a.dtype)
+    raise ValueError(f"unknown activation {activation!r}")
 
 
 # --------------------------------------------------------------------------

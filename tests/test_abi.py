@@ -60,6 +60,21 @@ def test_host_side_argument_checks_return_codes():
     assert L.dv_gather_transposed_gemv_f16(0x1000, 0x1000, 8, None, 0x1000, 8, 1, 8, 8, 4, 0x1000, None, 0, None) == -4
     assert L.dv_predictor_logits_f16(0x1000, 0x1000, 8, 0x1000, 8, 65, 8, 8, 8, 0x1000, 0x1000, None) == -2  # B > 64
     assert L.dv_qkv_proj_sparse_f16(0x1000, 0x1000, None, 0x1000, 0x1000, 17, 128, 4, 32, 2, 0x1000, None) == -2  # rows > 16
+    # outputs and scratch that the kernels write with vector stores must be aligned (checked before any launch)
+    A = 0x1000
+    assert L.dv_gather_transposed_gemv_f16(A, A, 8, None, A, 8, 1, 8, 8, 4, A + 2, A, 1 << 20, None) == -3  # y
+    assert L.dv_gather_transposed_gemv_f16(A, A, 8, None, A, 8, 1, 8, 8, 4, A, A + 4, 1 << 20, None) == -3  # workspace
+    assert L.dv_gather_transposed_gemv_static_f16(A, A, 8, None, A, 8, 1, 8, 8, 4, A + 2, None) in (-3, -2)  # y (or no GPU)
+    assert L.dv_out_proj_sparse_t_f16(A, A, 128, None, A, 1, 1, 1, 128, 128, A + 2, A, 1 << 20, None) == -3  # y
+    assert L.dv_out_proj_sparse_t_f16(A, A, 128, None, A, 1, 8, 1, 128, 128, A, A + 8, 1 << 20, None) == -3  # workspace
+    for fn in (L.dv_qkv_proj_batch_f16, L.dv_qkv_window_batch_f16):
+        if fn is L.dv_qkv_window_batch_f16:  # (.., nnz, tokens, nseq, d, H, hd, y, ...)
+            args_y = [A, 128, A, None, A, A, 1, 2, 2, 128, 1, 128, A + 2, A, A, None, 0, 0, 16, A, 1 << 20, None]
+            args_k = [A, 128, A, None, A, A, 1, 2, 2, 128, 1, 128, A, A + 4, A, None, 0, 0, 16, A, 1 << 20, None]
+        else:  # (.., live, live_stride, nnz, B, d, H, hd, y, ...)
+            args_y = [A, 128, A, None, A, A, 1, 1, 2, 128, 1, 128, A + 2, A, A, None, 0, 0, 16, A, 1 << 20, None]
+            args_k = [A, 128, A, None, A, A, 1, 1, 2, 128, 1, 128, A, A + 4, A, None, 0, 0, 16, A, 1 << 20, None]
+        assert fn(*args_y) == -3 and fn(*args_k) == -3
 
 
 def test_ops_refuse_cpu_tensors():

@@ -313,3 +313,27 @@ def test_predictor_first_product_long_rows_several_batch_rows_bit_exact(ops, B, 
     h_ref, l_ref = O.predictor_logits(x.numpy(), Wa.numpy(), Wb.numpy())
     assert np.array_equal(np16(hidden).view(np.uint16), h_ref.view(np.uint16)), "hidden vector differs"
     assert np.array_equal(np16(got).view(np.uint16), l_ref.view(np.uint16)), "logits differ"
+
+
+@pytest.mark.parametrize("act", ["gelu", "gelu_approx", "squared_relu", "relu", "id"])
+@pytest.mark.parametrize("B", [1, 4, 24])
+def test_gather_gemv_activations(ops, act, B):
+    """Every activation the reference's gathered fc1 accepts (gather_gemv.py:213), on the vector kernel
+    (one row), the per-tile matrix-core kernel (4 rows) and the X-shared split-K kernel (24 rows, where
+    the reduction launch applies bias and activation), against the oracle; and the sparse MLP with it."""
+    g = torch.Generator().manual_seed(40 + B)
+    N, Z, M = 1024, 4096, 1000
+    x = torch.randn(B, N, generator=g).half()
+    W = (torch.randn(Z, N, generator=g) * 0.04).half()
+    b = (torch.randn(Z, generator=g) * 0.2).half()
+    idx = torch.randperm(Z, generator=g)[:M].sort().values
+    print(f"case gather_gemv activation {act} B={B}", flush=True)
+    got = ops.gather_gemv(x.cuda(), W.cuda(), idx.cuda(), b.cuda(), activation=act)
+    torch.cuda.synchronize()
+    want = O.gather_gemv(x.numpy(), W.numpy(), idx.numpy(), b.numpy(), act)
+    assert_close(np16(got), want, f"fc1 with {act}")
+    W2t = (torch.randn(Z, N, generator=g) * 0.04).half()
+    out = ops.mlp_sparse(x.cuda(), W.cuda(), W2t.cuda(), idx.cuda(), b.cuda(), None, activation=act)
+    torch.cuda.synchronize()
+    want_out = O.gather_transposed_gemv(want, W2t.numpy(), idx.numpy())
+    assert_close(np16(out), want_out, f"sparse MLP with {act}")

@@ -689,3 +689,18 @@ def test_cpu_baseline_layer_step_follows_the_oracle():
         wout = np.ascontiguousarray(n["Wout_t"].reshape(H, hd, d).transpose(2, 0, 1))  # (d, H, hd)
         want_attn = O.out_proj_sparse(ctx, wout, want_heads, n["bout"])
         assert_close(attn.numpy(), want_attn, f"cpu baseline attention, batch {batch}")
+
+
+def test_oracle_activations_against_library_forms():
+    """The four activations of gather_gemv against torch's own (float64): relu, relu^2, erf GELU and
+    tanh GELU, plus their defining special values."""
+    x = np.linspace(-6, 6, 1201).astype(np.float32)
+    t = torch.from_numpy(x).double()
+    want = {"relu": torch.relu(t), "squared_relu": torch.relu(t) ** 2, "gelu": torch.nn.functional.gelu(t),
+            "gelu_approx": torch.nn.functional.gelu(t, approximate="tanh"), "id": t}
+    for name, w in want.items():
+        got = O._act(x, name).astype(np.float64)
+        assert np.allclose(got, w.numpy(), rtol=1e-6, atol=1e-7), name
+    assert O._act(np.float32([0.0]), "gelu")[0] == 0.0 and O._act(np.float32([-3.0]), "squared_relu")[0] == 0.0
+    with pytest.raises(ValueError):
+        O._act(x, "swish")

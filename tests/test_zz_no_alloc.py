@@ -70,3 +70,43 @@ def test_static_scratch_entry_point_rejects_shapes_beyond_the_array():
     assert lib.dv_gather_transposed_gemv_workspace_bytes(B, N, M) > 8 << 20
     rc = lib.dv_gather_transposed_gemv_static_f16(0x1000, 0x1000, N, None, 0x1000, 8, B, N, 49152, M, 0x1000, None)
     assert rc == -4
+
+
+def test_static_scratch_calls_on_two_streams_do_not_share_partial_sums():
+    """Two calls in flight at once on two streams (each stream has its own slot of the library's array):
+    both results equal the workspace entry point's; a third stream is refused with DV_ERR_UNSUPPORTED."""
+    from dejavu_amd._lib import lib
+
+    B, N, Z, M = 2, 4096, 8192, 2048
+    cases = []
+    for seed in (21, 22):
+        x, W, bias, idx = _inputs(B, N, Z, M, seed)
+        cases.append([t.cuda() for t in (x, W, bias, idx)])
+    nbytes = lib.dv_gather_transposed_gemv_workspace_bytes(B, N, M)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    want = []
+    for xd, Wd, bd, idd in cases:
+        y = torch.empty(B, N, dtype=torch.float16, device="cuda")
+        assert lib.dv_gather_transposed_gemv_f16(xd.data_ptr(), Wd.data_ptr(), N, bd.data_ptr(), idd.data_ptr(), 8, B, N,
+                                                 Z, M, y.data_ptr(), ws.data_ptr(), ws.numel(),
+                                                 torch.cuda.current_stream().cuda_stream) == 0
+        want.append(y)
+    torch.cuda.synchronize()
+    # the stream the other tests of this file used holds one slot; one more stream takes the second
+    streams = [torch.cuda.current_stream(), torch.cuda.Stream()]
+    got = [torch.full((B, N), float("nan"), dtype=torch.float16, device="cuda") for _ in cases]
+    print("case static scratch on two streams", flush=True)
+    for rep in range(8):  # several rounds in flight on both streams at once
+        for (xd, Wd, bd, idd), y, st in zip(cases, got, streams):
+            rc = lib.dv_gather_transposed_gemv_static_f16(xd.data_ptr(), Wd.data_ptr(), N, bd.data_ptr(), idd.data_ptr(),
+                                                          8, B, N, Z, M, y.data_ptr(), st.cuda_stream)
+            assert rc == 0, rc
+    torch.cuda.synchronize()
+    for y, w in zip(got, want):
+        assert torch.equal(y, w)
+    third = torch.cuda.Stream()
+    xd, Wd, bd, idd = cases[0]
+    rc = lib.dv_gather_transposed_gemv_static_f16(xd.data_ptr(), Wd.data_ptr(), N, bd.data_ptr(), idd.data_ptr(), 8, B, N,
+                                                  Z, M, got[0].data_ptr(), third.cuda_stream)
+    assert rc == -2, "a third stream has no slot"
+    torch.cuda.synchronize()
