@@ -413,7 +413,7 @@ def decode_bench(args):
     layers, vocab, prompt_len, new_tokens = args.decode_layers, 50272, 128, args.steps
     torch.cuda.set_device(0)
     conf = SparseGPTConfig(hidden_size=cfg["d"], num_attention_heads=cfg["H"], num_hidden_layers=layers,
-                           vocab_size=vocab, n_inner=cfg["ffn"], max_position_embeddings=2048, mlp_K=cfg["K"],
+                           vocab_size=vocab, n_inner=cfg["ffn"], max_position_embeddings=2304, mlp_K=cfg["K"],
                            mlp_sp_dim=cfg["r"], att_K=[cfg["Hk"], cfg["Hk"]], att_sp_dim=cfg["r"],
                            pad_vocab_size_multiple=8)
     model = GPTLMHeadModel(conf, device="cuda", dtype=torch.float16).eval()
@@ -442,6 +442,20 @@ def decode_bench(args):
         t_total, seq_cg = min((run(True) for _ in range(3)), key=lambda r: r[0])
         t_prompt, _ = min((run(True, prompt_len + 1) for _ in range(3)), key=lambda r: r[0])
         t_eager, seq_eager = run(False)
+        # longer prompts (prompt + one token): their dense products are compute-bound
+        prompt_ms_by_length = {}
+        for plen in (512, 2048):
+            pids = torch.randint(0, vocab, (1, plen), generator=gen, device="cuda")
+
+            def run_prompt():
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                model.generate(pids, max_length=plen + 1, cg=False, vocab_size=vocab)
+                torch.cuda.synchronize()
+                return time.perf_counter() - t0
+
+            run_prompt()
+            prompt_ms_by_length[str(plen)] = round(min(run_prompt() for _ in range(3)) * 1e3, 2)
         # roofline of the kernel that carries the largest share of a token's bytes (the QKV projection of
         # a sparse block, one launch per block and token), alone, graph-replayed between two HIP events
         from dejavu_amd import ops
@@ -472,7 +486,8 @@ def decode_bench(args):
         "config": {"workload": "opt-13b-shaped greedy decode", "layers": layers, "d": d, "ffn": ffn, "heads": H,
                    "K": K, "active_heads": Hk, "vocab": vocab, "prompt": prompt_len, "new_tokens": new_tokens,
                    "hip_graphs": "one graph per 16-token back-fill window"},
-        "prompt_ms": round(t_prompt * 1e3, 2), "total_ms": round(t_total * 1e3, 2),
+        "prompt_ms": round(t_prompt * 1e3, 2), "prompt_ms_by_length": prompt_ms_by_length,
+        "total_ms": round(t_total * 1e3, 2),
         "eager_total_ms": round(t_eager * 1e3, 2), "graph_equals_eager": same,
         "us_per_layer": round(decode_s / steps / layers * 1e6, 2),
         "weight_MB_per_token": round(token_bytes / 1e6, 1),
@@ -689,6 +704,7 @@ def other_workloads():
     else:
         out["decode"] = {"metric": d["metric"], "tokens_per_s": d["value"], "ms_per_token": d["ms_per_step"],
                          "us_per_layer": d["us_per_layer"], "prompt_ms": d["prompt_ms"],
+                         "prompt_ms_by_length": d.get("prompt_ms_by_length"),
                          "frac_of_hbm_peak": d["frac_of_hbm_peak"], "graph_equals_eager": d["graph_equals_eager"],
                          "new_tokens": d["steps"], "wall_s": round(secs, 1)}
     return out

@@ -114,8 +114,18 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_tiled_mfma_kernel(
   half_t* ws = xs + (size_t)2 * XROWS * LD + (size_t)wave * WROWS * LD;  // [WROWS][LD], wavefront-private
   const int l16 = lane & 15, kg = lane >> 4;
 
-  const int b0 = blockIdx.x * XROWS;
-  const int m0 = (blockIdx.y * WAVES + wave) * WROWS;  // first output row of this wavefront
+  // Several blocks of X against the same weight rows: the workgroups that share a weight tile are
+  // given consecutive slots of ONE XCD (workgroup ids go round the 8 XCDs, each with its own L2), so
+  // that the tile leaves HBM once and the other blocks find it in that L2.
+  int bx = blockIdx.x, by = blockIdx.y;
+  if (gridDim.x > 1 && gridDim.y % 8 == 0) {
+    const int lin = bx + (int)gridDim.x * by;
+    const int xcd = lin & 7, q = lin >> 3;
+    by = (q / (int)gridDim.x) * 8 + xcd;
+    bx = q % (int)gridDim.x;
+  }
+  const int b0 = bx * XROWS;
+  const int m0 = (by * WAVES + wave) * WROWS;  // first output row of this wavefront
   const int nchunks = (N + KC - 1) / KC;
   const int c_begin = SPLIT ? (int)blockIdx.z * chunks_per_split : 0;
   const int c_end = SPLIT ? (c_begin + chunks_per_split < nchunks ? c_begin + chunks_per_split : nchunks) : nchunks;

@@ -43,6 +43,11 @@ SIDE_STREAM_MIN_BATCH = 2
 # Prompt phase on this package's own kernels (dense products: dv_dense_linear_f16; causal attention
 # + cache fill: dv_prefill_attention_f16).  False: PyTorch's library GEMM and attention.
 USE_HIP_PROMPT = True
+# The dense products of a prompt are plain GEMMs.  Up to this many rows of X the package's X-shared
+# kernel is at least as fast as the library (it is bound by the weight stream: 85 against 96 us for
+# 128 rows x 12288 x 12288); beyond it the product is compute-bound and the library's GEMM is taken
+# (164 against 250 us at 512 rows, 515 against 763 us at 2048 rows on the same operands).
+HIP_PROMPT_MAX_ROWS = 192
 
 _side_streams: dict = {}
 _side_pending = False  # work was enqueued on the side stream since the last join_side_stream()
@@ -221,13 +226,13 @@ class ParallelFusedMLPDejavu(nn.Module):
 
 def decode_linear(linear: nn.Linear, x: torch.Tensor, activation: str = "id") -> torch.Tensor:
     """``activation(linear(x))``.  The rows of a decode step (x: (B, 1, d) with B <= 64, fp16, on the GPU)
-    always go to this package's row kernels (vector ALUs for one or two rows, matrix cores above).  Many
-    rows (the prompt phase) go to the X-shared matrix-core kernel when ``USE_HIP_PROMPT`` is set, else to
-    the library GEMM."""
+    always go to this package's row kernels (vector ALUs for one or two rows, matrix cores above).  The
+    rows of a prompt go to the X-shared matrix-core kernel while the product is bound by the weight
+    stream (``USE_HIP_PROMPT``, up to ``HIP_PROMPT_MAX_ROWS`` rows), else to the library GEMM."""
     on_hip = x.is_cuda and x.dtype == torch.float16 and linear.weight.dtype == torch.float16 and x.shape[-1] % 8 == 0
     if on_hip and x.dim() == 3 and x.shape[1] == 1 and x.shape[0] <= 64:
         return ops.dense_decode_linear(x, linear.weight, linear.bias, activation)
-    if on_hip and USE_HIP_PROMPT:
+    if on_hip and USE_HIP_PROMPT and x.numel() // x.shape[-1] <= HIP_PROMPT_MAX_ROWS:
         return ops.dense_linear(x, linear.weight, linear.bias, activation)
     y = linear(x)
     if activation == "relu":
