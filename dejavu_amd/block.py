@@ -52,7 +52,7 @@ class BlockMlpAttSparse(nn.Module):
             self.mixer.mlp_k = self.mlp.sp.K
         if hasattr(self.mixer, "sp"):
             self.mixer.att_k = self.mixer.sp.K
-        # ordinary head-sparse decode steps run as one fused call (eight launches); set to
+        # ordinary head-sparse decode steps run as one fused call (seven launches); set to
         # False to always go through the modules' own forwards
         self.use_fused_layer = True
 

@@ -108,7 +108,7 @@ def test_sparse_block_decode_step_matches_oracle(d, ffn, H, r, K, Hk, S):
                                             # OPT-13B- and OPT-66B-shaped layers: other launch plans
                                             (5120, 40, 20480, 1000, 2048, 16), (9216, 72, 36864, 1000, 4096, 24)])
 def test_fused_layer_equals_module_by_module_path(d, H, ffn, r, K, Hk):
-    """The eight-launch fused block step and the module-by-module path run the same kernel
+    """The fused block step and the module-by-module path run the same kernel
     bodies: outputs, predictions, caches and window state must agree bit for bit over a
     whole back-fill window and into the next one (the flush step is a fused step too, with every
     head active).  Every scratch
