@@ -1276,17 +1276,22 @@ int launch_attn_partials(const void* q, int64_t ldq, const void* k_cache, const 
   if (hd == 128)
     hipLaunchKernelGGL((decode_attn_kernel<128, kAttnWaves>), grid, dim3(kAttnWaves * 64), 0, s, qq,
                        ldq, kc, vc, hi, ln, n_len, H, S, scale, nsplit, part);
-  else
+  else if (hd == 64)
     hipLaunchKernelGGL((decode_attn_kernel<64, kAttnWaves>), grid, dim3(kAttnWaves * 64), 0, s, qq,
+                       ldq, kc, vc, hi, ln, n_len, H, S, scale, nsplit, part);
+  else
+    hipLaunchKernelGGL((decode_attn_kernel<32, kAttnWaves>), grid, dim3(kAttnWaves * 64), 0, s, qq,
                        ldq, kc, vc, hi, ln, n_len, H, S, scale, nsplit, part);
   return launch_status();
 }
 
+// hd32: the caller also has the 32-wide head kernels (the attention alone has; the entry points that
+// go on into out_proj do not)
 int check_attn_args(const void* q, int64_t ldq, const void* k_cache, const void* v_cache, int nheads,
-                    int n_len, int B, int H, int hd, int S) {
+                    int n_len, int B, int H, int hd, int S, bool hd32 = false) {
   if (!q || !k_cache || !v_cache || nheads < 0 || B < 1 || H <= 0 || S <= 0 || n_len < 1 || n_len > S)
     return DV_ERR_INVALID_ARG;
-  if (hd != 64 && hd != 128) return DV_ERR_UNSUPPORTED;
+  if (hd != 64 && hd != 128 && !(hd32 && hd == 32)) return DV_ERR_UNSUPPORTED;
   if (ldq % 8 || !aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache)) return DV_ERR_ALIGNMENT;
   return DV_OK;
 }
@@ -1296,7 +1301,7 @@ int dv_decode_attention_f16(const void* q, int64_t ldq, const void* k_cache, con
                             const void* head_idx, int nheads, const void* lengths, int n_len,
                             int B, int H, int hd, int S, float scale, void* out, int64_t ldo,
                             void* workspace, size_t workspace_bytes, void* stream) {
-  int rc = check_attn_args(q, ldq, k_cache, v_cache, nheads, n_len, B, H, hd, S);
+  int rc = check_attn_args(q, ldq, k_cache, v_cache, nheads, n_len, B, H, hd, S, true);
   if (rc != DV_OK) return rc;
   if (!out) return DV_ERR_INVALID_ARG;
   const int heads = head_idx ? nheads : H;
@@ -1314,8 +1319,11 @@ int dv_decode_attention_f16(const void* q, int64_t ldq, const void* k_cache, con
   if (hd == 128)
     hipLaunchKernelGGL((decode_attn_combine_kernel<128>), dim3(heads, B), dim3(128), 0, s, part,
                        hi, H, nsplit, oo, ldo);
-  else
+  else if (hd == 64)
     hipLaunchKernelGGL((decode_attn_combine_kernel<64>), dim3(heads, B), dim3(64), 0, s, part, hi,
+                       H, nsplit, oo, ldo);
+  else
+    hipLaunchKernelGGL((decode_attn_combine_kernel<32>), dim3(heads, B), dim3(32), 0, s, part, hi,
                        H, nsplit, oo, ldo);
   return launch_status();
 }

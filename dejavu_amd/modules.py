@@ -48,6 +48,11 @@ USE_HIP_PROMPT = True
 # 128 rows x 12288 x 12288); beyond it the product is compute-bound and the library's GEMM is taken
 # (164 against 250 us at 512 rows, 515 against 763 us at 2048 rows on the same operands).
 HIP_PROMPT_MAX_ROWS = 192
+# The package's causal-attention kernel (one wavefront per 16 queries, K / V straight from memory, cache fill
+# in the same launch) wins for short prompts (40 heads x 128: 29 us at 128 tokens against 36 us for the
+# library's attention plus the permuted cache copies) and loses from about 200 tokens on (512 tokens: 167
+# against 53 us; 2048: 1461 against 216 us): longer prompts take the library's attention and the copies.
+HIP_PROMPT_ATTN_MAX_TOKENS = 192
 
 _side_streams: dict = {}
 _side_pending = False  # work was enqueued on the side stream since the last join_side_stream()
@@ -285,7 +290,7 @@ class _MHABase(nn.Module):
     def _init_common(self, embed_dim, num_heads, process_group, bias, softmax_scale, causal, layer_idx,
                      rotary_emb_dim, device, dtype):
         _world_size(process_group)
-        assert rotary_emb_dim == 0, "OPT uses learned positions; rotary embedding is not built"
+        ops.require_no_rotary(rotary_emb_dim)
         self.embed_dim = embed_dim
         self.causal = causal
         self.layer_idx = layer_idx
@@ -315,7 +320,7 @@ class _MHABase(nn.Module):
         if inference_params is None or inference_params.sequence_len_offset == 0:
             causal = self.causal if inference_params is None else True
             if USE_HIP_PROMPT and qkv.is_cuda and qkv.dtype == torch.float16 and qkv.shape[-1] in (64, 128) \
-                    and (causal or s == 1):
+                    and (causal or s == 1) and s <= HIP_PROMPT_ATTN_MAX_TOKENS:
                 # causal attention and the cache fill in one launch (no permuted copy of K / V)
                 kc = vc = None
                 if inference_params is not None:

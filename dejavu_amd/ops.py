@@ -610,6 +610,15 @@ def kv_cache_copy_sparse(k, v, k_cache, v_cache, head_idx, seqlen_idx, padding=N
     _cache_copy(k, v, k_cache, v_cache, head_idx, seqlen_idx, padding)
 
 
+def require_no_rotary(rotary_emb_dim: int) -> None:
+    """The one place where a rotary embedding is turned down: OPT uses learned positions, and the
+    rotation that ``ft_attention.single_query_attention`` applies to q and k for ``rotary_emb_dim > 0``
+    (mha_dejavu.py:1439-1456) is not built here."""
+    if rotary_emb_dim != 0:
+        raise NotImplementedError(f"rotary_emb_dim = {rotary_emb_dim}: rotary position embedding is not built "
+                                  "(OPT uses learned positions)")
+
+
 def single_query_attention(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.Tensor],
                            k_cache: torch.Tensor, v_cache: torch.Tensor,
                            lengths_per_sample: Optional[torch.Tensor], timestep: int, rotary_emb_dim: int = 0,
@@ -624,10 +633,10 @@ def single_query_attention(q: torch.Tensor, k: Optional[torch.Tensor], v: Option
     and only their rows of the (B, H, hd) result are written.
     """
     _require_device(q, k, v, k_cache, v_cache, lengths_per_sample, head_idx)
-    assert rotary_emb_dim == 0, "OPT has no rotary embedding"
+    require_no_rotary(rotary_emb_dim)
     B, H, hd = q.shape
     S = v_cache.shape[2]
-    assert hd in [64, 128], "the decode attention kernels are built for head_dim 64 and 128"
+    assert hd in [32, 64, 128], "the decode attention kernels are built for head_dim 32, 64 and 128"
     assert q.dtype == torch.float16 and k_cache.dtype == torch.float16 and v_cache.dtype == torch.float16
     assert v_cache.shape == (B, H, S, hd) and k_cache.shape == (B, H, hd // 8, S, 8)
     assert k_cache.is_contiguous() and v_cache.is_contiguous()

@@ -325,7 +325,7 @@ DV_API int dv_kv_append_f16(const void* k, const void* v, int64_t ld_src, void* 
  * `out` for unlisted heads are not written.  Replaces the attention part of
  * ft_attention.single_query_attention (same call sites as dv_kv_append_f16).
  *   q (B, H, hd) with batch stride ldq; out (B, H, hd) with batch stride ldo;
- *   hd in {64, 128}; workspace: dv_decode_attention_workspace_bytes(...) bytes.
+ *   hd in {32, 64, 128}; workspace: dv_decode_attention_workspace_bytes(...) bytes.
  */
 DV_API size_t dv_decode_attention_workspace_bytes(int B, int nheads, int n_len, int hd);
 DV_API int dv_decode_attention_f16(const void* q, int64_t ldq, const void* k_cache,

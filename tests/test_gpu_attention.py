@@ -182,7 +182,7 @@ def test_cache_copy_sparse_bit_exact(ops, hd):
 
 # ------------------------------------------------------ decode attention
 @pytest.mark.parametrize("B,H,hd,S,t,nsel", [(1, 12, 128, 256, 200, 4), (2, 8, 64, 100, 99, 3), (1, 96, 128, 2048, 2047, 32),
-                                             (3, 4, 128, 70, 0, 4), (1, 6, 128, 130, 64, 2)])
+                                             (3, 4, 128, 70, 0, 4), (1, 6, 128, 130, 64, 2), (2, 16, 32, 300, 270, 5)])
 def test_single_query_attention(ops, B, H, hd, S, t, nsel):
     g = torch.Generator().manual_seed(4)
     q, k, v = (randh(g, B, H, hd) for _ in range(3))

@@ -87,31 +87,36 @@ def test_prefill_attention_matches_oracle(B, T, H, hd):
         assert np.array_equal(k_cache[b].cpu().numpy(), kn) and np.array_equal(v_cache[b].cpu().numpy(), vn)
 
 
-def test_prompt_runs_on_the_hip_kernels_and_matches_the_library_path():
+@pytest.mark.parametrize("T", [45, 230])
+def test_prompt_runs_on_the_hip_kernels_and_matches_the_library_path(T):
     """The prompt phase of a small model through dv_dense_linear_f16 / dv_prefill_attention_f16
     (USE_HIP_PROMPT) against PyTorch's library GEMM and attention on the same weights, and against
-    the oracle's model_prompt; the caches the two paths leave behind agree within fp16 rounding."""
+    the oracle's model_prompt; the caches the two paths leave behind agree within fp16 rounding.
+    The 230-token prompt is past both switch-over lengths (HIP_PROMPT_MAX_ROWS,
+    HIP_PROMPT_ATTN_MAX_TOKENS): its products and attention are the library's, the cache layout and
+    everything after the prompt are the package's."""
     import dejavu_amd.modules as M
     from dejavu_amd.gpt import GPTLMHeadModel, SparseGPTConfig
     from dejavu_amd.modules import InferenceParams
     from oracle import dejavu_oracle as O
     from tests.model_utils import load_model_params, make_model_params
 
-    L, d, H, ffn, r, V, P = 2, 256, 4, 1024, 32, 512, 96
+    L, d, H, ffn, r, V, P = 2, 256, 4, 1024, 32, 512, 256
     params = make_model_params(L, d, H, ffn, r, V, P, 256, [2, 2], seed=5)
     cfg = SparseGPTConfig(hidden_size=d, num_attention_heads=H, num_hidden_layers=L, vocab_size=V, n_inner=ffn,
                           max_position_embeddings=P, mlp_K=256, mlp_sp_dim=r, att_K=[2, 2], att_sp_dim=r)
     model = GPTLMHeadModel(cfg, device="cuda", dtype=torch.float16).eval()
     load_model_params(model, params)
-    prompt = [int(v) for v in torch.randint(0, V, (45,), generator=torch.Generator().manual_seed(1))]
+    assert (T <= M.HIP_PROMPT_ATTN_MAX_TOKENS) == (T == 45)
+    prompt = [int(v) for v in torch.randint(0, V, (T,), generator=torch.Generator().manual_seed(1))]
     ids = torch.tensor([prompt], device="cuda")
     outs, caches = [], []
     assert M.USE_HIP_PROMPT
     try:
         for flag in (True, False):
             M.USE_HIP_PROMPT = flag
-            ip = InferenceParams(max_sequence_len=64, max_batch_size=1)
-            print(f"case prompt phase, hip kernels={flag}", flush=True)
+            ip = InferenceParams(max_sequence_len=256, max_batch_size=1)
+            print(f"case prompt phase of {T} tokens, hip kernels={flag}", flush=True)
             with torch.no_grad():
                 logits = model(ids, inference_params=ip, last_token_only=True).logits[0, -1]
             torch.cuda.synchronize()
@@ -120,7 +125,7 @@ def test_prompt_runs_on_the_hip_kernels_and_matches_the_library_path():
                            (ip.key_value_memory_dict[l] for l in range(L))])
     finally:
         M.USE_HIP_PROMPT = True
-    state = O.new_decode_state(params, 64)
+    state = O.new_decode_state(params, 256)
     want = O.model_prompt(params, state, prompt).astype(np.float32)
     assert_close(outs[0], want, "prompt logits, hip kernels vs oracle", rel_tol=1.3e-3)
     assert_close(outs[1], want, "prompt logits, library path vs oracle", rel_tol=1.3e-3)
