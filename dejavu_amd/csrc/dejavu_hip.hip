@@ -13,6 +13,7 @@
 #include "gemm_cols16.hpp"
 #include "gemm_mfma.hpp"
 #include "gemm_tiled.hpp"
+#include "gemm_big.hpp"
 #include "gemv_cols.hpp"
 #include "gemv_rows.hpp"
 #include "layer_fused.hpp"
@@ -462,7 +463,9 @@ TiledPlan plan_tiled(int B, int N, int M) {
   return p;
 }
 
+bool big_applies(int B, int N);
 size_t tiled_workspace_bytes(int B, int N, int M) {
+  if (big_applies(B, N)) return 0;
   const TiledPlan p = plan_tiled(B, N, M);
   return p.nsplit > 1 ? (size_t)p.nsplit * B * M * sizeof(float) : 0;
 }
@@ -481,10 +484,58 @@ int launch_tiled(const TiledPlan& p, const half_t* X, int64_t ldx, const half_t*
   return DV_OK;
 }
 
+// Many rows of X (two or more 128-row blocks): the product is bound by the matrix cores and by what
+// the L2 delivers, and gemm_big_mfma_kernel (weights straight into MFMA operands, 64 * WT weight rows
+// per workgroup) is the faster kernel -- measured at 12288 x 12288 against gemm_tiled_mfma_kernel:
+// 256 rows 172 against 259 us, 512 rows 225 against 278 us, 2048 rows 793 against 797 us.  Same bits.
+// WT: the tile height that fills the device best; on a tie the larger (fewer L2 reads per flop).
+bool big_applies(int B, int N) { return B >= 200 && N % (kBgKC * kBgRing) == 0; }
+int big_pick_wt(int B, int M, int max_wt) {
+  const int cus = compute_units();
+  const int xblocks = (B + kBgXRows - 1) / kBgXRows;
+  int best_wt = 2;
+  double best_fill = -1.0;
+  for (int wt = 2; wt <= max_wt; ++wt) {
+    const int64_t wgs = (int64_t)xblocks * ((M + 64 * wt - 1) / (64 * wt));
+    const double fill = (double)wgs / (double)((wgs + cus - 1) / cus * cus);
+    if (fill >= best_fill - 1e-9) {
+      best_fill = fill;
+      best_wt = wt;
+    }
+  }
+  return best_wt;
+}
+template <int WT, bool QKV>
+int launch_big(const half_t* X, int64_t ldx, const half_t* W, int64_t ldw, const half_t* bias, const void* idx,
+               int idx_bytes, int B, int N, int Z, int M, half_t* Y, int64_t ldy, int act, const QkvScatter& qs,
+               hipStream_t s) {
+  auto kern = gemm_big_mfma_kernel<WT, QKV>;
+  static LdsGrant grant;
+  if (int rc = grant.ensure(reinterpret_cast<const void*>(kern), big_lds_bytes()); rc != DV_OK) return rc;
+  const dim3 grid((B + kBgXRows - 1) / kBgXRows, (M + 64 * WT - 1) / (64 * WT));
+  hipLaunchKernelGGL(kern, grid, dim3(256), big_lds_bytes(), s, X, ldx, W, ldw, bias, idx, idx_bytes, B, N, Z, M, Y,
+                     ldy, act, qs);
+  return launch_status();
+}
+template <bool QKV>
+int gemm_big(const half_t* X, int64_t ldx, const half_t* W, int64_t ldw, const half_t* bias, const void* idx,
+             int idx_bytes, int B, int N, int Z, int M, half_t* Y, int64_t ldy, int act, const QkvScatter& qs,
+             hipStream_t s) {
+  // (the scatter epilogue of the QKV form leaves no registers for the tallest tile)
+  constexpr int kMaxWt = QKV ? 3 : 4;
+  switch (big_pick_wt(B, M, kMaxWt)) {
+    case 2: return launch_big<2, QKV>(X, ldx, W, ldw, bias, idx, idx_bytes, B, N, Z, M, Y, ldy, act, qs, s);
+    case 3: return launch_big<3, QKV>(X, ldx, W, ldw, bias, idx, idx_bytes, B, N, Z, M, Y, ldy, act, qs, s);
+    default: return launch_big<(QKV ? 3 : 4), QKV>(X, ldx, W, ldw, bias, idx, idx_bytes, B, N, Z, M, Y, ldy, act, qs, s);
+  }
+}
+
 // QKV of the selected heads for B rows (see QkvScatter): M = 3 * Hk * hd output rows
 int gemm_tiled_qkv(const half_t* X, int64_t ldx, const half_t* W, const half_t* bias, int B, int d, half_t* Y,
                    const QkvScatter& qs, void* workspace, size_t workspace_bytes, hipStream_t s) {
   const int M = 3 * qs.Hk * qs.hd, Z = 3 * qs.H * qs.hd;
+  if (big_applies(B, d))
+    return gemm_big<true>(X, ldx, W, (int64_t)d, bias, nullptr, 4, B, d, Z, M, Y, (int64_t)Z, 0, qs, s);
   const TiledPlan p = plan_tiled(B, d, M);
   float* partial = nullptr;
   if (p.nsplit > 1) {
@@ -526,6 +577,8 @@ int gemm_tiled_qkv(const half_t* X, int64_t ldx, const half_t* W, const half_t* 
 int gemm_tiled(const half_t* X, int64_t ldx, const half_t* W, int64_t ldw, const half_t* bias, const void* idx,
                int idx_bytes, int B, int N, int Z, int M, int act, half_t* Y, int64_t ldy, void* workspace,
                size_t workspace_bytes, hipStream_t s) {
+  if (big_applies(B, N))
+    return gemm_big<false>(X, ldx, W, ldw, bias, idx, idx_bytes, B, N, Z, M, Y, ldy, act, QkvScatter{}, s);
   const TiledPlan p = plan_tiled(B, N, M);
   float* partial = nullptr;
   if (p.nsplit > 1) {

@@ -93,6 +93,47 @@ __device__ __forceinline__ void qkv_store4(const QkvScatter& q, half_t* __restri
   *reinterpret_cast<half4_t*>(p) = o;
 }
 
+// qkv_store4 in two halves, for kernels whose lanes keep many (X row, output row) pairs: what depends
+// on the X row alone and what depends on the output rows alone is worked out once each.
+struct QkvXRow {  // X row r
+  int s, b, dst;  // window token, sequence, cache position (-1: not cached)
+};
+struct QkvOutRows {  // output rows m .. m + 3, weight rows rid .. rid + 3 (one head)
+  int i, t, rid;
+  int64_t head_off;  // ((h) * (hd / 8) + j / 8) * S * 8 + (j & 7) for K, h * S * hd + j for V, without the sequence
+};
+__device__ __forceinline__ QkvXRow qkv_x_row(const QkvScatter& q, int r) {
+  QkvXRow x;
+  x.s = q.tokens > 1 ? r / q.nseq : 0;
+  x.b = r - x.s * q.nseq;
+  const int dst = (q.positions ? q.positions[q.per_sample ? x.b : 0] : 0) + q.pos_add + x.s;
+  x.dst = (dst >= 0 && dst < q.S) ? dst : -1;
+  return x;
+}
+__device__ __forceinline__ QkvOutRows qkv_out_rows(const QkvScatter& q, int m, int rid) {
+  QkvOutRows o;
+  o.i = (m % (q.Hk * q.hd)) / q.hd;
+  o.rid = rid;
+  o.t = rid >= 0 ? rid / (q.H * q.hd) : 0;
+  const int rem = rid - o.t * q.H * q.hd;
+  const int h = rem / q.hd, j = rem - h * q.hd;
+  o.head_off = o.t == 1 ? ((int64_t)h * (q.hd / 8) + j / 8) * q.S * 8 + (j & 7) : (int64_t)h * q.S * q.hd + j;
+  return o;
+}
+__device__ __forceinline__ void qkv_store4(const QkvScatter& q, half_t* __restrict__ Y, const QkvXRow& x,
+                                           const QkvOutRows& o, const float (&val)[4]) {
+  if (o.rid < 0) return;
+  if (q.live != nullptr && q.tokens > 1 &&
+      q.live[(int64_t)o.i * q.live_stride + (int64_t)x.s * q.live_tstride] < 0)
+    return;
+  const half4_t v = {(half_t)val[0], (half_t)val[1], (half_t)val[2], (half_t)val[3]};
+  if (x.s == q.y_token) *reinterpret_cast<half4_t*>(Y + (int64_t)x.b * 3 * q.H * q.hd + o.rid) = v;
+  if (q.k_cache == nullptr || o.t == 0 || x.dst < 0) return;
+  half_t* p = o.t == 1 ? q.k_cache + (int64_t)x.b * q.H * q.hd * q.S + o.head_off + (int64_t)x.dst * 8
+                       : q.v_cache + (int64_t)x.b * q.H * q.S * q.hd + o.head_off + (int64_t)x.dst * q.hd;
+  *reinterpret_cast<half4_t*>(p) = v;
+}
+
 template <int BT, int WT, int KC, bool QKV = false, int WAVES = kTgWaves>
 __global__ __launch_bounds__(WAVES * 64) void gemm_tiled_mfma_kernel(
     const half_t* __restrict__ X, int64_t ldx, const half_t* __restrict__ W, int64_t ldw,

@@ -100,12 +100,14 @@ def test_qkv_proj_batch_matches_oracle(B, H, hd, d, S):
 
 @pytest.mark.parametrize("tokens,nseq,H,hd,d,S,per_sample", [
     (2, 3, 4, 64, 512, 40, True), (5, 8, 6, 128, 776, 64, False), (16, 8, 4, 64, 512, 48, True),
-    (9, 17, 3, 32, 264, 40, True), (16, 32, 3, 128, 520, 40, False)])
+    (9, 17, 3, 32, 264, 40, True), (16, 32, 3, 128, 520, 40, False), (16, 32, 3, 128, 512, 40, False),
+    (13, 17, 5, 64, 768, 40, True)])
 def test_qkv_window_batch_matches_oracle(tokens, nseq, H, hd, d, S, per_sample):
     """All tokens of a shared back-fill window in one pass: (head, token) pairs the tracker marks are
     projected for every sequence and cached at position + token; the newest token's rows also go to
     `out`; everything else stays untouched.  Row counts cover one to four blocks of 128 rows, ragged
-    last column chunks and every batch-tile count of the kernel (6 .. 512 rows)."""
+    last column chunks and every batch-tile count of the kernel (6 .. 512 rows); the last two cases (200 rows
+    and more, d a multiple of 256) run on the kernel for compute-bound products."""
     from dejavu_amd import ops
     from dejavu_amd.workloads import pack_k_cache
 

@@ -19,7 +19,8 @@ def assert_close(got, want, what="", max_abs_tol=2e-2, rel_tol=1e-3):
 
 @pytest.mark.parametrize("rows,N,M,act", [(1, 768, 2304, "id"), (7, 520, 1001, "relu"), (16, 1024, 4096, "id"),
                                           (33, 776, 300, "relu"), (64, 2048, 640, "id"), (128, 1024, 4096, "relu"),
-                                          (130, 520, 2050, "id"), (300, 768, 3072, "relu"), (128, 5120, 15360, "id")])
+                                          (130, 520, 2050, "id"), (300, 768, 3072, "relu"), (128, 5120, 15360, "id"),
+                                          (520, 1024, 1000, "id"), (200, 256, 130, "relu"), (1030, 512, 2304, "id")])
 def test_dense_linear_matches_fp32_reference(rows, N, M, act):
     """Against the fp32-accumulated product of the same fp16 operands (max-abs 2e-2, relative L2 1e-3).
     Ragged cases: a last column chunk that is not full, output widths that are not multiples of 4 or
