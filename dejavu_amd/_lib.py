@@ -108,6 +108,9 @@ SIGNATURES = {
          _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr]),
     "dv_add_layer_norm_f16": (
         _c_int, [_c_ptr, _c_ptr, _c_ptr, _c_ptr, ctypes.c_float, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr]),
+    "dv_add_layer_norm_window_f16": (
+        _c_int, [_c_ptr, _c_ptr, _c_ptr, _c_ptr, ctypes.c_float, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                 _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr]),
     "dv_window_step_f16": (
         _c_int, [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr]),
     "dv_kv_append_f16": (

@@ -18,7 +18,22 @@ import torch.nn as nn
 from torch import Tensor
 
 from . import fused_layer, ops
+from . import modules as dv_modules
 from .modules import ParallelFusedMLPDejavu, ParallelMHADejavu, ParallelMHASparseAttMlp
+
+
+# Batched sparse decode: LayerNorm 1, the window buffer's row and the tracker step in one launch
+# (False: add_layer_norm, then dv_window_step_f16 inside the mixer).
+FOLD_WINDOW_STEP = True
+
+
+# Side-stream work (predictors, top-ks; batches of sequences) is waited for where its results are
+# needed instead of at the end of the module that started it: the attention module's selections before
+# fc1 (LayerNorm 2 runs without them), the MLP predictor's logits never on the main stream (the next
+# block's top-k is enqueued on the side stream behind them).  The block's outputs next_mlp_sp_logit /
+# next_att_idx are then good for the next block, or for anybody after modules.join_side_stream().
+# False: every module waits for its side work before it returns.
+LAZY_SIDE_JOIN = True
 
 
 def _add_norm(norm: nn.LayerNorm, hidden_states: Tensor, residual: Optional[Tensor]):
@@ -63,17 +78,37 @@ class BlockMlpAttSparse(nn.Module):
         (hidden_states, residual, next_mlp_sp_logit, next_att_idx)."""
         assert mixer_subset is None
         ip = None if mixer_kwargs is None else mixer_kwargs.get("inference_params")
+        dv_modules.join_heads()  # head_idx may be the pending selection of the block before
         if self.use_fused_layer and fused_layer.eligible(self, hidden_states, residual, head_idx, mlp_sp_logit, ip):
             return fused_layer.sparse_layer_decode(self, hidden_states, residual, head_idx, mlp_sp_logit, ip)
-        hidden_states, residual = _add_norm(self.norm1, hidden_states, residual)
         if mixer_kwargs is None:
             mixer_kwargs = {}
+        hidden_states, residual, window = self._norm1(hidden_states, residual, head_idx, ip)
+        lazy = LAZY_SIDE_JOIN and hidden_states.is_cuda
         hidden_states, mlp_idx, next_att_idx = self.mixer(hidden_states, residual=residual, head_idx=head_idx,
-                                                          mlp_sp_logit=mlp_sp_logit, **mixer_kwargs)
+                                                          mlp_sp_logit=mlp_sp_logit, window=window, defer_join=lazy,
+                                                          **mixer_kwargs)
         hidden_states, residual = _add_norm(self.norm2, hidden_states, residual)
-        hidden_states, next_mlp_sp_logit = self.mlp(hidden_states, residual, mlp_idx)
+        if lazy:
+            self.mixer.join_side()  # LayerNorm 2 did not need the selections; fc1 does
+        hidden_states, next_mlp_sp_logit = self.mlp(hidden_states, residual, mlp_idx, defer_join=lazy)
         return hidden_states, residual, next_mlp_sp_logit, next_att_idx
 
+
+    def _norm1(self, hidden_states, residual, head_idx, ip):
+        """LayerNorm 1; for B > 1 sequences at a sparse decode step the window row and the tracker step
+        ride in the same launch (FOLD_WINDOW_STEP).  Returns (hidden_states, residual, window)."""
+        window = None
+        if (FOLD_WINDOW_STEP and head_idx is not None and ip is not None and ip.sequence_len_offset > 0
+                and hidden_states.is_cuda and hidden_states.dtype == torch.float16 and hidden_states.size(0) > 1
+                and hidden_states.size(1) == 1 and hasattr(self.mixer, "begin_window_step")):
+            window = self.mixer.begin_window_step(hidden_states.size(0), head_idx, hidden_states.device)
+            hidden_states, residual = ops.add_layer_norm_window(
+                hidden_states, residual, self.norm1.weight, self.norm1.bias, self.norm1.eps, window["x_cache_row"],
+                window["tracker"], window["head_idx"], window["counter"], window["flush"], window["batch_idx"])
+        else:
+            hidden_states, residual = _add_norm(self.norm1, hidden_states, residual)
+        return hidden_states, residual, window
 
 class BlockDejavu(nn.Module):
     """Block with dense attention and a sparse MLP (block_dejavu.py:259-461)."""
@@ -95,9 +130,12 @@ class BlockDejavu(nn.Module):
         hidden_states, residual = _add_norm(self.norm1, hidden_states, residual)
         if mixer_kwargs is None:
             mixer_kwargs = {}
-        hidden_states, mlp_idx = self.mixer(hidden_states, mlp_sp_logit=mlp_sp_logit, **mixer_kwargs)
+        lazy = LAZY_SIDE_JOIN and hidden_states.is_cuda
+        hidden_states, mlp_idx = self.mixer(hidden_states, mlp_sp_logit=mlp_sp_logit, defer_join=lazy, **mixer_kwargs)
         hidden_states, residual = _add_norm(self.norm2, hidden_states, residual)
-        hidden_states, next_mlp_sp_logit = self.mlp(hidden_states, residual, mlp_idx)
+        if lazy:
+            self.mixer.join_side()
+        hidden_states, next_mlp_sp_logit = self.mlp(hidden_states, residual, mlp_idx, defer_join=lazy)
         return hidden_states, residual, next_mlp_sp_logit
 
 

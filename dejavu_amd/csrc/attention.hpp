@@ -367,6 +367,22 @@ __global__ __launch_bounds__(256) void window_step_kernel(
   window_tracker_step(tracker, head_idx, nnz, H, counter, flush, batch_idx);
 }
 
+// add + LayerNorm of `rows` rows (one workgroup each; a second copy of the normalised rows goes to
+// the window buffer's row of this step) and, in one more workgroup, the tracker step of the same
+// window position: add_layer_norm_kernel and window_step_kernel in one launch.
+template <int THREADS, int NV>
+__global__ __launch_bounds__(THREADS) void add_layer_norm_window_kernel(
+    const half_t* __restrict__ Hin, const half_t* __restrict__ R, const half_t* __restrict__ gamma,
+    const half_t* __restrict__ beta, float eps, int d, half_t* __restrict__ Y, half_t* __restrict__ Rout,
+    half_t* __restrict__ x_cache_row, int rows, int* __restrict__ tracker, const int* __restrict__ head_idx,
+    int nnz, int H, int counter, int flush, int* __restrict__ batch_idx) {
+  if ((int)blockIdx.x == rows) {
+    window_tracker_step(tracker, head_idx, nnz, H, counter, flush, batch_idx);
+    return;
+  }
+  add_layer_norm_body<THREADS, NV>(Hin, R, gamma, beta, eps, d, Y, Rout, x_cache_row, blockIdx.x);
+}
+
 // Appends the newest token: for every batch row b and head (all, or head_idx):
 //   k_cache[b, h, :, pos_b, :] = K[b, h, :],  v_cache[b, h, pos_b, :] = V[b, h, :]
 // with pos_b = lengths[b] if lengths else pos.  K / V: (B, H, hd) with batch

@@ -1613,6 +1613,40 @@ int dv_add_layer_norm_f16(const void* h, const void* residual, const void* gamma
   return launch_status();
 }
 
+int dv_add_layer_norm_window_f16(const void* h, const void* residual, const void* gamma, const void* beta,
+                                 float eps, int rows, int d, void* y, void* residual_out, void* x_cache_row,
+                                 void* tracker, const void* head_idx, int nnz, int H, int counter, int flush,
+                                 void* batch_idx, void* stream) {
+  if (!h || !gamma || !beta || !y || !x_cache_row || !tracker || !batch_idx || rows < 1 || d <= 0 || H <= 0 ||
+      nnz < 0 || counter < 0 || counter > 15 || (!flush && nnz > 0 && !head_idx))
+    return DV_ERR_INVALID_ARG;
+  if (d % 8 || !aligned16(h) || !aligned16(y) || !aligned16(gamma) || !aligned16(beta) || !aligned16(x_cache_row) ||
+      (residual && !aligned16(residual)) || (residual_out && !aligned16(residual_out)))
+    return DV_ERR_ALIGNMENT;
+  if (d > 256 * 8 * 16) return DV_ERR_UNSUPPORTED;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+#define DV_LNW(T, V)                                                                                          \
+  hipLaunchKernelGGL((add_layer_norm_window_kernel<T, V>), dim3(rows + 1), dim3(T), 0, s,                      \
+                     reinterpret_cast<const half_t*>(h), reinterpret_cast<const half_t*>(residual),           \
+                     reinterpret_cast<const half_t*>(gamma), reinterpret_cast<const half_t*>(beta), eps, d,    \
+                     reinterpret_cast<half_t*>(y), reinterpret_cast<half_t*>(residual_out),                   \
+                     reinterpret_cast<half_t*>(x_cache_row), rows, reinterpret_cast<int*>(tracker),            \
+                     reinterpret_cast<const int*>(head_idx), nnz, H, counter, flush,                          \
+                     reinterpret_cast<int*>(batch_idx))
+  if (d <= 256 * 8 * 1)
+    DV_LNW(256, 1);
+  else if (d <= 512 * 8 * 1)
+    DV_LNW(512, 1);
+  else if (d <= 1024 * 8 * 1)
+    DV_LNW(1024, 1);
+  else if (d <= 1024 * 8 * 2)
+    DV_LNW(1024, 2);
+  else
+    DV_LNW(1024, 4);
+#undef DV_LNW
+  return launch_status();
+}
+
 namespace {
 struct LayerPlan {
   size_t off_topk, off_res1, off_parts, off_acc, off_qkv, off_batch_idx, off_hp_hidden, off_mp_hidden, off_h,

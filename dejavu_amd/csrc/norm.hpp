@@ -290,8 +290,8 @@ template <int THREADS, int NV>
 __global__ __launch_bounds__(THREADS) void add_layer_norm_kernel(
     const half_t* __restrict__ H, const half_t* __restrict__ R, const half_t* __restrict__ gamma,
     const half_t* __restrict__ beta, float eps, int d, half_t* __restrict__ Y,
-    half_t* __restrict__ Rout) {
-  add_layer_norm_body<THREADS, NV>(H, R, gamma, beta, eps, d, Y, Rout, nullptr, blockIdx.x);
+    half_t* __restrict__ Rout, half_t* __restrict__ Y2 = nullptr) {
+  add_layer_norm_body<THREADS, NV>(H, R, gamma, beta, eps, d, Y, Rout, Y2, blockIdx.x);
 }
 
 }  // namespace dv

@@ -152,8 +152,16 @@ def _advance_window(m, flush):
         m.counter = 0
 
 
+def _join_side_stream():
+    """The launches read the predictions of the block before on the current stream; a block that went
+    module by module may have left them pending on the side stream (block.LAZY_SIDE_JOIN)."""
+    from .modules import join_side_stream
+    join_side_stream()
+
+
 def sparse_layer_decode(block, hidden_states, residual, head_idx, mlp_sp_logit, inference_params):
     """Returns (hidden_states, residual, next_mlp_sp_logit, next_att_idx) like the block's forward."""
+    _join_side_stream()
     a = SparseLayerArgs()
     outs, keep, flush = _fill_args(a, block, hidden_states, residual, head_idx, mlp_sp_logit, inference_params)
     hidden_out, residual_out, logit_out, att_idx_out, mlp_idx_out = outs
@@ -201,6 +209,7 @@ class LayerChain:
     def run(self):
         n = len(self._args)
         assert n > 0
+        _join_side_stream()
         arr = (SparseLayerArgs * n)(*self._args)
         ws = _workspace(self.outputs[0][0].device, self._nbytes)
         arr[0].workspace, arr[0].workspace_bytes = ws.data_ptr(), ws.numel()

@@ -176,6 +176,7 @@ class GPTModel(nn.Module):
                     and input_ids.shape[0] == 1)
         for layer in self.layers:
             if self.record is not None and input_ids.shape[1] == 1:
+                dv_modules.join_side_stream()  # the predictions of the block before may be pending on the side stream
                 self.record.append((None if next_att_idx is None else next_att_idx.clone(),
                                     None if next_mlp_sp_logit is None else next_mlp_sp_logit.clone()))
             if chaining and getattr(layer, "use_fused_layer", False) and fused_layer.eligible(

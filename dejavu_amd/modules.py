@@ -76,12 +76,32 @@ def side_stream(device=None) -> "torch.cuda.Stream":
     return st
 
 
+_heads_event = None  # head selection of the last block that left it pending on a side stream
+
+
+def mark_side_pending(heads_event=None) -> None:
+    """Work was left on the side stream (and this event covers the head selection among it)."""
+    global _side_pending, _heads_event
+    _side_pending = True
+    if heads_event is not None:
+        _heads_event = heads_event
+
+
+def join_heads() -> None:
+    """Makes the current stream wait for the head selection a block left pending on a side stream."""
+    global _heads_event
+    if _heads_event is not None:
+        torch.cuda.current_stream().wait_event(_heads_event)
+        _heads_event = None
+
+
 def join_side_stream() -> None:
     """Makes the current stream wait for everything enqueued on the side stream so far
     (e.g. before a graph capture that used the side stream ends)."""
-    global _side_pending
+    global _side_pending, _heads_event
     if _side_pending and _side_streams:
         _side_pending = False
+        _heads_event = None
         ev = torch.cuda.Event(enable_timing=False, blocking=False)
         st = side_stream()
         st.record_event(ev)
@@ -192,40 +212,56 @@ class ParallelFusedMLPDejavu(nn.Module):
         """fc2.weight as (hidden, out), contiguous; follows updates of fc2.weight."""
         return _transposed_copy(self, "fc2_weight_t", self.fc2.weight)
 
-    def forward(self, x, residual, idx=None):
+    def forward(self, x, residual, idx=None, defer_join=False):
         """x, residual: (B, 1, d) at decode (or (B, s, d) for the prompt).
         idx: (K,) active neurons or None for the dense MLP.
         Returns (out, mlp_logit); mlp_logit, the predictor output for the next
-        layer's MLP, only when decoding one token."""
+        layer's MLP, only when decoding one token.  defer_join: when the predictor runs on the side
+        stream, the current stream does not wait for it: mlp_logit is then only good for work
+        enqueued on the side stream (the next layer's top-k is) or after ``join_side_stream()``."""
         self._streams()
         curr_stream = torch.cuda.current_stream()
         do_token_generation = x.size(1) == 1
         # The predictor only needs `residual`, so it streams its weights on the side
         # stream while fc1 / fc2 run (the reference starts it after the MLP, to
         # overlap the tensor-parallel all-reduce that one GPU does not have).
+        # The side work is ENQUEUED AFTER the main work of the phase (it still starts from the event
+        # recorded here).  In a captured graph the first-captured successor of a node stays on its
+        # hardware queue and the others move to another one; a hand-over between queues costs about
+        # 10 us when the consumer is waiting for it, so the chain that is waited for -- fc1, fc2 --
+        # must be the one captured first (batch 8, OPT-175B shape: four such hand-overs per layer step).
         mlp_logit = None
         side = do_token_generation and side_stream_enabled(x.shape[0])
         if side:
+            curr_stream.record_event(self.event_mlp)
+        if idx != None:
+            assert x.size(1) == 1
+            h = ops.gather_gemv(x.squeeze(1), self.fc1.weight, idx, self.fc1.bias, activation=self.activation)
+        else:
+            h = decode_linear(self.fc1, x, self.activation)
+        if side:  # behind fc1: the main chain's first launch of the phase is captured, the rest follows
             global _side_pending
             _side_pending = True
-            curr_stream.record_event(self.event_mlp)
             with torch.cuda.stream(self.sp_stream):
                 self.sp_stream.wait_event(self.event_mlp)
                 mlp_logit = self.sp(residual)
                 self.sp_stream.record_event(self.event_mlp_sp)
-        elif do_token_generation:
-            mlp_logit = self.sp(residual)
         if idx != None:
-            assert x.size(1) == 1
-            out = ops.mlp_sparse(x.squeeze(1), self.fc1.weight, self.transposed_fc2(), idx, self.fc1.bias,
-                                 self.fc2.bias, activation=self.activation)
-            out = out.unsqueeze(1)
+            out = ops.gather_transposed_gemv(h, self.transposed_fc2(), idx, self.fc2.bias).unsqueeze(1)
         else:
-            h = decode_linear(self.fc1, x, self.activation)
             out = decode_linear(self.fc2, h)
         # (tensor parallel all-reduce of `out` is the identity on one GPU)
         if side:
-            curr_stream.wait_event(self.event_mlp_sp)
+            if defer_join:
+                # The predictor may still be reading `residual` when the caller lets go of it: the
+                # tensor stays referenced here until this module's next forward.  By then the current
+                # stream has waited for side work that was enqueued behind this predictor (the top-k
+                # that consumes mlp_logit), so its memory is not handed out again too early.
+                self._side_keep = residual
+            else:
+                curr_stream.wait_event(self.event_mlp_sp)
+        elif do_token_generation:
+            mlp_logit = self.sp(residual)
         return out, mlp_logit
 
 
@@ -306,12 +342,16 @@ class _MHABase(nn.Module):
         self.mlp_k = None
         self.sp_stream = None
         self._side_used = False
+        self._forked = False
+        self._side_keep = None
+        self._mlp_idx_event = False
 
     def _streams(self):
         if self.sp_stream is None:
             self.sp_stream = side_stream(self.Wqkv.weight.device)
             self.event_in = torch.cuda.Event(enable_timing=False, blocking=False)
             self.event_side = torch.cuda.Event(enable_timing=False, blocking=False)
+            self.event_mlp_idx = torch.cuda.Event(enable_timing=False, blocking=False)
 
     def _dense_context(self, qkv, inference_params):
         """qkv: (B, s, 3, H, hd) -> context (B, s, H*hd) for the prompt or a dense decode step."""
@@ -345,18 +385,25 @@ class _MHABase(nn.Module):
                                          self.rotary_emb_dim, softmax_scale=scale)
         return ctx.reshape(B, 1, -1)
 
+    def _side_fork(self, batch):
+        """Marks, at the start of the forward, the point from which the side work may run."""
+        self._forked = side_stream_enabled(batch)
+        if self._forked:
+            torch.cuda.current_stream().record_event(self.event_in)
+
     def _side_work(self, mlp_sp_logit, residual=None, att_sp=None, att_k=None, att_idx_out=None):
         """Everything that does not depend on this layer's attention runs on the
-        side stream from the start of the forward: the head predictor + top-k for
+        side stream from the point ``_side_fork`` marked: the head predictor + top-k for
         the next layer (from the residual stream) and the MLP top-k for this layer
-        (from the previous layer's logits).  The caller joins with ``_join_side``
-        before returning."""
+        (from the previous layer's logits).  The forward enqueues it AFTER its own launches
+        (see ParallelFusedMLPDejavu.forward: the chain that is waited for must be captured first)
+        and joins with ``_join_side`` before returning."""
         mlp_idx, att_idx = None, None
         self._side_used = False
         if mlp_sp_logit is None and att_sp is None:
             return mlp_idx, att_idx
         batch = residual.shape[0] if residual is not None else (mlp_sp_logit.shape[0] if mlp_sp_logit.dim() > 1 else 1)
-        if not side_stream_enabled(batch):
+        if not (side_stream_enabled(batch) and self._forked):
             if att_sp is not None:
                 att_idx = ops.topk_indices(att_sp(residual), att_k, dtype=torch.int32, out=att_idx_out)
             if mlp_sp_logit is not None:
@@ -365,18 +412,34 @@ class _MHABase(nn.Module):
         self._side_used = True
         global _side_pending
         _side_pending = True
-        torch.cuda.current_stream().record_event(self.event_in)
         with torch.cuda.stream(self.sp_stream):
             self.sp_stream.wait_event(self.event_in)
-            if att_sp is not None:
-                att_idx = ops.topk_indices(att_sp(residual), att_k, dtype=torch.int32, out=att_idx_out)
+            # the neuron selection first: fc1 of this layer waits for it, the head selection is for
+            # the next layer
             if mlp_sp_logit is not None:
                 mlp_idx = ops.topk_indices(mlp_sp_logit, self.mlp_k)
+                self.sp_stream.record_event(self.event_mlp_idx)
+            if att_sp is not None:
+                att_idx = ops.topk_indices(att_sp(residual), att_k, dtype=torch.int32, out=att_idx_out)
             self.sp_stream.record_event(self.event_side)
+        self._mlp_idx_event = mlp_sp_logit is not None
         return mlp_idx, att_idx
 
     def _join_side(self):
         if self._side_used:
+            torch.cuda.current_stream().wait_event(self.event_side)
+
+    def join_side(self):
+        """For a caller that passed ``defer_join=True`` to ``forward``: makes the current stream wait for
+        the neuron selection of that forward.  The head selection (for the next layer) stays pending:
+        whoever uses it calls ``join_heads()`` first (the blocks do at their start;
+        ``join_side_stream()`` covers it too)."""
+        if not self._side_used:
+            return
+        if self._mlp_idx_event:
+            torch.cuda.current_stream().wait_event(self.event_mlp_idx)
+            mark_side_pending(self.event_side)
+        else:
             torch.cuda.current_stream().wait_event(self.event_side)
 
 
@@ -390,16 +453,21 @@ class ParallelMHADejavu(_MHABase):
         self._init_common(embed_dim, num_heads, process_group, bias, softmax_scale, causal, layer_idx,
                           rotary_emb_dim, device, dtype)
 
-    def forward(self, x, mlp_sp_logit=None, seqlen=None, inference_params=None, **kwargs):
-        """x: (B, s, d).  Returns (out, mlp_idx)."""
+    def forward(self, x, mlp_sp_logit=None, seqlen=None, inference_params=None, defer_join=False, **kwargs):
+        """x: (B, s, d).  Returns (out, mlp_idx).  defer_join: the caller calls ``join_side()`` itself
+        before it uses mlp_idx."""
         assert seqlen is None, "sequence-parallel input layout is not used for generation"
         self._streams()
-        mlp_idx, _ = self._side_work(mlp_sp_logit)
+        self._side_fork(x.shape[0])
         qkv = decode_linear(self.Wqkv, x)
         qkv = qkv.view(x.shape[0], x.shape[1], 3, self.num_heads, self.head_dim)
         context = self._dense_context(qkv, inference_params)
         out = decode_linear(self.out_proj, context)
-        self._join_side()
+        mlp_idx, _ = self._side_work(mlp_sp_logit)
+        if defer_join:
+            self._side_keep = mlp_sp_logit
+        else:
+            self._join_side()
         return out, mlp_idx
 
 
@@ -479,7 +547,25 @@ class ParallelMHASparseAttMlp(_MHABase):
         self.counter += 1
         return qkv, head_idx, kc, vc
 
-    def _sparse_decode_batched(self, x, head_idx, inference_params):
+    def begin_window_step(self, B, head_idx, dev):
+        """What the block needs to fold this step's window write and tracker step into its
+        LayerNorm 1 launch (``ops.add_layer_norm_window``) for B > 1 sequences: the window buffer's
+        row of this position, the tracker, the head set of the step (all heads at the flush
+        position) and the slot list to fill.  The result goes back in as ``window=`` of ``forward``."""
+        d, H = self.embed_dim, self.num_heads
+        if self.x_cache_batch is None or self.x_cache_batch.shape[1] != B * d:
+            assert self.counter == 0, "the batch size cannot change inside a back-fill window"
+            self.x_cache_batch = torch.zeros((self.WINDOW, B * d), dtype=torch.float16, device=dev)
+        flush = self.counter == self.WINDOW - 1
+        if flush:
+            if self._all_heads is None:
+                self._all_heads = torch.arange(H, dtype=torch.int32, device=dev)
+            head_idx = self._all_heads
+        batch_idx = torch.empty(head_idx.shape[0], self.counter + 1, dtype=torch.int32, device=dev)
+        return {"x_cache_row": self.x_cache_batch[self.counter], "tracker": self.tracker, "head_idx": head_idx,
+                "counter": self.counter, "flush": flush, "batch_idx": batch_idx}
+
+    def _sparse_decode_batched(self, x, head_idx, inference_params, window=None):
         """x: (B, 1, d), B > 1 sequences that decode in lockstep and share the head set and the
         back-fill window (the reference's sparse attention is single-sequence, mha_dejavu.py:1469;
         this is its batch extension).  The window buffer holds the B LayerNorm rows of each of
@@ -493,17 +579,22 @@ class ParallelMHASparseAttMlp(_MHABase):
         if self.x_cache_batch is None or self.x_cache_batch.shape[1] != B * d:
             assert self.counter == 0, "the batch size cannot change inside a back-fill window"
             self.x_cache_batch = torch.zeros((self.WINDOW, B * d), dtype=torch.float16, device=dev)
-        flush = self.counter == self.WINDOW - 1
-        if flush:
-            if self._all_heads is None:
-                self._all_heads = torch.arange(H, dtype=torch.int32, device=dev)
-            head_idx = self._all_heads
-        nnz = head_idx.shape[0]
         nb = self.counter + 1
-        batch_idx = torch.empty(nnz, nb, dtype=torch.int32, device=dev)
-        check(lib.dv_window_step_f16(x.data_ptr(), self.x_cache_batch.data_ptr(), B * d, self.tracker.data_ptr(),
-                                     head_idx.data_ptr(), nnz, H, self.counter, int(flush), batch_idx.data_ptr(),
-                                     torch.cuda.current_stream().cuda_stream), "dv_window_step_f16")
+        if window is not None:  # the block's LayerNorm launch has written the window row and run the tracker
+            assert window["counter"] == self.counter and window["x_cache_row"].data_ptr() == \
+                self.x_cache_batch[self.counter].data_ptr()
+            head_idx, batch_idx = window["head_idx"], window["batch_idx"]
+        else:
+            flush = self.counter == self.WINDOW - 1
+            if flush:
+                if self._all_heads is None:
+                    self._all_heads = torch.arange(H, dtype=torch.int32, device=dev)
+                head_idx = self._all_heads
+            nnz = head_idx.shape[0]
+            batch_idx = torch.empty(nnz, nb, dtype=torch.int32, device=dev)
+            check(lib.dv_window_step_f16(x.data_ptr(), self.x_cache_batch.data_ptr(), B * d, self.tracker.data_ptr(),
+                                         head_idx.data_ptr(), nnz, H, self.counter, int(flush), batch_idx.data_ptr(),
+                                         torch.cuda.current_stream().cuda_stream), "dv_window_step_f16")
         k_cache, v_cache = inference_params.key_value_memory_dict[self.layer_idx]
         b0 = inference_params.batch_size_offset
         kc, vc = k_cache[b0:b0 + B], v_cache[b0:b0 + B]
@@ -524,10 +615,13 @@ class ParallelMHASparseAttMlp(_MHABase):
         self.counter += 1
         return qkv, head_idx, kc, vc
 
-    def forward(self, x, residual, head_idx=None, mlp_sp_logit=None, seqlen=None, inference_params=None, **kwargs):
+    def forward(self, x, residual, head_idx=None, mlp_sp_logit=None, seqlen=None, inference_params=None, window=None,
+                defer_join=False, **kwargs):
         """x, residual: (B, s, d).  head_idx: (Hk,) int32 heads to compute, or None
-        for dense attention.  mlp_sp_logit: predictor logits for this layer's MLP.
-        Returns (out, mlp_idx, att_idx)."""
+        for dense attention.  mlp_sp_logit: predictor logits for this layer's MLP.  window: the
+        result of ``begin_window_step`` when the caller's LayerNorm launch has already done the
+        window step.  defer_join: the caller calls ``join_side()`` itself before it uses mlp_idx / att_idx
+        (the block does, after LayerNorm 2, which does not need them).  Returns (out, mlp_idx, att_idx)."""
         assert seqlen is None, "sequence-parallel input layout is not used for generation"
         self._streams()
         do_token_generation = x.size(1) == 1
@@ -535,8 +629,7 @@ class ParallelMHASparseAttMlp(_MHABase):
             self._set_cache_offset(x.size(1), x.device)
             self.reset_window()
         sparse = inference_params is not None and inference_params.sequence_len_offset > 0 and head_idx != None
-        mlp_idx, att_idx = self._side_work(mlp_sp_logit, residual, self.sp if do_token_generation else None,
-                                           self.att_k, self.att_idx_out)
+        self._side_fork(x.shape[0])
         if sparse:
             assert x.size(1) == 1
             self.transposed_out_proj()
@@ -547,7 +640,7 @@ class ParallelMHASparseAttMlp(_MHABase):
                                              self.out_proj_weight_t, self.out_proj.bias,
                                              inference_params.lengths_per_sample, self.softmax_scale).unsqueeze(1)
             else:
-                qkv, head_idx, kc, vc = self._sparse_decode_batched(x, head_idx, inference_params)
+                qkv, head_idx, kc, vc = self._sparse_decode_batched(x, head_idx, inference_params, window)
                 ctx = ops.single_query_attention(qkv[:, 0], None, None, kc, vc, inference_params.lengths_per_sample,
                                                  inference_params.sequence_len_offset, self.rotary_emb_dim,
                                                  head_idx=head_idx, softmax_scale=self.softmax_scale)
@@ -561,5 +654,10 @@ class ParallelMHASparseAttMlp(_MHABase):
             qkv = qkv.view(x.shape[0], x.shape[1], 3, self.num_heads, self.head_dim)
             context = self._dense_context(qkv, inference_params)
             out = decode_linear(self.out_proj, context)
-        self._join_side()
+        mlp_idx, att_idx = self._side_work(mlp_sp_logit, residual, self.sp if do_token_generation else None,
+                                           self.att_k, self.att_idx_out)
+        if defer_join:
+            self._side_keep = (residual, mlp_sp_logit)  # read by the side work until join_side()
+        else:
+            self._join_side()
         return out, mlp_idx, att_idx

@@ -728,6 +728,37 @@ def add_layer_norm(hidden: torch.Tensor, residual: Optional[torch.Tensor], weigh
     return y, r_out
 
 
+def add_layer_norm_window(hidden: torch.Tensor, residual: Optional[torch.Tensor], weight: torch.Tensor,
+                          bias: torch.Tensor, eps: float, x_cache_row: torch.Tensor, tracker: torch.Tensor,
+                          head_idx: torch.Tensor, counter: int, flush: bool, batch_idx: torch.Tensor):
+    """``add_layer_norm`` for the rows of B sequences that share a back-fill window, with the window
+    step of the same position in the same launch: the normalised rows also go to ``x_cache_row``
+    ((B * d,) row ``counter`` of the window buffer) and the tracker hands out ``batch_idx``
+    ((nnz, counter + 1) int32; see ``dv_window_step_f16``).  Returns (normed, residual_out)."""
+    _require_device(hidden, residual, weight, bias, x_cache_row, tracker, head_idx, batch_idx)
+    assert hidden.dtype == torch.float16 and weight.dtype == torch.float16 and bias.dtype == torch.float16
+    d = hidden.shape[-1]
+    hidden = hidden.contiguous()
+    rows = hidden.numel() // d
+    if residual is not None:
+        assert residual.shape == hidden.shape and residual.dtype == hidden.dtype
+        residual = residual.contiguous()
+    assert x_cache_row.dtype == torch.float16 and x_cache_row.is_contiguous() and x_cache_row.numel() == rows * d
+    assert tracker.dtype == torch.int32 and head_idx.dtype == torch.int32 and batch_idx.dtype == torch.int32
+    assert tracker.is_contiguous() and batch_idx.is_contiguous() and head_idx.is_contiguous()
+    H = tracker.shape[0]
+    nnz = head_idx.shape[0]
+    assert batch_idx.numel() >= nnz * (counter + 1)
+    y = torch.empty_like(hidden)
+    r_out = torch.empty_like(hidden)
+    check(lib.dv_add_layer_norm_window_f16(_ptr(hidden), _ptr(residual), _ptr(weight.contiguous()),
+                                           _ptr(bias.contiguous()), float(eps), rows, d, _ptr(y), _ptr(r_out),
+                                           _ptr(x_cache_row), _ptr(tracker), _ptr(head_idx), nnz, H, int(counter),
+                                           int(flush), _ptr(batch_idx), _stream()),
+          "dv_add_layer_norm_window_f16")
+    return y, r_out
+
+
 def add_ln_parts(hidden: torch.Tensor, residual: Optional[torch.Tensor]):
     """First half of ``add_layer_norm`` for ONE row when the consumer of the row normalises it itself:
     ``r = hidden + residual`` (fp16) and the statistics pairs of r's 64-element parts (float32,

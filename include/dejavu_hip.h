@@ -432,6 +432,19 @@ DV_API int dv_add_layer_norm_f16(const void* h, const void* residual, const void
                                  void* residual_out, void* stream);
 
 /*
+ * dv_add_layer_norm_f16 and dv_window_step_f16 in one launch, for `rows` sequences that share a
+ * back-fill window: the normalised rows also go to x_cache_row (rows, d) -- the row of the window
+ * buffer that belongs to this step (x_cache + counter * rows * d) -- and one more workgroup runs the
+ * tracker step (block_dejavu.py:575-584 + mha_dejavu.py:1124-1149, 1318-1329).  Same outputs as the
+ * two separate calls.  Arguments as there; x_cache_row 16-byte aligned.
+ */
+DV_API int dv_add_layer_norm_window_f16(const void* h, const void* residual, const void* gamma,
+                                        const void* beta, float eps, int rows, int d, void* y,
+                                        void* residual_out, void* x_cache_row, void* tracker,
+                                        const void* head_idx, int nnz, int H, int counter, int flush,
+                                        void* batch_idx, void* stream);
+
+/*
  * Greedy step of the generation loop (batch 1): next = argmax(logits[0 .. vocab)), first index
  * among equal values; then, all on the device so that a captured step can be replayed:
  * token[0] = next, sequences[out_index[0]++] = next, position[0]++, seq_pos[0]++ and, with

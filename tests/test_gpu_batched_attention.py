@@ -377,3 +377,61 @@ def test_batched_block_step_same_bits_with_and_without_the_side_stream():
             assert torch.equal(xa, xb)
     for ca, cb in zip(results[0][1], results[1][1]):
         assert torch.equal(ca, cb)
+
+
+# switches that fold launches of the batched layer step; each must leave every bit where it was
+_FOLD_SWITCHES = [("dejavu_amd.block", "FOLD_WINDOW_STEP"), ("dejavu_amd.block", "LAZY_SIDE_JOIN")]
+
+
+@pytest.mark.parametrize("module_name,flag", _FOLD_SWITCHES)
+def test_batched_block_step_same_bits_with_and_without_folded_launches(module_name, flag):
+    """18 decode steps of a batch of sequences (a whole back-fill window with its flush step and the
+    start of the next) through the block with one launch-folding switch on and off: outputs,
+    residual stream, predictor logits, selections and both caches are the same bits."""
+    import copy
+    import importlib
+
+    import dejavu_amd.modules as M
+    from dejavu_amd.block import create_sparse_block, init_block_synthetic
+    from dejavu_amd.modules import InferenceParams
+    from dejavu_amd.workloads import pack_k_cache
+
+    mod = importlib.import_module(module_name)
+    B, d, ffn, H, r, K, Hk, S = 9, 1024, 4096, 8, 1000, 512, 3, 64
+    hd = d // H
+    blk = create_sparse_block(d, ffn, H, r, K, r, Hk, layer_idx=0)
+    init_block_synthetic(blk, seed=11)
+    g = torch.Generator().manual_seed(111)
+    kc = pack_k_cache(torch.randn(B, H, S, hd, generator=g).half())
+    vc = torch.randn(B, H, S, hd, generator=g).half()
+    assert getattr(mod, flag) is True
+    results = []
+    try:
+        for on in (True, False):
+            setattr(mod, flag, on)
+            b = copy.deepcopy(blk)
+            ip = InferenceParams(max_sequence_len=S, max_batch_size=B, sequence_len_offset=30)
+            ip.key_value_memory_dict[0] = (kc.clone().cuda(), vc.clone().cuda())
+            b.mixer._set_cache_offset(30, torch.device("cuda"))
+            gg = torch.Generator().manual_seed(112)
+            outs = []
+            for step in range(18):
+                hs = torch.randn(B, 1, d, generator=gg).half().cuda()
+                res = torch.randn(B, 1, d, generator=gg).half().cuda()
+                head_idx = torch.sort(torch.randperm(H, generator=gg)[:Hk]).values.int().cuda()
+                logit = (torch.randn(B, ffn, generator=gg) * 4).half().cuda()
+                print(f"case batched block, {flag}={on}, step {step}", flush=True)
+                with torch.no_grad():
+                    out = b(hs, res, mixer_kwargs={"inference_params": ip}, head_idx=head_idx, mlp_sp_logit=logit)
+                M.join_side_stream()
+                torch.cuda.synchronize()
+                outs.append([t.clone() for t in out])
+                ip.sequence_len_offset += 1
+            results.append((outs, ip.key_value_memory_dict[0]))
+    finally:
+        setattr(mod, flag, True)
+    for step, (oa, ob) in enumerate(zip(results[0][0], results[1][0])):
+        for xa, xb in zip(oa, ob):
+            assert torch.equal(xa, xb), f"step {step} differs"
+    for ca, cb in zip(results[0][1], results[1][1]):
+        assert torch.equal(ca, cb)
