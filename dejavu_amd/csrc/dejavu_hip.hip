@@ -939,13 +939,16 @@ int dv_topk_f16(const void* logits, int B, int n, int k, void* idx_out, int idx_
     return DV_ERR_WORKSPACE;
   unsigned* ws = reinterpret_cast<unsigned*>(workspace);
   const int blocks = (n + kTopkItemsPerBlock - 1) / kTopkItemsPerBlock;
-  if (B > 1 && B <= 64) {  // one wide pass reduces the batch to a row; the selection then reads that row
+  if (B > 1 && B <= 64) {
+    // one pass reduces the batch to a row of column-wise maxima and takes that row's coarse histogram;
+    // the selection then reads the row
     half_t* m = reinterpret_cast<half_t*>(reinterpret_cast<unsigned char*>(workspace) + topk_max_row_offset(n));
-    hipLaunchKernelGGL(topk_batch_max_kernel, dim3((n / 8 + 31) / 32), dim3(256), 0, s, lg, B, n, m);
+    hipLaunchKernelGGL(topk_batch_hist_kernel, dim3(blocks), dim3(256), 0, s, lg, B, n, m, ws);
     lg = m;
     B = 1;
+  } else {
+    hipLaunchKernelGGL(topk_hist_kernel, dim3(blocks), dim3(256), 0, s, lg, B, n, ws);
   }
-  hipLaunchKernelGGL(topk_hist_kernel, dim3(blocks), dim3(256), 0, s, lg, B, n, ws);
   hipLaunchKernelGGL(topk_count_kernel, dim3(blocks), dim3(256), 0, s, lg, B, n, k, ws);
   hipLaunchKernelGGL(topk_emit_kernel, dim3(blocks), dim3(256), 0, s, lg, B, n, k, ws, idx_out, idx_bytes);
   return launch_status();

@@ -224,7 +224,7 @@ __global__ __launch_bounds__(256) void topk_small_kernel(const half_t* __restric
 //     (ascending) positions.
 // Workspace layout (u32): wc[32][256], wf[32][256], above[32], meta[4] = {c*, columns above c*},
 // then (16-byte aligned) n fp16 values: the column-wise maximum of a batch
-// (topk_batch_max_kernel).
+// (topk_batch_hist_kernel).
 // ---------------------------------------------------------------------------
 constexpr int kTopkItemsPerBlock = 256 * 8;
 constexpr int kTopkBins = 256;
@@ -249,53 +249,6 @@ __device__ __forceinline__ void topk_load_keys(const half_t* __restrict__ logits
   }
 }
 
-// Column-wise "maximum" of a (B, n) batch, as a row of fp16 values: m[j] = the logit of
-// column j with the largest key.  Top-k over m equals top-k over the batch with the
-// maximum-over-rows score, so a batch costs one wide pass (n / 256 workgroups, the rows of a
-// column spread over 8 threads, every thread's loads issued together) and the three
-// selection kernels then read one row instead of B.  Requires n % 8 == 0, B <= 64.
-__global__ __launch_bounds__(256) void topk_batch_max_kernel(const half_t* __restrict__ logits, int B,
-                                                             int n, half_t* __restrict__ m) {
-  __shared__ unsigned s_best[8][32][8];  // [row group][octet][element] = key << 16 | fp16 bits
-  const int oct_l = threadIdx.x & 31, rg = threadIdx.x >> 5;
-  const int i0 = (blockIdx.x * 32 + oct_l) * 8;
-  unsigned best[8];
-#pragma unroll
-  for (int e = 0; e < 8; ++e) best[e] = 0u;
-  if (i0 < n) {
-    half8_t v[8];
-#pragma unroll
-    for (int u = 0; u < 8; ++u) {  // rows rg, rg + 8, ...: past the batch the last own row repeats
-      int b = rg + 8 * u;
-      if (b >= B) b = rg < B ? rg : 0;
-      v[u] = load8(logits + (int64_t)b * n + i0);
-    }
-#pragma unroll
-    for (int u = 0; u < 8; ++u)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const half_t hv = v[u][e];  // a copy: bit-casting a vector element in place gave wrong lanes
-        const unsigned packed = (topk_key(hv) << 16) | (unsigned)__builtin_bit_cast(unsigned short, hv);
-        best[e] = packed > best[e] ? packed : best[e];
-      }
-  }
-#pragma unroll
-  for (int e = 0; e < 8; ++e) s_best[rg][oct_l][e] = best[e];
-  __syncthreads();
-  if (rg == 0 && i0 < n) {
-    half8_t o;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      unsigned p = s_best[0][oct_l][e];
-#pragma unroll
-      for (int r = 1; r < 8; ++r) p = s_best[r][oct_l][e] > p ? s_best[r][oct_l][e] : p;
-      const unsigned short bits = (unsigned short)(p & 0xFFFFu);
-      o[e] = __builtin_bit_cast(half_t, bits);
-    }
-    store8(m + i0, o);
-  }
-}
-
 // A workgroup covers 256 * 8 columns with its first 256 threads (further threads, if the launch
 // has them, only take part in the barriers).
 __device__ __forceinline__ void topk_hist_body(const half_t* __restrict__ logits, int B, int n,
@@ -317,6 +270,50 @@ __device__ __forceinline__ void topk_hist_body(const half_t* __restrict__ logits
 __global__ __launch_bounds__(256) void topk_hist_kernel(const half_t* __restrict__ logits, int B, int n,
                                                         unsigned* __restrict__ ws) {
   topk_hist_body(logits, B, n, ws, blockIdx.x);
+}
+
+// A (B, n) batch: the column-wise "maximum" as a row of fp16 values -- m[j] = the logit of column j with
+// the largest key (among equal keys the larger bit pattern) -- and the coarse histogram of m's keys, in one
+// launch.  Top-k over m equals top-k over the batch with the maximum-over-rows score, so the count and
+// emit kernels then read one row instead of B.  Workgroup b owns columns [2048 b, 2048 (b + 1)), a thread
+// one 8-column vector of all B rows (loads in groups of eight rows).  Requires n % 8 == 0.
+__global__ __launch_bounds__(256) void topk_batch_hist_kernel(const half_t* __restrict__ logits, int B, int n,
+                                                              half_t* __restrict__ m, unsigned* __restrict__ ws) {
+  __shared__ unsigned s_coarse[kTopkBins];
+  s_coarse[threadIdx.x] = 0u;
+  __syncthreads();
+  const int i0 = (blockIdx.x * 256 + threadIdx.x) * 8;
+  if (i0 < n) {
+    unsigned best[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) best[e] = 0u;
+    for (int b0 = 0; b0 < B; b0 += 8) {
+      half8_t v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {  // past the batch the last row repeats (a maximum does not mind)
+        const int b = b0 + u < B ? b0 + u : B - 1;
+        v[u] = load8(logits + (int64_t)b * n + i0);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const half_t hv = v[u][e];
+          const unsigned packed = (topk_key(hv) << 16) | (unsigned)__builtin_bit_cast(unsigned short, hv);
+          best[e] = packed > best[e] ? packed : best[e];
+        }
+    }
+    half8_t o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const unsigned short bits = (unsigned short)(best[e] & 0xFFFFu);
+      o[e] = __builtin_bit_cast(half_t, bits);
+      atomicAdd(&s_coarse[best[e] >> 24], 1u);  // key >> 8
+    }
+    store8(m + i0, o);
+  }
+  __syncthreads();
+  ws[blockIdx.x * kTopkBins + threadIdx.x] = s_coarse[threadIdx.x];
 }
 
 // Inclusive prefix sum over the 256 threads of a workgroup (s_w: 4 words of LDS).
