@@ -125,6 +125,10 @@ SIGNATURES = {
     "dv_out_proj_sparse_f16": (
         _c_int, [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr]),
     "dv_out_proj_sparse_t_workspace_bytes": (_c_size, [_c_int, _c_int, _c_int, _c_int]),
+    "dv_out_proj_sparse_t_ln_workspace_bytes": (_c_size, [_c_int, _c_int, _c_int, _c_int]),
+    "dv_out_proj_sparse_t_ln_f16": (
+        _c_int, [_c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr,
+                 _c_ptr, ctypes.c_float, _c_ptr, _c_ptr, _c_ptr, _c_size, _c_ptr]),
     "dv_out_proj_sparse_t_f16": (
         _c_int,
         [_c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_size,

@@ -34,6 +34,9 @@ FOLD_WINDOW_STEP = True
 # next_att_idx are then good for the next block, or for anybody after modules.join_side_stream().
 # False: every module waits for its side work before it returns.
 LAZY_SIDE_JOIN = True
+# Batched sparse decode: the split reduction of out_proj, the residual add and LayerNorm 2 in one launch
+# (ops.out_proj_sparse_t_add_layer_norm).  False: out_proj with its reduction launch, then add_layer_norm.
+FOLD_NORM2 = True
 
 
 def _add_norm(norm: nn.LayerNorm, hidden_states: Tensor, residual: Optional[Tensor]):
@@ -85,15 +88,19 @@ class BlockMlpAttSparse(nn.Module):
             mixer_kwargs = {}
         hidden_states, residual, window = self._norm1(hidden_states, residual, head_idx, ip)
         lazy = LAZY_SIDE_JOIN and hidden_states.is_cuda
+        post_norm = (self.norm2, residual) if (FOLD_NORM2 and window is not None) else None
         hidden_states, mlp_idx, next_att_idx = self.mixer(hidden_states, residual=residual, head_idx=head_idx,
                                                           mlp_sp_logit=mlp_sp_logit, window=window, defer_join=lazy,
-                                                          **mixer_kwargs)
+                                                          post_norm=post_norm, **mixer_kwargs)
         if lazy:
             # fc1 needs the neuron selection.  The wait sits in front of LayerNorm 2, which does not need it:
             # measured there (and in front of out_proj) 12 us per step faster than between LayerNorm 2 and
             # fc1 (OPT-175B shape, batch 8 / 16 / 32), 9 us faster than in front of the attention.
             self.mixer.join_side()
-        hidden_states, residual = _add_norm(self.norm2, hidden_states, residual)
+        if isinstance(hidden_states, tuple):  # LayerNorm 2 rode in the projection's reduction launch
+            hidden_states, residual = hidden_states
+        else:
+            hidden_states, residual = _add_norm(self.norm2, hidden_states, residual)
         hidden_states, next_mlp_sp_logit = self.mlp(hidden_states, residual, mlp_idx, defer_join=lazy)
         return hidden_states, residual, next_mlp_sp_logit, next_att_idx
 

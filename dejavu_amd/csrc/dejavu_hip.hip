@@ -673,36 +673,74 @@ size_t cols_mfma_workspace_bytes(int B, int N, int M) {
   return (size_t)groups * B * N * sizeof(float);
 }
 
+// What follows a transposed product in the block: residual add + LayerNorm of its rows.  With a tail the
+// split reduction and the LayerNorm are ONE launch (norm.hpp: LnRowFromPartials); y itself is not stored.
+struct LnTail {
+  const half_t* residual;
+  const half_t* gamma;
+  const half_t* beta;
+  float eps;
+  half_t* normed;
+  half_t* residual_out;
+};
+
+// the reduction (groups > 1: from the partial sums; else y is complete) with or without the tail
+void launch_cols_reduce(const float* partial, const half_t* bias, int groups, int B, int N, half_t* y,
+                        const LnTail* tail, hipStream_t s) {
+  if (tail == nullptr) {
+    if (groups > 1) {
+      const int64_t total = (int64_t)B * N;
+      hipLaunchKernelGGL(cols_reduce_kernel<false>, dim3((unsigned)((total + 63) / 64)), dim3(256), 0, s, partial,
+                         bias, groups, B, N, y, (const half_t*)nullptr, (half_t*)nullptr);
+    }
+    return;
+  }
+#define DV_RLN(T, V)                                                                                              \
+  do {                                                                                                            \
+    if (groups > 1)                                                                                               \
+      hipLaunchKernelGGL((reduce_add_layer_norm_kernel<T, V>), dim3(B), dim3(T), 0, s, partial, bias, groups, B,  \
+                         tail->residual, tail->gamma, tail->beta, tail->eps, N, tail->normed, tail->residual_out); \
+    else                                                                                                          \
+      hipLaunchKernelGGL((add_layer_norm_kernel<T, V>), dim3(B), dim3(T), 0, s, (const half_t*)y, tail->residual,   \
+                         tail->gamma, tail->beta, tail->eps, N, tail->normed, tail->residual_out,                 \
+                         (half_t*)nullptr);                                                                       \
+  } while (0)
+  if (N <= 256 * 8 * 1)
+    DV_RLN(256, 1);
+  else if (N <= 512 * 8 * 1)
+    DV_RLN(512, 1);
+  else if (N <= 1024 * 8 * 1)
+    DV_RLN(1024, 1);
+  else if (N <= 1024 * 8 * 2)
+    DV_RLN(1024, 2);
+  else
+    DV_RLN(1024, 4);
+#undef DV_RLN
+}
+
 template <int BT, bool IDX64, bool BLOCKED>
 void launch_cols16(const Cols16Plan& p, const half_t* h, int64_t ldh, int x_expanded, const half_t* W, int64_t ldw,
                    const half_t* bias, const void* idx, int blk, int B, int N, int Z, int M, float* partial,
-                   half_t* y, hipStream_t s) {
+                   half_t* y, hipStream_t s, const LnTail* tail = nullptr) {
   hipLaunchKernelGGL((gather_cols_mfma16_kernel<BT, kC16Waves, IDX64, BLOCKED>), dim3(p.col_tiles, p.groups),
                      dim3(kC16Waves * 64), 0, s, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M,
                      p.rows_per_block, p.rows_per_wave, partial, y);
-  if (p.groups > 1) {
-    const int64_t total = (int64_t)B * N;
-    hipLaunchKernelGGL(cols_reduce_kernel<false>, dim3((unsigned)((total + 63) / 64)), dim3(256), 0, s, partial,
-                       bias, p.groups, B, N, y, (const half_t*)nullptr, (half_t*)nullptr);
-  }
+  launch_cols_reduce(partial, bias, p.groups, B, N, y, tail, s);
 }
 
 template <int BT, bool IDX64, bool BLOCKED, bool HVEC>
 void launch_cols_mfma(const ColsMfmaPlan& p, const half_t* h, int64_t ldh, int x_expanded, const half_t* W,
                       int64_t ldw, const half_t* bias, const void* idx, int blk, int B, int N, int Z, int M,
-                      float* partial, half_t* y, hipStream_t s) {
+                      float* partial, half_t* y, hipStream_t s, const LnTail* tail = nullptr) {
   hipLaunchKernelGGL((gather_cols_mfma_kernel<BT, IDX64, BLOCKED, HVEC>), dim3(p.col_tiles, p.groups), dim3(256), 0,
                      s, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M, p.rows_per_block, partial, y);
-  if (p.groups > 1) {
-    const int64_t total = (int64_t)B * N;
-    hipLaunchKernelGGL(cols_reduce_kernel<false>, dim3((unsigned)((total + 63) / 64)), dim3(256), 0, s, partial,
-                       bias, p.groups, B, N, y, (const half_t*)nullptr, (half_t*)nullptr);
-  }
+  launch_cols_reduce(partial, bias, p.groups, B, N, y, tail, s);
 }
 
 int gather_cols_mfma(const half_t* h, int64_t ldh, int x_expanded, const half_t* W, int64_t ldw,
                      const half_t* bias, const void* idx, int idx_bytes, int blk, int B, int N, int Z, int M,
-                     half_t* y, void* workspace, size_t workspace_bytes, hipStream_t s) {
+                     half_t* y, void* workspace, size_t workspace_bytes, hipStream_t s,
+                     const LnTail* tail = nullptr) {
   const ColsMfmaPlan p = plan_cols_mfma(B, N, M);
   if (workspace == nullptr || workspace_bytes < cols_mfma_workspace_bytes(B, N, M)) return DV_ERR_WORKSPACE;
   float* partial = reinterpret_cast<float*>(workspace);
@@ -715,11 +753,11 @@ int gather_cols_mfma(const half_t* h, int64_t ldh, int x_expanded, const half_t*
 #define DV_C16(BT)                                                                                                   \
   do {                                                                                                               \
     if (blocked) {                                                                                                   \
-      if (i64) launch_cols16<BT, true, true>(q, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M, partial, y, s);  \
-      else launch_cols16<BT, false, true>(q, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M, partial, y, s);     \
+      if (i64) launch_cols16<BT, true, true>(q, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M, partial, y, s, tail);  \
+      else launch_cols16<BT, false, true>(q, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M, partial, y, s, tail);     \
     } else {                                                                                                         \
-      if (i64) launch_cols16<BT, true, false>(q, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M, partial, y, s); \
-      else launch_cols16<BT, false, false>(q, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M, partial, y, s);    \
+      if (i64) launch_cols16<BT, true, false>(q, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M, partial, y, s, tail); \
+      else launch_cols16<BT, false, false>(q, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M, partial, y, s, tail);    \
     }                                                                                                                \
   } while (0)
     if (B <= 16) DV_C16(1);
@@ -727,7 +765,7 @@ int gather_cols_mfma(const half_t* h, int64_t ldh, int x_expanded, const half_t*
 #undef DV_C16
     return launch_status();
   }
-#define DV_ARGS p, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M, partial, y, s
+#define DV_ARGS p, h, ldh, x_expanded, W, ldw, bias, idx, blk, B, N, Z, M, partial, y, s, tail
 #define DV_CM3(BT, I64, BLK)                                   \
   do {                                                         \
     if (hvec) launch_cols_mfma<BT, I64, BLK, true>(DV_ARGS);   \
@@ -1561,6 +1599,35 @@ int dv_out_proj_sparse_t_f16(const void* x, const void* Wt, int64_t ldw, const v
                      reinterpret_cast<const half_t*>(Wt), ldw, reinterpret_cast<const half_t*>(bias),
                      head_idx, 4, hd, B, N, H * hd, nnz * hd, reinterpret_cast<half_t*>(y),
                      workspace, workspace_bytes, reinterpret_cast<hipStream_t>(stream), true);
+}
+
+int dv_out_proj_sparse_t_ln_f16(const void* x, const void* Wt, int64_t ldw, const void* bias, const void* head_idx,
+                                int nnz, int B, int H, int hd, int N, const void* residual, const void* gamma,
+                                const void* beta, float eps, void* normed, void* residual_out, void* workspace,
+                                size_t workspace_bytes, void* stream) {
+  if (!x || !Wt || !normed || !gamma || !beta || nnz < 1 || B < 1 || H <= 0 || hd <= 0 || N <= 0 || !head_idx)
+    return DV_ERR_INVALID_ARG;
+  if (B <= 4 || B > 64 || N > 256 * 8 * 16) return DV_ERR_UNSUPPORTED;  // the matrix-core path of dv_out_proj_sparse_t_f16
+  if (N % 8 || ldw % 8 || ldw < N || !aligned16(Wt) || !aligned16(normed) || !aligned16(gamma) || !aligned16(beta) ||
+      (residual && !aligned16(residual)) || (residual_out && !aligned16(residual_out)) ||
+      (workspace && !aligned16(workspace)))
+    return DV_ERR_ALIGNMENT;
+  // the product's own output row block (needed when a single row group stores it directly) sits behind the partials
+  const size_t part_bytes = cols_mfma_workspace_bytes(B, N, nnz * hd);
+  const size_t y_off = (part_bytes + 255) & ~(size_t)255;
+  if (!workspace || workspace_bytes < y_off + (size_t)B * N * sizeof(half_t)) return DV_ERR_WORKSPACE;
+  const LnTail tail{reinterpret_cast<const half_t*>(residual), reinterpret_cast<const half_t*>(gamma),
+                    reinterpret_cast<const half_t*>(beta), eps, reinterpret_cast<half_t*>(normed),
+                    reinterpret_cast<half_t*>(residual_out)};
+  half_t* y = reinterpret_cast<half_t*>(reinterpret_cast<unsigned char*>(workspace) + y_off);
+  return gather_cols_mfma(reinterpret_cast<const half_t*>(x), (int64_t)H * hd, 1, reinterpret_cast<const half_t*>(Wt),
+                          ldw, reinterpret_cast<const half_t*>(bias), head_idx, 4, hd, B, N, H * hd, nnz * hd, y,
+                          workspace, part_bytes, reinterpret_cast<hipStream_t>(stream), &tail);
+}
+
+size_t dv_out_proj_sparse_t_ln_workspace_bytes(int B, int nnz, int hd, int N) {
+  if (B <= 4 || B > 64 || nnz <= 0 || hd <= 0 || N <= 0) return 0;
+  return ((cols_mfma_workspace_bytes(B, N, nnz * hd) + 255) & ~(size_t)255) + (size_t)B * N * sizeof(half_t);
 }
 
 size_t dv_qkv_window_batch_workspace_bytes(int tokens, int nseq, int d, int nnz, int hd) {

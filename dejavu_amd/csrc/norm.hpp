@@ -144,9 +144,60 @@ struct LnNoHook {
 };
 // after_loads: called once the row's loads have been requested (a place to request memory the caller
 // needs later: requests queued before the row's loads would delay them, the load counter retires in order)
-template <int THREADS, int NV, class AfterLoads = LnNoHook>
-__device__ __forceinline__ void add_layer_norm_body(
-    const half_t* __restrict__ H, const half_t* __restrict__ R, const half_t* __restrict__ gamma,
+// Where the row to be added and normalised comes from: vector i (8 columns) of row `row`.
+struct LnRowFromMemory {
+  const half_t* __restrict__ H;
+  int d;
+  __device__ __forceinline__ half8_t operator()(int i, int64_t row) const { return load8(H + row * d + i * 8); }
+};
+// ... or from the fp32 partial sums of a split product, partial[(g * rows + row) * d + column], added
+// exactly as cols_reduce_kernel adds them (group g goes to accumulator g % 4 in ascending order, then
+// (a0 + a1) + (a2 + a3), + bias, rounded to fp16): the reduction launch folded into the LayerNorm launch.
+struct LnRowFromPartials {
+  const float* __restrict__ partial;
+  const half_t* __restrict__ bias;
+  int G, d;
+  int64_t total;  // rows * d
+  __device__ __forceinline__ half8_t operator()(int i, int64_t row) const {
+    const float* p = partial + row * d + i * 8;
+    float a[4][8];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) a[k][e] = 0.f;
+    for (int g0 = 0; g0 < G; g0 += 4) {
+      float4_t lo[4], hi[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {  // groups past G re-read the last one and are not added
+        const int g = g0 + k < G ? g0 + k : G - 1;
+        lo[k] = *reinterpret_cast<const float4_t*>(p + (int64_t)g * total);
+        hi[k] = *reinterpret_cast<const float4_t*>(p + (int64_t)g * total + 4);
+      }
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        if (g0 + k < G) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            a[k][e] += lo[k][e];
+            a[k][4 + e] += hi[k][e];
+          }
+        }
+      }
+    }
+    const half8_t bv = bias != nullptr ? load8(bias + i * 8) : zero8();
+    half8_t y;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float r = (a[0][e] + a[1][e]) + (a[2][e] + a[3][e]);
+      y[e] = (half_t)(r + (bias != nullptr ? (float)bv[e] : 0.f));
+    }
+    return y;
+  }
+};
+
+template <int THREADS, int NV, class AfterLoads = LnNoHook, class Src = LnRowFromMemory>
+__device__ __forceinline__ void add_layer_norm_src_body(
+    Src src, const half_t* __restrict__ R, const half_t* __restrict__ gamma,
     const half_t* __restrict__ beta, float eps, int d, half_t* __restrict__ Y,
     half_t* __restrict__ Rout, half_t* __restrict__ Y2, int64_t row, AfterLoads after_loads = AfterLoads()) {
   __shared__ float2 s_parts[kLnMaxParts];
@@ -157,8 +208,8 @@ __device__ __forceinline__ void add_layer_norm_body(
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
     const int i = threadIdx.x + j * THREADS;
-    v[j] = i < nvec ? load8(H + row * d + i * 8) : zero8();
     rr[j] = (R != nullptr && i < nvec) ? load8(R + row * d + i * 8) : zero8();
+    v[j] = i < nvec ? src(i, row) : zero8();
   }
   after_loads();
   if (EARLY) {
@@ -194,6 +245,15 @@ __device__ __forceinline__ void add_layer_norm_body(
       if (Y2 != nullptr) store8(Y2 + row * d + i * 8, o);
     }
   }
+}
+
+template <int THREADS, int NV, class AfterLoads = LnNoHook>
+__device__ __forceinline__ void add_layer_norm_body(
+    const half_t* __restrict__ H, const half_t* __restrict__ R, const half_t* __restrict__ gamma,
+    const half_t* __restrict__ beta, float eps, int d, half_t* __restrict__ Y,
+    half_t* __restrict__ Rout, half_t* __restrict__ Y2, int64_t row, AfterLoads after_loads = AfterLoads()) {
+  add_layer_norm_src_body<THREADS, NV, AfterLoads, LnRowFromMemory>(LnRowFromMemory{H, d}, R, gamma, beta, eps, d, Y,
+                                                                     Rout, Y2, row, after_loads);
 }
 
 // The same for a row that arrives as fixed-point sums (common.hpp: to_fixed): by a whole workgroup
@@ -292,6 +352,16 @@ __global__ __launch_bounds__(THREADS) void add_layer_norm_kernel(
     const half_t* __restrict__ beta, float eps, int d, half_t* __restrict__ Y,
     half_t* __restrict__ Rout, half_t* __restrict__ Y2 = nullptr) {
   add_layer_norm_body<THREADS, NV>(H, R, gamma, beta, eps, d, Y, Rout, Y2, blockIdx.x);
+}
+
+// add + LayerNorm of rows that arrive as the fp32 partial sums of a split product (LnRowFromPartials)
+template <int THREADS, int NV>
+__global__ __launch_bounds__(THREADS) void reduce_add_layer_norm_kernel(
+    const float* __restrict__ partial, const half_t* __restrict__ bias, int G, int rows,
+    const half_t* __restrict__ R, const half_t* __restrict__ gamma, const half_t* __restrict__ beta, float eps,
+    int d, half_t* __restrict__ Y, half_t* __restrict__ Rout) {
+  add_layer_norm_src_body<THREADS, NV, LnNoHook, LnRowFromPartials>(
+      LnRowFromPartials{partial, bias, G, d, (int64_t)rows * d}, R, gamma, beta, eps, d, Y, Rout, nullptr, blockIdx.x);
 }
 
 }  // namespace dv

@@ -434,7 +434,7 @@ class _MHABase(nn.Module):
         the neuron selection of that forward.  The head selection (for the next layer) stays pending:
         whoever uses it calls ``join_heads()`` first (the blocks do at their start;
         ``join_side_stream()`` covers it too)."""
-        if not self._side_used:
+        if not self._side_used or getattr(self, "_joined", False):
             return
         if self._mlp_idx_event:
             torch.cuda.current_stream().wait_event(self.event_mlp_idx)
@@ -616,12 +616,15 @@ class ParallelMHASparseAttMlp(_MHABase):
         return qkv, head_idx, kc, vc
 
     def forward(self, x, residual, head_idx=None, mlp_sp_logit=None, seqlen=None, inference_params=None, window=None,
-                defer_join=False, **kwargs):
+                defer_join=False, post_norm=None, **kwargs):
         """x, residual: (B, s, d).  head_idx: (Hk,) int32 heads to compute, or None
         for dense attention.  mlp_sp_logit: predictor logits for this layer's MLP.  window: the
         result of ``begin_window_step`` when the caller's LayerNorm launch has already done the
         window step.  defer_join: the caller calls ``join_side()`` itself before it uses mlp_idx / att_idx
-        (the block does, after LayerNorm 2, which does not need them).  Returns (out, mlp_idx, att_idx)."""
+        (the block does).  post_norm = (LayerNorm module, its residual input): the caller's residual add + LayerNorm
+        of `out`, done here when it can ride in the projection's reduction launch (batched sparse decode, five
+        rows and more); `out` is then the pair (normed, residual_out) instead of the projection.
+        Returns (out, mlp_idx, att_idx)."""
         assert seqlen is None, "sequence-parallel input layout is not used for generation"
         self._streams()
         do_token_generation = x.size(1) == 1
@@ -630,6 +633,8 @@ class ParallelMHASparseAttMlp(_MHABase):
             self.reset_window()
         sparse = inference_params is not None and inference_params.sequence_len_offset > 0 and head_idx != None
         self._side_fork(x.shape[0])
+        side_done = None
+        self._joined = False
         if sparse:
             assert x.size(1) == 1
             self.transposed_out_proj()
@@ -641,10 +646,28 @@ class ParallelMHASparseAttMlp(_MHABase):
                                              inference_params.lengths_per_sample, self.softmax_scale).unsqueeze(1)
             else:
                 qkv, head_idx, kc, vc = self._sparse_decode_batched(x, head_idx, inference_params, window)
+                # the side work right behind the QKV launch (the main chain's first launch of the module is
+                # captured, and the selections can be waited for in front of out_proj)
+                side_done = self._side_work(mlp_sp_logit, residual, self.sp if do_token_generation else None,
+                                            self.att_k, self.att_idx_out)
                 ctx = ops.single_query_attention(qkv[:, 0], None, None, kc, vc, inference_params.lengths_per_sample,
                                                  inference_params.sequence_len_offset, self.rotary_emb_dim,
                                                  head_idx=head_idx, softmax_scale=self.softmax_scale)
-                out = ops.out_proj_sparse_t(ctx, self.out_proj_weight_t, head_idx, self.out_proj.bias).unsqueeze(1)
+                if post_norm is not None and x.size(0) >= ops.OUT_PROJ_LN_MIN_ROWS:
+                    # the caller's residual add + LayerNorm ride in the projection's reduction launch; the
+                    # wait for the neuron selection, which the caller would place in front of its LayerNorm,
+                    # goes in front of the projection
+                    if defer_join:
+                        self.join_side()
+                        defer_join = None  # joined
+                    norm, norm_residual = post_norm
+                    out = ops.out_proj_sparse_t_add_layer_norm(ctx, self.out_proj_weight_t, head_idx,
+                                                               self.out_proj.bias, norm_residual, norm.weight,
+                                                               norm.bias, norm.eps)
+                    out = (out[0].unsqueeze(1), out[1].view_as(norm_residual))
+                else:
+                    out = ops.out_proj_sparse_t(ctx, self.out_proj_weight_t, head_idx,
+                                                self.out_proj.bias).unsqueeze(1)
             if self.counter == self.WINDOW:  # window complete: start the next one
                 self.counter = 0
                 if not self.hold_window:
@@ -654,10 +677,13 @@ class ParallelMHASparseAttMlp(_MHABase):
             qkv = qkv.view(x.shape[0], x.shape[1], 3, self.num_heads, self.head_dim)
             context = self._dense_context(qkv, inference_params)
             out = decode_linear(self.out_proj, context)
-        mlp_idx, att_idx = self._side_work(mlp_sp_logit, residual, self.sp if do_token_generation else None,
-                                           self.att_k, self.att_idx_out)
-        if defer_join:
-            self._side_keep = (residual, mlp_sp_logit)  # read by the side work until join_side()
+        if side_done is None:
+            side_done = self._side_work(mlp_sp_logit, residual, self.sp if do_token_generation else None,
+                                        self.att_k, self.att_idx_out)
+        mlp_idx, att_idx = side_done
+        if defer_join or defer_join is None:
+            self._side_keep = (residual, mlp_sp_logit)  # read by the side work until the next step
+            self._joined = defer_join is None
         else:
             self._join_side()
         return out, mlp_idx, att_idx

@@ -554,6 +554,43 @@ def out_proj_sparse_t(x: torch.Tensor, weight_t: torch.Tensor, head_idx: torch.T
     return output
 
 
+OUT_PROJ_LN_MIN_ROWS = 5  # the matrix-core path of out_proj_sparse_t
+
+
+def out_proj_sparse_t_add_layer_norm(x: torch.Tensor, weight_t: torch.Tensor, head_idx: torch.Tensor,
+                                     bias: Optional[torch.Tensor], residual: Optional[torch.Tensor],
+                                     ln_weight: torch.Tensor, ln_bias: torch.Tensor, eps: float):
+    """``add_layer_norm(out_proj_sparse_t(x, ...), residual, ...)`` for 5..64 rows with the split
+    reduction of the projection and the LayerNorm in one launch.  Returns (normed, residual_out), both
+    (batch, hidden_dim); same bits as the two ops."""
+    _require_device(x, weight_t, head_idx, bias, residual, ln_weight, ln_bias)
+    batch, nheads, head_dim = x.shape
+    rows, hidden_dim = weight_t.shape
+    assert rows == nheads * head_dim and head_idx.dtype == torch.int32
+    assert OUT_PROJ_LN_MIN_ROWS <= batch <= 64
+    assert x.dtype == weight_t.dtype == ln_weight.dtype == ln_bias.dtype == torch.float16
+    n_active = head_idx.shape[0]
+    x = x.contiguous()
+    if weight_t.stride(1) != 1:
+        weight_t = weight_t.contiguous()
+    if bias is not None:
+        bias = bias.contiguous()
+    if residual is not None:
+        residual = residual.contiguous()
+        assert residual.numel() == batch * hidden_dim and residual.dtype == torch.float16
+    head_idx = head_idx.contiguous()
+    normed = torch.empty(batch, hidden_dim, device=x.device, dtype=x.dtype)
+    r_out = torch.empty(batch, hidden_dim, device=x.device, dtype=x.dtype)
+    nbytes = lib.dv_out_proj_sparse_t_ln_workspace_bytes(batch, n_active, head_dim, hidden_dim)
+    ws = _workspace(x.device, nbytes)
+    check(lib.dv_out_proj_sparse_t_ln_f16(_ptr(x), _ptr(weight_t), weight_t.stride(0), _ptr(bias), _ptr(head_idx),
+                                          n_active, batch, nheads, head_dim, hidden_dim, _ptr(residual),
+                                          _ptr(ln_weight.contiguous()), _ptr(ln_bias.contiguous()), float(eps),
+                                          _ptr(normed), _ptr(r_out), _ptr(ws), ws.numel(), _stream()),
+          "dv_out_proj_sparse_t_ln_f16")
+    return normed, r_out
+
+
 def _cache_copy(k, v, k_cache, v_cache, head_idx, seqlen_idx, padding):
     src = k if k is not None else v
     _require_device(src, k_cache, v_cache, head_idx, seqlen_idx, padding)

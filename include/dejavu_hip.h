@@ -392,6 +392,22 @@ DV_API int dv_out_proj_sparse_t_f16(const void* x, const void* Wt, int64_t ldw, 
                                     void* stream);
 
 /*
+ * dv_out_proj_sparse_t_f16 for 5..64 rows followed by the block's residual add + LayerNorm 2
+ * (dv_add_layer_norm_f16 with h = the projection's output) with the split reduction and the LayerNorm
+ * in ONE launch: normed = LayerNorm(fp16(y + residual)) * gamma + beta, residual_out = fp16(y + residual);
+ * y itself is not returned.  Same bits as the two calls (attention_proj_sparse.py:194-305 +
+ * block_dejavu.py:626-634).
+ *   residual (B, N) or NULL; normed, residual_out (B, N), residual_out may be NULL; N <= 32768;
+ *   workspace: dv_out_proj_sparse_t_ln_workspace_bytes(...) bytes, 16-byte aligned.
+ */
+DV_API size_t dv_out_proj_sparse_t_ln_workspace_bytes(int B, int nnz, int hd, int N);
+DV_API int dv_out_proj_sparse_t_ln_f16(const void* x, const void* Wt, int64_t ldw, const void* bias,
+                                       const void* head_idx, int nnz, int B, int H, int hd, int N,
+                                       const void* residual, const void* gamma, const void* beta,
+                                       float eps, void* normed, void* residual_out, void* workspace,
+                                       size_t workspace_bytes, void* stream);
+
+/*
  * The two halves of that add + LayerNorm when the LayerNorm is applied by the consumer of the
  * row (the same reference lines, block_dejavu.py:575-584):
  *   dv_add_ln_parts_f16: r_out = fp16(h + residual) (h alone when residual is NULL) and, for

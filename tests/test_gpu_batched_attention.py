@@ -380,7 +380,8 @@ def test_batched_block_step_same_bits_with_and_without_the_side_stream():
 
 
 # switches that fold launches of the batched layer step; each must leave every bit where it was
-_FOLD_SWITCHES = [("dejavu_amd.block", "FOLD_WINDOW_STEP"), ("dejavu_amd.block", "LAZY_SIDE_JOIN")]
+_FOLD_SWITCHES = [("dejavu_amd.block", "FOLD_WINDOW_STEP"), ("dejavu_amd.block", "LAZY_SIDE_JOIN"),
+                  ("dejavu_amd.block", "FOLD_NORM2")]
 
 
 @pytest.mark.parametrize("module_name,flag", _FOLD_SWITCHES)
