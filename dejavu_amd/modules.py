@@ -345,6 +345,7 @@ class _MHABase(nn.Module):
         self._forked = False
         self._side_keep = None
         self._mlp_idx_event = False
+        self._joined = False
 
     def _streams(self):
         if self.sp_stream is None:
@@ -434,7 +435,7 @@ class _MHABase(nn.Module):
         the neuron selection of that forward.  The head selection (for the next layer) stays pending:
         whoever uses it calls ``join_heads()`` first (the blocks do at their start;
         ``join_side_stream()`` covers it too)."""
-        if not self._side_used or getattr(self, "_joined", False):
+        if not self._side_used or self._joined:
             return
         if self._mlp_idx_event:
             torch.cuda.current_stream().wait_event(self.event_mlp_idx)
@@ -634,6 +635,7 @@ class ParallelMHASparseAttMlp(_MHABase):
         sparse = inference_params is not None and inference_params.sequence_len_offset > 0 and head_idx != None
         self._side_fork(x.shape[0])
         side_done = None
+        joined_early = False
         self._joined = False
         if sparse:
             assert x.size(1) == 1
@@ -659,7 +661,7 @@ class ParallelMHASparseAttMlp(_MHABase):
                     # goes in front of the projection
                     if defer_join:
                         self.join_side()
-                        defer_join = None  # joined
+                        joined_early = True
                     norm, norm_residual = post_norm
                     out = ops.out_proj_sparse_t_add_layer_norm(ctx, self.out_proj_weight_t, head_idx,
                                                                self.out_proj.bias, norm_residual, norm.weight,
@@ -681,9 +683,9 @@ class ParallelMHASparseAttMlp(_MHABase):
             side_done = self._side_work(mlp_sp_logit, residual, self.sp if do_token_generation else None,
                                         self.att_k, self.att_idx_out)
         mlp_idx, att_idx = side_done
-        if defer_join or defer_join is None:
+        if defer_join:
             self._side_keep = (residual, mlp_sp_logit)  # read by the side work until the next step
-            self._joined = defer_join is None
+            self._joined = joined_early  # the caller's join_side() then has nothing left to do
         else:
             self._join_side()
         return out, mlp_idx, att_idx
