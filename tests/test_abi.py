@@ -67,6 +67,19 @@ def test_host_side_argument_checks_return_codes():
     assert L.dv_gather_transposed_gemv_static_f16(A, A, 8, None, A, 8, 1, 8, 8, 4, A + 2, None) in (-3, -2)  # y (or no GPU)
     assert L.dv_out_proj_sparse_t_f16(A, A, 128, None, A, 1, 1, 1, 128, 128, A + 2, A, 1 << 20, None) == -3  # y
     assert L.dv_out_proj_sparse_t_f16(A, A, 128, None, A, 1, 8, 1, 128, 128, A, A + 8, 1 << 20, None) == -3  # workspace
+    # the two LayerNorm entry points that fold a neighbouring launch
+    #   (h, residual, gamma, beta, eps, rows, d, y, residual_out, x_cache_row, tracker, head_idx, nnz, H, counter,
+    #    flush, batch_idx, stream)
+    assert L.dv_add_layer_norm_window_f16(A, None, A, A, 1e-5, 2, 128, A, A, A, A, A, 1, 4, 16, 0, A, None) == -1  # counter
+    assert L.dv_add_layer_norm_window_f16(A, None, A, A, 1e-5, 2, 128, A, A, None, A, A, 1, 4, 0, 0, A, None) == -1  # no row
+    assert L.dv_add_layer_norm_window_f16(A, None, A, A, 1e-5, 2, 124, A, A, A, A, A, 1, 4, 0, 0, A, None) == -3  # d % 8
+    assert L.dv_add_layer_norm_window_f16(A, None, A, A, 1e-5, 2, 128, A, A, A + 2, A, A, 1, 4, 0, 0, A, None) == -3
+    #   (x, Wt, ldw, bias, head_idx, nnz, B, H, hd, N, residual, gamma, beta, eps, normed, residual_out, ws, bytes, stream)
+    assert L.dv_out_proj_sparse_t_ln_f16(A, A, 128, None, A, 1, 4, 1, 128, 128, A, A, A, 1e-5, A, A, A, 1 << 20, None) == -2
+    assert L.dv_out_proj_sparse_t_ln_f16(A, A, 128, None, A, 1, 8, 1, 128, 128, A, A, A, 1e-5, A + 2, A, A, 1 << 20, None) == -3
+    assert L.dv_out_proj_sparse_t_ln_f16(A, A, 128, None, A, 1, 8, 1, 128, 128, A, A, A, 1e-5, A, A, A, 16, None) == -4
+    assert L.dv_out_proj_sparse_t_ln_workspace_bytes(4, 1, 128, 128) == 0
+    assert L.dv_out_proj_sparse_t_ln_workspace_bytes(8, 32, 128, 12288) >= 8 * 12288 * 2
     for fn in (L.dv_qkv_proj_batch_f16, L.dv_qkv_window_batch_f16):
         if fn is L.dv_qkv_window_batch_f16:  # (.., nnz, tokens, nseq, d, H, hd, y, ...)
             args_y = [A, 128, A, None, A, A, 1, 2, 2, 128, 1, 128, A + 2, A, A, None, 0, 0, 16, A, 1 << 20, None]

@@ -436,3 +436,62 @@ def test_batched_block_step_same_bits_with_and_without_folded_launches(module_na
             assert torch.equal(xa, xb), f"step {step} differs"
     for ca, cb in zip(results[0][1], results[1][1]):
         assert torch.equal(ca, cb)
+
+
+@pytest.mark.parametrize("B,H,hd,d,nnz", [(5, 8, 128, 1024, 3), (16, 6, 64, 520, 1), (32, 12, 128, 1536, 12),
+                                          (33, 4, 64, 256, 2), (9, 96, 128, 12288, 32)])
+def test_out_proj_with_layer_norm_in_the_reduction_launch_same_bits(B, H, hd, d, nnz):
+    """dv_out_proj_sparse_t_ln_f16 (split reduction + residual add + LayerNorm in one launch) against
+    out_proj_sparse_t followed by add_layer_norm: both outputs bit for bit.  Shapes with one and with
+    several row groups, both matrix-core kernels (up to 32 rows, above), with and without a residual."""
+    from dejavu_amd import ops
+
+    g = torch.Generator().manual_seed(B * 100 + nnz)
+    ctx = randh(g, B, H, hd).cuda()
+    Wt = randh(g, H * hd, d, std=0.05).cuda()
+    bias = randh(g, d, std=0.1).cuda()
+    res = randh(g, B, d).cuda()
+    gamma, beta = (1 + 0.1 * torch.randn(d, generator=g)).half().cuda(), randh(g, d, std=0.1).cuda()
+    head_idx = torch.sort(torch.randperm(H, generator=g)[:nnz]).values.int().cuda()
+    print(f"case out_proj + LayerNorm B={B} H={H} hd={hd} d={d} nnz={nnz}", flush=True)
+    for residual in (res, None):
+        y = ops.out_proj_sparse_t(ctx, Wt, head_idx, bias)
+        want_n, want_r = ops.add_layer_norm(y, residual, gamma, beta, 1e-5)
+        got_n, got_r = ops.out_proj_sparse_t_add_layer_norm(ctx, Wt, head_idx, bias, residual, gamma, beta, 1e-5)
+        torch.cuda.synchronize()
+        assert torch.equal(got_r, want_r), "residual stream differs"
+        assert torch.equal(got_n, want_n), "normalised rows differ"
+
+
+@pytest.mark.parametrize("B,d,H,nnz", [(2, 256, 4, 2), (8, 1024, 8, 3), (32, 12288, 96, 32)])
+def test_layer_norm_with_the_window_step_in_the_same_launch_same_results(B, d, H, nnz):
+    """dv_add_layer_norm_window_f16 against add_layer_norm followed by dv_window_step_f16 over a whole window
+    (flush position included): normalised rows, residual stream, window buffer, tracker and slot lists."""
+    from dejavu_amd import ops
+    from dejavu_amd._lib import check, lib
+
+    g = torch.Generator().manual_seed(B + d)
+    gamma, beta = (1 + 0.1 * torch.randn(d, generator=g)).half().cuda(), randh(g, d, std=0.1).cuda()
+    state = []
+    for _ in range(2):
+        state.append({"x_cache": torch.zeros(16, B * d, dtype=torch.float16, device="cuda"),
+                      "tracker": torch.arange(16, dtype=torch.int32).repeat(H, 1).cuda()})
+    all_heads = torch.arange(H, dtype=torch.int32, device="cuda")
+    for counter in range(16):
+        h, r = randh(g, B, 1, d).cuda(), randh(g, B, 1, d).cuda()
+        flush = counter == 15
+        heads = all_heads if flush else torch.sort(torch.randperm(H, generator=g)[:nnz]).values.int().cuda()
+        print(f"case LayerNorm + window step B={B} d={d} position {counter}", flush=True)
+        a, b = state
+        idx_a = torch.full((heads.shape[0], counter + 1), -7, dtype=torch.int32, device="cuda")
+        idx_b = idx_a.clone()
+        n_a, r_a = ops.add_layer_norm_window(h, r, gamma, beta, 1e-5, a["x_cache"][counter], a["tracker"], heads,
+                                             counter, flush, idx_a)
+        n_b, r_b = ops.add_layer_norm(h, r, gamma, beta, 1e-5)
+        check(lib.dv_window_step_f16(n_b.data_ptr(), b["x_cache"].data_ptr(), B * d, b["tracker"].data_ptr(),
+                                     heads.data_ptr(), heads.shape[0], H, counter, int(flush), idx_b.data_ptr(),
+                                     torch.cuda.current_stream().cuda_stream), "dv_window_step_f16")
+        torch.cuda.synchronize()
+        assert torch.equal(n_a, n_b) and torch.equal(r_a, r_b)
+        assert torch.equal(a["x_cache"], b["x_cache"]) and torch.equal(a["tracker"], b["tracker"])
+        assert torch.equal(idx_a, idx_b)
