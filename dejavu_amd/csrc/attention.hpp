@@ -509,6 +509,110 @@ __global__ __launch_bounds__(WAVES * 64) void decode_attn_kernel(
                               blockIdx.x, blockIdx.y, blockIdx.z, gridDim.y);
 }
 
+// ---------------------------------------------------------------------------
+// One-query attention for MANY (sequence, head) pairs (a batch of sequences: B * heads pairs fill
+// the device by themselves): ONE workgroup of sixteen wavefronts per pair walks all cached
+// positions, 1024 per turn (a wavefront its 64, as in decode_attn_body: lanes map to positions for
+// q.K and to (row, 8-wide slice) for p.V, all K and V loads of a turn issued before its
+// arithmetic), keeps a running maximum / sum / un-normalised output per wavefront (online softmax:
+// the output is rescaled by exp(old max - new max), a wavefront-uniform factor, so the sums over the
+// V rows stay spread over the lanes until the end), merges the sixteen wavefronts in LDS and writes
+// the normalised fp16 result.  No partial results in memory and no combine launch.
+// Grid (heads, B).  lengths as in decode_attn_body.
+// ---------------------------------------------------------------------------
+constexpr int kAttnRowWaves = 16;
+
+template <int HD>
+__global__ __launch_bounds__(kAttnRowWaves * 64) void decode_attn_rows_kernel(
+    const half_t* __restrict__ Q, int64_t ldq, const half_t* __restrict__ k_cache,
+    const half_t* __restrict__ v_cache, const int* __restrict__ head_idx, const int* __restrict__ lengths,
+    int n_len, int H, int S, float scale, half_t* __restrict__ out, int64_t ldo) {
+  constexpr int WAVES = kAttnRowWaves;
+  constexpr int PK = HD / 8;        // 16-byte packets per position / lanes per V row
+  constexpr int RPI = kWave / PK;   // V rows per load instruction
+  constexpr int VIT = kWave / RPI;  // V load instructions per wavefront and turn (= PK)
+  __shared__ float s_m[WAVES], s_l[WAVES];
+  __shared__ float s_o[WAVES][HD];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int i = blockIdx.x, b = blockIdx.y;
+  const int h = head_idx ? head_idx[i] : i;
+  if (h < 0 || h >= H) return;  // uniform over the workgroup
+  int len = lengths ? lengths[b] + 1 : n_len;
+  if (len > S) len = S;  // a device-side length can never address past the cache
+  const int grp = lane / PK, sub = lane % PK;
+  const int64_t bh = (int64_t)b * H + h;
+  const half_t* q = Q + (int64_t)b * ldq + (int64_t)h * HD;
+  half8_t qv[PK];
+#pragma unroll
+  for (int dp = 0; dp < PK; ++dp) qv[dp] = load8(q + dp * 8);
+  float m = -INFINITY, l = 0.f;
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  for (int p0 = wave * kWave; p0 < len; p0 += WAVES * kWave) {  // uniform over the wavefront
+    const int pos = p0 + lane;
+    const bool pos_ok = pos < len;
+    const int pos_c = pos_ok ? pos : len - 1;  // clamp: always a valid address
+    half8_t kp[PK];
+    const half_t* kbase = k_cache + (bh * PK * S + pos_c) * 8;
+#pragma unroll
+    for (int dp = 0; dp < PK; ++dp) kp[dp] = load8_stream(kbase + (int64_t)dp * S * 8);
+    half8_t vv[VIT];
+#pragma unroll
+    for (int it = 0; it < VIT; ++it) {
+      int row = p0 + it * RPI + grp;
+      if (row >= len) row = len - 1;
+      vv[it] = load8_stream(v_cache + (bh * S + row) * HD + sub * 8);
+    }
+    float sc = 0.f;
+#pragma unroll
+    for (int dp = 0; dp < PK; ++dp) sc = dot8_fast(kp[dp], qv[dp], sc);
+    sc = pos_ok ? sc * scale : -INFINITY;
+    const float m_new = fmaxf(m, butterfly_max<kWave>(sc));  // finite: position p0 is inside the length
+    const float rescale = m == -INFINITY ? 0.f : __expf(m - m_new);
+    const float p = pos_ok ? __expf(sc - m_new) : 0.f;
+    l = l * rescale + butterfly_sum<kWave>(p);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] *= rescale;
+#pragma unroll
+    for (int it = 0; it < VIT; ++it) {
+      const float pr = __shfl(p, it * RPI + grp, kWave);  // 0 for positions >= len
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(pr, (float)vv[it][e], acc[e]);
+    }
+    m = m_new;
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+#pragma unroll
+    for (int off = PK; off < kWave; off <<= 1) acc[e] += __shfl_xor(acc[e], off, kWave);
+  }
+  if (lane == 0) {
+    s_m[wave] = m;
+    s_l[wave] = l;
+  }
+  if (grp == 0) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s_o[wave][sub * 8 + e] = acc[e];
+  }
+  __syncthreads();
+  // merge the wavefronts (those without a position carry max = -inf, sum = 0) and normalise
+  if (threadIdx.x < HD) {
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) M = fmaxf(M, s_m[w]);
+    float num = 0.f, den = 0.f;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+      const float sw = s_m[w] == -INFINITY ? 0.f : __expf(s_m[w] - M);
+      den += sw * s_l[w];
+      num += sw * s_o[w][threadIdx.x];
+    }
+    out[(int64_t)b * ldo + (int64_t)h * HD + threadIdx.x] = (half_t)(num / den);
+  }
+}
+
 // out[b, h, :] = sum_s o_s * exp(m_s - m) / sum_s l_s * exp(m_s - m).  Grid (heads, B), HD threads.
 template <int HD>
 __global__ __launch_bounds__(HD) void decode_attn_combine_kernel(

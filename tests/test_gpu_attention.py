@@ -182,7 +182,11 @@ def test_cache_copy_sparse_bit_exact(ops, hd):
 
 # ------------------------------------------------------ decode attention
 @pytest.mark.parametrize("B,H,hd,S,t,nsel", [(1, 12, 128, 256, 200, 4), (2, 8, 64, 100, 99, 3), (1, 96, 128, 2048, 2047, 32),
-                                             (3, 4, 128, 70, 0, 4), (1, 6, 128, 130, 64, 2), (2, 16, 32, 300, 270, 5)])
+                                             (3, 4, 128, 70, 0, 4), (1, 6, 128, 130, 64, 2), (2, 16, 32, 300, 270, 5),
+                                             # two and more (sequence, head) pairs per compute unit: one
+                                             # workgroup per pair walks the whole sequence
+                                             (16, 40, 128, 1300, 1290, 33), (24, 24, 64, 1100, 1030, 24),
+                                             (40, 16, 32, 90, 17, 13), (32, 16, 128, 1500, 0, 16)])
 def test_single_query_attention(ops, B, H, hd, S, t, nsel):
     g = torch.Generator().manual_seed(4)
     q, k, v = (randh(g, B, H, hd) for _ in range(3))
@@ -218,16 +222,18 @@ def test_single_query_attention(ops, B, H, hd, S, t, nsel):
     assert torch.equal(out_na, out_all)
 
 
-def test_single_query_attention_lengths_per_sample(ops):
+@pytest.mark.parametrize("B,H", [(3, 4), (36, 16)])
+def test_single_query_attention_lengths_per_sample(ops, B, H):
     g = torch.Generator().manual_seed(5)
-    B, H, hd, S = 3, 4, 128, 160
+    hd, S = 128, 160
     q, k, v = (randh(g, B, H, hd) for _ in range(3))
     kc = randh(g, B, H, S, hd)
     vc = randh(g, B, H, S, hd)
     from dejavu_amd.workloads import pack_k_cache
 
     k_cache = pack_k_cache(kc)
-    lengths = torch.tensor([5, 159, 64], dtype=torch.int32)
+    lengths = torch.tensor([5, 159, 64] + [int(v) for v in torch.randint(0, 160, (B - 3,), generator=g)],
+                           dtype=torch.int32)
     kcd, vcd = k_cache.cuda(), vc.cuda()
     out = ops.single_query_attention(q.cuda(), k.cuda(), v.cuda(), kcd, vcd, lengths.cuda(), 159)
     torch.cuda.synchronize()
