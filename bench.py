@@ -211,10 +211,12 @@ def layer_step_inputs(L):
     return L["att_idx_in"], L["mlp_logit_in"]
 
 
-def layer_step(L):
-    """One decode step of one block at the first position of a back-fill window."""
+def layer_step(L, stream_in=None):
+    """One decode step of one block at the first position of a back-fill window.  stream_in: the
+    (hidden_states, residual) of the step before (default: the layer's own fixed inputs)."""
     head_idx, logit = layer_step_inputs(L)
-    return L["block"](L["hidden"], L["residual"], mixer_kwargs={"inference_params": L["ip"]},
+    hidden, residual = stream_in if stream_in is not None else (L["hidden"], L["residual"])
+    return L["block"](hidden, residual, mixer_kwargs={"inference_params": L["ip"]},
                       head_idx=head_idx, mlp_sp_logit=logit)
 
 
@@ -233,9 +235,10 @@ def window_step_inputs(L, c):
     return L["heads"][c], L["mlp_logit_in"]
 
 
-def window_step(L, c):
+def window_step(L, c, stream_in=None):
     head_idx, logit = window_step_inputs(L, c)
-    return L["block"](L["hidden"], L["residual"], mixer_kwargs={"inference_params": L["ip"]},
+    hidden, residual = stream_in if stream_in is not None else (L["hidden"], L["residual"])
+    return L["block"](hidden, residual, mixer_kwargs={"inference_params": L["ip"]},
                       head_idx=head_idx, mlp_sp_logit=logit)
 
 
@@ -745,8 +748,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying HIP graphs")
     ap.add_argument("--no-chain", action="store_true",
-                    help="batch 1: one dv_sparse_layer_decode_f16 call per step (seven launches, every step from the "
-                         "same fixed input) instead of chaining the steps of a graph in one call (six launches each)")
+                    help="every step from the same fixed input instead of the residual stream of the step before "
+                         "(batch 1: one dv_sparse_layer_decode_f16 call per step, seven launches, instead of one "
+                         "call per graph, six launches each; batches: fc2 keeps its reduction launch)")
     ap.add_argument("--side-stream", action="store_true",
                     help="module path: predictors / top-k on a side stream, as the reference's sp_stream (slower here)")
     ap.add_argument("--pmc-calibration", action="store_true",
@@ -820,23 +824,34 @@ def main():
     cycle = args.window == "cycle"
     period = N_LAYERS * (WINDOW if cycle else 1)
 
-    def step_fn(i):
+    def step_fn(i, stream_in=None):
         """i-th step of the repeating schedule: positions outermost, layers innermost."""
         if cycle:
             c, l = divmod(i % period, N_LAYERS)
-            return window_step(layers[l], c)
-        return layer_step(layers[i % N_LAYERS])
+            return window_step(layers[l], c, stream_in)
+        return layer_step(layers[i % N_LAYERS], stream_in)
 
-    chained = batch == 1 and not args.no_chain
+    chained = not args.no_chain
+    for L in layers:  # chained: a step's hidden_states go straight into the next step's LayerNorm 1
+        L["block"].defer_mlp_reduce = chained and batch > 1
 
     def run_steps(first, count):
-        """Enqueues steps first .. first+count-1.  Batch 1: as ONE call for consecutive blocks of a
-        model (dv_sparse_layers_decode_f16): the residual stream of a step feeds the next step, the
-        layers forming a ring, and the launch that ends a step prepares the next; the predictions a
-        step consumes are the schedule's own (heads re-drawn per position)."""
+        """Enqueues steps first .. first+count-1 as consecutive blocks of a model: the residual stream of a
+        step feeds the next step, the layers forming a ring; the predictions a step consumes are the
+        schedule's own (heads re-drawn per position).  Batch 1: ONE call (dv_sparse_layers_decode_f16), the
+        launch that ends a step prepares the next.  A batch of sequences: the blocks' own forwards, the
+        split reduction of a step's fc2 inside the next step's LayerNorm 1 launch (the last step's alone)."""
         if not chained:
             for i in range(first, first + count):
                 step_fn(i)
+            return
+        if batch > 1:
+            stream = None
+            for i in range(first, first + count):
+                out = step_fn(i, stream)
+                stream = (out[0], out[1])
+            if not torch.is_tensor(stream[0]):
+                stream[0].materialize()
             return
         from dejavu_amd.fused_layer import LayerChain
 
@@ -924,18 +939,24 @@ def main():
                 L["block"].mixer.cache_offset.fill_(cfg["S"] - 1)
                 L["offset_mode"] = "start"
         # eager warm-up: allocates workspaces, sets kernel attributes (every window position once)
+        def eager_step(i):  # a batch's step ends with its own fc2 reduction when nothing follows it
+            if batch > 1:
+                run_steps(i, 1)
+            else:
+                step_fn(i)
+
         for i in range(2 * period):
-            step_fn(i)
+            eager_step(i)
         dv_modules.join_side_stream()
         torch.cuda.synchronize()
         spread = None
         if args.no_graph:
             for i in range(args.warmup):
-                step_fn(i)
+                eager_step(i)
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             for i in range(args.warmup, args.warmup + args.steps):
-                step_fn(i)
+                eager_step(i)
             torch.cuda.synchronize()
             us_per_layer = (time.perf_counter() - t0) / args.steps * 1e6
             graph_mode = "none"
@@ -972,7 +993,7 @@ def main():
                 L["block"].mixer.cache_offset.fill_(cfg["S"] - 1)
                 L["offset_mode"] = "start"
             for i in range(N_LAYERS):
-                step_fn(i)
+                eager_step(i)
             torch.cuda.synchronize()
             window_start_us = run_timed(0, MAX_GRAPH_STEPS, 5 * MAX_GRAPH_STEPS)
             cycle, period, graphs = True, period_saved, graphs_saved
@@ -1061,9 +1082,11 @@ def main():
                    "layers_cycled": N_LAYERS, "window": args.window, "hip_graph": graph_mode,
                    "entry_point": ("dv_sparse_layers_decode_f16: the steps of a graph are consecutive blocks of one "
                                    "call, the residual stream of a step feeds the next (six launches per step)"
-                                   if chained and not args.no_graph else
+                                   if chained and batch == 1 and not args.no_graph else
                                    "dv_sparse_layer_decode_f16 per step (seven launches)" if batch == 1 else
-                                   "module path")},
+                                   "module path, the steps of a graph consecutive blocks (the residual stream of a "
+                                   "step feeds the next, fc2's reduction inside the next LayerNorm 1 launch)"
+                                   if chained else "module path, every step from the same fixed input")},
         "positions": {"steps_per_window_position": positions, "schedule_period": period},
         "roofline": roofline,
         "mlp_pair": table["mlp_pair"],

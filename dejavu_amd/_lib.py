@@ -111,6 +111,14 @@ SIGNATURES = {
     "dv_add_layer_norm_window_f16": (
         _c_int, [_c_ptr, _c_ptr, _c_ptr, _c_ptr, ctypes.c_float, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                  _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr]),
+    "dv_gather_transposed_gemv_partial_workspace_bytes": (_c_size, [_c_int, _c_int, _c_int]),
+    "dv_gather_transposed_gemv_partial_f16": (
+        _c_int, [_c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr,
+                 _c_size, ctypes.POINTER(ctypes.c_int), _c_ptr]),
+    "dv_reduce_rows_f16": (_c_int, [_c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr]),
+    "dv_reduce_add_layer_norm_window_f16": (
+        _c_int, [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, ctypes.c_float, _c_int, _c_int, _c_ptr,
+                 _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr]),
     "dv_window_step_f16": (
         _c_int, [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr]),
     "dv_kv_append_f16": (

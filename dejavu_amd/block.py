@@ -37,10 +37,15 @@ LAZY_SIDE_JOIN = True
 # Batched sparse decode: the split reduction of out_proj, the residual add and LayerNorm 2 in one launch
 # (ops.out_proj_sparse_t_add_layer_norm).  False: out_proj with its reduction launch, then add_layer_norm.
 FOLD_NORM2 = True
+# Batched sparse decode, blocks with ``defer_mlp_reduce`` set (whoever sets it consumes the block's
+# hidden_states with ops.add_layer_norm / add_layer_norm_window, as the next block and the model's
+# final LayerNorm do): the split reduction of fc2 is left to that LayerNorm's launch; the block
+# returns ops.PendingRows as hidden_states.  False: fc2 with its reduction launch.
+FOLD_NORM1 = True
 
 
 def _add_norm(norm: nn.LayerNorm, hidden_states: Tensor, residual: Optional[Tensor]):
-    if hidden_states.is_cuda and hidden_states.dtype == torch.float16:
+    if isinstance(hidden_states, ops.PendingRows) or (hidden_states.is_cuda and hidden_states.dtype == torch.float16):
         return ops.add_layer_norm(hidden_states, residual, norm.weight, norm.bias, norm.eps)
     residual = hidden_states + residual if residual is not None else hidden_states
     return norm(residual.to(dtype=norm.weight.dtype)), residual
@@ -73,10 +78,12 @@ class BlockMlpAttSparse(nn.Module):
         # ordinary head-sparse decode steps run as one fused call (seven launches); set to
         # False to always go through the modules' own forwards
         self.use_fused_layer = True
+        # set by a caller that hands hidden_states straight to the next add + LayerNorm (FOLD_NORM1)
+        self.defer_mlp_reduce = False
 
     def forward(self, hidden_states: Tensor, residual: Optional[Tensor] = None, mixer_subset=None,
                 mixer_kwargs=None, head_idx=None, mlp_sp_logit=None):
-        """hidden_states: output of the previous block's MLP; residual: its
+        """hidden_states: output of the previous block's MLP (or its ops.PendingRows); residual: its
         residual stream (None for the first block).  Returns
         (hidden_states, residual, next_mlp_sp_logit, next_att_idx)."""
         assert mixer_subset is None
@@ -101,7 +108,9 @@ class BlockMlpAttSparse(nn.Module):
             hidden_states, residual = hidden_states
         else:
             hidden_states, residual = _add_norm(self.norm2, hidden_states, residual)
-        hidden_states, next_mlp_sp_logit = self.mlp(hidden_states, residual, mlp_idx, defer_join=lazy)
+        hidden_states, next_mlp_sp_logit = self.mlp(
+            hidden_states, residual, mlp_idx, defer_join=lazy,
+            defer_reduce=FOLD_NORM1 and self.defer_mlp_reduce and window is not None)
         return hidden_states, residual, next_mlp_sp_logit, next_att_idx
 
 

@@ -383,6 +383,24 @@ __global__ __launch_bounds__(THREADS) void add_layer_norm_window_kernel(
   add_layer_norm_body<THREADS, NV>(Hin, R, gamma, beta, eps, d, Y, Rout, x_cache_row, blockIdx.x);
 }
 
+// The same for rows that arrive as the fp32 partial sums of a split product (the fc2 of the block
+// before: its reduction, the residual add, LayerNorm 1 and the window step are one launch).
+// tracker == nullptr: no window step (launch `rows` workgroups), x_cache_row may be nullptr.
+template <int THREADS, int NV>
+__global__ __launch_bounds__(THREADS) void reduce_add_layer_norm_window_kernel(
+    const float* __restrict__ partial, const half_t* __restrict__ bias, int G, const half_t* __restrict__ R,
+    const half_t* __restrict__ gamma, const half_t* __restrict__ beta, float eps, int d, half_t* __restrict__ Y,
+    half_t* __restrict__ Rout, half_t* __restrict__ x_cache_row, int rows, int* __restrict__ tracker,
+    const int* __restrict__ head_idx, int nnz, int H, int counter, int flush, int* __restrict__ batch_idx) {
+  if ((int)blockIdx.x == rows) {
+    window_tracker_step(tracker, head_idx, nnz, H, counter, flush, batch_idx);
+    return;
+  }
+  add_layer_norm_src_body<THREADS, NV, LnNoHook, LnRowFromPartials>(
+      LnRowFromPartials{partial, bias, G, d, (int64_t)rows * d}, R, gamma, beta, eps, d, Y, Rout, x_cache_row,
+      blockIdx.x);
+}
+
 // Appends the newest token: for every batch row b and head (all, or head_idx):
 //   k_cache[b, h, :, pos_b, :] = K[b, h, :],  v_cache[b, h, pos_b, :] = V[b, h, :]
 // with pos_b = lengths[b] if lengths else pos.  K / V: (B, H, hd) with batch

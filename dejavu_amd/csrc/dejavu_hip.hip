@@ -642,10 +642,14 @@ ColsMfmaPlan plan_cols_mfma(int B, int N, int M) {
 }
 
 // plan of gather_cols_mfma16_kernel (batch <= 32): 128 columns per workgroup of 4 wavefronts whose shares
-// are whole double steps (64 rows).  One batch tile: about three workgroups per compute unit (fc2 at the
-// OPT-175B shape, batch 8: 22.7 us with 8 row groups, 24.4 with 4, 24.2 with 2; the 32x32x16 kernel: 26.7);
-// two batch tiles write twice the partial sums per group: about one workgroup per compute unit
-// (batch 32: 30.6 us with 2 groups, 32.3 with 4, 33.0 with 8; the 32x32x16 kernel: 32.2).
+// are whole double steps (64 rows); as many row groups as give every compute unit at most one workgroup
+// (OPT-175B shape: 96 column tiles x 2 groups).  Alone the kernel is a little faster with more groups
+// (fc2, batch 8: 22.7 us with 8 row groups, 24.4 with 4, 24.2 with 2; the 32x32x16 kernel: 26.7), but
+// every group costs (B, N) fp32 partial sums written and read back, one workgroup per row reads all of
+// them when the reduction rides in a LayerNorm launch, and the concurrent stream's kernels find no free
+// compute unit: a whole layer step at batch 8 takes 213.3 / 217.4 / 211.7 / 234.2 us with 8 / 4 / 2 / 1 groups
+// (209.4 with 2 groups and both reductions inside LayerNorm launches), at batch 16 260.9 / 260.3 / 260.9 /
+// 288.1 us, at batch 32 350.6 us with 2 groups, 356.1 with 3 (288 workgroups: a second round), 387.6 with 1.
 struct Cols16Plan {
   int col_tiles, groups, rows_per_block, rows_per_wave;
 };
@@ -654,7 +658,7 @@ constexpr int kC16Waves = 4;
 Cols16Plan plan_cols16(int B, int N, int M) {
   Cols16Plan p;
   p.col_tiles = (N + kC16Cols - 1) / kC16Cols;
-  int groups = (B <= 16 ? 3 : 1) * compute_units() / p.col_tiles;
+  int groups = compute_units() / p.col_tiles;
   if (groups < 1) groups = 1;
   const int unit = kC16Waves * 2 * kC16Step;
   int rpb = ((M + groups - 1) / groups + unit - 1) / unit * unit;
@@ -682,11 +686,18 @@ struct LnTail {
   float eps;
   half_t* normed;
   half_t* residual_out;
+  // non-null: no reduction launch at all; the number of row groups goes here and the caller's
+  // consumer reduces (dv_reduce_add_layer_norm_window_f16, dv_reduce_rows_f16)
+  int* deferred_groups = nullptr;
 };
 
 // the reduction (groups > 1: from the partial sums; else y is complete) with or without the tail
 void launch_cols_reduce(const float* partial, const half_t* bias, int groups, int B, int N, half_t* y,
                         const LnTail* tail, hipStream_t s) {
+  if (tail != nullptr && tail->deferred_groups != nullptr) {
+    *tail->deferred_groups = groups;
+    return;
+  }
   if (tail == nullptr) {
     if (groups > 1) {
       const int64_t total = (int64_t)B * N;
@@ -981,7 +992,7 @@ int dv_topk_f16(const void* logits, int B, int n, int k, void* idx_out, int idx_
     // one pass reduces the batch to a row of column-wise maxima and takes that row's coarse histogram;
     // the selection then reads the row
     half_t* m = reinterpret_cast<half_t*>(reinterpret_cast<unsigned char*>(workspace) + topk_max_row_offset(n));
-    hipLaunchKernelGGL(topk_batch_hist_kernel, dim3(blocks), dim3(256), 0, s, lg, B, n, m, ws);
+    hipLaunchKernelGGL(topk_batch_hist_kernel, dim3(blocks), dim3(256 * topk_batch_groups(B)), 0, s, lg, B, n, m, ws);
     lg = m;
     B = 1;
   } else {
@@ -1140,6 +1151,34 @@ int dv_gather_transposed_gemv_f16(const void* x, const void* W, int64_t ldw, con
                      ldw, reinterpret_cast<const half_t*>(bias), idx, idx_bytes, 1, B, N, Z, M,
                      reinterpret_cast<half_t*>(y), workspace, workspace_bytes,
                      reinterpret_cast<hipStream_t>(stream));
+}
+
+size_t dv_gather_transposed_gemv_partial_workspace_bytes(int B, int N, int M) {
+  if (B <= kColsVecMaxBatch || B > 64 || N < 1 || M < 1) return 0;
+  return cols_mfma_workspace_bytes(B, N, M);
+}
+
+int dv_gather_transposed_gemv_partial_f16(const void* x, const void* W, int64_t ldw, const void* bias,
+                                          const void* idx, int idx_bytes, int B, int N, int Z, int M, void* y,
+                                          void* partial, size_t partial_bytes, int* groups, void* stream) {
+  if (!W || !y || !x || !idx || !groups || N <= 0 || Z <= 0 || M < 1 || !idx_ok(idx_bytes)) return DV_ERR_INVALID_ARG;
+  if (B <= kColsVecMaxBatch || B > 64) return DV_ERR_UNSUPPORTED;  // the matrix-core path of dv_gather_transposed_gemv_f16
+  if (N % 8 || ldw % 8 || ldw < N || !aligned16(W) || !aligned16(y) || (partial && !aligned16(partial)))
+    return DV_ERR_ALIGNMENT;
+  LnTail tail{};
+  tail.deferred_groups = groups;
+  return gather_cols_mfma(reinterpret_cast<const half_t*>(x), M, 0, reinterpret_cast<const half_t*>(W), ldw,
+                          reinterpret_cast<const half_t*>(bias), idx, idx_bytes, 1, B, N, Z, M,
+                          reinterpret_cast<half_t*>(y), partial, partial_bytes, reinterpret_cast<hipStream_t>(stream),
+                          &tail);
+}
+
+int dv_reduce_rows_f16(const void* partial, int groups, const void* bias, int rows, int N, void* y, void* stream) {
+  if (!y || groups < 1 || rows < 1 || N <= 0 || (groups > 1 && !partial)) return DV_ERR_INVALID_ARG;
+  if (N % 8 || !aligned16(y) || (partial && !aligned16(partial))) return DV_ERR_ALIGNMENT;
+  launch_cols_reduce(reinterpret_cast<const float*>(partial), reinterpret_cast<const half_t*>(bias), groups, rows, N,
+                     reinterpret_cast<half_t*>(y), nullptr, reinterpret_cast<hipStream_t>(stream));
+  return launch_status();
 }
 
 }  // extern "C"
@@ -1737,6 +1776,51 @@ int dv_add_layer_norm_window_f16(const void* h, const void* residual, const void
   else
     DV_LNW(1024, 4);
 #undef DV_LNW
+  return launch_status();
+}
+
+int dv_reduce_add_layer_norm_window_f16(const void* partial, int groups, const void* bias, const void* h,
+                                        const void* residual, const void* gamma, const void* beta, float eps,
+                                        int rows, int d, void* y, void* residual_out, void* x_cache_row,
+                                        void* tracker, const void* head_idx, int nnz, int H, int counter, int flush,
+                                        void* batch_idx, void* stream) {
+  if (!gamma || !beta || !y || groups < 1 || rows < 1 || d <= 0 || (groups > 1 ? !partial : !h))
+    return DV_ERR_INVALID_ARG;
+  if (tracker && (!x_cache_row || !batch_idx || H <= 0 || nnz < 0 || counter < 0 || counter > 15 ||
+                  (!flush && nnz > 0 && !head_idx)))
+    return DV_ERR_INVALID_ARG;
+  if (d % 8 || !aligned16(y) || !aligned16(gamma) || !aligned16(beta) || (partial && !aligned16(partial)) ||
+      (h && !aligned16(h)) || (x_cache_row && !aligned16(x_cache_row)) || (residual && !aligned16(residual)) ||
+      (residual_out && !aligned16(residual_out)) || (bias && !aligned16(bias)))
+    return DV_ERR_ALIGNMENT;
+  if (d > 256 * 8 * 16) return DV_ERR_UNSUPPORTED;
+  if (!tracker) x_cache_row = nullptr;  // the window row belongs to the window step
+  if (groups == 1) {  // the product stored its rows itself
+    if (tracker)
+      return dv_add_layer_norm_window_f16(h, residual, gamma, beta, eps, rows, d, y, residual_out, x_cache_row,
+                                          tracker, head_idx, nnz, H, counter, flush, batch_idx, stream);
+    return dv_add_layer_norm_f16(h, residual, gamma, beta, eps, rows, d, y, residual_out, stream);
+  }
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+#define DV_RLNW(T, V)                                                                                            \
+  hipLaunchKernelGGL((reduce_add_layer_norm_window_kernel<T, V>), dim3(rows + (tracker ? 1 : 0)), dim3(T), 0, s, \
+                     reinterpret_cast<const float*>(partial), reinterpret_cast<const half_t*>(bias), groups,     \
+                     reinterpret_cast<const half_t*>(residual), reinterpret_cast<const half_t*>(gamma),          \
+                     reinterpret_cast<const half_t*>(beta), eps, d, reinterpret_cast<half_t*>(y),                \
+                     reinterpret_cast<half_t*>(residual_out), reinterpret_cast<half_t*>(x_cache_row), rows,      \
+                     reinterpret_cast<int*>(tracker), reinterpret_cast<const int*>(head_idx), nnz, H, counter,   \
+                     flush, reinterpret_cast<int*>(batch_idx))
+  if (d <= 256 * 8 * 1)
+    DV_RLNW(256, 1);
+  else if (d <= 512 * 8 * 1)
+    DV_RLNW(512, 1);
+  else if (d <= 1024 * 8 * 1)
+    DV_RLNW(1024, 1);
+  else if (d <= 1024 * 8 * 2)
+    DV_RLNW(1024, 2);
+  else
+    DV_RLNW(1024, 4);
+#undef DV_RLNW
   return launch_status();
 }
 

@@ -275,19 +275,25 @@ __global__ __launch_bounds__(256) void topk_hist_kernel(const half_t* __restrict
 // A (B, n) batch: the column-wise "maximum" as a row of fp16 values -- m[j] = the logit of column j with
 // the largest key (among equal keys the larger bit pattern) -- and the coarse histogram of m's keys, in one
 // launch.  Top-k over m equals top-k over the batch with the maximum-over-rows score, so the count and
-// emit kernels then read one row instead of B.  Workgroup b owns columns [2048 b, 2048 (b + 1)), a thread
-// one 8-column vector of all B rows (loads in groups of eight rows).  Requires n % 8 == 0.
-__global__ __launch_bounds__(256) void topk_batch_hist_kernel(const half_t* __restrict__ logits, int B, int n,
-                                                              half_t* __restrict__ m, unsigned* __restrict__ ws) {
+// emit kernels then read one row instead of B.  Workgroup b owns columns [2048 b, 2048 (b + 1)); its
+// threads form blockDim.x / 256 groups (1..4) of 256, group q takes rows 8 q .. 8 q + 7 (then 8 more every
+// 8 * groups rows) of one 8-column vector per thread, all eight loads of a turn in flight together, and the
+// groups' maxima meet in LDS: up to 32 rows are one round trip to memory.  Requires n % 8 == 0.
+constexpr int kTopkBatchGroups = 4;
+inline int topk_batch_groups(int B) { return B > 24 ? 4 : B > 16 ? 3 : B > 8 ? 2 : 1; }
+
+__global__ __launch_bounds__(256 * kTopkBatchGroups) void topk_batch_hist_kernel(
+    const half_t* __restrict__ logits, int B, int n, half_t* __restrict__ m, unsigned* __restrict__ ws) {
   __shared__ unsigned s_coarse[kTopkBins];
-  s_coarse[threadIdx.x] = 0u;
-  __syncthreads();
-  const int i0 = (blockIdx.x * 256 + threadIdx.x) * 8;
-  if (i0 < n) {
-    unsigned best[8];
+  __shared__ unsigned s_best[kTopkBatchGroups - 1][8][256];
+  const int t = threadIdx.x & 255, q = threadIdx.x >> 8, groups = blockDim.x >> 8;
+  if (q == 0) s_coarse[t] = 0u;
+  const int i0 = (blockIdx.x * 256 + t) * 8;
+  unsigned best[8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) best[e] = 0u;
-    for (int b0 = 0; b0 < B; b0 += 8) {
+  for (int e = 0; e < 8; ++e) best[e] = 0u;  // below every packed value of a real row
+  if (i0 < n) {
+    for (int b0 = 8 * q; b0 < B; b0 += 8 * groups) {
       half8_t v[8];
 #pragma unroll
       for (int u = 0; u < 8; ++u) {  // past the batch the last row repeats (a maximum does not mind)
@@ -303,6 +309,20 @@ __global__ __launch_bounds__(256) void topk_batch_hist_kernel(const half_t* __re
           best[e] = packed > best[e] ? packed : best[e];
         }
     }
+  }
+  if (q > 0) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s_best[q - 1][e][t] = best[e];
+  }
+  __syncthreads();
+  if (q == 0 && i0 < n) {
+    for (int g = 1; g < groups; ++g) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const unsigned other = s_best[g - 1][e][t];
+        best[e] = other > best[e] ? other : best[e];
+      }
+    }
     half8_t o;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
@@ -313,7 +333,7 @@ __global__ __launch_bounds__(256) void topk_batch_hist_kernel(const half_t* __re
     store8(m + i0, o);
   }
   __syncthreads();
-  ws[blockIdx.x * kTopkBins + threadIdx.x] = s_coarse[threadIdx.x];
+  if (q == 0) ws[blockIdx.x * kTopkBins + t] = s_coarse[t];
 }
 
 // Inclusive prefix sum over the 256 threads of a workgroup (s_w: 4 words of LDS).

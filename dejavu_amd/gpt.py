@@ -147,6 +147,11 @@ class GPTModel(nn.Module):
         self.layers = nn.ModuleList([create_block(config, layer_idx=i, device=device, dtype=dtype)
                                      for i in range(config.num_hidden_layers)])
         self.ln_f = nn.LayerNorm(config.hidden_size, eps=config.layer_norm_epsilon, device=device, dtype=dtype)
+        # every block's hidden_states go straight into the next add + LayerNorm (the next block's, or ln_f):
+        # at a batched decode step the split reduction of fc2 runs in that launch
+        for layer in self.layers:
+            if hasattr(layer, "defer_mlp_reduce"):
+                layer.defer_mlp_reduce = True
         self.sparse = bool(getattr(config, "mlp_sparse", False) or getattr(config, "att_sparse", False))
         self.att_sparse = bool(getattr(config, "att_sparse", False))
         # when a list, every decode forward appends, per block, the lookahead inputs it

@@ -212,9 +212,12 @@ class ParallelFusedMLPDejavu(nn.Module):
         """fc2.weight as (hidden, out), contiguous; follows updates of fc2.weight."""
         return _transposed_copy(self, "fc2_weight_t", self.fc2.weight)
 
-    def forward(self, x, residual, idx=None, defer_join=False):
+    def forward(self, x, residual, idx=None, defer_join=False, defer_reduce=False):
         """x, residual: (B, 1, d) at decode (or (B, s, d) for the prompt).
         idx: (K,) active neurons or None for the dense MLP.
+        defer_reduce: the caller's next step is an ``ops.add_layer_norm`` / ``add_layer_norm_window`` of
+        ``out``; for 5..64 sequences ``out`` is then ``ops.PendingRows`` (the split reduction of fc2 runs
+        inside that LayerNorm launch).
         Returns (out, mlp_logit); mlp_logit, the predictor output for the next
         layer's MLP, only when decoding one token.  defer_join: when the predictor runs on the side
         stream, the current stream does not wait for it: mlp_logit is then only good for work
@@ -247,7 +250,9 @@ class ParallelFusedMLPDejavu(nn.Module):
                 mlp_logit = self.sp(residual)
                 self.sp_stream.record_event(self.event_mlp_sp)
         if idx != None:
-            out = ops.gather_transposed_gemv(h, self.transposed_fc2(), idx, self.fc2.bias).unsqueeze(1)
+            out = ops.gather_transposed_gemv(h, self.transposed_fc2(), idx, self.fc2.bias, defer_reduce=defer_reduce)
+            if not isinstance(out, ops.PendingRows):
+                out = out.unsqueeze(1)
         else:
             out = decode_linear(self.fc2, h)
         # (tensor parallel all-reduce of `out` is the identity on one GPU)

@@ -13,6 +13,7 @@ kernels are enqueued on ``torch.cuda.current_stream()``.
 """
 from __future__ import annotations
 
+import ctypes
 from typing import Optional
 
 import torch
@@ -274,14 +275,56 @@ def dense_decode_linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[to
     return y.view(*lead, weight.shape[0])
 
 
+DEFERRED_REDUCE_MIN_ROWS = 5  # the matrix-core path of gather_transposed_gemv
+
+
+class PendingRows:
+    """The (batch, 1, N) output of a transposed product whose last step -- adding up the fp32 sums of
+    its row groups -- has not run: ``add_layer_norm`` / ``add_layer_norm_window`` take it in place of
+    ``hidden`` and do that step in their own launch (the fc2 of one block and LayerNorm 1 of the
+    next).  ``materialize()`` runs the step alone and returns the tensor.  Shape queries answer as
+    the tensor would."""
+
+    def __init__(self, y: torch.Tensor, partial: torch.Tensor, groups: int, bias: Optional[torch.Tensor]):
+        self.y, self.partial, self.groups, self.bias = y, partial, groups, bias
+        self._reduced = groups == 1  # a single group stores the finished rows itself
+        self.shape = torch.Size((y.shape[0], 1, y.shape[1]))
+        self.dtype, self.device, self.is_cuda = y.dtype, y.device, True
+
+    def size(self, i: Optional[int] = None):
+        return self.shape if i is None else self.shape[i]
+
+    def dim(self) -> int:
+        return 3
+
+    def numel(self) -> int:
+        return self.y.numel()
+
+    def materialize(self) -> torch.Tensor:
+        if not self._reduced:
+            check(lib.dv_reduce_rows_f16(_ptr(self.partial), self.groups, _ptr(self.bias), self.y.shape[0],
+                                         self.y.shape[1], _ptr(self.y), _stream()), "dv_reduce_rows_f16")
+            self._reduced = True
+        return self.y.unsqueeze(1)
+
+
+def _rows_source(hidden):
+    """(partial, groups, bias, complete rows) of ``hidden`` as dv_reduce_add_layer_norm_window_f16 takes them."""
+    if hidden._reduced:
+        return None, 1, None, hidden.y
+    return hidden.partial, hidden.groups, hidden.bias, None
+
+
 def gather_transposed_gemv(x: torch.Tensor, weight: torch.Tensor, idx: torch.Tensor,
-                           bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+                           bias: Optional[torch.Tensor] = None, defer_reduce: bool = False):
     """Gathered rows of ``weight`` combined with the coefficients in ``x``:
     ``y[b, :] = sum_m x[b, m] * weight[idx[m], :] + bias`` (the fc2 of the sparse MLP over the
     transposed weight; interface of gather_gemv.py:572-636).
 
     Shapes: x (batch, M), weight (Z, N), idx (M,), bias (N,); returns (batch, N); batch 1..64.
     The split reduction has a fixed order: the result does not change from run to run.
+    defer_reduce (batch >= DEFERRED_REDUCE_MIN_ROWS): returns ``PendingRows`` instead, the reduction left
+    to the LayerNorm that consumes the rows.
     """
     _require_device(x, weight, idx, bias)
     _expect(x.dim() == 2 and weight.dim() == 2 and idx.dim() == 1 and x.shape[1] == idx.shape[0],
@@ -299,6 +342,16 @@ def gather_transposed_gemv(x: torch.Tensor, weight: torch.Tensor, idx: torch.Ten
         weight = weight.contiguous()
     idx = idx.contiguous()
     output = torch.empty(batch, N, device=x.device, dtype=x.dtype)
+    if defer_reduce and batch >= DEFERRED_REDUCE_MIN_ROWS and M >= 1:
+        # the partial sums outlive this call: a buffer of their own, not the stream's scratch
+        nbytes = lib.dv_gather_transposed_gemv_partial_workspace_bytes(batch, N, M)
+        partial = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
+        groups = ctypes.c_int(0)
+        check(lib.dv_gather_transposed_gemv_partial_f16(_ptr(x), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(idx),
+                                                        _idx_bytes(idx), batch, N, Z, M, _ptr(output), _ptr(partial),
+                                                        partial.numel(), ctypes.byref(groups), _stream()),
+              "dv_gather_transposed_gemv_partial_f16")
+        return PendingRows(output, partial, groups.value, bias)
     nbytes = lib.dv_gather_transposed_gemv_workspace_bytes(batch, N, M)
     ws = _workspace(x.device, nbytes)
     check(lib.dv_gather_transposed_gemv_f16(_ptr(x), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(idx),
@@ -748,7 +801,10 @@ def add_layer_norm(hidden: torch.Tensor, residual: Optional[torch.Tensor], weigh
     """``residual_out = hidden + residual`` (fp16) and ``LayerNorm(residual_out)``.
 
     hidden / residual: (..., d) fp16.  Returns (normed, residual_out), both shaped like hidden.
+    ``hidden`` may be ``PendingRows``: its reduction then runs in the same launch.
     """
+    if isinstance(hidden, PendingRows):
+        return _reduce_add_layer_norm(hidden, residual, weight, bias, eps, None)
     _require_device(hidden, residual, weight, bias)
     assert hidden.dtype == torch.float16 and weight.dtype == torch.float16 and bias.dtype == torch.float16
     d = hidden.shape[-1]
@@ -771,7 +827,11 @@ def add_layer_norm_window(hidden: torch.Tensor, residual: Optional[torch.Tensor]
     """``add_layer_norm`` for the rows of B sequences that share a back-fill window, with the window
     step of the same position in the same launch: the normalised rows also go to ``x_cache_row``
     ((B * d,) row ``counter`` of the window buffer) and the tracker hands out ``batch_idx``
-    ((nnz, counter + 1) int32; see ``dv_window_step_f16``).  Returns (normed, residual_out)."""
+    ((nnz, counter + 1) int32; see ``dv_window_step_f16``).  Returns (normed, residual_out).
+    ``hidden`` may be ``PendingRows``: its reduction then runs in the same launch."""
+    if isinstance(hidden, PendingRows):
+        return _reduce_add_layer_norm(hidden, residual, weight, bias, eps,
+                                      (x_cache_row, tracker, head_idx, counter, flush, batch_idx))
     _require_device(hidden, residual, weight, bias, x_cache_row, tracker, head_idx, batch_idx)
     assert hidden.dtype == torch.float16 and weight.dtype == torch.float16 and bias.dtype == torch.float16
     d = hidden.shape[-1]
@@ -793,6 +853,37 @@ def add_layer_norm_window(hidden: torch.Tensor, residual: Optional[torch.Tensor]
                                            _ptr(x_cache_row), _ptr(tracker), _ptr(head_idx), nnz, H, int(counter),
                                            int(flush), _ptr(batch_idx), _stream()),
           "dv_add_layer_norm_window_f16")
+    return y, r_out
+
+
+def _reduce_add_layer_norm(hidden: PendingRows, residual: Optional[torch.Tensor], weight: torch.Tensor,
+                           bias: torch.Tensor, eps: float, window):
+    """add_layer_norm / add_layer_norm_window of rows whose split reduction is still to run."""
+    _require_device(residual, weight, bias)
+    rows, d = hidden.y.shape
+    assert weight.dtype == torch.float16 and bias.dtype == torch.float16 and weight.shape == (d,) and bias.shape == (d,)
+    if residual is not None:
+        assert residual.numel() == rows * d and residual.dtype == torch.float16
+        residual = residual.contiguous()
+    partial, groups, pbias, complete = _rows_source(hidden)
+    y = torch.empty(rows, 1, d, dtype=torch.float16, device=hidden.device)
+    r_out = torch.empty_like(y)
+    if window is None:
+        x_cache_row = tracker = head_idx = batch_idx = None
+        nnz = H = counter = flush = 0
+    else:
+        x_cache_row, tracker, head_idx, counter, flush, batch_idx = window
+        _require_device(x_cache_row, tracker, head_idx, batch_idx)
+        assert x_cache_row.dtype == torch.float16 and x_cache_row.is_contiguous() and x_cache_row.numel() == rows * d
+        assert tracker.dtype == torch.int32 and head_idx.dtype == torch.int32 and batch_idx.dtype == torch.int32
+        assert tracker.is_contiguous() and batch_idx.is_contiguous() and head_idx.is_contiguous()
+        H, nnz = tracker.shape[0], head_idx.shape[0]
+        assert batch_idx.numel() >= nnz * (counter + 1)
+    check(lib.dv_reduce_add_layer_norm_window_f16(_ptr(partial), groups, _ptr(pbias), _ptr(complete), _ptr(residual),
+                                                  _ptr(weight.contiguous()), _ptr(bias.contiguous()), float(eps), rows,
+                                                  d, _ptr(y), _ptr(r_out), _ptr(x_cache_row), _ptr(tracker),
+                                                  _ptr(head_idx), nnz, H, int(counter), int(flush), _ptr(batch_idx),
+                                                  _stream()), "dv_reduce_add_layer_norm_window_f16")
     return y, r_out
 
 

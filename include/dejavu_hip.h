@@ -461,6 +461,37 @@ DV_API int dv_add_layer_norm_window_f16(const void* h, const void* residual, con
                                         void* batch_idx, void* stream);
 
 /*
+ * The fc2 of one block and LayerNorm 1 of the next without a reduction launch of their own, for
+ * 5..64 rows (the matrix-core path of dv_gather_transposed_gemv_f16):
+ *  - dv_gather_transposed_gemv_partial_f16 is dv_gather_transposed_gemv_f16 (gather_gemv.py:572-644)
+ *    without its last step: the fp32 sums of the row groups stay in `partial` (layout private to the
+ *    library), their number goes to *groups (host memory).  *groups == 1: there was nothing to split,
+ *    y (B, N) is complete and `partial` unused; otherwise y is not written.
+ *      partial: dv_gather_transposed_gemv_partial_workspace_bytes(B, N, M) bytes, 16-byte aligned,
+ *      left alone until one of the two consumers below has run.
+ *  - dv_reduce_rows_f16 is the last step alone: y = fp16(sum of the groups + bias); a no-op for groups == 1.
+ *  - dv_reduce_add_layer_norm_window_f16 is that step, the residual add and the LayerNorm that follow the
+ *    MLP in the next block (block_dejavu.py:575-584) and, with tracker != NULL, the window step of the
+ *    same position (dv_add_layer_norm_window_f16; mha_dejavu.py:1124-1149, 1318-1329) in ONE launch.
+ *    h: the complete rows, read instead of `partial` when groups == 1.  tracker == NULL: no window step,
+ *    x_cache_row .. batch_idx unused.  Other arguments as dv_add_layer_norm_window_f16.
+ * Same bits as dv_gather_transposed_gemv_f16 followed by dv_add_layer_norm(_window)_f16.
+ */
+DV_API size_t dv_gather_transposed_gemv_partial_workspace_bytes(int B, int N, int M);
+DV_API int dv_gather_transposed_gemv_partial_f16(const void* x, const void* W, int64_t ldw,
+                                                 const void* bias, const void* idx, int idx_bytes, int B,
+                                                 int N, int Z, int M, void* y, void* partial,
+                                                 size_t partial_bytes, int* groups, void* stream);
+DV_API int dv_reduce_rows_f16(const void* partial, int groups, const void* bias, int rows, int N,
+                              void* y, void* stream);
+DV_API int dv_reduce_add_layer_norm_window_f16(const void* partial, int groups, const void* bias,
+                                               const void* h, const void* residual, const void* gamma,
+                                               const void* beta, float eps, int rows, int d, void* y,
+                                               void* residual_out, void* x_cache_row, void* tracker,
+                                               const void* head_idx, int nnz, int H, int counter,
+                                               int flush, void* batch_idx, void* stream);
+
+/*
  * Greedy step of the generation loop (batch 1): next = argmax(logits[0 .. vocab)), first index
  * among equal values; then, all on the device so that a captured step can be replayed:
  * token[0] = next, sequences[out_index[0]++] = next, position[0]++, seq_pos[0]++ and, with

@@ -495,3 +495,109 @@ def test_layer_norm_with_the_window_step_in_the_same_launch_same_results(B, d, H
         assert torch.equal(n_a, n_b) and torch.equal(r_a, r_b)
         assert torch.equal(a["x_cache"], b["x_cache"]) and torch.equal(a["tracker"], b["tracker"])
         assert torch.equal(idx_a, idx_b)
+
+
+@pytest.mark.parametrize("B,M,N,Z", [(5, 512, 1024, 4096), (16, 200, 520, 700), (32, 4096, 12288, 49152),
+                                     (33, 96, 256, 300), (9, 24, 1024, 64)])
+def test_fc2_with_its_reduction_in_the_next_layer_norm_launch_same_bits(B, M, N, Z):
+    """gather_transposed_gemv(defer_reduce=True) and its three consumers against the plain op: the
+    reduction alone (materialize), add + LayerNorm, add + LayerNorm + window step.  Shapes with one
+    and with several row groups, both matrix-core kernels (up to 32 rows, above), with and without a
+    residual; bit for bit."""
+    from dejavu_amd import ops
+
+    g = torch.Generator().manual_seed(B * 1000 + M)
+    h = randh(g, B, M).cuda()
+    Wt = randh(g, Z, N, std=0.05).cuda()
+    bias = randh(g, N, std=0.1).cuda()
+    idx = torch.sort(torch.randperm(Z, generator=g)[:M]).values.cuda()
+    res = randh(g, B, 1, N).cuda()
+    gamma, beta = (1 + 0.1 * torch.randn(N, generator=g)).half().cuda(), randh(g, N, std=0.1).cuda()
+    H, nnz, counter = 8, 3, 4
+    heads = torch.sort(torch.randperm(H, generator=g)[:nnz]).values.int().cuda()
+    print(f"case fc2 with a deferred reduction B={B} M={M} N={N}", flush=True)
+    want = ops.gather_transposed_gemv(h, Wt, idx, bias)
+    pending = ops.gather_transposed_gemv(h, Wt, idx, bias, defer_reduce=True)
+    assert isinstance(pending, ops.PendingRows) and tuple(pending.shape) == (B, 1, N)
+    for residual in (res, None):
+        want_n, want_r = ops.add_layer_norm(want.unsqueeze(1), residual, gamma, beta, 1e-5)
+        got_n, got_r = ops.add_layer_norm(pending, residual, gamma, beta, 1e-5)
+        torch.cuda.synchronize()
+        assert torch.equal(got_r, want_r), "residual stream differs"
+        assert torch.equal(got_n, want_n), "normalised rows differ"
+        state = [{"x_cache": torch.zeros(16, B * N, dtype=torch.float16, device="cuda"),
+                  "tracker": torch.arange(16, dtype=torch.int32).repeat(H, 1).cuda(),
+                  "slots": torch.full((nnz, counter + 1), -7, dtype=torch.int32, device="cuda")} for _ in range(2)]
+        outs = [ops.add_layer_norm_window(hid, residual, gamma, beta, 1e-5, st["x_cache"][counter], st["tracker"],
+                                          heads, counter, False, st["slots"])
+                for hid, st in zip((pending, want.unsqueeze(1)), state)]
+        torch.cuda.synchronize()
+        assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+        for key in ("x_cache", "tracker", "slots"):
+            assert torch.equal(state[0][key], state[1][key]), key
+    assert torch.equal(pending.materialize(), want.unsqueeze(1))
+    # once reduced, the finished rows are what the consumers read
+    got_n, got_r = ops.add_layer_norm(pending, res, gamma, beta, 1e-5)
+    want_n, want_r = ops.add_layer_norm(want.unsqueeze(1), res, gamma, beta, 1e-5)
+    torch.cuda.synchronize()
+    assert torch.equal(got_n, want_n) and torch.equal(got_r, want_r)
+
+
+def test_two_chained_blocks_same_bits_with_fc2_reduction_deferred():
+    """18 decode steps of a batch through two chained blocks, the first handing its MLP output to the
+    second as pending rows (FOLD_NORM1) or as a tensor: the second block's outputs, the residual
+    stream, the selections and all caches are the same bits."""
+    import copy
+
+    import dejavu_amd.block as blk_mod
+    import dejavu_amd.modules as M
+    from dejavu_amd import ops
+    from dejavu_amd.block import create_sparse_block, init_block_synthetic
+    from dejavu_amd.modules import InferenceParams
+    from dejavu_amd.workloads import pack_k_cache
+
+    B, d, ffn, H, r, K, Hk, S = 9, 1024, 4096, 8, 1000, 512, 3, 64
+    hd = d // H
+    blocks = [create_sparse_block(d, ffn, H, r, K, r, Hk, layer_idx=l) for l in range(2)]
+    for l, b in enumerate(blocks):
+        init_block_synthetic(b, seed=21 + l)
+    g = torch.Generator().manual_seed(211)
+    caches = [(pack_k_cache(torch.randn(B, H, S, hd, generator=g).half()), torch.randn(B, H, S, hd, generator=g).half())
+              for _ in range(2)]
+    assert blk_mod.FOLD_NORM1 is True
+    results = []
+    try:
+        for on in (True, False):
+            blk_mod.FOLD_NORM1 = on
+            pair = copy.deepcopy(blocks)
+            pair[0].defer_mlp_reduce = True
+            ip = InferenceParams(max_sequence_len=S, max_batch_size=B, sequence_len_offset=30)
+            for l in range(2):
+                ip.key_value_memory_dict[l] = (caches[l][0].clone().cuda(), caches[l][1].clone().cuda())
+                pair[l].mixer._set_cache_offset(30, torch.device("cuda"))
+            gg = torch.Generator().manual_seed(212)
+            outs = []
+            for step in range(18):
+                hs = torch.randn(B, 1, d, generator=gg).half().cuda()
+                res = torch.randn(B, 1, d, generator=gg).half().cuda()
+                head_idx = torch.sort(torch.randperm(H, generator=gg)[:Hk]).values.int().cuda()
+                logit = (torch.randn(B, ffn, generator=gg) * 4).half().cuda()
+                print(f"case two chained blocks, FOLD_NORM1={on}, step {step}", flush=True)
+                with torch.no_grad():
+                    mid = pair[0](hs, res, mixer_kwargs={"inference_params": ip}, head_idx=head_idx, mlp_sp_logit=logit)
+                    assert isinstance(mid[0], ops.PendingRows) == on
+                    out = pair[1](mid[0], mid[1], mixer_kwargs={"inference_params": ip}, head_idx=mid[3],
+                                  mlp_sp_logit=mid[2])
+                M.join_side_stream()
+                torch.cuda.synchronize()
+                outs.append([t.clone() for t in out] + [mid[1].clone(), mid[2].clone(), mid[3].clone()])
+                ip.sequence_len_offset += 1
+            results.append((outs, [ip.key_value_memory_dict[l] for l in range(2)]))
+    finally:
+        blk_mod.FOLD_NORM1 = True
+    for step, (oa, ob) in enumerate(zip(results[0][0], results[1][0])):
+        for xa, xb in zip(oa, ob):
+            assert torch.equal(xa, xb), f"step {step} differs"
+    for la, lb in zip(results[0][1], results[1][1]):
+        for ca, cb in zip(la, lb):
+            assert torch.equal(ca, cb)

@@ -286,3 +286,48 @@ def test_opt13b_shaped_model_at_full_size_graphs_equal_eager_and_selections_are_
         assert torch.equal(g.sequences, eager.sequences), attempt
         assert torch.equal(g.scores, eager.scores), attempt
     assert "window" in model._decoding_cache.graphs
+
+
+def test_batched_model_steps_same_logits_with_fc2_reduction_inside_the_next_layer_norm():
+    """Six sequences through the whole model (prompt, then 20 decode steps over a back-fill window
+    boundary): every block hands its MLP output to the next add + LayerNorm (the next block's, or
+    ln_f) as pending rows.  Logits bit for bit those of the model whose blocks reduce fc2 themselves."""
+    import dejavu_amd.block as blk_mod
+    import dejavu_amd.modules as dv_modules
+    from dejavu_amd.modules import InferenceParams
+
+    L, d, H, ffn, r, V, P = 3, 256, 4, 2048, 64, 512, 96
+    model, _ = build(L, d, H, ffn, r, V, P, 512, (2, 3), seed=31)
+    B, T = 6, 7
+    g = torch.Generator().manual_seed(5)
+    prompt = torch.randint(0, V, (B, T), generator=g).cuda()
+    assert blk_mod.FOLD_NORM1 is True
+    assert all(layer.defer_mlp_reduce for layer in model.transformer.layers if hasattr(layer, "defer_mlp_reduce"))
+    runs = []
+    try:
+        for on in (True, False):
+            blk_mod.FOLD_NORM1 = on
+            for mixer in model._sparse_mixers():
+                mixer.reset_window() if hasattr(mixer, "reset_window") else None
+            ip = InferenceParams(max_sequence_len=64, max_batch_size=B)
+            print(f"case batched model, FOLD_NORM1={on}: prompt", flush=True)
+            with torch.no_grad():
+                logits = model(prompt, inference_params=ip, last_token_only=True).logits[:, -1]
+            ip.sequence_len_offset = T
+            steps = [logits.clone()]
+            for s in range(20):
+                token = logits.argmax(-1, keepdim=True)
+                pos = torch.full((B, 1), T + s, dtype=torch.long, device="cuda")
+                print(f"case batched model, FOLD_NORM1={on}: step {s}", flush=True)
+                with torch.no_grad():
+                    logits = model(token, position_ids=pos, inference_params=ip).logits[:, -1]
+                dv_modules.join_side_stream()
+                torch.cuda.synchronize()
+                steps.append(logits.clone())
+                ip.sequence_len_offset += 1
+            runs.append(steps)
+    finally:
+        blk_mod.FOLD_NORM1 = True
+    for s, (a, b) in enumerate(zip(*runs)):
+        assert torch.isfinite(a).all()
+        assert torch.equal(a, b), f"step {s} differs"
