@@ -160,6 +160,7 @@ struct LnRowFromPartials {
   int64_t total;  // rows * d
   __device__ __forceinline__ half8_t operator()(int i, int64_t row) const {
     const float* p = partial + row * d + i * 8;
+    const half8_t bv = bias != nullptr ? load8(bias + i * 8) : zero8();  // requested with the first groups
     float a[4][8];
 #pragma unroll
     for (int k = 0; k < 4; ++k)
@@ -184,7 +185,6 @@ struct LnRowFromPartials {
         }
       }
     }
-    const half8_t bv = bias != nullptr ? load8(bias + i * 8) : zero8();
     half8_t y;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {

@@ -498,7 +498,7 @@ def test_layer_norm_with_the_window_step_in_the_same_launch_same_results(B, d, H
 
 
 @pytest.mark.parametrize("B,M,N,Z", [(5, 512, 1024, 4096), (16, 200, 520, 700), (32, 4096, 12288, 49152),
-                                     (33, 96, 256, 300), (9, 24, 1024, 64)])
+                                     (33, 96, 256, 300), (9, 24, 1024, 64), (7, 20, 256, 64)])
 def test_fc2_with_its_reduction_in_the_next_layer_norm_launch_same_bits(B, M, N, Z):
     """gather_transposed_gemv(defer_reduce=True) and its three consumers against the plain op: the
     reduction alone (materialize), add + LayerNorm, add + LayerNorm + window step.  Shapes with one
