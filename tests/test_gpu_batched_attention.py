@@ -601,3 +601,59 @@ def test_two_chained_blocks_same_bits_with_fc2_reduction_deferred():
     for la, lb in zip(results[0][1], results[1][1]):
         for ca, cb in zip(la, lb):
             assert torch.equal(ca, cb)
+
+
+def test_graph_of_two_chained_batched_block_steps_replays_the_eager_result():
+    """Two chained blocks at the first position of a back-fill window (side stream, deferred waits, fc2's
+    reduction inside the second block's LayerNorm 1) captured in one HIP graph: every replay -- with eager work
+    and synchronisations of the program between the replays -- gives the eager step's outputs bit for bit."""
+    import dejavu_amd.modules as M
+    from dejavu_amd import ops
+    from dejavu_amd.block import create_sparse_block, init_block_synthetic
+    from dejavu_amd.modules import InferenceParams
+    from dejavu_amd.workloads import pack_k_cache
+
+    B, d, ffn, H, r, K, Hk, S = 12, 1024, 4096, 8, 1000, 512, 3, 64
+    hd = d // H
+    blocks = [create_sparse_block(d, ffn, H, r, K, r, Hk, layer_idx=l) for l in range(2)]
+    g = torch.Generator().manual_seed(311)
+    ip = InferenceParams(max_sequence_len=S, max_batch_size=B, sequence_len_offset=S - 1)
+    for l, b in enumerate(blocks):
+        init_block_synthetic(b, seed=31 + l)
+        ip.key_value_memory_dict[l] = (pack_k_cache(torch.randn(B, H, S, hd, generator=g).half()).cuda(),
+                                       torch.randn(B, H, S, hd, generator=g).half().cuda())
+        b.mixer._set_cache_offset(S - 1, torch.device("cuda"))
+        b.mixer.hold_window = True  # every step is the first of a window that sits at the end of the cache
+    blocks[0].defer_mlp_reduce = True
+    hs = torch.randn(B, 1, d, generator=g).half().cuda()
+    res = torch.randn(B, 1, d, generator=g).half().cuda()
+    head_idx = torch.sort(torch.randperm(H, generator=g)[:Hk]).values.int().cuda()
+    logit = (torch.randn(B, ffn, generator=g) * 4).half().cuda()
+
+    def step():
+        for b in blocks:
+            b.mixer.counter = 0
+        with torch.no_grad():
+            mid = blocks[0](hs, res, mixer_kwargs={"inference_params": ip}, head_idx=head_idx, mlp_sp_logit=logit)
+            assert isinstance(mid[0], ops.PendingRows)
+            out = blocks[1](mid[0], mid[1], mixer_kwargs={"inference_params": ip}, head_idx=mid[3], mlp_sp_logit=mid[2])
+        M.join_side_stream()
+        return out
+
+    print("case chained batched blocks, eager", flush=True)
+    want = [t.clone() for t in step()]
+    step()  # every scratch buffer exists before the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    print("case chained batched blocks, capture", flush=True)
+    with torch.cuda.graph(graph):
+        got = step()
+    for replay in range(4):
+        print(f"case chained batched blocks, replay {replay}", flush=True)
+        for t in got:
+            t.zero_()
+        (hs.float() @ torch.ones(d, 8, device="cuda")).sum().item()  # eager work of the program in between
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b in zip(got, want):
+            assert torch.equal(a, b), f"replay {replay} differs"
