@@ -262,10 +262,12 @@ int gather_cols(const half_t* x, int64_t ldx, int x_expanded, const half_t* W, i
 }
 
 // Largest batch the vector-ALU kernels take; above it the MFMA kernels are faster (measured at
-// the OPT-175B shape: fc1 19 us on MFMA against 24 / 39 us at batch 3 / 4, fc2 22-24 us on the
-// vector ALUs against 30 us on MFMA up to batch 4).
+// the OPT-175B shape: fc1 19 us on MFMA against 24 / 39 us at batch 3 / 4; fc2 alone 22-24 us on the
+// vector ALUs against 25 us on MFMA up to batch 4, but the matrix-core path writes two row groups of
+// partial sums instead of sixteen and its reductions ride in the LayerNorm launches that follow: a whole
+// batched layer step takes 170.3 against 177.5 us at batch 3 and 177.7 against 187.5 us at batch 4).
 constexpr int kRowsVecMaxBatch = 2;
-constexpr int kColsVecMaxBatch = 4;
+constexpr int kColsVecMaxBatch = 2;
 
 // ---- batched gathered GEMMs on the matrix cores (5 <= B <= 64) -------------------
 #ifndef DV_ROWS_XLDS
@@ -1639,7 +1641,7 @@ int dv_out_proj_sparse_f16(const void* x, const void* W, const void* bias, const
 
 size_t dv_out_proj_sparse_t_workspace_bytes(int B, int N, int nnz, int hd) {
   if (B < 1 || N < 1 || nnz < 0 || hd < 1) return 0;
-  return B > 4 ? cols_mfma_workspace_bytes(B, N, nnz * hd) : cols_workspace_bytes(B, N, nnz * hd);
+  return B > kColsVecMaxBatch ? cols_mfma_workspace_bytes(B, N, nnz * hd) : cols_workspace_bytes(B, N, nnz * hd);
 }
 
 int dv_out_proj_sparse_t_f16(const void* x, const void* Wt, int64_t ldw, const void* bias,
@@ -1650,12 +1652,12 @@ int dv_out_proj_sparse_t_f16(const void* x, const void* Wt, int64_t ldw, const v
   if (B > 64) return DV_ERR_UNSUPPORTED;
   if (N % 8 || ldw % 8 || ldw < N || !aligned16(Wt) || !aligned16(y) || (workspace && !aligned16(workspace)))
     return DV_ERR_ALIGNMENT;
-  if (B > 4)
+  if (B > kColsVecMaxBatch)
     return gather_cols_mfma(reinterpret_cast<const half_t*>(x), (int64_t)H * hd, 1,
                             reinterpret_cast<const half_t*>(Wt), ldw, reinterpret_cast<const half_t*>(bias),
                             head_idx, 4, hd, B, N, H * hd, nnz * hd, reinterpret_cast<half_t*>(y), workspace,
                             workspace_bytes, reinterpret_cast<hipStream_t>(stream));
-  // up to four rows: partial sums added in fixed point, the bits of dv_attention_out_proj_f16 and of
+  // one and two rows: partial sums added in fixed point, the bits of dv_attention_out_proj_f16 and of
   // the fused layer step
   return gather_cols(reinterpret_cast<const half_t*>(x), (int64_t)H * hd, 1,
                      reinterpret_cast<const half_t*>(Wt), ldw, reinterpret_cast<const half_t*>(bias),
@@ -1669,7 +1671,7 @@ int dv_out_proj_sparse_t_ln_f16(const void* x, const void* Wt, int64_t ldw, cons
                                 size_t workspace_bytes, void* stream) {
   if (!x || !Wt || !normed || !gamma || !beta || nnz < 1 || B < 1 || H <= 0 || hd <= 0 || N <= 0 || !head_idx)
     return DV_ERR_INVALID_ARG;
-  if (B <= 4 || B > 64 || N > 256 * 8 * 16) return DV_ERR_UNSUPPORTED;  // the matrix-core path of dv_out_proj_sparse_t_f16
+  if (B <= kColsVecMaxBatch || B > 64 || N > 256 * 8 * 16) return DV_ERR_UNSUPPORTED;  // the matrix-core path of dv_out_proj_sparse_t_f16
   if (N % 8 || ldw % 8 || ldw < N || !aligned16(Wt) || !aligned16(normed) || !aligned16(gamma) || !aligned16(beta) ||
       (residual && !aligned16(residual)) || (residual_out && !aligned16(residual_out)) ||
       (workspace && !aligned16(workspace)))
@@ -1688,7 +1690,7 @@ int dv_out_proj_sparse_t_ln_f16(const void* x, const void* Wt, int64_t ldw, cons
 }
 
 size_t dv_out_proj_sparse_t_ln_workspace_bytes(int B, int nnz, int hd, int N) {
-  if (B <= 4 || B > 64 || nnz <= 0 || hd <= 0 || N <= 0) return 0;
+  if (B <= kColsVecMaxBatch || B > 64 || nnz <= 0 || hd <= 0 || N <= 0) return 0;
   return ((cols_mfma_workspace_bytes(B, N, nnz * hd) + 255) & ~(size_t)255) + (size_t)B * N * sizeof(half_t);
 }
 

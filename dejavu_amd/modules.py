@@ -216,7 +216,7 @@ class ParallelFusedMLPDejavu(nn.Module):
         """x, residual: (B, 1, d) at decode (or (B, s, d) for the prompt).
         idx: (K,) active neurons or None for the dense MLP.
         defer_reduce: the caller's next step is an ``ops.add_layer_norm`` / ``add_layer_norm_window`` of
-        ``out``; for 5..64 sequences ``out`` is then ``ops.PendingRows`` (the split reduction of fc2 runs
+        ``out``; for 3..64 sequences ``out`` is then ``ops.PendingRows`` (the split reduction of fc2 runs
         inside that LayerNorm launch).
         Returns (out, mlp_logit); mlp_logit, the predictor output for the next
         layer's MLP, only when decoding one token.  defer_join: when the predictor runs on the side

@@ -275,7 +275,7 @@ def dense_decode_linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[to
     return y.view(*lead, weight.shape[0])
 
 
-DEFERRED_REDUCE_MIN_ROWS = 5  # the matrix-core path of gather_transposed_gemv
+DEFERRED_REDUCE_MIN_ROWS = 3  # the matrix-core path of gather_transposed_gemv
 
 
 class PendingRows:
@@ -607,13 +607,13 @@ def out_proj_sparse_t(x: torch.Tensor, weight_t: torch.Tensor, head_idx: torch.T
     return output
 
 
-OUT_PROJ_LN_MIN_ROWS = 5  # the matrix-core path of out_proj_sparse_t
+OUT_PROJ_LN_MIN_ROWS = 3  # the matrix-core path of out_proj_sparse_t
 
 
 def out_proj_sparse_t_add_layer_norm(x: torch.Tensor, weight_t: torch.Tensor, head_idx: torch.Tensor,
                                      bias: Optional[torch.Tensor], residual: Optional[torch.Tensor],
                                      ln_weight: torch.Tensor, ln_bias: torch.Tensor, eps: float):
-    """``add_layer_norm(out_proj_sparse_t(x, ...), residual, ...)`` for 5..64 rows with the split
+    """``add_layer_norm(out_proj_sparse_t(x, ...), residual, ...)`` for 3..64 rows with the split
     reduction of the projection and the LayerNorm in one launch.  Returns (normed, residual_out), both
     (batch, hidden_dim); same bits as the two ops."""
     _require_device(x, weight_t, head_idx, bias, residual, ln_weight, ln_bias)

@@ -338,7 +338,8 @@ DV_API int dv_decode_attention_f16(const void* q, int64_t ldq, const void* k_cac
  * dv_decode_attention_f16 followed by dv_out_proj_sparse_t_f16 without
  * materialising the context: the out_proj kernel merges the attention split
  * partials while it loads its activations.  Same arithmetic (the merged
- * context is rounded to fp16 as a stored one would be).
+ * context is rounded to fp16 as a stored one would be; the same bits for one and two rows, where
+ * dv_out_proj_sparse_t_f16 adds its partial sums in fixed point too).
  *   head_idx (nheads,) int32, required; Wt (H*hd, N) row stride ldw; y (B, N);
  *   B <= 4; workspace: dv_attention_out_proj_workspace_bytes(...) bytes, no
  *   initialisation needed.
@@ -392,7 +393,7 @@ DV_API int dv_out_proj_sparse_t_f16(const void* x, const void* Wt, int64_t ldw, 
                                     void* stream);
 
 /*
- * dv_out_proj_sparse_t_f16 for 5..64 rows followed by the block's residual add + LayerNorm 2
+ * dv_out_proj_sparse_t_f16 for 3..64 rows followed by the block's residual add + LayerNorm 2
  * (dv_add_layer_norm_f16 with h = the projection's output) with the split reduction and the LayerNorm
  * in ONE launch: normed = LayerNorm(fp16(y + residual)) * gamma + beta, residual_out = fp16(y + residual);
  * y itself is not returned.  Same bits as the two calls (attention_proj_sparse.py:194-305 +
@@ -462,7 +463,7 @@ DV_API int dv_add_layer_norm_window_f16(const void* h, const void* residual, con
 
 /*
  * The fc2 of one block and LayerNorm 1 of the next without a reduction launch of their own, for
- * 5..64 rows (the matrix-core path of dv_gather_transposed_gemv_f16):
+ * 3..64 rows (the matrix-core path of dv_gather_transposed_gemv_f16):
  *  - dv_gather_transposed_gemv_partial_f16 is dv_gather_transposed_gemv_f16 (gather_gemv.py:572-644)
  *    without its last step: the fp32 sums of the row groups stay in `partial` (layout private to the
  *    library), their number goes to *groups (host memory).  *groups == 1: there was nothing to split,

@@ -75,21 +75,21 @@ def test_host_side_argument_checks_return_codes():
     assert L.dv_add_layer_norm_window_f16(A, None, A, A, 1e-5, 2, 124, A, A, A, A, A, 1, 4, 0, 0, A, None) == -3  # d % 8
     assert L.dv_add_layer_norm_window_f16(A, None, A, A, 1e-5, 2, 128, A, A, A + 2, A, A, 1, 4, 0, 0, A, None) == -3
     #   (x, Wt, ldw, bias, head_idx, nnz, B, H, hd, N, residual, gamma, beta, eps, normed, residual_out, ws, bytes, stream)
-    assert L.dv_out_proj_sparse_t_ln_f16(A, A, 128, None, A, 1, 4, 1, 128, 128, A, A, A, 1e-5, A, A, A, 1 << 20, None) == -2
+    assert L.dv_out_proj_sparse_t_ln_f16(A, A, 128, None, A, 1, 2, 1, 128, 128, A, A, A, 1e-5, A, A, A, 1 << 20, None) == -2
     assert L.dv_out_proj_sparse_t_ln_f16(A, A, 128, None, A, 1, 8, 1, 128, 128, A, A, A, 1e-5, A + 2, A, A, 1 << 20, None) == -3
     assert L.dv_out_proj_sparse_t_ln_f16(A, A, 128, None, A, 1, 8, 1, 128, 128, A, A, A, 1e-5, A, A, A, 16, None) == -4
-    assert L.dv_out_proj_sparse_t_ln_workspace_bytes(4, 1, 128, 128) == 0
+    assert L.dv_out_proj_sparse_t_ln_workspace_bytes(2, 1, 128, 128) == 0
     assert L.dv_out_proj_sparse_t_ln_workspace_bytes(8, 32, 128, 12288) >= 8 * 12288 * 2
     # fc2 without its reduction launch and the consumers of its partial sums
     import ctypes
 
     groups = ctypes.c_int(0)
     #   (x, W, ldw, bias, idx, idx_bytes, B, N, Z, M, y, partial, partial_bytes, groups, stream)
-    assert L.dv_gather_transposed_gemv_partial_f16(A, A, 128, None, A, 8, 4, 128, 64, 8, A, A, 1 << 20, ctypes.byref(groups), None) == -2
+    assert L.dv_gather_transposed_gemv_partial_f16(A, A, 128, None, A, 8, 2, 128, 64, 8, A, A, 1 << 20, ctypes.byref(groups), None) == -2
     assert L.dv_gather_transposed_gemv_partial_f16(A, A, 128, None, A, 8, 8, 128, 64, 8, A, A, 1 << 20, None, None) == -1
     assert L.dv_gather_transposed_gemv_partial_f16(A, A, 128, None, A, 8, 8, 128, 64, 8, A + 2, A, 1 << 20, ctypes.byref(groups), None) == -3
     assert L.dv_gather_transposed_gemv_partial_f16(A, A, 128, None, A, 8, 8, 128, 64, 8, A, A, 16, ctypes.byref(groups), None) == -4
-    assert L.dv_gather_transposed_gemv_partial_workspace_bytes(4, 128, 8) == 0
+    assert L.dv_gather_transposed_gemv_partial_workspace_bytes(2, 128, 8) == 0
     assert L.dv_gather_transposed_gemv_partial_workspace_bytes(8, 12288, 4096) >= 8 * 12288 * 4
     #   (partial, groups, bias, rows, N, y, stream)
     assert L.dv_reduce_rows_f16(None, 2, None, 8, 128, A, None) == -1

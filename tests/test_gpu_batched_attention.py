@@ -438,11 +438,12 @@ def test_batched_block_step_same_bits_with_and_without_folded_launches(module_na
         assert torch.equal(ca, cb)
 
 
-@pytest.mark.parametrize("B,H,hd,d,nnz", [(5, 8, 128, 1024, 3), (16, 6, 64, 520, 1), (32, 12, 128, 1536, 12),
+@pytest.mark.parametrize("B,H,hd,d,nnz", [(3, 8, 128, 1024, 3), (4, 96, 128, 12288, 32), (5, 8, 128, 1024, 3),
+                                          (16, 6, 64, 520, 1), (32, 12, 128, 1536, 12),
                                           (33, 4, 64, 256, 2), (9, 96, 128, 12288, 32)])
 def test_out_proj_with_layer_norm_in_the_reduction_launch_same_bits(B, H, hd, d, nnz):
     """dv_out_proj_sparse_t_ln_f16 (split reduction + residual add + LayerNorm in one launch) against
-    out_proj_sparse_t followed by add_layer_norm: both outputs bit for bit.  Shapes with one and with
+    out_proj_sparse_t followed by add_layer_norm: both outputs bit for bit.  Three rows and more; shapes with one and with
     several row groups, both matrix-core kernels (up to 32 rows, above), with and without a residual."""
     from dejavu_amd import ops
 
@@ -497,7 +498,8 @@ def test_layer_norm_with_the_window_step_in_the_same_launch_same_results(B, d, H
         assert torch.equal(idx_a, idx_b)
 
 
-@pytest.mark.parametrize("B,M,N,Z", [(5, 512, 1024, 4096), (16, 200, 520, 700), (32, 4096, 12288, 49152),
+@pytest.mark.parametrize("B,M,N,Z", [(3, 512, 1024, 4096), (4, 4096, 12288, 49152), (5, 512, 1024, 4096),
+                                     (16, 200, 520, 700), (32, 4096, 12288, 49152),
                                      (33, 96, 256, 300), (9, 24, 1024, 64), (7, 20, 256, 64)])
 def test_fc2_with_its_reduction_in_the_next_layer_norm_launch_same_bits(B, M, N, Z):
     """gather_transposed_gemv(defer_reduce=True) and its three consumers against the plain op: the
