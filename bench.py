@@ -602,8 +602,7 @@ def mlp_bench(args):
                              "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
             out["fc1_fc2"]["TFLOP/s"] = round(2.0 * B * (weight_bytes / 2) / out["fc1_fc2"]["us"] / 1e6, 2)
             out["tokens_per_s"] = round(B / (out["block"]["us"] * 1e-6), 1)
-            out["path"] = ("vector ALU gather-GEMV" if B <= 2 else
-                           "fc1 on MFMA tiles, fc2 vector ALU" if B <= 4 else "MFMA tiles (fc1 LDS-staged, fc2 register-transposed)")
+            out["path"] = ("vector ALU gather-GEMV" if B <= 2 else "MFMA tiles (fc1 LDS-staged, fc2 register-transposed)")
             results[str(B)] = out
     # roofline: the fc1 gather alone at the largest batch of the sweep; CPU baseline: the same block at batch 1
     Bmax = max(args.batches)
