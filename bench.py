@@ -776,7 +776,7 @@ def main():
     if args.traffic_from:
         return write_traffic(*args.traffic_from)
 
-    # The headline run also reports the other BASELINE workloads (batched layer, end-to-end decode).  Every
+    # The headline run also reports the other workloads of the reference (batched layer, end-to-end decode).  Every
     # leg, the headline one first, is then a child process of this script and this process never touches
     # the GPU (a child must not be forked from a process that holds the device, and the headline figure is
     # taken before the other legs have heated the part: measured after them it read 3 % higher).
