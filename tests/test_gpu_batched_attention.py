@@ -240,8 +240,8 @@ def _block_params(block, H, hd, d, K, Hk):
                 mlp_K=K, att_K=Hk)
 
 
-@pytest.mark.parametrize("cfg,B", [("opt-125m", 3), ("opt-125m", 16), ("opt-66b", 16), ("opt-175b", 8),
-                                   ("opt-175b", 32)])
+@pytest.mark.parametrize("cfg,B", [("opt-125m", 3), ("opt-125m", 16), ("opt-66b", 16), ("opt-175b", 4),
+                                   ("opt-175b", 8), ("opt-175b", 32)])
 def test_batched_sparse_block_decode_step_matches_oracle(cfg, B):
     """One decode step of a whole block for B sequences (OPT-66B shape at batch 16, OPT-175B shape at
     batch 8 and 32, full-size weights and caches) against block_decode_step_batched.  Up to 8 rows
